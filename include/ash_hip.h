@@ -1,0 +1,193 @@
+/*
+ * ash_hip.h -- C ABI of libash_hip.so, the MI355X (gfx950) implementation of
+ * torch-ash's two data-parallel hot paths:
+ *
+ *   1. the collision-free int32[dim] -> int32 index hash map
+ *      (reference: the pybind class `HashMap`, ash/src/pybind.cpp:9-23,
+ *       ash/src/hashmap.h:18-61, kernels in ash/src/hashmap_gpu.cuh);
+ *   2. the sparse-dense grid trilinear query, forward / backward /
+ *      double-backward (reference: ash/src/pybind.cpp:25-29, ash/src/grid.h:6-82,
+ *      kernels in ash/src/grid.cu:68-451).
+ *
+ * Conventions
+ *   - plain C, no torch types: device pointers are raw `void*` / typed pointers
+ *     obtained from `Tensor.data_ptr()`; `stream` is a `hipStream_t` passed as
+ *     `void*` (NULL = the null stream);
+ *   - every function returns 0 on success, non-zero on failure; the message of
+ *     the last failure on the calling thread is `ash_last_error()`;
+ *   - nothing here allocates or frees device memory: table storage, outputs and
+ *     temporaries are caller-owned buffers (the Python layer hands in torch
+ *     tensors, so all device memory stays inside torch's caching allocator);
+ *   - launches are asynchronous on `stream`; only `ash_map_status` /
+ *     `ash_map_size` (which return host values) synchronise that stream;
+ *   - a map handle is not thread-safe; operations on one handle must be issued
+ *     in order on one stream (as the reference issues them on the null stream).
+ */
+#ifndef ASH_HIP_H_
+#define ASH_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ash_map ash_map_t;
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* ash_last_error(void);
+
+/* ABI version, bumped on incompatible changes. */
+int ash_abi_version(void);
+
+/* ------------------------------------------------------------------ hash map */
+
+/* Storage needed for a table of `capacity` entries with `key_dim` int32 key
+ * components (1..4, as ash/src/dispatch.h:50-68).
+ *   table_bytes   : mandatory workspace (bucket array + device counters)
+ *   general_bytes : optional second region, only needed once a key arrives
+ *                   whose components do not fit the packed 64-bit code
+ *                   (see ash_map_attach_general). */
+int ash_map_workspace_bytes(int key_dim, int64_t capacity,
+                            int64_t* table_bytes, int64_t* general_bytes);
+
+/* Replaces `HashMap(key_dim, capacity, heap, device)` (ash/src/pybind.cpp:10,
+ * ash/src/hashmap_impl.h:11-24).  `heap` is the caller-owned int32[capacity]
+ * free list (the `_heap` state-dict buffer, ash/core.py:72-74); the map aliases
+ * and mutates it exactly like the reference does.  `table_ws` is a 256-byte
+ * aligned device buffer of at least `table_bytes` bytes.  The table is cleared
+ * (heap := 0..capacity-1, size := 0) before the call returns control of the
+ * stream. */
+int ash_map_create(int key_dim, int64_t capacity, int32_t* heap,
+                   void* table_ws, int64_t table_bytes, int device,
+                   void* stream, ash_map_t** out);
+
+/* Hands the map its second region (device buffer of >= general_bytes bytes).
+ * Idempotent per handle: a second attach is an error. */
+int ash_map_attach_general(ash_map_t* map, void* general_ws,
+                           int64_t general_bytes, void* stream);
+
+/* Releases the host-side handle only (device buffers are caller-owned). */
+int ash_map_destroy(ash_map_t* map);
+
+/* Replaces `HashMap::find` (ash/src/hashmap_gpu.cuh:163-208).
+ * keys int32[n,key_dim] contiguous; indices int64[n]; masks uint8/bool[n].
+ * Every output element is written: masks[i] = found, indices[i] = found ?
+ * index : 0. */
+int ash_map_find(ash_map_t* map, const int32_t* keys, int64_t n,
+                 int64_t* indices, uint8_t* masks, void* stream);
+
+/* Replaces `HashMap::insert_keys` (ash/src/hashmap_gpu.cuh:211-247).  New keys
+ * pop one index each from the heap; duplicates (in the table or within the
+ * batch) are ignored.  Keys beyond `capacity` are dropped and counted
+ * (ash_map_status), where the reference reads past the heap. */
+int ash_map_insert_keys(ash_map_t* map, const int32_t* keys, int64_t n,
+                        void* stream);
+
+/* 1 when ash_map_insert needs the `assigned` temporary for these rows. */
+int ash_map_insert_needs_scratch(int n_values, const int64_t* row_bytes);
+
+/* Replaces `HashMap::insert(keys, values, external_values)`
+ * (ash/src/hashmap_gpu.cuh:249-313).  For value tensor j, the row
+ * src[j] + i*row_bytes[j] of every newly inserted key i is copied to
+ * dst[j] + index*row_bytes[j].  `assigned` is an int32[n] device temporary,
+ * required (non-NULL) only when ash_map_insert_needs_scratch(...) is 1. */
+int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n,
+                   int n_values, const void* const* src, void* const* dst,
+                   const int64_t* row_bytes, int32_t* assigned, void* stream);
+
+/* Replaces `HashMap::erase` (ash/src/hashmap_gpu.cuh:316-351): found keys are
+ * removed and their indices pushed back on the heap; duplicates inside the
+ * batch erase once. */
+int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n, void* stream);
+
+/* Replaces `HashMap::clear` (ash/src/hashmap_gpu.cuh:354-358,
+ * ash/src/hashmap_impl.h:26-33). */
+int ash_map_clear(ash_map_t* map, void* stream);
+
+/* Host read-back of the device counters; synchronises `stream`.
+ *   out[0] size (= heap counter, ash/src/hashmap_gpu.cuh:157)
+ *   out[1] keys dropped because the map was full (since the last clear)
+ *   out[2] tombstoned slots
+ *   out[3] keys that are waiting for ash_map_attach_general (re-issue the
+ *          insert after attaching; the counter is reset by the attach)
+ *   out[4] duplicate (key,index) pairs seen by ash_map_load */
+int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
+
+/* Replaces `HashMap::size` (ash/src/hashmap_gpu.cuh:157); synchronises. */
+int ash_map_size(ash_map_t* map, int64_t* size, void* stream);
+
+/* Replaces `HashMap::items` (ash/src/hashmap_gpu.cuh:360-405): writes the
+ * live (key, index) pairs in unspecified order.  keys_out int32[n_expected,
+ * key_dim], indices_out int64[n_expected]; n_expected must be the current
+ * size (rows beyond it are never written). */
+int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
+                  int64_t n_expected, void* stream);
+
+/* Replaces `HashMap::load_states` (ash/src/hashmap_gpu.cuh:407-450): the map
+ * is emptied, then (keys[i] -> indices[i]) are stored, size := n and the heap
+ * := heap_src (skipped when heap_src is NULL or already the map's heap). */
+int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
+                 int64_t n, const int32_t* heap_src, void* stream);
+
+/* Generic row scatter used by the wide-row path of ash_map_insert, exported
+ * because the Python layer reuses it: dst[assigned[i]] = src[i] for
+ * assigned[i] >= 0. */
+int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
+                     int64_t n, int64_t row_bytes, void* stream);
+
+/* -------------------------------------------------------- trilinear queries */
+
+enum { ASH_INTERP_LINEAR = 0, ASH_INTERP_SMOOTH_STEP = 1 };
+enum { ASH_F32 = 0, ASH_F64 = 1 };
+
+/* Operands shared by the three query entry points (ash/src/grid.h:6-82):
+ *   embeddings   scalar[B, M, E]   (M = cells per block, E <= 16)
+ *   offsets      float32[N, 3]     (always fp32, ash/src/grid.cu:71)
+ *   grid_indices int64[N], cell_indices int64[N], masks uint8/bool[N]
+ *   lut_grid_nb2grid_idx int64[B, 8]  (-1 = missing neighbour block)
+ *   lut_cell_nb2cell_idx int64[M, 8], lut_cell_nb2grid_nb int64[M, 8] */
+typedef struct ash_query_args {
+    const void* embeddings;
+    const float* offsets;
+    const int64_t* grid_indices;
+    const int64_t* cell_indices;
+    const uint8_t* masks;
+    const int64_t* lut_grid_nb2grid_idx;
+    const int64_t* lut_cell_nb2cell_idx;
+    const int64_t* lut_cell_nb2grid_nb;
+    int64_t num_queries;    /* N */
+    int64_t num_embeddings; /* B */
+    int64_t cells_per_grid; /* M */
+    int64_t embedding_dim;  /* E */
+    int32_t interpolation;  /* ASH_INTERP_* */
+    int32_t dtype;          /* ASH_F32 / ASH_F64: dtype of embeddings & grads */
+} ash_query_args;
+
+/* Replaces `query_forward` (ash/src/grid.cu:68-175).  output scalar[N, E];
+ * every row is written (zeros for masked-out queries and for queries with a
+ * missing neighbour block, ash/src/grid.cu:84-86,109-111). */
+int ash_query_forward(const ash_query_args* a, void* output, void* stream);
+
+/* Replaces `query_backward_forward` (ash/src/grid.cu:177-307).
+ * z scalar[N, E]; grad_embeddings scalar[B, M, E] (zero-filled here, then
+ * accumulated); grad_offsets scalar[N, 3] (every row written). */
+int ash_query_backward_forward(const ash_query_args* a, const void* z,
+                               void* grad_embeddings, void* grad_offsets,
+                               void* stream);
+
+/* Replaces `query_backward_backward` (ash/src/grid.cu:309-451).
+ * grad_grad_offsets scalar[N,3], z scalar[N,E]; outputs grad_z scalar[N,E]
+ * (every row written) and grad_embeddings scalar[B,M,E] (zero-filled here).
+ * As in the reference the incoming grad_grad_embeddings is not used and the
+ * offsets gradient is identically zero (ash/src/grid.cu:417-426); the caller
+ * produces that zero tensor itself. */
+int ash_query_backward_backward(const ash_query_args* a,
+                                const void* grad_grad_offsets, const void* z,
+                                void* grad_z, void* grad_embeddings,
+                                void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASH_HIP_H_ */

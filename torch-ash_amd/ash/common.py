@@ -1,0 +1,610 @@
+"""Loader and thin Python face of libash_hip.so.
+
+The reference binds its native code with pybind11 (`import __ash`,
+ash/common.py:4-15 and ash/src/pybind.cpp:8-38).  Here the native side is a
+plain C-ABI shared library (include/ash_hip.h) loaded with ctypes; this module
+rebuilds the exact surface the rest of the package expects from the extension
+module: a `HashMap` class and the three `query_*` functions.
+
+There is no CPU or PyTorch fallback: if the library is missing, or a tensor is
+not on a HIP device, the calls raise.
+"""
+import ctypes
+import os
+import warnings
+from typing import Dict, Optional, Tuple
+
+import torch
+
+_LIB_NAME = "libash_hip.so"
+_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+
+_I64 = ctypes.c_int64
+_PTR = ctypes.c_void_p
+
+
+class DotDict(dict):
+    """dict whose items are also attributes (ash/common.py:19-22)."""
+
+    __getattr__ = dict.__getitem__
+    __setattr__ = dict.__setitem__
+    __delattr__ = dict.__delitem__
+
+
+class _QueryArgs(ctypes.Structure):
+    _fields_ = [
+        ("embeddings", _PTR),
+        ("offsets", _PTR),
+        ("grid_indices", _PTR),
+        ("cell_indices", _PTR),
+        ("masks", _PTR),
+        ("lut_grid_nb2grid_idx", _PTR),
+        ("lut_cell_nb2cell_idx", _PTR),
+        ("lut_cell_nb2grid_nb", _PTR),
+        ("num_queries", _I64),
+        ("num_embeddings", _I64),
+        ("cells_per_grid", _I64),
+        ("embedding_dim", _I64),
+        ("interpolation", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
+# name -> (restype, argtypes); mirrors include/ash_hip.h
+_SIGNATURES = {
+    "ash_last_error": (ctypes.c_char_p, []),
+    "ash_abi_version": (ctypes.c_int, []),
+    "ash_map_workspace_bytes": (
+        ctypes.c_int,
+        [ctypes.c_int, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)],
+    ),
+    "ash_map_create": (
+        ctypes.c_int,
+        [ctypes.c_int, _I64, _PTR, _PTR, _I64, ctypes.c_int, _PTR, ctypes.POINTER(_PTR)],
+    ),
+    "ash_map_attach_general": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
+    "ash_map_destroy": (ctypes.c_int, [_PTR]),
+    "ash_map_find": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR, _PTR, _PTR]),
+    "ash_map_insert_keys": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
+    "ash_map_insert_needs_scratch": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_I64)]),
+    "ash_map_insert": (
+        ctypes.c_int,
+        [
+            _PTR,
+            _PTR,
+            _I64,
+            ctypes.c_int,
+            ctypes.POINTER(_PTR),
+            ctypes.POINTER(_PTR),
+            ctypes.POINTER(_I64),
+            _PTR,
+            _PTR,
+        ],
+    ),
+    "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
+    "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
+    "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_map_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_map_items": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
+    "ash_map_load": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR, _PTR]),
+    "ash_scatter_rows": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _I64, _PTR]),
+    "ash_query_forward": (ctypes.c_int, [ctypes.POINTER(_QueryArgs), _PTR, _PTR]),
+    "ash_query_backward_forward": (
+        ctypes.c_int,
+        [ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR],
+    ),
+    "ash_query_backward_backward": (
+        ctypes.c_int,
+        [ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR, _PTR],
+    ),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_INTERPOLATION = {"linear": 0, "smooth_step": 1}
+_DTYPE = {torch.float32: 0, torch.float64: 1}
+
+
+def library_path() -> str:
+    return os.environ.get("ASH_HIP_LIBRARY", os.path.join(_LIB_DIR, _LIB_NAME))
+
+
+def load_library(path: Optional[str] = None) -> ctypes.CDLL:
+    """dlopen the C-ABI library and attach the prototypes."""
+    lib = ctypes.CDLL(path or library_path())
+    for name, (restype, argtypes) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+def _stream_of(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_hip(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what} must live on a HIP device, got {t.device}")
+
+
+class _Backend:
+    """Stands where the reference's `__ash` extension module stands."""
+
+    def __init__(self, lib: ctypes.CDLL):
+        self.lib = lib
+        backend = self
+
+        class HashMap(_HashMap):
+            _backend = backend
+
+        self.HashMap = HashMap
+
+    # -- error plumbing -------------------------------------------------
+    def check(self, status: int) -> None:
+        if status != 0:
+            msg = self.lib.ash_last_error()
+            raise RuntimeError(msg.decode() if msg else "libash_hip call failed")
+
+    # -- trilinear queries (ash/src/pybind.cpp:25-29) ---------------------
+    def _query_args(
+        self,
+        embeddings,
+        offsets,
+        grid_indices,
+        cell_indices,
+        masks,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        interpolation,
+    ):
+        if interpolation not in _INTERPOLATION:
+            raise RuntimeError(f"Unknown interpolation functor: {interpolation}")
+        if embeddings.dtype not in _DTYPE:
+            raise RuntimeError(f"embeddings must be float32 or float64, got {embeddings.dtype}")
+        if embeddings.dim() != 3:
+            raise RuntimeError("embeddings must be (num_embeddings, cells_per_grid, dim)")
+        _require_hip(embeddings, "embeddings")
+        dev = embeddings.device
+        n = grid_indices.shape[0]
+
+        def prep(t, dtype, shape, name):
+            if t.device != dev:
+                raise RuntimeError(f"{name} is on {t.device}, embeddings on {dev}")
+            if t.dtype != dtype:
+                raise RuntimeError(f"{name} must be {dtype}, got {t.dtype}")
+            if tuple(t.shape) != shape and t.numel() != _numel(shape):
+                raise RuntimeError(f"{name} has shape {tuple(t.shape)}, expected {shape}")
+            return t.contiguous()
+
+        b, m, e = embeddings.shape
+        held = [
+            prep(embeddings, embeddings.dtype, (b, m, e), "embeddings"),
+            prep(offsets, torch.float32, (n, 3), "offsets"),
+            prep(grid_indices, torch.int64, (n,), "grid_indices"),
+            prep(cell_indices, torch.int64, (n,), "cell_indices"),
+            prep(masks, torch.bool, (n,), "masks"),
+            prep(lut_grid_nb2grid_idx, torch.int64, (b, 8), "lut_grid_nb2grid_idx"),
+            prep(lut_cell_nb2cell_idx, torch.int64, (m, 8), "lut_cell_nb2cell_idx"),
+            prep(lut_cell_nb2grid_nb, torch.int64, (m, 8), "lut_cell_nb2grid_nb"),
+        ]
+        args = _QueryArgs(
+            *[t.data_ptr() for t in held],
+            n,
+            b,
+            m,
+            e,
+            _INTERPOLATION[interpolation],
+            _DTYPE[embeddings.dtype],
+        )
+        return args, held, dev
+
+    def query_forward(
+        self,
+        embeddings,
+        offsets,
+        grid_indices,
+        cell_indices,
+        masks,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        grid_dim,
+        interpolation,
+    ) -> torch.Tensor:
+        args, held, dev = self._query_args(
+            embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+            interpolation,
+        )
+        out = torch.empty(
+            (args.num_queries, args.embedding_dim), dtype=embeddings.dtype, device=dev
+        )
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_query_forward(ctypes.byref(args), out.data_ptr(), _stream_of(dev))
+            )
+        return out
+
+    def query_backward_forward(
+        self,
+        z,
+        embeddings,
+        offsets,
+        grid_indices,
+        cell_indices,
+        masks,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        grid_dim,
+        interpolation,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        args, held, dev = self._query_args(
+            embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+            interpolation,
+        )
+        z = _as_like(z, embeddings, (args.num_queries, args.embedding_dim), "z")
+        grad_embeddings = torch.empty_like(held[0])
+        grad_offsets = torch.empty((args.num_queries, 3), dtype=embeddings.dtype, device=dev)
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_query_backward_forward(
+                    ctypes.byref(args),
+                    z.data_ptr(),
+                    grad_embeddings.data_ptr(),
+                    grad_offsets.data_ptr(),
+                    _stream_of(dev),
+                )
+            )
+        return grad_embeddings, grad_offsets
+
+    def query_backward_backward(
+        self,
+        grad_grad_embeddings,
+        grad_grad_offsets,
+        z,
+        embeddings,
+        offsets,
+        grid_indices,
+        cell_indices,
+        masks,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        grid_dim,
+        interpolation,
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        args, held, dev = self._query_args(
+            embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+            interpolation,
+        )
+        n, e = args.num_queries, args.embedding_dim
+        z = _as_like(z, embeddings, (n, e), "z")
+        gg_off = _as_like(grad_grad_offsets, embeddings, (n, 3), "grad_grad_offsets")
+        grad_z = torch.empty((n, e), dtype=embeddings.dtype, device=dev)
+        grad_embeddings = torch.empty_like(held[0])
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_query_backward_backward(
+                    ctypes.byref(args),
+                    gg_off.data_ptr(),
+                    z.data_ptr(),
+                    grad_z.data_ptr(),
+                    grad_embeddings.data_ptr(),
+                    _stream_of(dev),
+                )
+            )
+        # the offsets second-order term is not produced (ash/src/grid.cu:417-418)
+        grad_offsets = torch.zeros((n, 3), dtype=embeddings.dtype, device=dev)
+        return grad_z, grad_embeddings, grad_offsets
+
+
+def _numel(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= s
+    return n
+
+
+def _as_like(t: torch.Tensor, ref: torch.Tensor, shape, name: str) -> torch.Tensor:
+    if t.device != ref.device:
+        raise RuntimeError(f"{name} is on {t.device}, embeddings on {ref.device}")
+    if t.dtype != ref.dtype:
+        raise RuntimeError(f"{name} must be {ref.dtype}, got {t.dtype}")
+    if t.numel() != _numel(shape):
+        raise RuntimeError(f"{name} has shape {tuple(t.shape)}, expected {shape}")
+    return t.contiguous()
+
+
+class _HashMap:
+    """Same surface as the pybind class `HashMap` (ash/src/pybind.cpp:9-23).
+
+    Owns the table workspace as torch tensors and a native handle.  `heap` is
+    the caller's int32[capacity] buffer and is mutated in place by the kernels.
+    """
+
+    _backend: "_Backend" = None
+
+    def __init__(self, key_dim: int, capacity: int, heap: torch.Tensor, device):
+        device = torch.device(device)
+        if device.type != "cuda":
+            # the reference has no CPU map either (ash/src/hashmap_cpu.cpp:8)
+            raise RuntimeError("Not implemented: ash hash maps exist on HIP devices only")
+        if heap.dtype != torch.int32 or heap.numel() != capacity or not heap.is_contiguous():
+            raise RuntimeError("heap must be a contiguous int32 tensor of `capacity` elements")
+        _require_hip(heap, "heap")
+        lib = self._backend.lib
+        self._lib = lib
+        self._handle = None
+        self._device = heap.device
+        self.key_dim = int(key_dim)
+        self.capacity = int(capacity)
+        self._heap = heap
+        table_bytes, general_bytes = _I64(0), _I64(0)
+        self._check(
+            lib.ash_map_workspace_bytes(
+                self.key_dim, self.capacity, ctypes.byref(table_bytes), ctypes.byref(general_bytes)
+            )
+        )
+        self._general_bytes = general_bytes.value
+        self._table = torch.empty(table_bytes.value, dtype=torch.uint8, device=self._device)
+        self._general = None
+        handle = _PTR()
+        with torch.cuda.device(self._device):
+            self._check(
+                lib.ash_map_create(
+                    self.key_dim,
+                    self.capacity,
+                    heap.data_ptr(),
+                    self._table.data_ptr(),
+                    table_bytes.value,
+                    self._device.index,
+                    self._stream(),
+                    ctypes.byref(handle),
+                )
+            )
+        self._handle = handle
+
+    def __del__(self):
+        handle, self._handle = getattr(self, "_handle", None), None
+        if handle:
+            self._lib.ash_map_destroy(handle)
+
+    # -- helpers ---------------------------------------------------------
+    def _check(self, status: int) -> None:
+        self._backend.check(status)
+
+    def _stream(self) -> int:
+        return _stream_of(self._device)
+
+    def _keys(self, keys: torch.Tensor) -> torch.Tensor:
+        if keys.dim() != 2 or keys.shape[1] != self.key_dim:
+            raise RuntimeError(f"keys must be (N, {self.key_dim}), got {tuple(keys.shape)}")
+        if keys.device != self._device:
+            raise RuntimeError(f"keys are on {keys.device}, the map on {self._device}")
+        if keys.dtype != torch.int32:
+            keys = keys.to(torch.int32)
+        return keys.contiguous()
+
+    def _attach_general_if_needed(self) -> bool:
+        """After an insert/load: keys that need the second region are counted by
+        the kernel; attach the region once and let the caller re-issue."""
+        st = self.status()
+        if st["exotic_pending"] == 0:
+            return False
+        if self._general is not None:
+            raise RuntimeError("internal error: unpackable keys pending with region attached")
+        self._general = torch.empty(self._general_bytes, dtype=torch.uint8, device=self._device)
+        with torch.cuda.device(self._device):
+            self._check(
+                self._lib.ash_map_attach_general(
+                    self._handle, self._general.data_ptr(), self._general_bytes, self._stream()
+                )
+            )
+        return True
+
+    # -- pybind surface --------------------------------------------------
+    def device(self) -> torch.device:
+        return self._device
+
+    def status(self) -> Dict[str, int]:
+        out = (_I64 * 5)()
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_map_status(self._handle, out, self._stream()))
+        return {
+            "size": out[0],
+            "dropped": out[1],
+            "tombstones": out[2],
+            "exotic_pending": out[3],
+            "load_duplicates": out[4],
+        }
+
+    def size(self) -> int:
+        n = _I64(0)
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_map_size(self._handle, ctypes.byref(n), self._stream()))
+        return n.value
+
+    def find(self, keys: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        keys = self._keys(keys)
+        n = keys.shape[0]
+        indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        masks = torch.empty(n, dtype=torch.bool, device=self._device)
+        with torch.cuda.device(self._device):
+            self._check(
+                self._lib.ash_map_find(
+                    self._handle, keys.data_ptr(), n, indices.data_ptr(), masks.data_ptr(),
+                    self._stream(),
+                )
+            )
+        return indices, masks
+
+    def insert_keys(self, keys: torch.Tensor) -> None:
+        keys = self._keys(keys)
+        for _ in range(2):
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_map_insert_keys(
+                        self._handle, keys.data_ptr(), keys.shape[0], self._stream()
+                    )
+                )
+            if not self._attach_general_if_needed():
+                break
+
+    def insert(
+        self,
+        keys: torch.Tensor,
+        values: Dict[str, torch.Tensor],
+        external_values: Dict[str, torch.Tensor],
+    ) -> None:
+        keys = self._keys(keys)
+        n = keys.shape[0]
+        names = list(values.keys())
+        if not names:
+            return self.insert_keys(keys)
+        src, dst, row_bytes = [], [], []
+        for name in names:
+            v, ext = values[name], external_values[name]
+            if v.shape[0] != n:
+                raise RuntimeError(f"value '{name}' has {v.shape[0]} rows for {n} keys")
+            if v.dtype != ext.dtype or v.shape[1:] != ext.shape[1:]:
+                raise RuntimeError(f"value '{name}' does not match its destination buffer")
+            if v.device != self._device or ext.device != self._device:
+                raise RuntimeError(f"value '{name}' is not on {self._device}")
+            if not ext.is_contiguous():
+                raise RuntimeError(f"destination buffer '{name}' must be contiguous")
+            if ext.shape[0] != self.capacity:
+                raise RuntimeError(f"destination buffer '{name}' must have `capacity` rows")
+            v = v.contiguous()
+            src.append(v)
+            dst.append(ext)
+            row_bytes.append((v.numel() // max(n, 1)) * v.element_size() if n else 0)
+        if n == 0:
+            return
+        k = len(names)
+        c_rows = (_I64 * k)(*row_bytes)
+        c_src = (_PTR * k)(*[t.data_ptr() for t in src])
+        c_dst = (_PTR * k)(*[t.data_ptr() for t in dst])
+        assigned = None
+        if self._lib.ash_map_insert_needs_scratch(k, c_rows):
+            assigned = torch.empty(n, dtype=torch.int32, device=self._device)
+        for _ in range(2):
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_map_insert(
+                        self._handle,
+                        keys.data_ptr(),
+                        n,
+                        k,
+                        c_src,
+                        c_dst,
+                        c_rows,
+                        assigned.data_ptr() if assigned is not None else None,
+                        self._stream(),
+                    )
+                )
+            if not self._attach_general_if_needed():
+                break
+
+    def erase(self, keys: torch.Tensor) -> None:
+        keys = self._keys(keys)
+        with torch.cuda.device(self._device):
+            self._check(
+                self._lib.ash_map_erase(
+                    self._handle, keys.data_ptr(), keys.shape[0], self._stream()
+                )
+            )
+
+    def clear(self) -> None:
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_map_clear(self._handle, self._stream()))
+
+    def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        n = self.size()
+        keys = torch.empty((n, self.key_dim), dtype=torch.int32, device=self._device)
+        indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        if n > 0:
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_map_items(
+                        self._handle, keys.data_ptr(), indices.data_ptr(), n, self._stream()
+                    )
+                )
+        return keys, indices
+
+    def load_states(self, states: Dict[str, torch.Tensor]) -> None:
+        keys = self._keys(states["active_keys"])
+        indices = states["active_indices"].to(self._device, torch.int64).contiguous()
+        heap = states["heap"].to(self._device, torch.int32).contiguous()
+        n = keys.shape[0]
+        if indices.numel() != n:
+            raise RuntimeError("active_keys and active_indices differ in length")
+        if heap.numel() != self.capacity:
+            raise RuntimeError("heap length differs from the capacity")
+        for _ in range(2):
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_map_load(
+                        self._handle,
+                        keys.data_ptr() if n else None,
+                        indices.data_ptr() if n else None,
+                        n,
+                        heap.data_ptr(),
+                        self._stream(),
+                    )
+                )
+            if not self._attach_general_if_needed():
+                break
+        dup = self.status()["load_duplicates"]
+        if dup:
+            warnings.warn(f"load_states met {dup} duplicate keys; they were stored once")
+
+
+class _MissingBackend:
+    """Placeholder used when libash_hip.so cannot be loaded: every use raises."""
+
+    def __init__(self, reason: str):
+        self._reason = reason
+
+    def __getattr__(self, name):
+        raise RuntimeError(
+            f"libash_hip.so is not available ({self._reason}); build it with "
+            "`python torch-ash_amd/build.py`. There is no CPU or PyTorch fallback."
+        )
+
+
+_BACKEND = None
+
+
+def _get_c_extension():
+    """Counterpart of ash/common.py:4-15: returns the native backend object."""
+    global _BACKEND
+    if _BACKEND is None:
+        try:
+            _BACKEND = _Backend(load_library())
+        except OSError as exc:
+            warnings.warn(f"HIP extension {_LIB_NAME} could not be loaded: {exc}")
+            _BACKEND = _MissingBackend(str(exc))
+    return _BACKEND

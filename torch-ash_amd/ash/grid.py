@@ -1,0 +1,414 @@
+"""Sparse-dense grids: a hash map of active blocks, each a dense G^3 array of
+cells carrying an embedding row.
+
+Public names, shapes and semantics follow ash/grid.py:29-863 for what lies on
+the query path (allocation, query, interpolation, enumeration, neighbour
+tables, coordinate transforms).  Ray sampling, filtering and surface extraction
+belong to other native kernels of the reference and are not provided.
+"""
+from typing import Literal, Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+
+from .common import _get_c_extension
+from .core import ASHEngine, ASHModule
+from .grid_nns import enumerate_neighbor_coord_offsets
+from .grid_query import SparseDenseGridQuery
+from .hashmap import HashSet
+
+backend = _get_c_extension()
+
+Interpolation = Literal["nearest", "linear", "smooth_step"]
+
+
+class SparseDenseGrid(ASHModule):
+    """Grid addressed in cell units: position x lies in block floor(x / G) and,
+    inside it, in cell floor(x - G * block).
+
+    `embeddings` has shape (num_embeddings, G**3, embedding_dim); the row of a
+    cell is `embeddings[grid_index, cell_index]` with
+    cell_index = cx + G * cy + G**2 * cz.
+    """
+
+    def __init__(
+        self,
+        in_dim: int,
+        num_embeddings: int,
+        embedding_dim: int,
+        grid_dim: int,
+        device: Optional[Union[str, torch.device]] = torch.device("cpu"),
+    ):
+        assert in_dim == 3, "Only 3D sparse-dense grid is supported for now."
+        assert embedding_dim <= 16, "Embedding dim must be <= 16 for now."
+        super().__init__()
+
+        self.transform_world_to_cell = lambda x: x
+        self.transform_cell_to_world = lambda x: x
+
+        self.in_dim = in_dim
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        self.grid_dim = grid_dim
+        self.device = torch.device(device) if isinstance(device, str) else device
+
+        self.engine = ASHEngine(in_dim, num_embeddings, device)
+        self.num_cells_per_grid = grid_dim**in_dim
+        self.embeddings = nn.Parameter(
+            torch.zeros(num_embeddings, self.num_cells_per_grid, embedding_dim, device=device)
+        )
+
+        # Per-cell constants: the dense part has the same structure in every block.
+        self.cell_indices = torch.arange(
+            self.num_cells_per_grid, dtype=torch.long, device=self.device
+        )
+        self.cell_coords = self._delinearize_cell_indices(self.cell_indices)
+        assert self.cell_coords.shape == (self.num_cells_per_grid, in_dim)
+        self.lut_cell_nb2grid_nb, self.lut_cell_nb2cell_idx = self.construct_cell_neighbor_lut(
+            radius=1, bidirectional=False
+        )
+
+        # Per-block tables exist only once blocks have been activated.
+        self.grid_indices = None
+        self.grid_coords = None
+        self.lut_grid_nb2grid_idx = None
+
+    # ------------------------------------------------------------ activation
+    def spatial_init_(
+        self, points: torch.Tensor, dilation: int = 1, bidirectional: bool = False
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Activates the blocks containing `points` (world coordinates) and their
+        neighbours within `dilation` blocks (ash/grid.py:121-159).
+
+        Returns the touched blocks in broadcastable form:
+        grid_coords (n, 1, 3), cell_coords (1, M, 3), grid_indices (n, 1),
+        cell_indices (1, M).
+        """
+        cells = self.transform_world_to_cell(points)
+        block_coords = self.grids_in_bound(torch.floor(cells / self.grid_dim).int())
+
+        nb_offsets, _ = enumerate_neighbor_coord_offsets(
+            self.in_dim, dilation, bidirectional=bidirectional, device=self.device
+        )
+        candidates = (block_coords.view(-1, 1, 3) + nb_offsets).view(-1, 3)
+
+        unique_coords = self.grids_in_bound(self._unique_keys(candidates, len(block_coords)))
+
+        self.engine.insert_keys(unique_coords)
+        grid_indices, masks = self.engine.find(unique_coords)
+        assert masks.all()
+
+        return (
+            unique_coords.view(-1, 1, self.in_dim),
+            self.cell_coords.view(1, -1, self.in_dim),
+            grid_indices.view(-1, 1),
+            self.cell_indices.view(1, -1),
+        )
+
+    def _unique_keys(self, candidates: torch.Tensor, num_sources: int) -> torch.Tensor:
+        """Distinct rows of `candidates` through a scratch hash set.  The
+        reference sizes that set by the number of source points
+        (ash/grid.py:145), which is too small when few points are dilated
+        widely; here a set that turns out too small is retried at the size that
+        cannot fail."""
+        if len(candidates) == 0:
+            return candidates
+        first_try = min(len(candidates), max(num_sources, 1024))
+        for capacity in (first_try, len(candidates)):
+            scratch = HashSet(key_dim=3, capacity=capacity, device=self.device)
+            scratch.engine.backend.insert_keys(candidates.int().contiguous())
+            if capacity == len(candidates) or scratch.engine.backend.status()["dropped"] == 0:
+                return scratch.keys()
+        raise AssertionError("unreachable")
+
+    def ray_init_(self, ray_o, rays_d, rays_near, rays_far, dilation: int = 3) -> None:
+        raise NotImplementedError("Ray-tracing initialization not implemented yet")
+
+    # ----------------------------------------------------------------- query
+    def query(
+        self, x: torch.Tensor
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Splits positions (cell units) into block / cell / fractional parts
+        (ash/grid.py:183-199).
+
+        Returns grid_indices (N,), cell_indices (N,), offsets (N, 3) in [0, 1),
+        masks (N,) = block is active.
+        """
+        g = self.grid_dim
+        x_sparse = (x / g).floor()
+        x_dense = x - x_sparse * g
+        # For tiny negative x the subtraction rounds to exactly g in fp32; that
+        # position is cell 0 of the next block, not a cell index out of range.
+        spill = (x_dense >= g).to(x_dense.dtype)
+        x_sparse = x_sparse + spill
+        x_dense = x_dense - spill * g
+        offsets = x_dense - x_dense.floor()
+
+        grid_indices, masks = self.engine.find(x_sparse.int())
+        cell_indices = self._linearize_cell_coords(x_dense.int())
+        return grid_indices, cell_indices, offsets, masks
+
+    def forward(
+        self, x: torch.Tensor, interpolation: Interpolation = "smooth_step"
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Embeddings at world positions x (N, 3): features (N, E) and the mask
+        of positions that fall into an active block (ash/grid.py:201-238)."""
+        x = self.transform_world_to_cell(x)
+        grid_indices, cell_indices, offsets, masks = self.query(x)
+
+        if interpolation == "nearest":
+            return self.embeddings[grid_indices, cell_indices], masks
+        if interpolation not in ("linear", "smooth_step"):
+            raise ValueError(f"Unknown interpolation: {interpolation}")
+
+        if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
+            self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+        features = SparseDenseGridQuery.apply(
+            self.embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            self.lut_grid_nb2grid_idx,
+            self.lut_cell_nb2cell_idx,
+            self.lut_cell_nb2grid_nb,
+            self.grid_dim,
+            interpolation,
+        )
+        return features, masks
+
+    def items(self) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Active blocks in broadcastable form (ash/grid.py:240-266):
+        grid_coords (n, 1, 3), cell_coords (1, M, 3), grid_indices (n, 1),
+        cell_indices (1, M); integer cell positions are
+        grid_coords * G + cell_coords and their rows
+        embeddings[grid_indices, cell_indices]."""
+        grid_coords, grid_indices = self.engine.items()
+        return (
+            grid_coords.view(-1, 1, self.in_dim),
+            self.cell_coords.view(1, -1, self.in_dim),
+            grid_indices.view(-1, 1),
+            self.cell_indices.view(1, -1),
+        )
+
+    # ------------------------------------------------------------ transforms
+    @torch.no_grad()
+    def get_bbox(self):
+        return self.bbox_min, self.bbox_max
+
+    def cell_to_world(self, grid_coords: torch.Tensor, cell_coords: torch.Tensor) -> torch.Tensor:
+        """(n,1,3) block coords x (1,M,3) cell coords -> (n*M, 3) world positions."""
+        cells = grid_coords.view(-1, 1, self.in_dim) * self.grid_dim + cell_coords.view(
+            1, -1, self.in_dim
+        )
+        return self.transform_cell_to_world(cells).view(-1, self.in_dim)
+
+    def grids_in_bound(self, grid_coords: torch.Tensor) -> torch.Tensor:
+        """Unbounded by default; the bounded grid filters here."""
+        return grid_coords
+
+    @torch.no_grad()
+    def _linearize_cell_coords(self, cell_coords: torch.Tensor) -> torch.Tensor:
+        """(N, 3) cell coordinates -> int64 cell index cx + G*cy + G^2*cz."""
+        assert cell_coords.dim() == 2 and cell_coords.shape[1] == self.in_dim
+        index = torch.zeros(cell_coords.shape[0], dtype=torch.long, device=cell_coords.device)
+        for d in range(self.in_dim):
+            index += cell_coords[:, d].long() * self.grid_dim**d
+        return index
+
+    @torch.no_grad()
+    def _delinearize_cell_indices(self, cell_indices: torch.Tensor) -> torch.Tensor:
+        """Inverse of `_linearize_cell_coords`; int32 coordinates, last dim 3."""
+        rest = cell_indices.clone()
+        coords = []
+        for _ in range(self.in_dim):
+            coords.append(rest % self.grid_dim)
+            rest = torch.div(rest, self.grid_dim, rounding_mode="floor")
+        return torch.stack(coords, dim=-1).int()
+
+    # -------------------------------------------------------------- sampling
+    def uniform_sample(
+        self, num_samples: int, space: Literal["occupied", "empty"] = "occupied"
+    ) -> torch.Tensor:
+        """World positions drawn uniformly inside randomly chosen active blocks
+        (ash/grid.py:405-430)."""
+        if space != "occupied":
+            raise NotImplementedError("empty space sampling not implemented")
+        active_coords, _ = self.engine.items()
+        pick = torch.randint(len(active_coords), (num_samples,), device=self.device)
+        inside = torch.rand(num_samples, self.in_dim, device=self.device)
+        return self.transform_cell_to_world((active_coords[pick].float() + inside) * self.grid_dim)
+
+    # Native kernels of the reference that are not part of the query path.
+    def ray_sample(self, *args, **kwargs):
+        raise NotImplementedError("ray_sample is not provided by this build")
+
+    def ray_find_near_far(self, *args, **kwargs):
+        raise NotImplementedError("ray_find_near_far is not provided by this build")
+
+    def gaussian_filter_(self, *args, **kwargs):
+        raise NotImplementedError("gaussian_filter_ is not provided by this build")
+
+    def convolution(self, *args, **kwargs):
+        raise NotImplementedError("convolution is not provided by this build")
+
+    def marching_cubes(self, *args, **kwargs):
+        raise NotImplementedError("marching_cubes is not provided by this build")
+
+    # ------------------------------------------------------ neighbour tables
+    @torch.no_grad()
+    def construct_cell_neighbor_lut(
+        self, radius: int, bidirectional: bool
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Per-cell tables (ash/grid.py:525-564).  For cell p and window offset
+        o_k: the neighbour lies in block offset floor((p + o_k) / G), reported
+        as its row in the block-offset window, at cell (p + o_k) mod G.
+
+        Returns (lut_cell_nb2grid_nb, lut_cell_nb2cell_idx), both int64 (M, K).
+        """
+        cell_offsets, _ = enumerate_neighbor_coord_offsets(
+            self.in_dim, radius, bidirectional, self.device
+        )
+        block_radius = (radius + self.grid_dim - 1) // self.grid_dim
+        _, block_offset2idx = enumerate_neighbor_coord_offsets(
+            self.in_dim, block_radius, bidirectional, self.device
+        )
+        assert self.cell_coords is not None
+        shifted = (
+            self.cell_coords.view(-1, 1, self.in_dim) + cell_offsets.view(1, -1, self.in_dim)
+        ).view(-1, self.in_dim)
+        block_shift = torch.div(shifted, self.grid_dim, rounding_mode="floor").long()
+        wrapped = torch.remainder(shifted, self.grid_dim)
+
+        lut_cell_nb2grid_nb = block_offset2idx(block_shift).view(self.num_cells_per_grid, -1)
+        lut_cell_nb2cell_idx = self._linearize_cell_coords(wrapped).view(
+            self.num_cells_per_grid, -1
+        )
+        return lut_cell_nb2grid_nb, lut_cell_nb2cell_idx
+
+    @torch.no_grad()
+    def construct_grid_neighbor_lut(
+        self, radius: int, bidirectional: bool
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Per-block tables over all `num_embeddings` rows (ash/grid.py:566-617):
+        grid_coords int32 (B, 3) and lut_grid_nb2grid_idx int64 (B, K), both -1
+        in rows of inactive blocks and for missing neighbours."""
+        active_coords, active_indices = self.engine.items()
+        nb_offsets, _ = enumerate_neighbor_coord_offsets(
+            self.in_dim, radius, bidirectional, self.device
+        )
+        num_nbs = len(nb_offsets)
+
+        grid_coords = torch.full(
+            (self.num_embeddings, self.in_dim), -1, dtype=torch.int32, device=self.device
+        )
+        lut = torch.full(
+            (self.num_embeddings, num_nbs), -1, dtype=torch.int64, device=self.device
+        )
+        if len(active_coords) == 0:
+            return grid_coords, lut
+
+        nb_coords = (
+            active_coords.view(-1, 1, self.in_dim).int() + nb_offsets.view(1, -1, self.in_dim).int()
+        ).view(-1, self.in_dim)
+        nb_indices, nb_found = self.engine.find(nb_coords)
+        nb_indices[~nb_found] = -1
+
+        grid_coords[active_indices] = active_coords
+        lut[active_indices] = nb_indices.view(-1, num_nbs)
+        return grid_coords, lut
+
+    @torch.no_grad()
+    def construct_grid_neighbor_lut_(self, radius: int, bidirectional: bool) -> None:
+        """Caches the per-block tables; callers rebuild them after activating or
+        erasing blocks (they are not invalidated automatically, as in the
+        reference, ash/grid.py:221-222)."""
+        self.grid_coords, self.lut_grid_nb2grid_idx = self.construct_grid_neighbor_lut(
+            radius, bidirectional
+        )
+
+
+class UnBoundedSparseDenseGrid(SparseDenseGrid):
+    """Grid with a fixed metric cell size and no fixed extent
+    (ash/grid.py:714-775): world = cell * cell_size."""
+
+    def __init__(
+        self,
+        in_dim: int,
+        num_embeddings: int,
+        embedding_dim: int,
+        grid_dim: int,
+        cell_size: float = 0.01,
+        device: Optional[Union[str, torch.device]] = torch.device("cpu"),
+    ):
+        super().__init__(in_dim, num_embeddings, embedding_dim, grid_dim, device)
+        self.cell_size = cell_size
+        self.transform_world_to_cell = lambda x: x / self.cell_size
+        self.transform_cell_to_world = lambda x: x * self.cell_size
+        self.bbox_min = None
+        self.bbox_max = None
+
+    @torch.no_grad()
+    def compute_bbox_(self):
+        """World-space box spanned by the active blocks."""
+        active_coords, _ = self.engine.items()
+        lo = active_coords.min(dim=0)[0]
+        hi = active_coords.max(dim=0)[0] + 1
+        self.bbox_min = self.transform_cell_to_world(lo * self.grid_dim)
+        self.bbox_max = self.transform_cell_to_world(hi * self.grid_dim)
+
+    @torch.no_grad()
+    def get_bbox(self, force_recompute: bool = False):
+        if self.bbox_min is None or self.bbox_max is None or force_recompute:
+            self.compute_bbox_()
+        return self.bbox_min, self.bbox_max
+
+
+class BoundedSparseDenseGrid(SparseDenseGrid):
+    """Grid covering a fixed box with sparse_grid_dim^3 potential blocks
+    (ash/grid.py:778-863).  The cell size is chosen so that
+    sparse_grid_dim * grid_dim cell *corners* span the box:
+    cell_size = min((bbox_max - bbox_min) / (sparse_grid_dim * grid_dim - 1))."""
+
+    def __init__(
+        self,
+        in_dim: int,
+        num_embeddings: int,
+        embedding_dim: int,
+        grid_dim: int = 8,
+        sparse_grid_dim: int = 128,
+        bbox_min: torch.Tensor = None,
+        bbox_max: torch.Tensor = None,
+        device: Optional[Union[str, torch.device]] = None,
+    ):
+        assert in_dim == 3, "Only 3D is supported now"
+        super().__init__(in_dim, num_embeddings, embedding_dim, grid_dim, device)
+        self.sparse_grid_dim = sparse_grid_dim
+        self.bbox_min = (
+            bbox_min.to(self.device)
+            if bbox_min is not None
+            else -torch.ones(self.in_dim, device=self.device)
+        )
+        self.bbox_max = (
+            bbox_max.to(self.device)
+            if bbox_max is not None
+            else torch.ones(self.in_dim, device=self.device)
+        )
+        extent = self.bbox_max - self.bbox_min
+        self.cell_size = (extent / (sparse_grid_dim * grid_dim - 1)).min().item()
+        self.transform_world_to_cell = lambda x: (x - self.bbox_min) / self.cell_size
+        self.transform_cell_to_world = lambda x: x * self.cell_size + self.bbox_min
+
+    def grids_in_bound(self, grid_coords: torch.Tensor) -> torch.Tensor:
+        inside = ((grid_coords >= 0) & (grid_coords < self.sparse_grid_dim)).all(dim=-1)
+        return grid_coords[inside]
+
+    def dense_init_(self):
+        """Activates every block of the box."""
+        axis = torch.arange(self.sparse_grid_dim)
+        all_blocks = (
+            torch.stack(torch.meshgrid(*[axis] * self.in_dim, indexing="ij"))
+            .reshape(self.in_dim, -1)
+            .T.to(self.device)
+        )
+        self.engine.insert_keys(all_blocks)

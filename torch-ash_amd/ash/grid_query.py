@@ -1,0 +1,123 @@
+"""Autograd wiring of the trilinear query: forward, backward, backward of the
+backward.  Two chained Functions with the same operands and return
+conventions as the reference (ash/grid_query.py:10-283); each one is a single
+call into the HIP library.
+"""
+from typing import Literal
+
+import torch
+
+from .common import _get_c_extension
+
+backend = _get_c_extension()
+
+_N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
+
+
+class SparseDenseGridQuery(torch.autograd.Function):
+    """y[i] = sum over the 8 cell corners c of w_c(offsets[i]) * embeddings[row_c(i)].
+
+    Differentiable with respect to `embeddings` and `offsets`; the indices,
+    masks and neighbour tables only address memory.
+    """
+
+    @staticmethod
+    def forward(
+        ctx,
+        embeddings: torch.Tensor,
+        offsets: torch.Tensor,
+        grid_indices: torch.Tensor,
+        cell_indices: torch.Tensor,
+        masks: torch.Tensor,
+        lut_grid_nb2grid_idx: torch.Tensor,
+        lut_cell_nb2cell_idx: torch.Tensor,
+        lut_cell_nb2grid_nb: torch.Tensor,
+        grid_dim: int,
+        interpolation: Literal["linear", "smooth_step"] = "smooth_step",
+    ) -> torch.Tensor:
+        """embeddings (B, M, E), offsets (N, 3) in [0, 1), grid/cell indices and
+        masks (N,), tables (B, 8), (M, 8), (M, 8); returns (N, E)."""
+        operands = (
+            embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+        )
+        ctx.save_for_backward(*operands)
+        ctx.grid_dim = grid_dim
+        ctx.interpolation = interpolation
+        return backend.query_forward(*operands, grid_dim, interpolation)
+
+    @staticmethod
+    def backward(ctx, z: torch.Tensor):
+        """Delegates to SparseDenseGridQueryBackward so that this step is itself
+        differentiable (needed for gradient-norm losses)."""
+        grad_embeddings, grad_offsets = SparseDenseGridQueryBackward.apply(
+            z.contiguous(), *ctx.saved_tensors, ctx.grid_dim, ctx.interpolation
+        )
+        return (grad_embeddings, grad_offsets) + (None,) * _N_TABLE_ARGS
+
+
+class SparseDenseGridQueryBackward(torch.autograd.Function):
+    """(z, embeddings, offsets) -> (grad_embeddings, grad_offsets) with
+
+        grad_embeddings[row_c(i)] += w_c(offsets[i]) * z[i]
+        grad_offsets[i] = sum_c (embeddings[row_c(i)] . z[i]) * dw_c/doffsets
+
+    `z` may carry a graph itself (autograd.grad(..., create_graph=True)).
+    """
+
+    @staticmethod
+    def forward(
+        ctx,
+        z,
+        embeddings,
+        offsets,
+        grid_indices,
+        cell_indices,
+        masks,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        grid_dim,
+        interpolation,
+    ):
+        operands = (
+            z,
+            embeddings,
+            offsets,
+            grid_indices,
+            cell_indices,
+            masks,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+        )
+        ctx.save_for_backward(*operands)
+        ctx.grid_dim = grid_dim
+        ctx.interpolation = interpolation
+        return backend.query_backward_forward(*operands, grid_dim, interpolation)
+
+    @staticmethod
+    def backward(ctx, grad_grad_embeddings: torch.Tensor, grad_grad_offsets: torch.Tensor):
+        """Given u = d loss / d grad_offsets, returns
+
+            grad_z[i]                = sum_c (dw_c/doffsets . u[i]) * embeddings[row_c(i)]
+            grad_embeddings[row_c(i)] += (dw_c/doffsets . u[i]) * z[i]
+
+        Exactly like the reference (ash/grid_query.py:209-283,
+        ash/src/grid.cu:417-426) the incoming `grad_grad_embeddings` is not used
+        and no gradient flows to `offsets` at second order.
+        """
+        grad_z, grad_embeddings, _ = backend.query_backward_backward(
+            grad_grad_embeddings,
+            grad_grad_offsets,
+            *ctx.saved_tensors,
+            ctx.grid_dim,
+            ctx.interpolation,
+        )
+        return (grad_z, grad_embeddings) + (None,) * (_N_TABLE_ARGS + 1)

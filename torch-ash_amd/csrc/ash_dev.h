@@ -1,0 +1,96 @@
+// Shared host/device definitions for libash_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+namespace ash {
+
+// ---------------------------------------------------------------- errors
+void set_error(const std::string& msg);
+
+#define ASH_FAIL(msg)                 \
+    do {                              \
+        ::ash::set_error(msg);        \
+        return 1;                     \
+    } while (0)
+
+#define ASH_HIP(expr)                                                        \
+    do {                                                                     \
+        hipError_t _e = (expr);                                              \
+        if (_e != hipSuccess) {                                              \
+            ::ash::set_error(std::string(#expr) + ": " +                     \
+                             hipGetErrorString(_e));                         \
+            return 1;                                                        \
+        }                                                                    \
+    } while (0)
+
+#define ASH_LAUNCH_CHECK() ASH_HIP(hipGetLastError())
+
+// ------------------------------------------------------- table geometry
+// One bucket is one 128-byte line read by a group of 8 lanes, 16 bytes each:
+//   dwords [ 0,20)  ten 64-bit packed key codes
+//   dwords [20,30)  ten int32 indices (slot s -> dword 20+s)
+//   dwords [30,32)  unused
+constexpr int kGroup = 8;                       // lanes per bucket
+constexpr int kBucketDwords = kGroup * 4;       // 32
+constexpr int kBucketQwords = kGroup * 2;       // 16
+constexpr int kSlots = (kGroup * 16) / 12;      // 10
+constexpr int kValDword0 = 2 * kSlots;          // 20
+constexpr int kTargetFill = 6;                  // entries per bucket at capacity
+
+constexpr uint64_t kEmpty = ~0ull;
+constexpr uint64_t kTomb = ~0ull - 1ull;
+
+// Device counters kept in the first 256 bytes of the table workspace.
+enum Counter {
+    kCtrSize = 0,      // heap counter == number of live entries
+    kCtrDropped = 1,   // keys refused because the heap was exhausted
+    kCtrTombs = 2,     // tombstoned slots (packed + general)
+    kCtrExotic = 3,    // unpackable keys seen while no general region exists
+    kCtrLoadDup = 4,   // duplicate pairs met by load
+    kCtrCursor = 5,    // output cursor of items()
+    kNumCounters = 64
+};
+constexpr int64_t kHeaderBytes = 256;
+
+// General region: open addressing over 32-bit state words + 16-byte keys.
+constexpr int32_t kGenEmpty = -1;
+constexpr int32_t kGenLocked = -2;
+constexpr int32_t kGenTomb = -3;
+constexpr int32_t kGenNoIndex = -4;  // key visible, index not yet assigned
+
+struct MapDev {
+    uint64_t* buckets;   // nb * 16 qwords
+    int32_t* ctr;        // kNumCounters int32
+    int32_t* heap;       // capacity int32 (caller-owned)
+    int32_t* gstate;     // general region state/index words (or nullptr)
+    int32_t* gkeys;      // general region keys, 4 int32 per slot
+    uint32_t nb;         // number of buckets
+    uint32_t gslots;     // general slots (power of two) or 0
+    int32_t capacity;
+};
+
+inline int64_t num_buckets(int64_t capacity) {
+    int64_t nb = (capacity + kTargetFill - 1) / kTargetFill;
+    return nb < 2 ? 2 : nb;
+}
+
+inline int64_t general_slots(int64_t capacity) {
+    int64_t s = 64;
+    while (s < 2 * capacity) s <<= 1;
+    return s;
+}
+
+}  // namespace ash
+
+struct ash_map {
+    int key_dim;
+    int64_t capacity;
+    int device;
+    ash::MapDev d;
+    int64_t table_bytes;
+    bool general_attached;
+};

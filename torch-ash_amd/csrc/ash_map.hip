@@ -1,0 +1,1184 @@
+// Hash map of libash_hip.so: a bucketed open-addressing table for gfx950.
+//
+// Layout.  A bucket is one 128-byte line holding ten 64-bit key codes followed
+// by their ten int32 indices, so a lookup that hits touches one line.  A key
+// int32[dim] is packed into a 64-bit code (dim 1: 32 bits, dim 2: 2x32 biased,
+// dim 3: 3x21 biased, dim 4: 4x16 biased); a slot is claimed with one 64-bit
+// compare-and-swap of the code, which is also what makes duplicate keys inside
+// one batch collapse without locks.  Keys whose components do not fit the code
+// ("exotic" keys) live in a second, lock-based open-addressing region that is
+// only attached once such a key shows up.
+//
+// Probing.  A wavefront takes 64 keys.  Each group of 8 lanes owns 8 of them
+// and probes them one after the other: the 8 lanes read the 8 x 16 bytes of
+// the key's bucket in one coalesced request, compare, and agree through
+// ballots.  All 8 bucket reads of a group are issued before the first compare,
+// so a wavefront keeps 64 lines in flight.  If the bucket neither holds the key
+// nor an empty slot the key moves on to the next bucket.
+//
+// Index allocation follows the reference's heap protocol
+// (ash/src/hashmap_gpu.cuh:211-232,316-336): a new key takes heap[counter++],
+// an erased key stores its index at heap[--counter]; here the counter is
+// advanced once per 256-thread block instead of once per key.
+#include "ash_dev.h"
+
+#include "../../include/ash_hip.h"
+
+namespace ash {
+
+static thread_local std::string g_last_error;
+void set_error(const std::string& msg) { g_last_error = msg; }
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxFusedValues = 4;
+constexpr int kMaxFusedRowDwords = 16;
+constexpr uint32_t kSpinLimit = 1u << 22;
+
+// ------------------------------------------------------------ key codec
+template <int DIM>
+__device__ __forceinline__ bool pack_key(const int32_t (&k)[DIM],
+                                         uint64_t& code) {
+    if constexpr (DIM == 1) {
+        code = static_cast<uint32_t>(k[0]);
+        return true;
+    } else if constexpr (DIM == 2) {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) ^ 0x80000000u;
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) ^ 0x80000000u;
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 32);
+        return code < kTomb;
+    } else if constexpr (DIM == 3) {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) + (1u << 20);
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) + (1u << 20);
+        const uint32_t u2 = static_cast<uint32_t>(k[2]) + (1u << 20);
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 21) |
+               (static_cast<uint64_t>(u2) << 42);
+        return (u0 | u1 | u2) < (1u << 21);
+    } else {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) + 32768u;
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) + 32768u;
+        const uint32_t u2 = static_cast<uint32_t>(k[2]) + 32768u;
+        const uint32_t u3 = static_cast<uint32_t>(k[3]) + 32768u;
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 16) |
+               (static_cast<uint64_t>(u2) << 32) |
+               (static_cast<uint64_t>(u3) << 48);
+        return (u0 | u1 | u2 | u3) < 65536u && code < kTomb;
+    }
+}
+
+template <int DIM>
+__device__ __forceinline__ void unpack_key(uint64_t code, int32_t (&k)[DIM]) {
+    if constexpr (DIM == 1) {
+        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code));
+    } else if constexpr (DIM == 2) {
+        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code) ^ 0x80000000u);
+        k[1] = static_cast<int32_t>(static_cast<uint32_t>(code >> 32) ^
+                                    0x80000000u);
+    } else if constexpr (DIM == 3) {
+        k[0] = static_cast<int32_t>(code & 0x1FFFFFu) - (1 << 20);
+        k[1] = static_cast<int32_t>((code >> 21) & 0x1FFFFFu) - (1 << 20);
+        k[2] = static_cast<int32_t>((code >> 42) & 0x1FFFFFu) - (1 << 20);
+    } else {
+        k[0] = static_cast<int32_t>(code & 0xFFFFu) - 32768;
+        k[1] = static_cast<int32_t>((code >> 16) & 0xFFFFu) - 32768;
+        k[2] = static_cast<int32_t>((code >> 32) & 0xFFFFu) - 32768;
+        k[3] = static_cast<int32_t>((code >> 48) & 0xFFFFu) - 32768;
+    }
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t h) {
+    h ^= h >> 33;
+    h *= 0xff51afd7ed558ccdull;
+    h ^= h >> 33;
+    h *= 0xc4ceb9fe1a85ec53ull;
+    h ^= h >> 33;
+    return h;
+}
+
+__device__ __forceinline__ uint32_t bucket_of(uint64_t code, uint32_t nb) {
+    return __umulhi(static_cast<uint32_t>(mix64(code) >> 32), nb);
+}
+
+__device__ __forceinline__ uint32_t next_bucket(uint32_t b, uint32_t nb) {
+    return (b + 1 == nb) ? 0u : b + 1;
+}
+
+__device__ __forceinline__ uint32_t spread8(uint32_t x) {
+    x = (x | (x << 4)) & 0x0F0Fu;
+    x = (x | (x << 2)) & 0x3333u;
+    x = (x | (x << 1)) & 0x5555u;
+    return x;
+}
+
+__device__ __forceinline__ unsigned long long* slot_ptr(const MapDev& m,
+                                                        uint32_t b, int s) {
+    return reinterpret_cast<unsigned long long*>(
+            m.buckets + static_cast<size_t>(b) * kBucketQwords + s);
+}
+
+__device__ __forceinline__ int32_t* value_ptr(const MapDev& m, uint32_t b,
+                                              int s) {
+    return reinterpret_cast<int32_t*>(m.buckets) +
+           static_cast<size_t>(b) * kBucketDwords + kValDword0 + s;
+}
+
+// -------------------------------------------------- cooperative probe pass
+enum { kProbeFound = 0, kProbeHasEmpty = 1, kProbeFull = 2 };
+
+struct ProbeResult {
+    int status;      // kProbe*
+    int slot;        // matching slot (status == kProbeFound)
+    int32_t val;     // index stored with the matching slot
+    uint32_t emask;  // bit s set <=> slot s was empty in this snapshot
+};
+
+// Every lane of the wavefront calls this together.  Lane L owns key L; in
+// round r the 8 lanes of a group read the bucket `b` of the group's r-th key
+// (16 bytes per lane) and the result lands in that key's owner lane.  Keys
+// that are not pending cost no memory traffic.
+__device__ __forceinline__ void probe_pass(const MapDev& m, uint64_t code,
+                                           uint32_t b, bool pend, int lane,
+                                           ProbeResult& out) {
+    const int j = lane & (kGroup - 1);
+    const int gbase = lane & ~(kGroup - 1);
+    const bool v0 = (2 * j) < kSlots;
+    const bool v1 = (2 * j + 1) < kSlots;
+
+    uint4 line[kGroup];
+#pragma unroll
+    for (int r = 0; r < kGroup; ++r) {
+        const int src = gbase | r;
+        const uint32_t br = __shfl(b, src);
+        const int pr = __shfl(static_cast<int>(pend), src);
+        line[r] = make_uint4(0u, 0u, 0u, 0u);
+        if (pr) {
+            line[r] = *(reinterpret_cast<const uint4*>(
+                                m.buckets +
+                                static_cast<size_t>(br) * kBucketQwords) +
+                        j);
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < kGroup; ++r) {
+        const int src = gbase | r;
+        const uint64_t cr = __shfl(code, src);
+        const uint64_t qa =
+                static_cast<uint64_t>(line[r].x) |
+                (static_cast<uint64_t>(line[r].y) << 32);
+        const uint64_t qb =
+                static_cast<uint64_t>(line[r].z) |
+                (static_cast<uint64_t>(line[r].w) << 32);
+        const uint32_t gm0 =
+                static_cast<uint32_t>(__ballot(v0 && qa == cr) >> gbase) & 0xFFu;
+        const uint32_t gm1 =
+                static_cast<uint32_t>(__ballot(v1 && qb == cr) >> gbase) & 0xFFu;
+        const uint32_t ge0 =
+                static_cast<uint32_t>(__ballot(v0 && qa == kEmpty) >> gbase) &
+                0xFFu;
+        const uint32_t ge1 =
+                static_cast<uint32_t>(__ballot(v1 && qb == kEmpty) >> gbase) &
+                0xFFu;
+        int slot = -1;
+        if (gm0) {
+            slot = 2 * __builtin_ctz(gm0);
+        } else if (gm1) {
+            slot = 2 * __builtin_ctz(gm1) + 1;
+        }
+        const uint32_t emask = spread8(ge0) | (spread8(ge1) << 1);
+        const int t = kValDword0 + (slot < 0 ? 0 : slot);
+        const int comp = t & 3;
+        const uint32_t sel = comp == 0   ? line[r].x
+                             : comp == 1 ? line[r].y
+                             : comp == 2 ? line[r].z
+                                         : line[r].w;
+        const int32_t val = __shfl(static_cast<int>(sel), gbase + (t >> 2));
+        if (j == r) {
+            out.status = slot >= 0 ? kProbeFound
+                                   : (emask ? kProbeHasEmpty : kProbeFull);
+            out.slot = slot;
+            out.val = val;
+            out.emask = emask;
+        }
+    }
+}
+
+// ------------------------------------------------ general (exotic) region
+template <int DIM>
+__device__ __forceinline__ uint32_t gen_home(const int32_t (&k)[DIM],
+                                             uint32_t gslots) {
+    uint64_t h = 0xcbf29ce484222325ull;
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) {
+        h ^= static_cast<uint32_t>(k[d]);
+        h *= 0x100000001b3ull;
+    }
+    return static_cast<uint32_t>(mix64(h)) & (gslots - 1);
+}
+
+__device__ __forceinline__ int32_t gen_load(const int32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int DIM>
+__device__ __forceinline__ bool gen_key_equal(const MapDev& m, uint32_t p,
+                                              const int32_t (&k)[DIM]) {
+    bool eq = true;
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) {
+        eq = eq && (gen_load(m.gkeys + static_cast<size_t>(p) * 4 + d) == k[d]);
+    }
+    return eq;
+}
+
+// Returns true and the stored index when the key is present.
+template <int DIM>
+__device__ bool gen_find(const MapDev& m, const int32_t (&k)[DIM],
+                         int32_t& idx, uint32_t& pos) {
+    if (m.gstate == nullptr) return false;
+    const uint32_t mask = m.gslots - 1;
+    uint32_t p = gen_home<DIM>(k, m.gslots);
+    for (uint32_t step = 0; step < m.gslots; ++step) {
+        const int32_t w = gen_load(m.gstate + p);
+        if (w == kGenEmpty) return false;
+        if (w >= 0 && gen_key_equal<DIM>(m, p, k)) {
+            idx = w;
+            pos = p;
+            return true;
+        }
+        p = (p + 1) & mask;
+    }
+    return false;
+}
+
+enum { kGenWon = 0, kGenDup = 1, kGenFull = 2, kGenNoRegion = 3 };
+
+// Claims a slot for an exotic key.  The slot word goes EMPTY -> LOCKED ->
+// NOINDEX (key readable); the caller later stores the index.  A thread that
+// meets LOCKED re-reads the word; the holder finishes its few stores inside
+// the same loop trip, and the wait is bounded by kSpinLimit.
+template <int DIM>
+__device__ int gen_claim(const MapDev& m, const int32_t (&k)[DIM],
+                         uint32_t& pos) {
+    if (m.gstate == nullptr) return kGenNoRegion;
+    const uint32_t mask = m.gslots - 1;
+    uint32_t p = gen_home<DIM>(k, m.gslots);
+    uint32_t step = 0;
+    uint32_t spins = 0;
+    int result = kGenFull;
+    bool done = false;
+    while (!done) {
+        int32_t w = gen_load(m.gstate + p);
+        if (w == kGenEmpty) {
+            const int32_t old = atomicCAS(m.gstate + p, kGenEmpty, kGenLocked);
+            if (old == kGenEmpty) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    __hip_atomic_store(
+                            m.gkeys + static_cast<size_t>(p) * 4 + d,
+                            d < DIM ? k[d < DIM ? d : 0] : 0, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+                }
+                __hip_atomic_store(m.gstate + p, kGenNoIndex, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                pos = p;
+                result = kGenWon;
+                done = true;
+                w = kGenNoIndex;
+            } else {
+                w = old;
+            }
+        }
+        if (!done) {
+            if (w == kGenLocked) {
+                if (++spins >= kSpinLimit) done = true;  // give up: kGenFull
+            } else {
+                if (w != kGenTomb && w != kGenEmpty) {
+                    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+                    if (gen_key_equal<DIM>(m, p, k)) {
+                        result = kGenDup;
+                        done = true;
+                    }
+                }
+                if (!done && w != kGenEmpty) {
+                    p = (p + 1) & mask;
+                    if (++step >= m.gslots) done = true;
+                }
+            }
+        }
+    }
+    return result;
+}
+
+// ------------------------------------------------------------- kernels
+template <int DIM>
+__device__ __forceinline__ void load_key(const int32_t* __restrict__ keys,
+                                         int64_t i, bool active,
+                                         int32_t (&k)[DIM]) {
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) k[d] = active ? keys[i * DIM + d] : 0;
+}
+
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void find_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n,
+        int64_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const bool active = i < n;
+    int32_t k[DIM];
+    load_key<DIM>(keys, i, active, k);
+    uint64_t code;
+    const bool fits = pack_key<DIM>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+    int32_t res = 0;
+    bool found = false;
+    while (__ballot(pend)) {
+        ProbeResult p;
+        probe_pass(m, code, b, pend, lane, p);
+        if (pend) {
+            if (p.status == kProbeFound) {
+                found = true;
+                res = p.val;
+                pend = false;
+            } else if (p.status == kProbeHasEmpty) {
+                pend = false;
+            } else {
+                b = next_bucket(b, m.nb);
+                if (++steps >= m.nb) pend = false;
+            }
+        }
+    }
+    if (active && !fits) {
+        uint32_t pos;
+        found = gen_find<DIM>(m, k, res, pos);
+    }
+    if (active) {
+        idx_out[i] = found ? static_cast<int64_t>(res) : 0;
+        mask_out[i] = found ? 1 : 0;
+    }
+}
+
+struct ValueArgs {
+    int n;
+    const uint32_t* src[kMaxFusedValues];
+    uint32_t* dst[kMaxFusedValues];
+    int32_t row_dwords[kMaxFusedValues];
+};
+
+enum InsertMode {
+    kInsertKeys = 0,    // allocate indices only
+    kInsertFused = 1,   // + copy narrow value rows in the same kernel
+    kInsertAssign = 2,  // + report the allocated index per input row
+    kInsertLoad = 3     // indices are given (state-dict load), heap untouched
+};
+
+template <int DIM, int MODE>
+__global__ __launch_bounds__(kBlock) void insert_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n, ValueArgs va,
+        int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const bool active = i < n;
+    int32_t k[DIM];
+    load_key<DIM>(keys, i, active, k);
+    uint64_t code;
+    const bool fits = pack_key<DIM>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+
+    bool won = false;      // claimed a packed slot (wb, ws)
+    bool gwon = false;     // claimed a general slot gp
+    bool refused = false;  // no room anywhere
+    uint32_t wb = 0, gp = 0;
+    int ws = 0;
+
+    // Phase A: claim a slot per new key.
+    while (__ballot(pend)) {
+        ProbeResult p;
+        probe_pass(m, code, b, pend, lane, p);
+        if (pend) {
+            if (p.status == kProbeFound) {
+                pend = false;
+                if constexpr (MODE == kInsertLoad) {
+                    atomicAdd(m.ctr + kCtrLoadDup, 1);
+                }
+            } else {
+                uint32_t em = p.emask;
+                while (em) {
+                    const int s = __builtin_ctz(em);
+                    const unsigned long long old =
+                            atomicCAS(slot_ptr(m, b, s), kEmpty, code);
+                    if (old == kEmpty) {
+                        won = true;
+                        wb = b;
+                        ws = s;
+                        pend = false;
+                        break;
+                    }
+                    if (old == code) {
+                        pend = false;
+                        if constexpr (MODE == kInsertLoad) {
+                            atomicAdd(m.ctr + kCtrLoadDup, 1);
+                        }
+                        break;
+                    }
+                    em &= em - 1;
+                }
+                if (pend) {
+                    b = next_bucket(b, m.nb);
+                    if (++steps >= m.nb) {
+                        pend = false;
+                        refused = true;
+                    }
+                }
+            }
+        }
+    }
+    if (active && !fits) {
+        const int g = gen_claim<DIM>(m, k, gp);
+        if (g == kGenWon) {
+            gwon = true;
+        } else if (g == kGenFull) {
+            refused = true;
+        } else if (g == kGenNoRegion) {
+            atomicAdd(m.ctr + kCtrExotic, 1);
+        } else if constexpr (MODE == kInsertLoad) {
+            atomicAdd(m.ctr + kCtrLoadDup, 1);
+        }
+    }
+    if (refused) atomicAdd(m.ctr + kCtrDropped, 1);
+
+    // Phase B: one heap-counter update per block, indices for the winners.
+    const bool w = won || gwon;
+    int32_t idx = -1;
+    if constexpr (MODE == kInsertLoad) {
+        if (w) idx = static_cast<int32_t>(given[i]);
+    } else {
+        __shared__ int s_cnt[kBlock / 64];
+        __shared__ int s_base;
+        const uint64_t wm = __ballot(w);
+        const int nw = __popcll(wm);
+        const int rank = __popcll(wm & ((1ull << lane) - 1ull));
+        if (lane == 0) s_cnt[wave] = nw;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int tot = 0;
+#pragma unroll
+            for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+            int base = 0;
+            if (tot > 0) {
+                base = atomicAdd(m.ctr + kCtrSize, tot);
+                if (base + tot > m.capacity) {
+                    const int lo = base > m.capacity ? base : m.capacity;
+                    const int excess = base + tot - lo;
+                    atomicSub(m.ctr + kCtrSize, excess);
+                    atomicAdd(m.ctr + kCtrDropped, excess);
+                }
+            }
+            s_base = base;
+        }
+        __syncthreads();
+        int top = s_base + rank;
+        for (int q = 0; q < wave; ++q) top += s_cnt[q];
+        if (w) {
+            if (top < m.capacity) {
+                idx = m.heap[top];
+            } else {
+                // Heap exhausted: give the slot up again.
+                if (won) {
+                    atomicExch(slot_ptr(m, wb, ws), kTomb);
+                } else {
+                    __hip_atomic_store(m.gstate + gp, kGenTomb,
+                                       __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+                atomicAdd(m.ctr + kCtrTombs, 1);
+            }
+        }
+    }
+    if (idx >= 0) {
+        if (won) {
+            *value_ptr(m, wb, ws) = idx;
+        } else {
+            __hip_atomic_store(m.gstate + gp, idx, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if constexpr (MODE == kInsertFused) {
+#pragma unroll
+            for (int v = 0; v < kMaxFusedValues; ++v) {
+                if (v < va.n) {
+                    const int rd = va.row_dwords[v];
+                    const uint32_t* s = va.src[v] + i * rd;
+                    uint32_t* d = va.dst[v] + static_cast<int64_t>(idx) * rd;
+                    for (int q = 0; q < rd; ++q) d[q] = s[q];
+                }
+            }
+        }
+    }
+    if constexpr (MODE == kInsertAssign) {
+        if (active) assigned[i] = idx;
+    }
+}
+
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void erase_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const bool active = i < n;
+    int32_t k[DIM];
+    load_key<DIM>(keys, i, active, k);
+    uint64_t code;
+    const bool fits = pack_key<DIM>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+    bool won = false;
+    bool tomb = false;
+    int32_t idx = 0;
+    while (__ballot(pend)) {
+        ProbeResult p;
+        probe_pass(m, code, b, pend, lane, p);
+        if (pend) {
+            if (p.status == kProbeFound) {
+                // A bucket that still has an empty slot has never been full,
+                // so no key was ever pushed past it: the slot can go straight
+                // back to empty.  Otherwise leave a tombstone.
+                const bool reuse = p.emask != 0;
+                const unsigned long long old = atomicCAS(
+                        slot_ptr(m, b, p.slot), code, reuse ? kEmpty : kTomb);
+                if (old == code) {
+                    won = true;
+                    tomb = !reuse;
+                    idx = p.val;
+                }
+                pend = false;
+            } else if (p.status == kProbeHasEmpty) {
+                pend = false;
+            } else {
+                b = next_bucket(b, m.nb);
+                if (++steps >= m.nb) pend = false;
+            }
+        }
+    }
+    if (active && !fits) {
+        int32_t gi;
+        uint32_t pos;
+        if (gen_find<DIM>(m, k, gi, pos)) {
+            if (atomicCAS(m.gstate + pos, gi, kGenTomb) == gi) {
+                won = true;
+                tomb = true;
+                idx = gi;
+            }
+        }
+    }
+    __shared__ int s_cnt[kBlock / 64];
+    __shared__ int s_base;
+    const uint64_t wm = __ballot(won);
+    const int nw = __popcll(wm);
+    const int rank = __popcll(wm & ((1ull << lane) - 1ull));
+    const int nt = __popcll(__ballot(tomb));
+    if (lane == 0) {
+        s_cnt[wave] = nw;
+        if (nt) atomicAdd(m.ctr + kCtrTombs, nt);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int tot = 0;
+#pragma unroll
+        for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+        s_base = tot > 0 ? atomicSub(m.ctr + kCtrSize, tot) : 0;
+    }
+    __syncthreads();
+    if (won) {
+        int below = rank;
+        for (int q = 0; q < wave; ++q) below += s_cnt[q];
+        const int pos = s_base - 1 - below;
+        if (pos >= 0 && pos < m.capacity) m.heap[pos] = idx;
+    }
+}
+
+// items(): thread t reads the 16-byte unit t of the bucket array (two code
+// slots, or index words for the last lanes of a line), four units per thread.
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void items_kernel(
+        MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out,
+        int64_t n_expected) {
+    constexpr int kUnroll = 4;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int j = lane & (kGroup - 1);
+    const bool v0 = (2 * j) < kSlots;
+    const bool v1 = (2 * j + 1) < kSlots;
+    const uint64_t units = static_cast<uint64_t>(m.nb) * kGroup;
+    const uint64_t t0 = static_cast<uint64_t>(blockIdx.x) * (kBlock * kUnroll) +
+                        threadIdx.x;
+    uint64_t qa[kUnroll], qb[kUnroll];
+    bool l0[kUnroll], l1[kUnroll];
+    int cnt = 0;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t t = t0 + static_cast<uint64_t>(u) * kBlock;
+        uint4 q = make_uint4(~0u, ~0u, ~0u, ~0u);
+        if (t < units) q = reinterpret_cast<const uint4*>(m.buckets)[t];
+        qa[u] = static_cast<uint64_t>(q.x) | (static_cast<uint64_t>(q.y) << 32);
+        qb[u] = static_cast<uint64_t>(q.z) | (static_cast<uint64_t>(q.w) << 32);
+        l0[u] = v0 && qa[u] < kTomb;
+        l1[u] = v1 && qb[u] < kTomb;
+        cnt += (l0[u] ? 1 : 0) + (l1[u] ? 1 : 0);
+    }
+    // exclusive scan of cnt over the block
+    int incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    __shared__ int s_cnt[kBlock / 64];
+    __shared__ int s_base;
+    if (lane == 63) s_cnt[wave] = incl;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int tot = 0;
+#pragma unroll
+        for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+        s_base = tot > 0 ? atomicAdd(m.ctr + kCtrCursor, tot) : 0;
+    }
+    __syncthreads();
+    int64_t pos = s_base + (incl - cnt);
+    for (int q = 0; q < wave; ++q) pos += s_cnt[q];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t t = t0 + static_cast<uint64_t>(u) * kBlock;
+        const uint32_t bkt = static_cast<uint32_t>(t / kGroup);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const bool live = h == 0 ? l0[u] : l1[u];
+            if (live) {
+                const uint64_t code = h == 0 ? qa[u] : qb[u];
+                const int32_t val = *value_ptr(m, bkt, 2 * j + h);
+                if (pos < n_expected) {
+                    int32_t k[DIM];
+                    unpack_key<DIM>(code, k);
+#pragma unroll
+                    for (int d = 0; d < DIM; ++d) keys_out[pos * DIM + d] = k[d];
+                    idx_out[pos] = val;
+                }
+                ++pos;
+            }
+        }
+    }
+}
+
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void items_general_kernel(
+        MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out,
+        int64_t n_expected) {
+    const uint32_t p = blockIdx.x * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    int32_t w = kGenEmpty;
+    if (p < m.gslots) w = m.gstate[p];
+    const bool live = w >= 0;
+    const uint64_t lm = __ballot(live);
+    if (lm == 0) return;
+    const int rank = __popcll(lm & ((1ull << lane) - 1ull));
+    int base = 0;
+    if (lane == 0) base = atomicAdd(m.ctr + kCtrCursor, __popcll(lm));
+    base = __shfl(base, 0);
+    if (live) {
+        const int64_t pos = static_cast<int64_t>(base) + rank;
+        if (pos < n_expected) {
+#pragma unroll
+            for (int d = 0; d < DIM; ++d) {
+                keys_out[pos * DIM + d] = m.gkeys[static_cast<size_t>(p) * 4 + d];
+            }
+            idx_out[pos] = w;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void fill16_kernel(uint4* __restrict__ p,
+                                                        int64_t n16,
+                                                        uint32_t word) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    const uint4 v = make_uint4(word, word, word, word);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+         i < n16; i += stride) {
+        p[i] = v;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void reset_heap_kernel(
+        int32_t* __restrict__ heap, int64_t capacity, int32_t* __restrict__ ctr,
+        int32_t size_value, bool write_heap) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (write_heap && i < capacity) heap[i] = static_cast<int32_t>(i);
+    if (i < kNumCounters) ctr[i] = (i == kCtrSize) ? size_value : 0;
+}
+
+__global__ void set_counter_kernel(int32_t* ctr, int which, int32_t value) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) ctr[which] = value;
+}
+
+template <typename Unit>
+__global__ __launch_bounds__(kBlock) void scatter_rows_kernel(
+        const Unit* __restrict__ src, Unit* __restrict__ dst,
+        const int32_t* __restrict__ assigned, int64_t n, int64_t units_per_row) {
+    const int64_t total = n * units_per_row;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+         t < total; t += stride) {
+        const int64_t row = t / units_per_row;
+        const int64_t u = t - row * units_per_row;
+        const int32_t a = assigned[row];
+        if (a >= 0) dst[static_cast<int64_t>(a) * units_per_row + u] = src[t];
+    }
+}
+
+// ---------------------------------------------------------------- host
+struct DeviceGuard {
+    int prev = -1;
+    bool switched = false;
+    hipError_t enter(int device) {
+        hipError_t e = hipGetDevice(&prev);
+        if (e != hipSuccess) return e;
+        if (prev != device) {
+            e = hipSetDevice(device);
+            switched = (e == hipSuccess);
+        }
+        return e;
+    }
+    ~DeviceGuard() {
+        if (switched) (void)hipSetDevice(prev);
+    }
+};
+
+inline unsigned grid_for(int64_t n, int per_block = kBlock) {
+    return static_cast<unsigned>((n + per_block - 1) / per_block);
+}
+
+inline unsigned capped_grid(int64_t n) {
+    int64_t g = (n + kBlock - 1) / kBlock;
+    const int64_t cap = 256 * 32;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return static_cast<unsigned>(g);
+}
+
+int check_map(const ash_map* map) {
+    if (map == nullptr) ASH_FAIL("null map handle");
+    return 0;
+}
+
+int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size) {
+    const int64_t n16 = static_cast<int64_t>(map->d.nb) * kGroup;
+    fill16_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
+            reinterpret_cast<uint4*>(map->d.buckets), n16, 0xFFFFFFFFu);
+    ASH_LAUNCH_CHECK();
+    if (map->general_attached) {
+        const int64_t g16 = static_cast<int64_t>(map->d.gslots) / 4;
+        fill16_kernel<<<capped_grid(g16), kBlock, 0, s>>>(
+                reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
+        ASH_LAUNCH_CHECK();
+    }
+    int64_t span = map->capacity > kNumCounters ? map->capacity : kNumCounters;
+    reset_heap_kernel<<<grid_for(span), kBlock, 0, s>>>(
+            map->d.heap, map->capacity, map->d.ctr, size, write_heap);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+template <int MODE>
+int launch_insert(ash_map* map, const int32_t* keys, int64_t n,
+                  const ValueArgs& va, int32_t* assigned, const int64_t* given,
+                  hipStream_t s) {
+    const unsigned g = grid_for(n);
+    switch (map->key_dim) {
+        case 1:
+            insert_kernel<1, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+                                                        assigned, given);
+            break;
+        case 2:
+            insert_kernel<2, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+                                                        assigned, given);
+            break;
+        case 3:
+            insert_kernel<3, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+                                                        assigned, given);
+            break;
+        default:
+            insert_kernel<4, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+                                                        assigned, given);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int check_batch(const ash_map* map, const void* keys, int64_t n) {
+    if (check_map(map)) return 1;
+    if (n < 0) ASH_FAIL("negative key count");
+    if (n > 0 && keys == nullptr) ASH_FAIL("null keys pointer");
+    if (n > (int64_t{1} << 31) - kBlock) ASH_FAIL("too many keys in one call");
+    return 0;
+}
+
+}  // namespace
+}  // namespace ash
+
+using namespace ash;
+
+extern "C" {
+
+const char* ash_last_error(void) { return g_last_error.c_str(); }
+
+int ash_abi_version(void) { return 1; }
+
+int ash_map_workspace_bytes(int key_dim, int64_t capacity, int64_t* table_bytes,
+                            int64_t* general_bytes) {
+    if (key_dim < 1 || key_dim > 4) ASH_FAIL("key_dim must be in 1..4");
+    if (capacity < 1 || capacity > 0x7FFFFFF0ll) {
+        ASH_FAIL("capacity must be in 1..2^31-16");
+    }
+    if (table_bytes) {
+        *table_bytes = kHeaderBytes + num_buckets(capacity) * kBucketDwords * 4;
+    }
+    if (general_bytes) *general_bytes = general_slots(capacity) * 20;
+    return 0;
+}
+
+int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
+                   int64_t table_bytes, int device, void* stream,
+                   ash_map_t** out) {
+    if (out == nullptr) ASH_FAIL("null output handle");
+    *out = nullptr;
+    int64_t need = 0;
+    if (ash_map_workspace_bytes(key_dim, capacity, &need, nullptr)) return 1;
+    if (heap == nullptr || table_ws == nullptr) ASH_FAIL("null device buffer");
+    if (table_bytes < need) ASH_FAIL("table workspace too small");
+    if (reinterpret_cast<uintptr_t>(table_ws) % 256 != 0) {
+        ASH_FAIL("table workspace must be 256-byte aligned");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(device));
+    ash_map* map = new ash_map();
+    map->key_dim = key_dim;
+    map->capacity = capacity;
+    map->device = device;
+    map->table_bytes = table_bytes;
+    map->general_attached = false;
+    map->d.ctr = static_cast<int32_t*>(table_ws);
+    map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
+                                                 kHeaderBytes);
+    map->d.heap = heap;
+    map->d.gstate = nullptr;
+    map->d.gkeys = nullptr;
+    map->d.nb = static_cast<uint32_t>(num_buckets(capacity));
+    map->d.gslots = 0;
+    map->d.capacity = static_cast<int32_t>(capacity);
+    if (clear_table(map, static_cast<hipStream_t>(stream), true, 0)) {
+        delete map;
+        return 1;
+    }
+    *out = map;
+    return 0;
+}
+
+int ash_map_attach_general(ash_map_t* map, void* general_ws,
+                           int64_t general_bytes, void* stream) {
+    if (check_map(map)) return 1;
+    if (map->general_attached) ASH_FAIL("general region already attached");
+    const int64_t slots = general_slots(map->capacity);
+    if (general_ws == nullptr || general_bytes < slots * 20) {
+        ASH_FAIL("general workspace too small");
+    }
+    if (reinterpret_cast<uintptr_t>(general_ws) % 256 != 0) {
+        ASH_FAIL("general workspace must be 256-byte aligned");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // keys first (16 B per slot, keeps them 16-byte aligned), then states
+    map->d.gkeys = static_cast<int32_t*>(general_ws);
+    map->d.gstate = map->d.gkeys + slots * 4;
+    map->d.gslots = static_cast<uint32_t>(slots);
+    map->general_attached = true;
+    fill16_kernel<<<capped_grid(slots / 4), kBlock, 0, s>>>(
+            reinterpret_cast<uint4*>(map->d.gstate), slots / 4, 0xFFFFFFFFu);
+    ASH_LAUNCH_CHECK();
+    set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrExotic, 0);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_map_destroy(ash_map_t* map) {
+    delete map;
+    return 0;
+}
+
+int ash_map_find(ash_map_t* map, const int32_t* keys, int64_t n,
+                 int64_t* indices, uint8_t* masks, void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n == 0) return 0;
+    if (indices == nullptr || masks == nullptr) ASH_FAIL("null output pointer");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned g = grid_for(n);
+    switch (map->key_dim) {
+        case 1:
+            find_kernel<1><<<g, kBlock, 0, s>>>(map->d, keys, n, indices, masks);
+            break;
+        case 2:
+            find_kernel<2><<<g, kBlock, 0, s>>>(map->d, keys, n, indices, masks);
+            break;
+        case 3:
+            find_kernel<3><<<g, kBlock, 0, s>>>(map->d, keys, n, indices, masks);
+            break;
+        default:
+            find_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys, n, indices, masks);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_map_insert_keys(ash_map_t* map, const int32_t* keys, int64_t n,
+                        void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n == 0) return 0;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    ValueArgs va = {};
+    return launch_insert<kInsertKeys>(map, keys, n, va, nullptr, nullptr,
+                                      static_cast<hipStream_t>(stream));
+}
+
+int ash_map_insert_needs_scratch(int n_values, const int64_t* row_bytes) {
+    if (n_values <= 0) return 0;
+    if (n_values > kMaxFusedValues) return 1;
+    for (int v = 0; v < n_values; ++v) {
+        if (row_bytes[v] % 4 != 0 || row_bytes[v] > kMaxFusedRowDwords * 4) {
+            return 1;
+        }
+    }
+    return 0;
+}
+
+int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
+                     int64_t n, int64_t row_bytes, void* stream) {
+    if (n == 0 || row_bytes == 0) return 0;
+    if (src == nullptr || dst == nullptr || assigned == nullptr) {
+        ASH_FAIL("null pointer in scatter");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uintptr_t align = reinterpret_cast<uintptr_t>(src) |
+                            reinterpret_cast<uintptr_t>(dst) |
+                            static_cast<uintptr_t>(row_bytes);
+    if (align % 16 == 0) {
+        const int64_t upr = row_bytes / 16;
+        scatter_rows_kernel<uint4><<<capped_grid(n * upr), kBlock, 0, s>>>(
+                static_cast<const uint4*>(src), static_cast<uint4*>(dst),
+                assigned, n, upr);
+    } else if (align % 4 == 0) {
+        const int64_t upr = row_bytes / 4;
+        scatter_rows_kernel<uint32_t><<<capped_grid(n * upr), kBlock, 0, s>>>(
+                static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst),
+                assigned, n, upr);
+    } else {
+        scatter_rows_kernel<uint8_t><<<capped_grid(n * row_bytes), kBlock, 0,
+                                       s>>>(static_cast<const uint8_t*>(src),
+                                            static_cast<uint8_t*>(dst),
+                                            assigned, n, row_bytes);
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
+                   const void* const* src, void* const* dst,
+                   const int64_t* row_bytes, int32_t* assigned, void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n_values < 0) ASH_FAIL("negative value count");
+    if (n_values == 0) return ash_map_insert_keys(map, keys, n, stream);
+    if (src == nullptr || dst == nullptr || row_bytes == nullptr) {
+        ASH_FAIL("null value tables");
+    }
+    for (int v = 0; v < n_values; ++v) {
+        if (src[v] == nullptr || dst[v] == nullptr) ASH_FAIL("null value tensor");
+        if (row_bytes[v] <= 0) ASH_FAIL("value rows must not be empty");
+    }
+    if (n == 0) return 0;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ValueArgs va = {};
+    if (!ash_map_insert_needs_scratch(n_values, row_bytes)) {
+        va.n = n_values;
+        for (int v = 0; v < n_values; ++v) {
+            va.src[v] = static_cast<const uint32_t*>(src[v]);
+            va.dst[v] = static_cast<uint32_t*>(dst[v]);
+            va.row_dwords[v] = static_cast<int32_t>(row_bytes[v] / 4);
+        }
+        return launch_insert<kInsertFused>(map, keys, n, va, nullptr, nullptr,
+                                           s);
+    }
+    if (assigned == nullptr) {
+        ASH_FAIL("these value rows need the `assigned` temporary");
+    }
+    if (launch_insert<kInsertAssign>(map, keys, n, va, assigned, nullptr, s)) {
+        return 1;
+    }
+    for (int v = 0; v < n_values; ++v) {
+        if (ash_scatter_rows(src[v], dst[v], assigned, n, row_bytes[v], stream)) {
+            return 1;
+        }
+    }
+    return 0;
+}
+
+int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
+                  void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n == 0) return 0;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned g = grid_for(n);
+    switch (map->key_dim) {
+        case 1:
+            erase_kernel<1><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            break;
+        case 2:
+            erase_kernel<2><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            break;
+        case 3:
+            erase_kernel<3><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            break;
+        default:
+            erase_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_map_clear(ash_map_t* map, void* stream) {
+    if (check_map(map)) return 1;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    return clear_table(map, static_cast<hipStream_t>(stream), true, 0);
+}
+
+int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
+    if (check_map(map)) return 1;
+    if (out == nullptr) ASH_FAIL("null status output");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    int32_t host[8] = {0};
+    ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(host), hipMemcpyDeviceToHost,
+                           s));
+    ASH_HIP(hipStreamSynchronize(s));
+    out[0] = host[kCtrSize];
+    out[1] = host[kCtrDropped];
+    out[2] = host[kCtrTombs];
+    out[3] = host[kCtrExotic];
+    out[4] = host[kCtrLoadDup];
+    return 0;
+}
+
+int ash_map_size(ash_map_t* map, int64_t* size, void* stream) {
+    if (size == nullptr) ASH_FAIL("null size output");
+    int64_t st[5];
+    if (ash_map_status(map, st, stream)) return 1;
+    *size = st[0];
+    return 0;
+}
+
+int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
+                  int64_t n_expected, void* stream) {
+    if (check_map(map)) return 1;
+    if (n_expected < 0) ASH_FAIL("negative item count");
+    if (n_expected == 0) return 0;
+    if (keys_out == nullptr || indices_out == nullptr) {
+        ASH_FAIL("null output pointer");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrCursor, 0);
+    ASH_LAUNCH_CHECK();
+    const int64_t units = static_cast<int64_t>(map->d.nb) * kGroup;
+    const unsigned g = grid_for(units, kBlock * 4);
+    switch (map->key_dim) {
+        case 1:
+            items_kernel<1><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+                                                 n_expected);
+            break;
+        case 2:
+            items_kernel<2><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+                                                 n_expected);
+            break;
+        case 3:
+            items_kernel<3><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+                                                 n_expected);
+            break;
+        default:
+            items_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+                                                 n_expected);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
+    if (map->general_attached) {
+        const unsigned gg = grid_for(map->d.gslots);
+        switch (map->key_dim) {
+            case 1:
+                items_general_kernel<1><<<gg, kBlock, 0, s>>>(
+                        map->d, keys_out, indices_out, n_expected);
+                break;
+            case 2:
+                items_general_kernel<2><<<gg, kBlock, 0, s>>>(
+                        map->d, keys_out, indices_out, n_expected);
+                break;
+            case 3:
+                items_general_kernel<3><<<gg, kBlock, 0, s>>>(
+                        map->d, keys_out, indices_out, n_expected);
+                break;
+            default:
+                items_general_kernel<4><<<gg, kBlock, 0, s>>>(
+                        map->d, keys_out, indices_out, n_expected);
+                break;
+        }
+        ASH_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
+                 int64_t n, const int32_t* heap_src, void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n > map->capacity) ASH_FAIL("more pairs than capacity");
+    if (n > 0 && indices == nullptr) ASH_FAIL("null indices pointer");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (clear_table(map, s, false, static_cast<int32_t>(n))) return 1;
+    if (heap_src != nullptr && heap_src != map->d.heap) {
+        ASH_HIP(hipMemcpyAsync(map->d.heap, heap_src,
+                               static_cast<size_t>(map->capacity) * 4,
+                               hipMemcpyDeviceToDevice, s));
+    }
+    if (n == 0) return 0;
+    ValueArgs va = {};
+    return launch_insert<kInsertLoad>(map, keys, n, va, nullptr, indices, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,735 @@
+// Trilinear query kernels of libash_hip.so (gfx950): forward, backward and
+// double backward of the sparse-dense grid interpolation
+//   y[i,:] = sum_c w_c(offset_i) * embeddings[g_c, cell_c, :]
+// with the reference's addressing (ash/src/grid.cu:68-132): the 8 corner rows
+// of query i are found through three neighbour tables,
+//   nbn = lut_cell_nb2grid_nb[cell_i][c]     which neighbour block (0..7)
+//   g_c = lut_grid_nb2grid_idx[grid_i][nbn]  its block index, -1 if missing
+//   cell_c = lut_cell_nb2cell_idx[cell_i][c] the cell inside that block
+// and a query with any missing neighbour block yields zeros.
+//
+// Mapping.  LPQ lanes share one query and each lane owns VEC consecutive
+// channels, so one request of a wavefront covers whole embedding rows
+// (E = 16 fp32: 4 lanes x 16 B = one 64-byte row; a wavefront reads 16 rows per
+// instruction and writes 1 KiB of contiguous output).  The two per-cell tables
+// are staged once per workgroup in LDS as uint16/uint8; workgroups are
+// persistent and walk the query tiles of "their" XCD (workgroup id mod 8) so
+// that neighbouring queries meet in one L2.  Gradients for the embeddings are
+// accumulated with hardware floating-point atomics; with MERGE, consecutive
+// queries of a wavefront that hit the same row are summed in registers first
+// and issue one atomic per run.
+#include "ash_dev.h"
+
+#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
+
+#include <cstdlib>
+
+#include "../../include/ash_hip.h"
+
+namespace ash {
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kXcds = 8;
+constexpr int64_t kMaxLdsCells = 2048;  // 2048 * 8 * 3 B = 48 KiB
+
+struct QDev {
+    const void* emb;
+    const float* off;
+    const int64_t* gidx;
+    const int64_t* cidx;
+    const uint8_t* mask;
+    const int64_t* lut_g;
+    const int64_t* lut_c2c;
+    const int64_t* lut_c2g;
+    int64_t N;
+    int64_t B;
+    int64_t M;
+    int E;
+    int smooth;  // 0 linear, 1 smooth step
+};
+
+// Interpolation basis (ash/src/grid.cu:7-41).
+template <typename T>
+__device__ __forceinline__ T basis(T x, int smooth) {
+    return smooth ? x * x * (T(3) - T(2) * x) : x;
+}
+template <typename T>
+__device__ __forceinline__ T dbasis(T x, int smooth) {
+    return smooth ? T(6) * x * (T(1) - x) : T(1);
+}
+
+// Per-axis factors of the corner weights and of their derivatives
+// (ash/src/grid.cu:113-118,229-241): side 0 is the "1 - o" side.
+template <typename T>
+struct AxisTerms {
+    T w[3][2];
+    T dw[3][2];
+};
+
+template <typename T>
+__device__ __forceinline__ void axis_terms(const float (&o)[3], int smooth,
+                                           AxisTerms<T>& t) {
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        const T x1 = static_cast<T>(o[d]);
+        const T x0 = static_cast<T>(1.0f - o[d]);
+        t.w[d][0] = basis<T>(x0, smooth);
+        t.w[d][1] = basis<T>(x1, smooth);
+        t.dw[d][0] = -dbasis<T>(x0, smooth);
+        t.dw[d][1] = dbasis<T>(x1, smooth);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T corner_weight(const AxisTerms<T>& t, int c) {
+    T w = T(1);
+    w *= t.w[0][c & 1];
+    w *= t.w[1][(c >> 1) & 1];
+    w *= t.w[2][(c >> 2) & 1];
+    return w;
+}
+
+template <typename T>
+__device__ __forceinline__ void corner_weight_grad(const AxisTerms<T>& t, int c,
+                                                   T (&g)[3]) {
+    const int b0 = c & 1, b1 = (c >> 1) & 1, b2 = (c >> 2) & 1;
+    g[0] = t.dw[0][b0] * t.w[1][b1] * t.w[2][b2];
+    g[1] = t.w[0][b0] * t.dw[1][b1] * t.w[2][b2];
+    g[2] = t.w[0][b0] * t.w[1][b1] * t.dw[2][b2];
+}
+
+// The two per-cell tables, either staged in LDS or read through the caches.
+template <bool LDS>
+struct CellLut {
+    const uint16_t* c2c;
+    const uint8_t* c2g;
+    const int64_t* g_c2c;
+    const int64_t* g_c2g;
+    int64_t M;
+    __device__ __forceinline__ void get(int64_t cell, int c, int& nb_cell,
+                                        int& nb_grid) const {
+        if constexpr (LDS) {
+            nb_cell = c2c[cell * 8 + c];
+            nb_grid = c2g[cell * 8 + c];
+        } else {
+            int64_t v = g_c2c[cell * 8 + c];
+            v = v < 0 ? 0 : (v >= M ? M - 1 : v);
+            nb_cell = static_cast<int>(v);
+            nb_grid = static_cast<int>(g_c2g[cell * 8 + c]) & 7;
+        }
+    }
+};
+
+template <bool LDS>
+__device__ __forceinline__ CellLut<LDS> stage_cell_lut(const QDev& a,
+                                                       unsigned char* smem) {
+    CellLut<LDS> lut;
+    lut.g_c2c = a.lut_c2c;
+    lut.g_c2g = a.lut_c2g;
+    lut.M = a.M;
+    lut.c2c = nullptr;
+    lut.c2g = nullptr;
+    if constexpr (LDS) {
+        uint16_t* s_c2c = reinterpret_cast<uint16_t*>(smem);
+        uint8_t* s_c2g = smem + a.M * 8 * 2;
+        const int64_t n = a.M * 8;
+        for (int64_t t = threadIdx.x; t < n; t += kBlock) {
+            int64_t v = a.lut_c2c[t];
+            v = v < 0 ? 0 : (v >= a.M ? a.M - 1 : v);
+            s_c2c[t] = static_cast<uint16_t>(v);
+            s_c2g[t] = static_cast<uint8_t>(a.lut_c2g[t] & 7);
+        }
+        __syncthreads();
+        lut.c2c = s_c2c;
+        lut.c2g = s_c2g;
+    }
+    return lut;
+}
+
+// Tile walk: workgroup w serves XCD (w mod 8); each XCD owns a contiguous
+// eighth of the tiles and its workgroups stride through it.
+struct TileWalk {
+    int64_t next;
+    int64_t end;
+    int64_t step;
+    __device__ __forceinline__ TileWalk(int64_t ntiles) {
+        const int64_t per_xcd = (ntiles + kXcds - 1) / kXcds;
+        const int xcd = blockIdx.x % kXcds;
+        const int slot = blockIdx.x / kXcds;
+        step = (gridDim.x + kXcds - 1 - xcd) / kXcds;  // workgroups on this XCD
+        next = xcd * per_xcd + slot;
+        end = (xcd + 1) * per_xcd;
+        if (end > ntiles) end = ntiles;
+        if (step < 1) step = 1;
+    }
+};
+
+// Resolves the 8 corner rows of one query.  Returns false (all rows invalid)
+// when the query is masked out or any neighbour block is missing.
+template <bool LDS>
+__device__ __forceinline__ bool resolve_rows(const QDev& a,
+                                             const CellLut<LDS>& lut, int64_t q,
+                                             bool in_range, int64_t (&row)[8],
+                                             float (&o)[3]) {
+    bool valid = in_range && a.mask[q] != 0;
+    int64_t gi = 0, ci = 0;
+    o[0] = o[1] = o[2] = 0.f;
+    if (valid) {
+        gi = a.gidx[q];
+        ci = a.cidx[q];
+        o[0] = a.off[q * 3 + 0];
+        o[1] = a.off[q * 3 + 1];
+        o[2] = a.off[q * 3 + 2];
+        valid = gi >= 0 && gi < a.B;
+        ci = ci < 0 ? 0 : (ci >= a.M ? a.M - 1 : ci);
+    }
+    int64_t g0 = -1;
+    if (valid) g0 = a.lut_g[gi * 8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        row[c] = -1;
+        if (valid) {
+            int nb_cell, nb_grid;
+            lut.get(ci, c, nb_cell, nb_grid);
+            int64_t g = g0;
+            if (nb_grid != 0) g = a.lut_g[gi * 8 + nb_grid];
+            if (g < 0 || g >= a.B) {
+                valid = false;
+            } else {
+                row[c] = g * a.M + nb_cell;
+            }
+        }
+    }
+    return valid;
+}
+
+template <typename T, int VEC>
+struct VecOf;
+template <>
+struct VecOf<float, 4> {
+    using type = float4;
+};
+template <>
+struct VecOf<float, 1> {
+    using type = float;
+};
+template <>
+struct VecOf<double, 1> {
+    using type = double;
+};
+
+// ------------------------------------------------------------- forward
+template <typename T, int VEC, int LPQ, bool LDS>
+__global__ __launch_bounds__(kBlock) void query_forward_kernel(
+        QDev a, T* __restrict__ out) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
+    constexpr int kQpb = kBlock / LPQ;
+    const int sub = threadIdx.x % LPQ;
+    const int ch0 = sub * VEC;
+    const bool chv = ch0 < a.E;
+    const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
+        const bool in_range = q < a.N;
+        int64_t row[8];
+        float o[3];
+        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
+        T acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = T(0);
+        if (valid && chv) {
+            AxisTerms<T> t;
+            axis_terms<T>(o, a.smooth, t);
+            using V = typename VecOf<T, VEC>::type;
+            V e[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                e[c] = *reinterpret_cast<const V*>(emb + row[c] * a.E + ch0);
+            }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const T w = corner_weight<T>(t, c);
+                const T* ev = reinterpret_cast<const T*>(&e[c]);
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] += w * ev[v];
+            }
+        }
+        if (in_range && chv) {
+            using V = typename VecOf<T, VEC>::type;
+            *reinterpret_cast<V*>(out + q * a.E + ch0) =
+                    *reinterpret_cast<const V*>(acc);
+        }
+    }
+}
+
+// ------------------------------------------------- run merge for atomics
+template <int LPQ>
+__device__ __forceinline__ void run_flags(int64_t row, int lane, bool& head,
+                                          bool& tail) {
+    constexpr int kGroups = 64 / LPQ;
+    const int grp = lane / LPQ;
+    const int64_t prev = __shfl_up(row, LPQ);
+    const int64_t next = __shfl_down(row, LPQ);
+    head = (grp == 0) || (prev != row);
+    tail = (grp == kGroups - 1) || (next != row);
+}
+
+// Inclusive segmented sum over the query groups of a wavefront: after the
+// call the last group of every run of equal rows holds the run's total.
+template <typename T, int LPQ>
+__device__ __forceinline__ T run_sum(T v, bool head, int lane) {
+    constexpr int kGroups = 64 / LPQ;
+    const int grp = lane / LPQ;
+    int f = head ? 1 : 0;
+#pragma unroll
+    for (int d = 1; d < kGroups; d <<= 1) {
+        const T vu = __shfl_up(v, d * LPQ);
+        const int fu = __shfl_up(f, d * LPQ);
+        if (grp >= d && !f) {
+            v += vu;
+            f |= fu;
+        }
+    }
+    return v;
+}
+
+template <typename T, int LPQ, bool MERGE>
+__device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
+                                               int64_t row, int E, int ch,
+                                               bool on, T v, int lane) {
+    if constexpr (MERGE) {
+        bool head, tail;
+        run_flags<LPQ>(on ? row : -1 - static_cast<int64_t>(lane / LPQ), lane,
+                       head, tail);
+        v = run_sum<T, LPQ>(on ? v : T(0), head, lane);
+        if (on && tail) unsafeAtomicAdd(grad_emb + row * E + ch, v);
+    } else {
+        if (on) unsafeAtomicAdd(grad_emb + row * E + ch, v);
+    }
+}
+
+// --------------------------------------------------- backward (first order)
+// grad_embeddings[row_c, k] += w_c * z[i,k];
+// grad_offsets[i,:] = sum_c (emb[row_c,:] . z[i,:]) * grad w_c
+// (ash/src/grid.cu:177-255).  One lane per channel.
+template <typename T, int LPQ, bool LDS, bool MERGE>
+__global__ __launch_bounds__(kBlock) void query_backward_forward_kernel(
+        QDev a, const T* __restrict__ z, T* __restrict__ grad_emb,
+        T* __restrict__ grad_off) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
+    constexpr int kQpb = kBlock / LPQ;
+    const int lane = threadIdx.x & 63;
+    const int ch = threadIdx.x % LPQ;
+    const bool chv = ch < a.E;
+    const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
+        const bool in_range = q < a.N;
+        int64_t row[8];
+        float o[3];
+        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
+        const bool on = valid && chv;
+        AxisTerms<T> t;
+        axis_terms<T>(o, a.smooth, t);
+        const T zk = on ? z[q * a.E + ch] : T(0);
+        T e[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            e[c] = on ? emb[row[c] * a.E + ch] : T(0);
+        }
+        T go[3] = {T(0), T(0), T(0)};
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const T w = corner_weight<T>(t, c);
+            T gw[3];
+            corner_weight_grad<T>(t, c, gw);
+            accumulate_row<T, LPQ, MERGE>(grad_emb, row[c], a.E, ch, on, w * zk,
+                                          lane);
+            T dot = e[c] * zk;
+#pragma unroll
+            for (int s = 1; s < LPQ; s <<= 1) dot += __shfl_xor(dot, s);
+            go[0] += dot * gw[0];
+            go[1] += dot * gw[1];
+            go[2] += dot * gw[2];
+        }
+        if (in_range && ch == 0) {
+            grad_off[q * 3 + 0] = valid ? go[0] : T(0);
+            grad_off[q * 3 + 1] = valid ? go[1] : T(0);
+            grad_off[q * 3 + 2] = valid ? go[2] : T(0);
+        }
+    }
+}
+
+// -------------------------------------------------- backward of backward
+// d_c = grad w_c . gg_off[i];  grad_embeddings[row_c,k] += d_c * z[i,k];
+// grad_z[i,k] = sum_c d_c * emb[row_c,k]   (ash/src/grid.cu:309-387).
+template <typename T, int LPQ, bool LDS, bool MERGE>
+__global__ __launch_bounds__(kBlock) void query_backward_backward_kernel(
+        QDev a, const T* __restrict__ gg_off, const T* __restrict__ z,
+        T* __restrict__ grad_z, T* __restrict__ grad_emb) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
+    constexpr int kQpb = kBlock / LPQ;
+    const int lane = threadIdx.x & 63;
+    const int ch = threadIdx.x % LPQ;
+    const bool chv = ch < a.E;
+    const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
+        const bool in_range = q < a.N;
+        int64_t row[8];
+        float o[3];
+        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
+        const bool on = valid && chv;
+        AxisTerms<T> t;
+        axis_terms<T>(o, a.smooth, t);
+        const T zk = on ? z[q * a.E + ch] : T(0);
+        T gg[3] = {T(0), T(0), T(0)};
+        if (valid) {
+            gg[0] = gg_off[q * 3 + 0];
+            gg[1] = gg_off[q * 3 + 1];
+            gg[2] = gg_off[q * 3 + 2];
+        }
+        T e[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            e[c] = on ? emb[row[c] * a.E + ch] : T(0);
+        }
+        T gz = T(0);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            T gw[3];
+            corner_weight_grad<T>(t, c, gw);
+            const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
+            accumulate_row<T, LPQ, MERGE>(grad_emb, row[c], a.E, ch, on, d * zk,
+                                          lane);
+            gz += d * e[c];
+        }
+        if (in_range && chv) grad_z[q * a.E + ch] = on ? gz : T(0);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p,
+                                                        int64_t n16) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    const uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+         i < n16; i += stride) {
+        p[i] = v;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void zero1_kernel(
+        unsigned char* __restrict__ p, int64_t n) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+         i < n; i += stride) {
+        p[i] = 0;
+    }
+}
+
+// ---------------------------------------------------------------- host
+int zero_fill(void* ptr, int64_t bytes, hipStream_t s) {
+    if (bytes <= 0) return 0;
+    unsigned char* p = static_cast<unsigned char*>(ptr);
+    // unaligned head
+    const int64_t mis = (16 - reinterpret_cast<uintptr_t>(p) % 16) % 16;
+    const int64_t head = mis < bytes ? mis : bytes;
+    if (head > 0) {
+        zero1_kernel<<<1, kBlock, 0, s>>>(p, head);
+        ASH_LAUNCH_CHECK();
+    }
+    const int64_t n16 = (bytes - head) / 16;
+    if (n16 > 0) {
+        int64_t g = (n16 + kBlock - 1) / kBlock;
+        if (g > 256 * 64) g = 256 * 64;
+        zero16_kernel<<<static_cast<unsigned>(g), kBlock, 0, s>>>(
+                reinterpret_cast<uint4*>(p + head), n16);
+        ASH_LAUNCH_CHECK();
+    }
+    const int64_t tail = bytes - head - n16 * 16;
+    if (tail > 0) {
+        zero1_kernel<<<1, kBlock, 0, s>>>(p + head + n16 * 16, tail);
+        ASH_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int check_args(const ash_query_args* a, QDev& d) {
+    if (a == nullptr) ASH_FAIL("null query arguments");
+    if (a->num_queries < 0) ASH_FAIL("negative query count");
+    if (a->num_embeddings < 1 || a->cells_per_grid < 1) {
+        ASH_FAIL("embeddings must have at least one block and one cell");
+    }
+    if (a->embedding_dim < 1 || a->embedding_dim > 16) {
+        ASH_FAIL("embedding_dim must be in 1..16");
+    }
+    if (a->interpolation != ASH_INTERP_LINEAR &&
+        a->interpolation != ASH_INTERP_SMOOTH_STEP) {
+        ASH_FAIL("Unknown interpolation functor");
+    }
+    if (a->dtype != ASH_F32 && a->dtype != ASH_F64) ASH_FAIL("unknown dtype");
+    if (a->embeddings == nullptr || a->lut_grid_nb2grid_idx == nullptr ||
+        a->lut_cell_nb2cell_idx == nullptr || a->lut_cell_nb2grid_nb == nullptr) {
+        ASH_FAIL("null table pointer");
+    }
+    if (a->num_queries > 0 &&
+        (a->offsets == nullptr || a->grid_indices == nullptr ||
+         a->cell_indices == nullptr || a->masks == nullptr)) {
+        ASH_FAIL("null query pointer");
+    }
+    d.emb = a->embeddings;
+    d.off = a->offsets;
+    d.gidx = a->grid_indices;
+    d.cidx = a->cell_indices;
+    d.mask = a->masks;
+    d.lut_g = a->lut_grid_nb2grid_idx;
+    d.lut_c2c = a->lut_cell_nb2cell_idx;
+    d.lut_c2g = a->lut_cell_nb2grid_nb;
+    d.N = a->num_queries;
+    d.B = a->num_embeddings;
+    d.M = a->cells_per_grid;
+    d.E = static_cast<int>(a->embedding_dim);
+    d.smooth = a->interpolation == ASH_INTERP_SMOOTH_STEP ? 1 : 0;
+    return 0;
+}
+
+int pow2_ceil(int v) {
+    int p = 1;
+    while (p < v) p <<= 1;
+    return p;
+}
+
+unsigned persistent_grid(int64_t ntiles) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount,
+                                  dev) == hipSuccess &&
+            n > 0) {
+            cus = n;
+        } else {
+            cus = 256;
+        }
+    }
+    int64_t g = static_cast<int64_t>(cus) * 8;
+    if (g > ntiles) g = ntiles;
+    g = (g + kXcds - 1) / kXcds * kXcds;  // whole rounds over the XCDs
+    if (g < kXcds) g = kXcds;
+    return static_cast<unsigned>(g);
+}
+
+bool merge_enabled() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = std::getenv("ASH_BWD_MERGE");
+        v = (e != nullptr && e[0] == '0') ? 0 : 1;
+    }
+    return v == 1;
+}
+
+size_t lds_bytes(const QDev& d, bool lds) {
+    return lds ? static_cast<size_t>(d.M) * 8 * 3 : 0;
+}
+
+template <typename T, int VEC, int LPQ>
+int launch_forward(const QDev& d, void* out, hipStream_t s) {
+    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
+    const unsigned g = persistent_grid(ntiles);
+    const bool lds = d.M <= kMaxLdsCells;
+    if (lds) {
+        query_forward_kernel<T, VEC, LPQ, true>
+                <<<g, kBlock, lds_bytes(d, true), s>>>(d, static_cast<T*>(out));
+    } else {
+        query_forward_kernel<T, VEC, LPQ, false>
+                <<<g, kBlock, 0, s>>>(d, static_cast<T*>(out));
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T, int LPQ>
+int launch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
+                   hipStream_t s) {
+    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
+    const unsigned g = persistent_grid(ntiles);
+    const bool lds = d.M <= kMaxLdsCells;
+    const bool merge = merge_enabled();
+#define ASH_BF(L, M)                                                          \
+    query_backward_forward_kernel<T, LPQ, L, M>                               \
+            <<<g, kBlock, lds_bytes(d, L), s>>>(d, static_cast<const T*>(z),  \
+                                                static_cast<T*>(ge),          \
+                                                static_cast<T*>(go))
+    if (lds && merge) {
+        ASH_BF(true, true);
+    } else if (lds) {
+        ASH_BF(true, false);
+    } else if (merge) {
+        ASH_BF(false, true);
+    } else {
+        ASH_BF(false, false);
+    }
+#undef ASH_BF
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T, int LPQ>
+int launch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
+                   void* ge, hipStream_t s) {
+    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
+    const unsigned g = persistent_grid(ntiles);
+    const bool lds = d.M <= kMaxLdsCells;
+    const bool merge = merge_enabled();
+#define ASH_BB(L, M)                                                          \
+    query_backward_backward_kernel<T, LPQ, L, M>                              \
+            <<<g, kBlock, lds_bytes(d, L), s>>>(                              \
+                    d, static_cast<const T*>(gg), static_cast<const T*>(z),   \
+                    static_cast<T*>(gz), static_cast<T*>(ge))
+    if (lds && merge) {
+        ASH_BB(true, true);
+    } else if (lds) {
+        ASH_BB(true, false);
+    } else if (merge) {
+        ASH_BB(false, true);
+    } else {
+        ASH_BB(false, false);
+    }
+#undef ASH_BB
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T>
+int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
+    if constexpr (sizeof(T) == 4) {
+        if (d.E % 4 == 0) {
+            switch (d.E / 4) {
+                case 1:
+                    return launch_forward<float, 4, 1>(d, out, s);
+                case 2:
+                    return launch_forward<float, 4, 2>(d, out, s);
+                default:
+                    return launch_forward<float, 4, 4>(d, out, s);
+            }
+        }
+    }
+    switch (pow2_ceil(d.E)) {
+        case 1:
+            return launch_forward<T, 1, 1>(d, out, s);
+        case 2:
+            return launch_forward<T, 1, 2>(d, out, s);
+        case 4:
+            return launch_forward<T, 1, 4>(d, out, s);
+        case 8:
+            return launch_forward<T, 1, 8>(d, out, s);
+        default:
+            return launch_forward<T, 1, 16>(d, out, s);
+    }
+}
+
+template <typename T>
+int dispatch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
+                     hipStream_t s) {
+    switch (pow2_ceil(d.E)) {
+        case 1:
+            return launch_bwd_fwd<T, 1>(d, z, ge, go, s);
+        case 2:
+            return launch_bwd_fwd<T, 2>(d, z, ge, go, s);
+        case 4:
+            return launch_bwd_fwd<T, 4>(d, z, ge, go, s);
+        case 8:
+            return launch_bwd_fwd<T, 8>(d, z, ge, go, s);
+        default:
+            return launch_bwd_fwd<T, 16>(d, z, ge, go, s);
+    }
+}
+
+template <typename T>
+int dispatch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
+                     void* ge, hipStream_t s) {
+    switch (pow2_ceil(d.E)) {
+        case 1:
+            return launch_bwd_bwd<T, 1>(d, gg, z, gz, ge, s);
+        case 2:
+            return launch_bwd_bwd<T, 2>(d, gg, z, gz, ge, s);
+        case 4:
+            return launch_bwd_bwd<T, 4>(d, gg, z, gz, ge, s);
+        case 8:
+            return launch_bwd_bwd<T, 8>(d, gg, z, gz, ge, s);
+        default:
+            return launch_bwd_bwd<T, 16>(d, gg, z, gz, ge, s);
+    }
+}
+
+int64_t elem_bytes(int dtype) { return dtype == ASH_F64 ? 8 : 4; }
+
+}  // namespace
+}  // namespace ash
+
+using namespace ash;
+
+extern "C" {
+
+int ash_query_forward(const ash_query_args* a, void* output, void* stream) {
+    QDev d;
+    if (check_args(a, d)) return 1;
+    if (d.N == 0) return 0;
+    if (output == nullptr) ASH_FAIL("null output pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return a->dtype == ASH_F64 ? dispatch_forward<double>(d, output, s)
+                               : dispatch_forward<float>(d, output, s);
+}
+
+int ash_query_backward_forward(const ash_query_args* a, const void* z,
+                               void* grad_embeddings, void* grad_offsets,
+                               void* stream) {
+    QDev d;
+    if (check_args(a, d)) return 1;
+    if (grad_embeddings == nullptr) ASH_FAIL("null grad_embeddings pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
+        return 1;
+    }
+    if (d.N == 0) return 0;
+    if (z == nullptr || grad_offsets == nullptr) ASH_FAIL("null pointer");
+    return a->dtype == ASH_F64
+                   ? dispatch_bwd_fwd<double>(d, z, grad_embeddings,
+                                              grad_offsets, s)
+                   : dispatch_bwd_fwd<float>(d, z, grad_embeddings,
+                                             grad_offsets, s);
+}
+
+int ash_query_backward_backward(const ash_query_args* a,
+                                const void* grad_grad_offsets, const void* z,
+                                void* grad_z, void* grad_embeddings,
+                                void* stream) {
+    QDev d;
+    if (check_args(a, d)) return 1;
+    if (grad_embeddings == nullptr) ASH_FAIL("null grad_embeddings pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
+        return 1;
+    }
+    if (d.N == 0) return 0;
+    if (z == nullptr || grad_grad_offsets == nullptr || grad_z == nullptr) {
+        ASH_FAIL("null pointer");
+    }
+    return a->dtype == ASH_F64
+                   ? dispatch_bwd_bwd<double>(d, grad_grad_offsets, z, grad_z,
+                                              grad_embeddings, s)
+                   : dispatch_bwd_bwd<float>(d, grad_grad_offsets, z, grad_z,
+                                             grad_embeddings, s);
+}
+
+}  // extern "C"
