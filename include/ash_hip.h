@@ -130,6 +130,20 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
 int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
                  int64_t n, const int32_t* heap_src, void* stream);
 
+/* Erasing from buckets that have been full, and refusing keys of an overfull
+ * batch, leaves tombstoned slots behind.  `ash_map_should_rebuild` (host
+ * arithmetic only) says whether, with `size` live entries, `tombstones`
+ * tombstones and `incoming` keys about to arrive, fewer than a fifth of the
+ * slots would stay empty.  `ash_map_rebuild` then re-places the `n` = size live
+ * (key, index) pairs into a cleared table; indices, heap and size are
+ * untouched.  keys_scratch int32[n,key_dim] and indices_scratch int64[n] are
+ * device temporaries.  No counterpart in the reference, whose container
+ * recycles slots itself. */
+int ash_map_should_rebuild(ash_map_t* map, int64_t size, int64_t tombstones,
+                           int64_t incoming);
+int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
+                    int64_t* indices_scratch, int64_t n, void* stream);
+
 /* Generic row scatter used by the wide-row path of ash_map_insert, exported
  * because the Python layer reuses it: dst[assigned[i]] = src[i] for
  * assigned[i] >= 0. */

@@ -1,0 +1,327 @@
+"""GPU parity tests of the trilinear query kernels against the CPU oracle on
+identical seeded inputs.  fp32 tolerance (north-star): 1e-5 relative / 1e-6
+absolute; gradients accumulated by atomics in a different order are compared
+with the same tolerance scaled by the number of accumulated terms where noted.
+fp64 runs use 1e-12 / 1e-13."""
+import pytest
+import torch
+
+import workloads
+from helpers import torch_query
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+RTOL32, ATOL32 = 1e-5, 1e-6
+
+
+def _tol(dtype):
+    return dict(rtol=RTOL32, atol=ATOL32) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-13)
+
+
+def _make_grid(ash, grid_dim, embedding_dim, bound, dtype=torch.float32, seed=0, holes=0):
+    """Blocks -bound..bound in each axis (minus `holes` random ones) with
+    uniform(-1,1) embeddings and the neighbour table built."""
+    g = torch.Generator().manual_seed(seed)
+    side = 2 * bound + 1
+    grid = ash.SparseDenseGrid(3, side**3 + 5, embedding_dim, grid_dim, device=DEV)
+    r = torch.arange(-bound, bound + 1, dtype=torch.int32)
+    blocks = torch.stack(torch.meshgrid(r, r, r, indexing="ij"), dim=-1).view(-1, 3)
+    if holes:
+        blocks = blocks[torch.randperm(len(blocks), generator=g)[holes:]]
+    grid.engine.insert_keys(blocks.to(DEV))
+    with torch.no_grad():
+        grid.embeddings.copy_((torch.rand(grid.embeddings.shape, generator=g) * 2 - 1).to(DEV))
+    if dtype != torch.float32:
+        grid.embeddings.data = grid.embeddings.data.to(dtype)
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    return grid
+
+
+def _queries(grid_dim, bound, n, seed, margin=0.0):
+    g = torch.Generator().manual_seed(seed)
+    lo, hi = -grid_dim * bound - margin, grid_dim * (bound + 1) + margin
+    return (torch.rand(n, 3, generator=g) * (hi - lo) + lo).to(DEV)
+
+
+def _operands(grid, x):
+    gi, ci, off, masks = grid.query(x)
+    return (
+        grid.embeddings.detach(), off, gi, ci, masks,
+        grid.lut_grid_nb2grid_idx, grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb,
+    )
+
+
+def _to_cpu(ops):
+    return tuple(o.cpu() for o in ops)
+
+
+def _compare_all(ash, oracle, grid, x, interpolation, seed=0, grad_scale=1.0):
+    ops = _operands(grid, x)
+    cops = _to_cpu(ops)
+    dtype = ops[0].dtype
+    n, e, g_dim = x.shape[0], ops[0].shape[2], grid.grid_dim
+    backend = ash.grid_query.backend
+    gen = torch.Generator().manual_seed(seed)
+    z = (torch.rand(n, e, generator=gen, dtype=torch.float64) - 0.5).to(dtype)
+    u = (torch.rand(n, 3, generator=gen, dtype=torch.float64) - 0.5).to(dtype)
+    tol = _tol(dtype)
+    gtol = dict(rtol=tol["rtol"], atol=tol["atol"] * grad_scale)
+
+    y = backend.query_forward(*ops, g_dim, interpolation)
+    y_ref = oracle.query_forward(*cops, g_dim, interpolation)
+    assert torch.allclose(y.cpu(), y_ref, **tol), (y.cpu() - y_ref).abs().max()
+
+    ge, go = backend.query_backward_forward(z.to(DEV), *ops, g_dim, interpolation)
+    ge_ref, go_ref = oracle.query_backward_forward(z, *cops, g_dim, interpolation)
+    assert torch.allclose(go.cpu(), go_ref, **gtol), (go.cpu() - go_ref).abs().max()
+    assert torch.allclose(ge.cpu(), ge_ref, **gtol), (ge.cpu() - ge_ref).abs().max()
+
+    gz, ge2, goff2 = backend.query_backward_backward(
+        torch.zeros_like(ops[0]), u.to(DEV), z.to(DEV), *ops, g_dim, interpolation
+    )
+    gz_ref, ge2_ref, _ = oracle.query_backward_backward(None, u, z, *cops, g_dim, interpolation)
+    assert torch.allclose(gz.cpu(), gz_ref, **gtol), (gz.cpu() - gz_ref).abs().max()
+    assert torch.allclose(ge2.cpu(), ge2_ref, **gtol), (ge2.cpu() - ge2_ref).abs().max()
+    assert float(goff2.abs().sum()) == 0.0
+    return ops
+
+
+@pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
+@pytest.mark.parametrize("embedding_dim", [1, 2, 3, 4, 5, 8, 12, 16])
+def test_all_embedding_dims_fp32(gpu_ash, oracle, interpolation, embedding_dim):
+    grid = _make_grid(gpu_ash, 4, embedding_dim, 1, seed=embedding_dim, holes=3)
+    x = _queries(4, 1, 6000, seed=100 + embedding_dim, margin=2.0)
+    # a few queries per cell: sums of a handful of O(1) terms
+    _compare_all(gpu_ash, oracle, grid, x, interpolation, seed=embedding_dim, grad_scale=8.0)
+
+
+@pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
+@pytest.mark.parametrize("grid_dim", [1, 2, 8, 16])
+def test_all_grid_dims_fp32(gpu_ash, oracle, interpolation, grid_dim):
+    """grid_dim 16 has 4096 cells per block: the per-cell tables no longer fit
+    the LDS staging and are read through the caches."""
+    grid = _make_grid(gpu_ash, grid_dim, 4, 1, seed=grid_dim, holes=2)
+    x = _queries(grid_dim, 1, 5000, seed=200 + grid_dim, margin=1.0)
+    _compare_all(gpu_ash, oracle, grid, x, interpolation, seed=grid_dim, grad_scale=64.0)
+
+
+@pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
+@pytest.mark.parametrize("embedding_dim", [1, 4, 7, 16])
+def test_fp64(gpu_ash, oracle, interpolation, embedding_dim):
+    grid = _make_grid(gpu_ash, 4, embedding_dim, 1, dtype=torch.float64, seed=7, holes=3)
+    x = _queries(4, 1, 4000, seed=300 + embedding_dim, margin=2.0)
+    _compare_all(gpu_ash, oracle, grid, x, interpolation, seed=3, grad_scale=100.0)
+
+
+def test_repeated_cells_merge_path(gpu_ash, oracle):
+    """Ray-like input: long runs of consecutive queries in one cell, the case
+    the per-wavefront pre-reduction of atomics is for."""
+    grid = _make_grid(gpu_ash, 8, 4, 1, seed=11)
+    g = torch.Generator().manual_seed(12)
+    starts = torch.rand(300, 1, 3, generator=g) * 20 - 6
+    steps = torch.arange(64).view(1, -1, 1) * torch.rand(300, 1, 3, generator=g) * 0.05
+    x = (starts + steps).view(-1, 3).to(DEV)
+    for interpolation in ("linear", "smooth_step"):
+        _compare_all(gpu_ash, oracle, grid, x, interpolation, seed=13, grad_scale=64.0)
+
+
+def test_empty_batch_and_bad_arguments(gpu_ash):
+    grid = _make_grid(gpu_ash, 2, 3, 1, seed=5)
+    backend = gpu_ash.grid_query.backend
+    x = _queries(2, 1, 10, seed=1)
+    ops = _operands(grid, x)
+    empty = (ops[0], ops[1][:0], ops[2][:0], ops[3][:0], ops[4][:0]) + ops[5:]
+    y = backend.query_forward(*empty, 2, "linear")
+    assert y.shape == (0, 3)
+    ge, go = backend.query_backward_forward(torch.zeros((0, 3), device=DEV), *empty, 2, "linear")
+    assert ge.shape == ops[0].shape and float(ge.abs().sum()) == 0 and go.shape == (0, 3)
+    with pytest.raises(RuntimeError, match="Unknown interpolation"):
+        backend.query_forward(*ops, 2, "cubic")
+    with pytest.raises(RuntimeError):
+        backend.query_forward(ops[0].cpu(), *ops[1:], 2, "linear")
+
+
+@pytest.mark.parametrize("grid_dim", [1, 4, 8])
+def test_reference_forward_closed_form(gpu_ash, grid_dim):
+    """unittests/test_sparsedense_grid.py:139-181: embeddings := coordinates."""
+    bound = 3
+    grid = gpu_ash.SparseDenseGrid(3, 1000, 3, grid_dim, device=DEV)
+    r = torch.arange(-bound, bound + 1, dtype=torch.int, device=DEV)
+    blocks = grid_dim * torch.stack(torch.meshgrid(r, r, r, indexing="ij"), dim=-1).view(-1, 3)
+    grid.spatial_init_(blocks, dilation=0)
+    gc, cc, gi, ci = grid.items()
+    coords = (gc * grid_dim + cc).view(-1, 3).float()
+    with torch.no_grad():
+        grid.embeddings[gi, ci, :3] = coords.view(gi.shape[0], ci.shape[1], 3)
+    q = (2 * grid_dim * bound - 1) * torch.rand(1000, 3, device=DEV) - grid_dim * bound
+    emb, masks = grid(q, interpolation="linear")
+    assert torch.allclose(emb[..., :3], q, rtol=1e-5, atol=1e-4)
+    assert bool(masks.all())
+    feats, masks = grid(coords, interpolation="nearest")
+    gi2, ci2, off, _ = grid.query(coords)
+    assert torch.allclose(off, torch.zeros_like(off))
+    assert torch.equal(feats, grid.embeddings[gi2, ci2])
+    feats.sum().backward()
+    assert grid.embeddings.grad is not None
+
+
+class _SineMLP(torch.nn.Module):
+    """Small sine network standing in for the reference tests' SirenNet."""
+
+    def __init__(self, d_in, d_hidden=32):
+        super().__init__()
+        self.a = torch.nn.Linear(d_in, d_hidden)
+        self.b = torch.nn.Linear(d_hidden, 1)
+
+    def forward(self, x):
+        return self.b(torch.sin(3.0 * self.a(x)))
+
+
+@pytest.mark.parametrize("embedding_dim,grid_dim", [(2, 1), (1, 2), (4, 4), (8, 8)])
+def test_reference_gradcheck(gpu_ash, embedding_dim, grid_dim):
+    """unittests/test_sparsedense_grid.py:183-281: gradcheck w.r.t. positions
+    and w.r.t. embeddings through a small network, fp32, eps 1e-3, tol 1e-2."""
+    torch.manual_seed(15213)
+    grid = gpu_ash.SparseDenseGrid(3, 8, embedding_dim, grid_dim, device=DEV)
+    r = torch.arange(0, 2, dtype=torch.int, device=DEV)
+    blocks = grid_dim * torch.stack(torch.meshgrid(r, r, r, indexing="ij"), dim=-1).view(-1, 3)
+    grid.spatial_init_(blocks, dilation=0)
+    torch.nn.init.uniform_(grid.embeddings, -1, 1)
+    eps = 1e-3
+    cells = torch.randint(high=grid_dim * 2 - 1, size=(200, 3), device=DEV)
+    frac = torch.rand(200, 3, device=DEV).clamp(2 * eps, 1 - 2 * eps)
+    positions = (cells + frac).requires_grad_(True)
+    net = _SineMLP(embedding_dim + 3).to(DEV)
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+
+    def run(embeddings, x_in, interpolation):
+        gi, ci, off, masks = grid.query(grid.transform_world_to_cell(x_in))
+        assert bool(masks.all())
+        feats = gpu_ash.SparseDenseGridQuery.apply(
+            embeddings, off, gi, ci, masks, grid.lut_grid_nb2grid_idx,
+            grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, grid.grid_dim, interpolation,
+        )
+        return net(torch.cat((feats, x_in), dim=-1))
+
+    torch.autograd.gradcheck(
+        lambda x: run(grid.embeddings, x, "linear"), (positions,), eps=eps, atol=1e-2, rtol=1e-2,
+        nondet_tol=1e-4,
+    )
+    torch.autograd.gradcheck(
+        lambda e: run(e, positions, "smooth_step"), (grid.embeddings,), eps=eps, atol=1e-2,
+        rtol=1e-2, nondet_tol=1e-4,
+    )
+
+
+def test_double_backward_gradcheck_fp64(gpu_ash):
+    """unittests/test_sparsedense_grid.py:283-347 (defined upstream, never
+    called): fp64 gradcheck of SparseDenseGridQueryBackward w.r.t. embeddings
+    and w.r.t. z."""
+    torch.manual_seed(1)
+    grid_dim, e = 4, 3
+    grid = gpu_ash.SparseDenseGrid(3, 8, e, grid_dim, device=DEV)
+    r = torch.arange(0, 2, dtype=torch.int, device=DEV)
+    blocks = grid_dim * torch.stack(torch.meshgrid(r, r, r, indexing="ij"), dim=-1).view(-1, 3)
+    grid.spatial_init_(blocks, dilation=0)
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    cells = torch.randint(high=grid_dim * 2 - 1, size=(60, 3), device=DEV)
+    positions = cells + torch.rand(60, 3, device=DEV).clamp(0.01, 0.99)
+    gi, ci, off, masks = grid.query(positions)
+    emb64 = (torch.rand(grid.embeddings.shape, device=DEV, dtype=torch.float64) * 2 - 1).requires_grad_(True)
+    z = torch.rand(60, e, device=DEV, dtype=torch.float64).requires_grad_(True)
+
+    def grad_offsets(embeddings, zz):
+        return gpu_ash.SparseDenseGridQueryBackward.apply(
+            zz, embeddings, off, gi, ci, masks, grid.lut_grid_nb2grid_idx,
+            grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, grid.grid_dim, "smooth_step",
+        )[1]
+
+    torch.autograd.gradcheck(grad_offsets, (emb64, z), eps=1e-6, atol=1e-6, rtol=1e-6, nondet_tol=1e-9)
+
+
+@pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
+def test_eikonal_training_step_matches_autograd(gpu_ash, interpolation):
+    """The flow of configuration 4 end to end through the module: value loss +
+    gradient-norm loss, second-order backward to the embeddings; compared with
+    float64 autograd of the independent torch formula.  The offsets-Hessian
+    term the reference leaves out (ash/src/grid.cu:417-418) is removed from the
+    comparison by detaching the positions inside the formula's gradient."""
+    grid = _make_grid(gpu_ash, 4, 4, 1, seed=21)
+    x = _queries(4, 1, 3000, seed=22).requires_grad_(True)
+
+    feats, masks = grid(x, interpolation)
+    sdf = feats[:, 0]
+    (grad_x,) = torch.autograd.grad(sdf.sum(), x, create_graph=True)
+    loss = (feats[:, 1:] ** 2).mean() + ((grad_x.norm(dim=-1) - 1) ** 2).mean()
+    loss.backward()
+    got = grid.embeddings.grad.detach().cpu().double()
+
+    gi, ci, off, masks2 = grid.query(x.detach())
+    ops = [o.cpu() for o in (gi, ci, masks2, grid.lut_grid_nb2grid_idx,
+                             grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)]
+    emb = grid.embeddings.detach().cpu().double().requires_grad_(True)
+    off_leaf = off.detach().cpu().requires_grad_(True)
+    y = torch_query(emb, off_leaf, *ops, interpolation)
+    (gx,) = torch.autograd.grad(y[:, 0].sum(), off_leaf, create_graph=True)
+    ref_loss = (y[:, 1:] ** 2).mean() + ((gx.norm(dim=-1) - 1) ** 2).mean()
+    (ref,) = torch.autograd.grad(ref_loss, emb)
+    assert abs(loss.item() - ref_loss.item()) < 1e-5 * max(1.0, abs(ref_loss.item()))
+    assert torch.allclose(got, ref, rtol=1e-4, atol=1e-6), (got - ref).abs().max()
+
+
+def _config_grid(gpu_ash, embedding_dim, num_blocks=3000, sparse=64):
+    return workloads.build_grid(
+        gpu_ash, num_blocks, embedding_dim, grid_dim=8, sparse_grid_dim=sparse, device=DEV
+    )
+
+
+def test_config3_reduced_against_oracle(gpu_ash, oracle):
+    """Configuration 3 at reduced size: bounded grid, 8^3 cells, E = 16,
+    queries uniform in active blocks plus 10 % in empty space."""
+    grid, _, _ = _config_grid(gpu_ash, 16)
+    x = workloads.uniform_queries(grid, 60000)
+    cells = grid.transform_world_to_cell(x)
+    for interpolation in ("linear", "smooth_step"):
+        ops = _operands(grid, cells)
+        masks = ops[4]
+        assert 0.85 < float(masks.float().mean()) < 0.95
+        y = gpu_ash.grid_query.backend.query_forward(*ops, 8, interpolation)
+        y_ref = oracle.query_forward(*_to_cpu(ops), 8, interpolation)
+        assert torch.allclose(y.cpu(), y_ref, rtol=RTOL32, atol=ATOL32)
+        assert float(y[~masks].abs().sum()) == 0.0
+        feats, m2 = grid(x, interpolation)
+        assert torch.equal(m2, masks) and torch.equal(feats.detach(), y)
+
+
+def test_config4_reduced_against_oracle(gpu_ash, oracle):
+    """Configuration 4 at reduced size: E = 4, ray-ordered stratified samples,
+    forward + backward + double backward."""
+    grid, radii, centres = _config_grid(gpu_ash, 4)
+    x = workloads.ray_queries(grid, radii, centres, num_rays=512, samples_per_ray=128)
+    cells = grid.transform_world_to_cell(x)
+    ops = _compare_all(gpu_ash, oracle, grid, cells, "smooth_step", seed=31, grad_scale=256.0)
+    assert float(ops[4].float().mean()) > 0.5
+
+
+def test_full_size_forward_properties(gpu_ash):
+    """Configuration 3 at full size (200 k blocks, E = 16, 4.4 M queries),
+    through properties that need no oracle: linearity in the embeddings,
+    constants reproduced where all 8 corners exist, masked rows zero."""
+    grid, _, _ = workloads.build_grid(gpu_ash, device=DEV)
+    x = workloads.uniform_queries(grid)
+    ops = list(_operands(grid, grid.transform_world_to_cell(x)))
+    backend = gpu_ash.grid_query.backend
+    y1 = backend.query_forward(*ops, 8, "smooth_step")
+    masks = ops[4]
+    assert float(y1[~masks].abs().sum()) == 0.0
+    emb = ops[0]
+    ops[0] = emb * 3.0
+    y3 = backend.query_forward(*ops, 8, "smooth_step")
+    assert torch.allclose(y3, 3.0 * y1, rtol=1e-5, atol=1e-7)
+    ops[0] = torch.ones_like(emb)
+    yc = backend.query_forward(*ops, 8, "smooth_step")
+    row_sum = yc.sum(dim=1)
+    complete = row_sum != 0
+    assert bool((complete <= masks).all())
+    assert float(complete.float().mean()) > 0.7
+    assert torch.allclose(yc[complete], torch.ones_like(yc[complete]), rtol=1e-5, atol=0)

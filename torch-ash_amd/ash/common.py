@@ -87,6 +87,8 @@ _SIGNATURES = {
     "ash_map_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_items": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_map_load": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR, _PTR]),
+    "ash_map_should_rebuild": (ctypes.c_int, [_PTR, _I64, _I64, _I64]),
+    "ash_map_rebuild": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_scatter_rows": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _I64, _PTR]),
     "ash_query_forward": (ctypes.c_int, [ctypes.POINTER(_QueryArgs), _PTR, _PTR]),
     "ash_query_backward_forward": (
@@ -371,6 +373,7 @@ class _HashMap:
         self._general_bytes = general_bytes.value
         self._table = torch.empty(table_bytes.value, dtype=torch.uint8, device=self._device)
         self._general = None
+        self._maybe_tombstones = False
         handle = _PTR()
         with torch.cuda.device(self._device):
             self._check(
@@ -408,10 +411,36 @@ class _HashMap:
             keys = keys.to(torch.int32)
         return keys.contiguous()
 
+    def _make_room(self, incoming: int) -> None:
+        """Before an insert: if earlier erases or refused keys may have left
+        tombstones, look at the counters and re-place the live entries into a
+        cleared table when too few empty slots remain."""
+        if not self._maybe_tombstones:
+            return
+        st = self.status()
+        self._maybe_tombstones = st["tombstones"] > 0
+        if not self._lib.ash_map_should_rebuild(
+            self._handle, st["size"], st["tombstones"], incoming
+        ):
+            return
+        n = st["size"]
+        keys = torch.empty((n, self.key_dim), dtype=torch.int32, device=self._device)
+        indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        with torch.cuda.device(self._device):
+            self._check(
+                self._lib.ash_map_rebuild(
+                    self._handle, keys.data_ptr() if n else None,
+                    indices.data_ptr() if n else None, n, self._stream(),
+                )
+            )
+        self._maybe_tombstones = False
+
     def _attach_general_if_needed(self) -> bool:
         """After an insert/load: keys that need the second region are counted by
         the kernel; attach the region once and let the caller re-issue."""
         st = self.status()
+        if st["dropped"] > 0 or st["tombstones"] > 0:
+            self._maybe_tombstones = True
         if st["exotic_pending"] == 0:
             return False
         if self._general is not None:
@@ -463,6 +492,7 @@ class _HashMap:
 
     def insert_keys(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)
+        self._make_room(keys.shape[0])
         for _ in range(2):
             with torch.cuda.device(self._device):
                 self._check(
@@ -510,6 +540,7 @@ class _HashMap:
         assigned = None
         if self._lib.ash_map_insert_needs_scratch(k, c_rows):
             assigned = torch.empty(n, dtype=torch.int32, device=self._device)
+        self._make_room(n)
         for _ in range(2):
             with torch.cuda.device(self._device):
                 self._check(
@@ -530,6 +561,7 @@ class _HashMap:
 
     def erase(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)
+        self._maybe_tombstones = True
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_erase(
@@ -540,6 +572,7 @@ class _HashMap:
     def clear(self) -> None:
         with torch.cuda.device(self._device):
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
+        self._maybe_tombstones = False
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
         n = self.size()

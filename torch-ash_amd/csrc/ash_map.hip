@@ -1162,6 +1162,49 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     return 0;
 }
 
+int ash_map_should_rebuild(ash_map_t* map, int64_t size, int64_t tombstones,
+                           int64_t incoming) {
+    if (map == nullptr || tombstones <= 0) return 0;
+    int64_t room = map->capacity - size;
+    if (room < 0) room = 0;
+    const int64_t arriving = incoming < room ? incoming : room;
+    int64_t slots = static_cast<int64_t>(map->d.nb) * kSlots;
+    if (map->general_attached && map->d.gslots < slots) slots = map->d.gslots;
+    // keep at least a fifth of the slots truly empty
+    return (size + tombstones + arriving) * 5 > slots * 4 ? 1 : 0;
+}
+
+int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
+                    int64_t* indices_scratch, int64_t n, void* stream) {
+    if (check_map(map)) return 1;
+    if (n < 0 || n > map->capacity) ASH_FAIL("rebuild: bad entry count");
+    if (n > 0 && (keys_scratch == nullptr || indices_scratch == nullptr)) {
+        ASH_FAIL("rebuild: null scratch pointer");
+    }
+    if (n > 0 && ash_map_items(map, keys_scratch, indices_scratch, n, stream)) {
+        return 1;
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t n16 = static_cast<int64_t>(map->d.nb) * kGroup;
+    fill16_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
+            reinterpret_cast<uint4*>(map->d.buckets), n16, 0xFFFFFFFFu);
+    ASH_LAUNCH_CHECK();
+    if (map->general_attached) {
+        const int64_t g16 = static_cast<int64_t>(map->d.gslots) / 4;
+        fill16_kernel<<<capped_grid(g16), kBlock, 0, s>>>(
+                reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
+        ASH_LAUNCH_CHECK();
+    }
+    set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrTombs, 0);
+    ASH_LAUNCH_CHECK();
+    if (n == 0) return 0;
+    ValueArgs va = {};
+    return launch_insert<kInsertLoad>(map, keys_scratch, n, va, nullptr,
+                                      indices_scratch, s);
+}
+
 int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
                  int64_t n, const int32_t* heap_src, void* stream) {
     if (check_batch(map, keys, n)) return 1;
