@@ -1,0 +1,361 @@
+"""Benchmark of the two hot paths on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-trilinear] [--no-cpu]
+
+Headline (`value`): configuration 2 of the baseline -- HashMap with values
+{color: fp32[3], depth: fp32[1]}, 16 M distinct voxel keys into capacity 24 M,
+16 M queries (70 % hits), full items() enumeration.  One step is
+clear + insert + find + items through the public Python API (including its
+host read-backs), inputs resident in HBM; `value` counts the 32 M keys that
+were inserted or looked up per step.
+
+Beside it, on the same JSON line:
+  roofline      the step's longest kernel, timed alone with HIP events on the
+                stream it runs on (raw C-ABI call, no host read-back inside),
+                priced with the algorithmic bytes per key of that operation;
+  kernels       the same figures for every hash kernel and for the trilinear
+                query kernels of configurations 3 and 4;
+  cpu_baseline  the CPU oracle (OpenMP) on a bounded sample of the same
+                workload, on this machine's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for sub in ("torch-ash_amd", "oracle", ""):
+    path = os.path.join(ROOT, sub) if sub else ROOT
+    if path not in sys.path:
+        sys.path.insert(0, path)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X, published
+
+# Algorithmic bytes per unit of work.  A stored slot counts as 16 B (12 B key +
+# 4 B index) whatever the physical layout; E = embedding width; fp32.
+FIND_BYTES = 12 + 16 + 8 + 1                 # key in, slot, index out, mask out
+INSERT_KEY_BYTES = 12 + 16 + 16 + 4          # key in, probe, slot write, heap pop (all unique)
+VALUE_ROW_BYTES = 2 * (12 + 4)               # color + depth, read and written
+
+
+def items_bytes(slots: int, n: int) -> int:
+    return 16 * slots + 20 * n
+
+
+def fwd_bytes(e: int) -> int:
+    return 29 + 36 * e
+
+
+def bwd_bytes(e: int) -> int:
+    return 41 + 100 * e
+
+
+def bwd2_bytes(e: int) -> int:
+    return 41 + 104 * e
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--keys", type=int, default=16_000_000, help="distinct keys (configuration 2)")
+    ap.add_argument("--capacity", type=int, default=24_000_000)
+    ap.add_argument("--no-trilinear", action="store_true", help="skip the trilinear kernel figures")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-keys", type=int, default=4_000_000, help="CPU baseline sample size")
+    return ap.parse_args()
+
+
+class EventTimer:
+    """Average duration of a region on torch's current stream, in ms."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.pairs = []
+
+    def __call__(self, fn):
+        start = self.torch.cuda.Event(enable_timing=True)
+        end = self.torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        self.pairs.append((start, end))
+
+    def mean_ms(self):
+        self.torch.cuda.synchronize()
+        times = [s.elapsed_time(e) for s, e in self.pairs]
+        return sum(times) / max(len(times), 1)
+
+
+def roofline_entry(name, alg_bytes, ms, traffic=None):
+    achieved = alg_bytes / (ms * 1e-3) / 1e9 if ms > 0 else 0.0
+    return {
+        "kernel": name,
+        "bound": "hbm",
+        "achieved": round(achieved, 2),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 5),
+        "traffic": traffic,
+        "ms": round(ms, 4),
+    }
+
+
+def bench_hash(torch, ash, workloads, args, dev):
+    w = workloads.hashmap_sphere_voxels(num_keys=args.keys, device=dev)
+    n = args.keys
+    hm = ash.HashMap(3, {"color": 3, "depth": 1}, args.capacity, dev)
+    values = {"color": w["color"], "depth": w["depth"]}
+
+    def step():
+        hm.clear()
+        hm.insert(w["keys"], values)
+        masks, indices = hm.find(w["query_keys"])
+        keys_out, idx_out = hm.items()
+        return masks, keys_out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        masks, keys_out = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert keys_out.shape[0] == n
+    hits = int(masks.sum())
+    ms_per_step = elapsed / args.steps * 1e3
+
+    # Kernel-only timings through the raw C ABI (no host read-back inside).
+    backend = hm.engine.backend
+    lib, handle = backend._lib, backend._handle
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    keys, queries = w["keys"], w["query_keys"]
+    k = 2
+    c_rows = (ctypes.c_int64 * k)(12, 4)
+    c_src = (ctypes.c_void_p * k)(w["color"].data_ptr(), w["depth"].data_ptr())
+    c_dst = (ctypes.c_void_p * k)(hm.values["color"].data_ptr(), hm.values["depth"].data_ptr())
+    idx_out = torch.empty(n, dtype=torch.int64, device=dev)
+    mask_out = torch.empty(n, dtype=torch.bool, device=dev)
+    items_keys = torch.empty((n, 3), dtype=torch.int32, device=dev)
+    items_idx = torch.empty(n, dtype=torch.int64, device=dev)
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError(lib.ash_last_error().decode())
+
+    t_clear, t_insert, t_insert_keys, t_find, t_items = (EventTimer(torch) for _ in range(5))
+    for it in range(args.warmup + args.steps):
+        timed = it >= args.warmup
+        run = (lambda timer, fn: timer(fn)) if timed else (lambda timer, fn: fn())
+        run(t_clear, lambda: check(lib.ash_map_clear(handle, stream)))
+        run(t_insert_keys, lambda: check(lib.ash_map_insert_keys(handle, keys.data_ptr(), n, stream)))
+        check(lib.ash_map_clear(handle, stream))
+        run(t_insert, lambda: check(lib.ash_map_insert(
+            handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows, None, stream)))
+        run(t_find, lambda: check(lib.ash_map_find(
+            handle, queries.data_ptr(), n, idx_out.data_ptr(), mask_out.data_ptr(), stream)))
+        run(t_items, lambda: check(lib.ash_map_items(
+            handle, items_keys.data_ptr(), items_idx.data_ptr(), n, stream)))
+    assert int(mask_out.sum()) == hits
+    slots = (backend._table.numel() - 256) // 128 * 10
+    kernels = {
+        "insert_values": roofline_entry(
+            "insert_kernel<3,fused>", (INSERT_KEY_BYTES + VALUE_ROW_BYTES) * n, t_insert.mean_ms()),
+        "insert_keys": roofline_entry("insert_kernel<3,keys>", INSERT_KEY_BYTES * n, t_insert_keys.mean_ms()),
+        "find": roofline_entry("find_kernel<3>", FIND_BYTES * n, t_find.mean_ms()),
+        "items": roofline_entry("items_kernel<3>", items_bytes(slots, n), t_items.mean_ms()),
+        "clear": roofline_entry("fill16+reset_heap", 16 * slots + 4 * args.capacity, t_clear.mean_ms()),
+    }
+    for name in ("insert_values", "insert_keys", "find"):
+        kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
+    kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
+    del hm, w
+    torch.cuda.empty_cache()
+    return ms_per_step, hits, kernels
+
+
+def bench_trilinear(torch, ash, workloads, args, dev):
+    """Kernel figures of configurations 3 (E=16 forward) and 4 (E=4 forward,
+    backward, double backward) plus the module-level autograd step of
+    configuration 4."""
+    out = {}
+    backend = ash.grid_query.backend
+    reps = max(args.steps, 3)
+
+    # configuration 3
+    grid, _, _ = workloads.build_grid(ash, 200_000, 16, device=dev)
+    x = workloads.uniform_queries(grid, 4_000_000)
+    gi, ci, off, mk = grid.query(grid.transform_world_to_cell(x))
+    ops = (grid.embeddings.detach(), off, gi, ci, mk, grid.lut_grid_nb2grid_idx,
+           grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)
+    n3 = x.shape[0]
+    for interp in ("linear", "smooth_step"):
+        t = EventTimer(torch)
+        for it in range(2 + reps):
+            if it < 2:
+                backend.query_forward(*ops, 8, interp)
+            else:
+                t(lambda: backend.query_forward(*ops, 8, interp))
+        n_live = int(mk.sum())
+        alg = fwd_bytes(16) * n_live + (29 + 64) * (n3 - n_live)
+        e = roofline_entry(f"query_forward_kernel<f32,E16> {interp}", alg, t.mean_ms())
+        e["Mqueries_per_s"] = round(n3 / e["ms"] / 1e3, 1)
+        out[f"cfg3_forward_{interp}"] = e
+    del grid, ops, x
+    torch.cuda.empty_cache()
+
+    # configuration 4
+    grid, radii, centres = workloads.build_grid(ash, 200_000, 4, device=dev)
+    x = workloads.ray_queries(grid, radii, centres, 32768, 128)
+    n4 = x.shape[0]
+    gi, ci, off, mk = grid.query(grid.transform_world_to_cell(x))
+    ops = (grid.embeddings.detach(), off, gi, ci, mk, grid.lut_grid_nb2grid_idx,
+           grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)
+    n_live = int(mk.sum())
+    z = torch.rand(n4, 4, device=dev) - 0.5
+    u = torch.rand(n4, 3, device=dev) - 0.5
+    dense = 4 * grid.embeddings.numel()
+    t_f, t_b, t_bb = EventTimer(torch), EventTimer(torch), EventTimer(torch)
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        run(t_f, lambda: backend.query_forward(*ops, 8, "smooth_step"))
+        run(t_b, lambda: backend.query_backward_forward(z, *ops, 8, "smooth_step"))
+        run(t_bb, lambda: backend.query_backward_backward(None, u, z, *ops, 8, "smooth_step"))
+    masked = n4 - n_live
+    entries = {
+        "cfg4_forward": roofline_entry(
+            "query_forward_kernel<f32,E4>", fwd_bytes(4) * n_live + (29 + 16) * masked, t_f.mean_ms()),
+        "cfg4_backward": roofline_entry(
+            "zero16 + query_backward_forward_kernel<f32,E4>",
+            bwd_bytes(4) * n_live + (29 + 12) * masked + dense, t_b.mean_ms()),
+        "cfg4_double_backward": roofline_entry(
+            "zero16 + query_backward_backward_kernel<f32,E4>",
+            bwd2_bytes(4) * n_live + (29 + 16) * masked + dense, t_bb.mean_ms()),
+    }
+    for name, e in entries.items():
+        e["Mqueries_per_s"] = round(n4 / e["ms"] / 1e3, 1)
+        out[name] = e
+    fb_ms = entries["cfg4_forward"]["ms"] + entries["cfg4_backward"]["ms"]
+    fb_bytes = (fwd_bytes(4) + bwd_bytes(4)) * n_live + (58 + 28) * masked + dense
+    e = roofline_entry("cfg4 forward + backward kernels", fb_bytes, fb_ms)
+    e["Mqueries_per_s"] = round(n4 / fb_ms / 1e3, 1)
+    out["cfg4_forward_plus_backward"] = e
+    out["cfg4_live_fraction"] = round(n_live / n4, 4)
+
+    # module-level training step: value loss + gradient-norm loss
+    xq = x.clone().requires_grad_(True)
+
+    def train_step():
+        grid.embeddings.grad = None
+        feats, _ = grid(xq, "smooth_step")
+        (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+        loss = (feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
+        loss.backward()
+
+    for _ in range(2):
+        train_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        train_step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / reps * 1e3
+    out["cfg4_module_train_step"] = {"ms": round(ms, 3), "Mqueries_per_s": round(n4 / ms / 1e3, 1)}
+    return out
+
+
+def cpu_baseline(torch, workloads, args):
+    """The oracle (OpenMP) on a bounded sample of configuration 2: same
+    generator, `--cpu-keys` distinct keys, capacity 1.5x, insert + find + items."""
+    import ash_oracle
+
+    oracle = ash_oracle.OracleBackend()
+    n = args.cpu_keys
+    cap = n * 3 // 2
+    w = workloads.hashmap_sphere_voxels(num_keys=n, device="cpu")
+    heap = torch.arange(cap, dtype=torch.int32)
+    omap = oracle.HashMap(3, cap, heap)
+    stores = {"color": torch.zeros(cap, 3), "depth": torch.zeros(cap, 1)}
+    values = {"color": w["color"], "depth": w["depth"]}
+    best = None
+    for _ in range(2):
+        omap.clear()
+        t0 = time.perf_counter()
+        omap.insert(w["keys"], values, stores)
+        t1 = time.perf_counter()
+        omap.find(w["query_keys"])
+        t2 = time.perf_counter()
+        omap.items()
+        t3 = time.perf_counter()
+        if best is None or t3 - t0 < best[0]:
+            best = (t3 - t0, t1 - t0, t2 - t1, t3 - t2)
+    total, t_ins, t_find, t_items = best
+    return {
+        "value": round(2 * n / total / 1e6, 2),
+        "unit": "Mkeys/s",
+        "cores": oracle.num_threads(),
+        "kind": "port",
+        "sample": f"configuration 2 generator at {n} keys, capacity {cap}: insert+find+items, best of 2",
+        "insert_Mkeys_per_s": round(n / t_ins / 1e6, 2),
+        "find_Mkeys_per_s": round(n / t_find / 1e6, 2),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has one GPU and the path "
+              "has no multi-GPU part; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import ash
+    import workloads
+    from ash.common import _Backend
+
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    assert isinstance(ash.core.backend, _Backend), "libash_hip.so is not loaded"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    ms_per_step, hits, kernels = bench_hash(torch, ash, workloads, args, dev)
+    if not args.no_trilinear:
+        kernels.update(bench_trilinear(torch, ash, workloads, args, dev))
+    dominant = max(("insert_values", "find", "items"), key=lambda k: kernels[k]["ms"])
+    roof = dict(kernels[dominant])
+    value = 2 * args.keys / (ms_per_step * 1e-3) / 1e6
+    line = {
+        "metric": "Mkeys/s insert+find (16M int3); Mqueries/s trilinear fwd+bwd; % HBM roofline",
+        "value": round(value, 1),
+        "unit": "Mkeys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u64 keys / int32 indices; fp32 trilinear",
+        "data": "synthetic",
+        "config": {
+            "workload": "configuration 2: HashMap{color fp32[3], depth fp32[1]}, "
+                        f"{args.keys} distinct int3 voxel keys into capacity {args.capacity}, "
+                        f"{args.keys} finds ({hits} hits), items(); step = clear+insert+find+items "
+                        "through the Python API",
+            "keys": args.keys,
+            "capacity": args.capacity,
+        },
+        "roofline": roof,
+        "kernels": kernels,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(torch, workloads, args)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
