@@ -66,6 +66,8 @@ def parse_args():
     ap.add_argument("--no-trilinear", action="store_true", help="skip the trilinear kernel figures")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-keys", type=int, default=4_000_000, help="CPU baseline sample size")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="run a 1 GiB device copy first (reference point for HBM counters)")
     return ap.parse_args()
 
 
@@ -321,6 +323,17 @@ def main():
     assert isinstance(ash.core.backend, _Backend), "libash_hip.so is not loaded"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate:
+        # A plain 1 GiB device-to-device copy: the reference point for scaling
+        # rocprofv3's FETCH_SIZE / WRITE_SIZE counters to bytes.
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     ms_per_step, hits, kernels = bench_hash(torch, ash, workloads, args, dev)
     if not args.no_trilinear:
