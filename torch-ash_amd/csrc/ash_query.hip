@@ -8,16 +8,22 @@
 //   cell_c = lut_cell_nb2cell_idx[cell_i][c] the cell inside that block
 // and a query with any missing neighbour block yields zeros.
 //
-// Mapping.  LPQ lanes share one query and each lane owns VEC consecutive
-// channels, so one request of a wavefront covers whole embedding rows
-// (E = 16 fp32: 4 lanes x 16 B = one 64-byte row; a wavefront reads 16 rows per
-// instruction and writes 1 KiB of contiguous output).  The two per-cell tables
-// are staged once per workgroup in LDS as uint16/uint8; workgroups are
-// persistent and walk the query tiles of "their" XCD (workgroup id mod 8) so
-// that neighbouring queries meet in one L2.  Gradients for the embeddings are
-// accumulated with hardware floating-point atomics; with MERGE, consecutive
-// queries of a wavefront that hit the same row are summed in registers first
-// and issue one atomic per run.
+// Structure.  A workgroup of 256 threads takes tiles of 256 queries.
+//   Phase 1 (one thread per query) reads the query's indices, offsets and mask
+//   with coalesced loads, walks the neighbour tables (the two per-cell tables
+//   are staged once per workgroup in LDS as uint16/uint8) and leaves the 8 row
+//   numbers g_c * M + cell_c and the 3 offsets of every query in LDS.
+//   Phase 2 re-maps the threads so that LPQ lanes share one query and each lane
+//   owns VEC consecutive channels: one request of a wavefront then covers whole
+//   embedding rows (E = 16 fp32: 4 lanes x 16 B = one 64-byte row, 16 rows per
+//   instruction, 1 KiB of contiguous output), and the per-query address work is
+//   not repeated per channel.  When one lane covers the row (LPQ = 1) both
+//   phases run in registers without the LDS round trip.
+// Workgroups are persistent and walk the tiles of "their" XCD (workgroup id
+// mod 8), so neighbouring queries meet in one L2.  Gradients for the embeddings
+// are accumulated with hardware floating-point atomics; consecutive queries of
+// a wavefront that hit the same row are summed in registers first and issue
+// one atomic per run (ray-ordered samples produce long runs).
 #include "ash_dev.h"
 
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
@@ -32,6 +38,8 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kXcds = 8;
 constexpr int64_t kMaxLdsCells = 2048;  // 2048 * 8 * 3 B = 48 KiB
+constexpr uint32_t kNoRow = 0xFFFFFFFFu;
+constexpr int kLdsPerCu = 160 * 1024;
 
 struct QDev {
     const void* emb;
@@ -46,7 +54,9 @@ struct QDev {
     int64_t B;
     int64_t M;
     int E;
-    int smooth;  // 0 linear, 1 smooth step
+    int smooth;    // 0 linear, 1 smooth step
+    int lds_lut;   // per-cell tables staged in LDS
+    int merge;     // pre-reduce runs of equal rows before the atomics
 };
 
 // Interpolation basis (ash/src/grid.cu:7-41).
@@ -67,7 +77,7 @@ struct AxisTerms {
     T dw[3][2];
 };
 
-template <typename T>
+template <typename T, bool GRAD>
 __device__ __forceinline__ void axis_terms(const float (&o)[3], int smooth,
                                            AxisTerms<T>& t) {
 #pragma unroll
@@ -76,8 +86,10 @@ __device__ __forceinline__ void axis_terms(const float (&o)[3], int smooth,
         const T x0 = static_cast<T>(1.0f - o[d]);
         t.w[d][0] = basis<T>(x0, smooth);
         t.w[d][1] = basis<T>(x1, smooth);
-        t.dw[d][0] = -dbasis<T>(x0, smooth);
-        t.dw[d][1] = dbasis<T>(x1, smooth);
+        if constexpr (GRAD) {
+            t.dw[d][0] = -dbasis<T>(x0, smooth);
+            t.dw[d][1] = dbasis<T>(x1, smooth);
+        }
     }
 }
 
@@ -99,38 +111,39 @@ __device__ __forceinline__ void corner_weight_grad(const AxisTerms<T>& t, int c,
     g[2] = t.w[0][b0] * t.w[1][b1] * t.dw[2][b2];
 }
 
-// The two per-cell tables, either staged in LDS or read through the caches.
-template <bool LDS>
+// ------------------------------------------------------------ LDS layout
+// [ tile: row[8][256] uint32, off[3][256] float ]  (only when LPQ > 1)
+// [ per-cell tables: c2c[M*8] uint16, c2g[M*8] uint8 ]  (only when lds_lut)
+struct Tile {
+    uint32_t row[8][kBlock];
+    float off[3][kBlock];
+};
+
 struct CellLut {
     const uint16_t* c2c;
     const uint8_t* c2g;
-    const int64_t* g_c2c;
-    const int64_t* g_c2g;
-    int64_t M;
-    __device__ __forceinline__ void get(int64_t cell, int c, int& nb_cell,
-                                        int& nb_grid) const {
-        if constexpr (LDS) {
-            nb_cell = c2c[cell * 8 + c];
-            nb_grid = c2g[cell * 8 + c];
-        } else {
-            int64_t v = g_c2c[cell * 8 + c];
-            v = v < 0 ? 0 : (v >= M ? M - 1 : v);
-            nb_cell = static_cast<int>(v);
-            nb_grid = static_cast<int>(g_c2g[cell * 8 + c]) & 7;
-        }
-    }
 };
 
-template <bool LDS>
-__device__ __forceinline__ CellLut<LDS> stage_cell_lut(const QDev& a,
-                                                       unsigned char* smem) {
-    CellLut<LDS> lut;
-    lut.g_c2c = a.lut_c2c;
-    lut.g_c2g = a.lut_c2g;
-    lut.M = a.M;
+__device__ __forceinline__ void cell_neighbor(const QDev& a, const CellLut& lut,
+                                              int64_t cell, int c, int& nb_cell,
+                                              int& nb_grid) {
+    if (a.lds_lut) {
+        nb_cell = lut.c2c[cell * 8 + c];
+        nb_grid = lut.c2g[cell * 8 + c];
+    } else {
+        int64_t v = a.lut_c2c[cell * 8 + c];
+        v = v < 0 ? 0 : (v >= a.M ? a.M - 1 : v);
+        nb_cell = static_cast<int>(v);
+        nb_grid = static_cast<int>(a.lut_c2g[cell * 8 + c]) & 7;
+    }
+}
+
+__device__ __forceinline__ CellLut stage_cell_lut(const QDev& a,
+                                                  unsigned char* smem) {
+    CellLut lut;
     lut.c2c = nullptr;
     lut.c2g = nullptr;
-    if constexpr (LDS) {
+    if (a.lds_lut) {
         uint16_t* s_c2c = reinterpret_cast<uint16_t*>(smem);
         uint8_t* s_c2g = smem + a.M * 8 * 2;
         const int64_t n = a.M * 8;
@@ -165,14 +178,12 @@ struct TileWalk {
     }
 };
 
-// Resolves the 8 corner rows of one query.  Returns false (all rows invalid)
-// when the query is masked out or any neighbour block is missing.
-template <bool LDS>
-__device__ __forceinline__ bool resolve_rows(const QDev& a,
-                                             const CellLut<LDS>& lut, int64_t q,
-                                             bool in_range, int64_t (&row)[8],
+// Phase 1 for one query: the 8 corner rows (kNoRow in row[0] when the query is
+// masked out, out of range, or misses a neighbour block) and the offsets.
+__device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
+                                             int64_t q, uint32_t (&row)[8],
                                              float (&o)[3]) {
-    bool valid = in_range && a.mask[q] != 0;
+    bool valid = q < a.N && a.mask[q] != 0;
     int64_t gi = 0, ci = 0;
     o[0] = o[1] = o[2] = 0.f;
     if (valid) {
@@ -188,21 +199,61 @@ __device__ __forceinline__ bool resolve_rows(const QDev& a,
     if (valid) g0 = a.lut_g[gi * 8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-        row[c] = -1;
+        row[c] = 0;
         if (valid) {
             int nb_cell, nb_grid;
-            lut.get(ci, c, nb_cell, nb_grid);
+            cell_neighbor(a, lut, ci, c, nb_cell, nb_grid);
             int64_t g = g0;
             if (nb_grid != 0) g = a.lut_g[gi * 8 + nb_grid];
             if (g < 0 || g >= a.B) {
                 valid = false;
             } else {
-                row[c] = g * a.M + nb_cell;
+                row[c] = static_cast<uint32_t>(g * a.M + nb_cell);
             }
         }
     }
-    return valid;
+    if (!valid) row[0] = kNoRow;
 }
+
+// Runs phase 1 for the tile and hands every thread the rows / offsets of the
+// query it serves in pass `p` of phase 2.
+template <int LPQ>
+struct TileStage {
+    static constexpr int kPasses = LPQ;
+    static constexpr int kQpp = kBlock / LPQ;  // queries per pass
+
+    static __device__ __forceinline__ void fill(const QDev& a,
+                                                const CellLut& lut,
+                                                int64_t tile, Tile* s,
+                                                uint32_t (&row)[8],
+                                                float (&o)[3]) {
+        resolve_rows(a, lut, tile * kBlock + threadIdx.x, row, o);
+        if constexpr (LPQ > 1) {
+            __syncthreads();  // previous tile fully consumed
+#pragma unroll
+            for (int c = 0; c < 8; ++c) s->row[c][threadIdx.x] = row[c];
+#pragma unroll
+            for (int d = 0; d < 3; ++d) s->off[d][threadIdx.x] = o[d];
+            __syncthreads();
+        }
+    }
+
+    static __device__ __forceinline__ int64_t fetch(int64_t tile, int p,
+                                                    const Tile* s,
+                                                    uint32_t (&row)[8],
+                                                    float (&o)[3]) {
+        if constexpr (LPQ > 1) {
+            const int qi = p * kQpp + threadIdx.x / LPQ;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) row[c] = s->row[c][qi];
+#pragma unroll
+            for (int d = 0; d < 3; ++d) o[d] = s->off[d][qi];
+            return tile * kBlock + qi;
+        } else {
+            return tile * kBlock + threadIdx.x;
+        }
+    }
+};
 
 template <typename T, int VEC>
 struct VecOf;
@@ -220,66 +271,60 @@ struct VecOf<double, 1> {
 };
 
 // ------------------------------------------------------------- forward
-template <typename T, int VEC, int LPQ, bool LDS>
+template <typename T, int VEC, int LPQ>
 __global__ __launch_bounds__(kBlock) void query_forward_kernel(
         QDev a, T* __restrict__ out) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
-    constexpr int kQpb = kBlock / LPQ;
-    const int sub = threadIdx.x % LPQ;
-    const int ch0 = sub * VEC;
+    Tile* tile_s = reinterpret_cast<Tile*>(smem);
+    const CellLut lut =
+            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ>;
+    using V = typename VecOf<T, VEC>::type;
+    const int ch0 = (threadIdx.x % LPQ) * VEC;
     const bool chv = ch0 < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
-    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
-        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
-        const bool in_range = q < a.N;
-        int64_t row[8];
+        uint32_t row[8];
         float o[3];
-        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
-        T acc[VEC];
+        Stage::fill(a, lut, tile, tile_s, row, o);
+#pragma unroll 1
+        for (int p = 0; p < Stage::kPasses; ++p) {
+            const int64_t q = Stage::fetch(tile, p, tile_s, row, o);
+            const bool valid = row[0] != kNoRow;
+            alignas(16) T acc[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) acc[v] = T(0);
-        if (valid && chv) {
-            AxisTerms<T> t;
-            axis_terms<T>(o, a.smooth, t);
-            using V = typename VecOf<T, VEC>::type;
-            V e[8];
+            for (int v = 0; v < VEC; ++v) acc[v] = T(0);
+            if (valid && chv) {
+                V e[8];
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                e[c] = *reinterpret_cast<const V*>(emb + row[c] * a.E + ch0);
+                for (int c = 0; c < 8; ++c) {
+                    e[c] = *reinterpret_cast<const V*>(
+                            emb + static_cast<int64_t>(row[c]) * a.E + ch0);
+                }
+                AxisTerms<T> t;
+                axis_terms<T, false>(o, a.smooth, t);
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const T w = corner_weight<T>(t, c);
+                    const T* ev = reinterpret_cast<const T*>(&e[c]);
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] += w * ev[v];
+                }
             }
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const T w = corner_weight<T>(t, c);
-                const T* ev = reinterpret_cast<const T*>(&e[c]);
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) acc[v] += w * ev[v];
+            if (q < a.N && chv) {
+                *reinterpret_cast<V*>(out + q * a.E + ch0) =
+                        *reinterpret_cast<const V*>(acc);
             }
-        }
-        if (in_range && chv) {
-            using V = typename VecOf<T, VEC>::type;
-            *reinterpret_cast<V*>(out + q * a.E + ch0) =
-                    *reinterpret_cast<const V*>(acc);
         }
     }
 }
 
 // ------------------------------------------------- run merge for atomics
-template <int LPQ>
-__device__ __forceinline__ void run_flags(int64_t row, int lane, bool& head,
-                                          bool& tail) {
-    constexpr int kGroups = 64 / LPQ;
-    const int grp = lane / LPQ;
-    const int64_t prev = __shfl_up(row, LPQ);
-    const int64_t next = __shfl_down(row, LPQ);
-    head = (grp == 0) || (prev != row);
-    tail = (grp == kGroups - 1) || (next != row);
-}
-
-// Inclusive segmented sum over the query groups of a wavefront: after the
-// call the last group of every run of equal rows holds the run's total.
+// Inclusive segmented sum over the query groups of a wavefront: `head` marks
+// the first group of a run of equal rows; afterwards the last group of every
+// run holds the run's total.
 template <typename T, int LPQ>
 __device__ __forceinline__ T run_sum(T v, bool head, int lane) {
     constexpr int kGroups = 64 / LPQ;
@@ -297,18 +342,27 @@ __device__ __forceinline__ T run_sum(T v, bool head, int lane) {
     return v;
 }
 
-template <typename T, int LPQ, bool MERGE>
+// Adds v to grad_emb[row, ch] for the lanes that are `on`.
+template <typename T, int LPQ>
 __device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
-                                               int64_t row, int E, int ch,
-                                               bool on, T v, int lane) {
-    if constexpr (MERGE) {
-        bool head, tail;
-        run_flags<LPQ>(on ? row : -1 - static_cast<int64_t>(lane / LPQ), lane,
-                       head, tail);
+                                               uint32_t row, int E, int ch,
+                                               bool on, T v, int lane,
+                                               int merge) {
+    if (merge) {
+        constexpr int kGroups = 64 / LPQ;
+        const int grp = lane / LPQ;
+        // lanes that are off get a row number no neighbour shares
+        const uint32_t id = on ? row : (kNoRow - static_cast<uint32_t>(grp & 1));
+        const uint32_t prev = __shfl_up(id, LPQ);
+        const uint32_t next = __shfl_down(id, LPQ);
+        const bool head = (grp == 0) || (prev != id) || !on;
+        const bool tail = (grp == kGroups - 1) || (next != id);
         v = run_sum<T, LPQ>(on ? v : T(0), head, lane);
-        if (on && tail) unsafeAtomicAdd(grad_emb + row * E + ch, v);
-    } else {
-        if (on) unsafeAtomicAdd(grad_emb + row * E + ch, v);
+        if (on && tail) {
+            unsafeAtomicAdd(grad_emb + static_cast<int64_t>(row) * E + ch, v);
+        }
+    } else if (on) {
+        unsafeAtomicAdd(grad_emb + static_cast<int64_t>(row) * E + ch, v);
     }
 }
 
@@ -316,53 +370,58 @@ __device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
 // grad_embeddings[row_c, k] += w_c * z[i,k];
 // grad_offsets[i,:] = sum_c (emb[row_c,:] . z[i,:]) * grad w_c
 // (ash/src/grid.cu:177-255).  One lane per channel.
-template <typename T, int LPQ, bool LDS, bool MERGE>
+template <typename T, int LPQ>
 __global__ __launch_bounds__(kBlock) void query_backward_forward_kernel(
         QDev a, const T* __restrict__ z, T* __restrict__ grad_emb,
         T* __restrict__ grad_off) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
-    constexpr int kQpb = kBlock / LPQ;
+    Tile* tile_s = reinterpret_cast<Tile*>(smem);
+    const CellLut lut =
+            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ>;
     const int lane = threadIdx.x & 63;
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
-    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
-        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
-        const bool in_range = q < a.N;
-        int64_t row[8];
+        uint32_t row[8];
         float o[3];
-        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
-        const bool on = valid && chv;
-        AxisTerms<T> t;
-        axis_terms<T>(o, a.smooth, t);
-        const T zk = on ? z[q * a.E + ch] : T(0);
-        T e[8];
+        Stage::fill(a, lut, tile, tile_s, row, o);
+#pragma unroll 1
+        for (int p = 0; p < Stage::kPasses; ++p) {
+            const int64_t q = Stage::fetch(tile, p, tile_s, row, o);
+            const bool valid = row[0] != kNoRow;
+            const bool on = valid && chv;
+            const T zk = on ? z[q * a.E + ch] : T(0);
+            T e[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            e[c] = on ? emb[row[c] * a.E + ch] : T(0);
-        }
-        T go[3] = {T(0), T(0), T(0)};
+            for (int c = 0; c < 8; ++c) {
+                e[c] = on ? emb[static_cast<int64_t>(row[c]) * a.E + ch] : T(0);
+            }
+            AxisTerms<T> t;
+            axis_terms<T, true>(o, a.smooth, t);
+            T go[3] = {T(0), T(0), T(0)};
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const T w = corner_weight<T>(t, c);
-            T gw[3];
-            corner_weight_grad<T>(t, c, gw);
-            accumulate_row<T, LPQ, MERGE>(grad_emb, row[c], a.E, ch, on, w * zk,
-                                          lane);
-            T dot = e[c] * zk;
+            for (int c = 0; c < 8; ++c) {
+                const T w = corner_weight<T>(t, c);
+                T gw[3];
+                corner_weight_grad<T>(t, c, gw);
+                accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk,
+                                       lane, a.merge);
+                T dot = e[c] * zk;
 #pragma unroll
-            for (int s = 1; s < LPQ; s <<= 1) dot += __shfl_xor(dot, s);
-            go[0] += dot * gw[0];
-            go[1] += dot * gw[1];
-            go[2] += dot * gw[2];
-        }
-        if (in_range && ch == 0) {
-            grad_off[q * 3 + 0] = valid ? go[0] : T(0);
-            grad_off[q * 3 + 1] = valid ? go[1] : T(0);
-            grad_off[q * 3 + 2] = valid ? go[2] : T(0);
+                for (int s = 1; s < LPQ; s <<= 1) dot += __shfl_xor(dot, s);
+                go[0] += dot * gw[0];
+                go[1] += dot * gw[1];
+                go[2] += dot * gw[2];
+            }
+            if (q < a.N && ch == 0) {
+                grad_off[q * 3 + 0] = valid ? go[0] : T(0);
+                grad_off[q * 3 + 1] = valid ? go[1] : T(0);
+                grad_off[q * 3 + 2] = valid ? go[2] : T(0);
+            }
         }
     }
 }
@@ -370,51 +429,56 @@ __global__ __launch_bounds__(kBlock) void query_backward_forward_kernel(
 // -------------------------------------------------- backward of backward
 // d_c = grad w_c . gg_off[i];  grad_embeddings[row_c,k] += d_c * z[i,k];
 // grad_z[i,k] = sum_c d_c * emb[row_c,k]   (ash/src/grid.cu:309-387).
-template <typename T, int LPQ, bool LDS, bool MERGE>
+template <typename T, int LPQ>
 __global__ __launch_bounds__(kBlock) void query_backward_backward_kernel(
         QDev a, const T* __restrict__ gg_off, const T* __restrict__ z,
         T* __restrict__ grad_z, T* __restrict__ grad_emb) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const CellLut<LDS> lut = stage_cell_lut<LDS>(a, smem);
-    constexpr int kQpb = kBlock / LPQ;
+    Tile* tile_s = reinterpret_cast<Tile*>(smem);
+    const CellLut lut =
+            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ>;
     const int lane = threadIdx.x & 63;
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
-    const int64_t ntiles = (a.N + kQpb - 1) / kQpb;
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
-        const int64_t q = tile * kQpb + threadIdx.x / LPQ;
-        const bool in_range = q < a.N;
-        int64_t row[8];
+        uint32_t row[8];
         float o[3];
-        const bool valid = resolve_rows<LDS>(a, lut, q, in_range, row, o);
-        const bool on = valid && chv;
-        AxisTerms<T> t;
-        axis_terms<T>(o, a.smooth, t);
-        const T zk = on ? z[q * a.E + ch] : T(0);
-        T gg[3] = {T(0), T(0), T(0)};
-        if (valid) {
-            gg[0] = gg_off[q * 3 + 0];
-            gg[1] = gg_off[q * 3 + 1];
-            gg[2] = gg_off[q * 3 + 2];
-        }
-        T e[8];
+        Stage::fill(a, lut, tile, tile_s, row, o);
+#pragma unroll 1
+        for (int p = 0; p < Stage::kPasses; ++p) {
+            const int64_t q = Stage::fetch(tile, p, tile_s, row, o);
+            const bool valid = row[0] != kNoRow;
+            const bool on = valid && chv;
+            const T zk = on ? z[q * a.E + ch] : T(0);
+            T gg[3] = {T(0), T(0), T(0)};
+            if (valid) {
+                gg[0] = gg_off[q * 3 + 0];
+                gg[1] = gg_off[q * 3 + 1];
+                gg[2] = gg_off[q * 3 + 2];
+            }
+            T e[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            e[c] = on ? emb[row[c] * a.E + ch] : T(0);
-        }
-        T gz = T(0);
+            for (int c = 0; c < 8; ++c) {
+                e[c] = on ? emb[static_cast<int64_t>(row[c]) * a.E + ch] : T(0);
+            }
+            AxisTerms<T> t;
+            axis_terms<T, true>(o, a.smooth, t);
+            T gz = T(0);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            T gw[3];
-            corner_weight_grad<T>(t, c, gw);
-            const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
-            accumulate_row<T, LPQ, MERGE>(grad_emb, row[c], a.E, ch, on, d * zk,
-                                          lane);
-            gz += d * e[c];
+            for (int c = 0; c < 8; ++c) {
+                T gw[3];
+                corner_weight_grad<T>(t, c, gw);
+                const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
+                accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk,
+                                       lane, a.merge);
+                gz += d * e[c];
+            }
+            if (q < a.N && chv) grad_z[q * a.E + ch] = on ? gz : T(0);
         }
-        if (in_range && chv) grad_z[q * a.E + ch] = on ? gz : T(0);
     }
 }
 
@@ -464,6 +528,15 @@ int zero_fill(void* ptr, int64_t bytes, hipStream_t s) {
     return 0;
 }
 
+bool merge_enabled() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = std::getenv("ASH_BWD_MERGE");
+        v = (e != nullptr && e[0] == '0') ? 0 : 1;
+    }
+    return v == 1;
+}
+
 int check_args(const ash_query_args* a, QDev& d) {
     if (a == nullptr) ASH_FAIL("null query arguments");
     if (a->num_queries < 0) ASH_FAIL("negative query count");
@@ -478,6 +551,10 @@ int check_args(const ash_query_args* a, QDev& d) {
         ASH_FAIL("Unknown interpolation functor");
     }
     if (a->dtype != ASH_F32 && a->dtype != ASH_F64) ASH_FAIL("unknown dtype");
+    if (a->num_embeddings > 0x7FFFFFFFll ||
+        a->num_embeddings * a->cells_per_grid >= 0xFFFFFFFFll) {
+        ASH_FAIL("num_embeddings * cells_per_grid must stay below 2^32 - 1");
+    }
     if (a->embeddings == nullptr || a->lut_grid_nb2grid_idx == nullptr ||
         a->lut_cell_nb2cell_idx == nullptr || a->lut_cell_nb2grid_nb == nullptr) {
         ASH_FAIL("null table pointer");
@@ -500,6 +577,8 @@ int check_args(const ash_query_args* a, QDev& d) {
     d.M = a->cells_per_grid;
     d.E = static_cast<int>(a->embedding_dim);
     d.smooth = a->interpolation == ASH_INTERP_SMOOTH_STEP ? 1 : 0;
+    d.lds_lut = d.M <= kMaxLdsCells ? 1 : 0;
+    d.merge = merge_enabled() ? 1 : 0;
     return 0;
 }
 
@@ -509,7 +588,14 @@ int pow2_ceil(int v) {
     return p;
 }
 
-unsigned persistent_grid(int64_t ntiles) {
+size_t smem_bytes(const QDev& d, int lpq) {
+    size_t bytes = lpq > 1 ? sizeof(Tile) : 0;
+    if (d.lds_lut) bytes += static_cast<size_t>(d.M) * 8 * 3;
+    return bytes;
+}
+
+// Enough persistent workgroups to fill every CU as far as LDS allows.
+unsigned persistent_grid(int64_t ntiles, size_t smem) {
     static int cus = 0;
     if (cus == 0) {
         int dev = 0, n = 0;
@@ -522,38 +608,24 @@ unsigned persistent_grid(int64_t ntiles) {
             cus = 256;
         }
     }
-    int64_t g = static_cast<int64_t>(cus) * 8;
+    int per_cu = 8;
+    if (smem > 0) {
+        const int fit = static_cast<int>(kLdsPerCu / smem);
+        if (fit < per_cu) per_cu = fit < 1 ? 1 : fit;
+    }
+    int64_t g = static_cast<int64_t>(cus) * per_cu;
     if (g > ntiles) g = ntiles;
     g = (g + kXcds - 1) / kXcds * kXcds;  // whole rounds over the XCDs
     if (g < kXcds) g = kXcds;
     return static_cast<unsigned>(g);
 }
 
-bool merge_enabled() {
-    static int v = -1;
-    if (v < 0) {
-        const char* e = std::getenv("ASH_BWD_MERGE");
-        v = (e != nullptr && e[0] == '0') ? 0 : 1;
-    }
-    return v == 1;
-}
-
-size_t lds_bytes(const QDev& d, bool lds) {
-    return lds ? static_cast<size_t>(d.M) * 8 * 3 : 0;
-}
-
 template <typename T, int VEC, int LPQ>
 int launch_forward(const QDev& d, void* out, hipStream_t s) {
-    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
-    const unsigned g = persistent_grid(ntiles);
-    const bool lds = d.M <= kMaxLdsCells;
-    if (lds) {
-        query_forward_kernel<T, VEC, LPQ, true>
-                <<<g, kBlock, lds_bytes(d, true), s>>>(d, static_cast<T*>(out));
-    } else {
-        query_forward_kernel<T, VEC, LPQ, false>
-                <<<g, kBlock, 0, s>>>(d, static_cast<T*>(out));
-    }
+    const size_t smem = smem_bytes(d, LPQ);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    query_forward_kernel<T, VEC, LPQ>
+            <<<g, kBlock, smem, s>>>(d, static_cast<T*>(out));
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -561,25 +633,11 @@ int launch_forward(const QDev& d, void* out, hipStream_t s) {
 template <typename T, int LPQ>
 int launch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
                    hipStream_t s) {
-    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
-    const unsigned g = persistent_grid(ntiles);
-    const bool lds = d.M <= kMaxLdsCells;
-    const bool merge = merge_enabled();
-#define ASH_BF(L, M)                                                          \
-    query_backward_forward_kernel<T, LPQ, L, M>                               \
-            <<<g, kBlock, lds_bytes(d, L), s>>>(d, static_cast<const T*>(z),  \
-                                                static_cast<T*>(ge),          \
-                                                static_cast<T*>(go))
-    if (lds && merge) {
-        ASH_BF(true, true);
-    } else if (lds) {
-        ASH_BF(true, false);
-    } else if (merge) {
-        ASH_BF(false, true);
-    } else {
-        ASH_BF(false, false);
-    }
-#undef ASH_BF
+    const size_t smem = smem_bytes(d, LPQ);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    query_backward_forward_kernel<T, LPQ><<<g, kBlock, smem, s>>>(
+            d, static_cast<const T*>(z), static_cast<T*>(ge),
+            static_cast<T*>(go));
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -587,33 +645,23 @@ int launch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
 template <typename T, int LPQ>
 int launch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
                    void* ge, hipStream_t s) {
-    const int64_t ntiles = (d.N + kBlock / LPQ - 1) / (kBlock / LPQ);
-    const unsigned g = persistent_grid(ntiles);
-    const bool lds = d.M <= kMaxLdsCells;
-    const bool merge = merge_enabled();
-#define ASH_BB(L, M)                                                          \
-    query_backward_backward_kernel<T, LPQ, L, M>                              \
-            <<<g, kBlock, lds_bytes(d, L), s>>>(                              \
-                    d, static_cast<const T*>(gg), static_cast<const T*>(z),   \
-                    static_cast<T*>(gz), static_cast<T*>(ge))
-    if (lds && merge) {
-        ASH_BB(true, true);
-    } else if (lds) {
-        ASH_BB(true, false);
-    } else if (merge) {
-        ASH_BB(false, true);
-    } else {
-        ASH_BB(false, false);
-    }
-#undef ASH_BB
+    const size_t smem = smem_bytes(d, LPQ);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    query_backward_backward_kernel<T, LPQ><<<g, kBlock, smem, s>>>(
+            d, static_cast<const T*>(gg), static_cast<const T*>(z),
+            static_cast<T*>(gz), static_cast<T*>(ge));
     ASH_LAUNCH_CHECK();
     return 0;
+}
+
+bool aligned16(const void* p) {
+    return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
 
 template <typename T>
 int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
     if constexpr (sizeof(T) == 4) {
-        if (d.E % 4 == 0) {
+        if (d.E % 4 == 0 && aligned16(d.emb) && aligned16(out)) {
             switch (d.E / 4) {
                 case 1:
                     return launch_forward<float, 4, 1>(d, out, s);
