@@ -40,6 +40,18 @@ INSERT_KEY_BYTES = 12 + 16 + 16 + 4          # key in, probe, slot write, heap p
 VALUE_ROW_BYTES = 2 * (12 + 4)               # color + depth, read and written
 
 
+# HBM bytes per launch (read + written) at the default sizes, from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
+# counters read for a plain 1 GiB copy: FETCH_SIZE x 1024 / 0.50,
+# WRITE_SIZE x 1024 / 1.00.  Only attached when the run uses those sizes.
+MEASURED_TRAFFIC_BYTES = {
+    "insert_values": 2_563_000_000 + 1_819_000_000,
+    "insert_keys": 2_303_000_000 + 1_564_000_000,
+    "find": 2_230_000_000 + 146_000_000,
+    "items": 947_000_000 + 775_000_000,
+}
+
+
 def items_bytes(slots: int, n: int) -> int:
     return 16 * slots + 20 * n
 
@@ -104,6 +116,44 @@ def roofline_entry(name, alg_bytes, ms, traffic=None):
         "traffic": traffic,
         "ms": round(ms, 4),
     }
+
+
+def measure_ceilings(torch, ash, dev, table_bytes, n):
+    """What this device's memory system delivers for the two access patterns
+    that bound the table kernels, measured with the library's probes on a
+    buffer of the table's size: random 128-byte line reads (a probe) and random
+    line read + compare-and-swap + dword store (an insert); plus a plain
+    device-to-device copy for the streaming rate."""
+    lib = ash.core.backend.lib
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    buf = torch.empty(table_bytes // 128 * 128, dtype=torch.uint8, device=dev).fill_(255)
+    sink = torch.empty(n, dtype=torch.int32, device=dev)
+    out = {}
+    for mode, name in ((0, "random_line_reads"), (1, "random_line_updates")):
+        timer = EventTimer(torch)
+        for it in range(6):
+            call = lambda: lib.ash_diag_random_lines(
+                mode, buf.data_ptr(), buf.numel(), n, sink.data_ptr(), 7919 * it, stream)
+            if it == 0:
+                assert call() == 0, lib.ash_last_error().decode()
+            else:
+                timer(call)
+        ms = timer.mean_ms()
+        out[name] = {"Glines_per_s": round(n / ms / 1e6, 2), "ms": round(ms, 4)}
+    src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    timer = EventTimer(torch)
+    for it in range(6):
+        if it == 0:
+            dst.copy_(src)
+        else:
+            timer(lambda: dst.copy_(src))
+    ms = timer.mean_ms()
+    out["copy_1GiB"] = {"GB_per_s_read_plus_write": round(2 * src.numel() * 4 / ms / 1e6, 1),
+                        "ms": round(ms, 4)}
+    del buf, sink, src, dst
+    torch.cuda.empty_cache()
+    return out
 
 
 def bench_hash(torch, ash, workloads, args, dev):
@@ -175,6 +225,9 @@ def bench_hash(torch, ash, workloads, args, dev):
     for name in ("insert_values", "insert_keys", "find"):
         kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
+    if n == 16_000_000 and args.capacity == 24_000_000:
+        for name, traffic in MEASURED_TRAFFIC_BYTES.items():
+            kernels[name]["traffic"] = traffic
     del hm, w
     torch.cuda.empty_cache()
     return ms_per_step, hits, kernels
@@ -340,6 +393,13 @@ def main():
         kernels.update(bench_trilinear(torch, ash, workloads, args, dev))
     dominant = max(("insert_values", "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
+    table_bytes = (args.capacity + 5) // 6 * 128
+    ceilings = measure_ceilings(torch, ash, dev, table_bytes, 16 << 20)
+    kernels["find"]["of_random_line_read_rate"] = round(
+        kernels["find"]["Mkeys_per_s"] / 1e3 / ceilings["random_line_reads"]["Glines_per_s"], 3)
+    for name in ("insert_values", "insert_keys"):
+        kernels[name]["of_random_line_update_rate"] = round(
+            kernels[name]["Mkeys_per_s"] / 1e3 / ceilings["random_line_updates"]["Glines_per_s"], 3)
     value = 2 * args.keys / (ms_per_step * 1e-3) / 1e6
     line = {
         "metric": "Mkeys/s insert+find (16M int3); Mqueries/s trilinear fwd+bwd; % HBM roofline",
@@ -364,6 +424,7 @@ def main():
         },
         "roofline": roof,
         "kernels": kernels,
+        "ceilings": ceilings,
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch, workloads, args)

@@ -201,6 +201,19 @@ int ash_query_backward_backward(const ash_query_args* a,
                                 void* grad_z, void* grad_embeddings,
                                 void* stream);
 
+/* -------------------------------------------------------------- diagnostics */
+
+/* Measures the device's random-access ceilings that bound the table kernels
+ * (no counterpart in the reference).  `buf` is a 128-byte aligned device
+ * buffer of `buf_bytes` bytes treated as 128-byte lines; `n` (a multiple of
+ * 256) pseudo-random lines are touched and `sink` (uint32[n]) receives values
+ * that keep the accesses alive.  The caller times the call.
+ *   mode 0: every line is read in full by 8 lanes x 16 bytes (a table probe);
+ *   mode 1: per line one 64-bit read, one 64-bit compare-and-swap and one
+ *           32-bit store (the accesses of an insert); modifies `buf`. */
+int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes, int64_t n,
+                          uint32_t* sink, uint64_t seed, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -90,6 +90,10 @@ _SIGNATURES = {
     "ash_map_should_rebuild": (ctypes.c_int, [_PTR, _I64, _I64, _I64]),
     "ash_map_rebuild": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_scatter_rows": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _I64, _PTR]),
+    "ash_diag_random_lines": (
+        ctypes.c_int,
+        [ctypes.c_int, _PTR, _I64, _I64, _PTR, ctypes.c_uint64, _PTR],
+    ),
     "ash_query_forward": (ctypes.c_int, [ctypes.POINTER(_QueryArgs), _PTR, _PTR]),
     "ash_query_backward_forward": (
         ctypes.c_int,

@@ -1,0 +1,96 @@
+// Memory-system probes of libash_hip.so.  The hash kernels are bound by how
+// many random 128-byte lines per second the device can read or update, not by
+// streaming bandwidth; these kernels measure those ceilings on the device at
+// hand so that a benchmark can price the table kernels against them.
+#include "ash_dev.h"
+
+#include "../../include/ash_hip.h"
+
+namespace ash {
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ uint64_t mix64(uint64_t h) {
+    h ^= h >> 33;
+    h *= 0xff51afd7ed558ccdull;
+    h ^= h >> 33;
+    h *= 0xc4ceb9fe1a85ec53ull;
+    h ^= h >> 33;
+    return h;
+}
+
+// Every group of 8 lanes reads 8 pseudo-random 128-byte lines, 16 bytes per
+// lane, all 8 reads in flight at once: the access pattern of a table probe.
+__global__ __launch_bounds__(kBlock) void probe_line_reads(
+        const uint4* __restrict__ buf, uint32_t nlines, int64_t n,
+        uint32_t* __restrict__ sink, uint64_t seed) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 7;
+    const int gbase = lane & ~7;
+    const uint32_t line = __umulhi(
+            static_cast<uint32_t>(mix64(static_cast<uint64_t>(t) + seed) >> 32),
+            nlines);
+    uint4 v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const uint32_t lr = __shfl(line, gbase | r);
+        v[r] = buf[static_cast<size_t>(lr) * 8 + j];
+    }
+    uint32_t s = 0;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) s += v[r].x ^ v[r].y ^ v[r].z ^ v[r].w;
+    if (t < n) sink[t] = s;
+}
+
+// One thread per line: read one 64-bit word, compare-and-swap it, store one
+// dword elsewhere in the line -- the three accesses an insert makes.
+__global__ __launch_bounds__(kBlock) void probe_line_updates(
+        unsigned long long* __restrict__ buf, uint32_t nlines, int64_t n,
+        uint32_t* __restrict__ sink, uint64_t seed) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const uint64_t key = mix64(static_cast<uint64_t>(t) + seed);
+    const uint32_t line = __umulhi(static_cast<uint32_t>(key >> 32), nlines);
+    const int slot = static_cast<int>(key % 10);
+    unsigned long long* p = buf + static_cast<size_t>(line) * 16 + slot;
+    const unsigned long long seen = *p;
+    const unsigned long long old = atomicCAS(p, seen, key | 1ull);
+    reinterpret_cast<uint32_t*>(buf + static_cast<size_t>(line) * 16)[20 + slot] =
+            static_cast<uint32_t>(t);
+    if (t < n) sink[t] = static_cast<uint32_t>(old);
+}
+
+}  // namespace
+}  // namespace ash
+
+using namespace ash;
+
+extern "C" int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes,
+                                     int64_t n, uint32_t* sink, uint64_t seed,
+                                     void* stream) {
+    if (buf == nullptr || sink == nullptr) ASH_FAIL("null buffer");
+    if (buf_bytes < 128 || buf_bytes / 128 > 0xFFFFFFFFll) {
+        ASH_FAIL("buffer must hold between 1 and 2^32-1 lines of 128 bytes");
+    }
+    if (n <= 0 || n % kBlock != 0 || n > (int64_t{1} << 31)) {
+        ASH_FAIL("n must be a positive multiple of 256 below 2^31");
+    }
+    if (reinterpret_cast<uintptr_t>(buf) % 128 != 0) {
+        ASH_FAIL("buffer must be 128-byte aligned");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t nlines = static_cast<uint32_t>(buf_bytes / 128);
+    const unsigned g = static_cast<unsigned>(n / kBlock);
+    if (mode == 0) {
+        probe_line_reads<<<g, kBlock, 0, s>>>(static_cast<const uint4*>(buf),
+                                              nlines, n, sink, seed);
+    } else if (mode == 1) {
+        probe_line_updates<<<g, kBlock, 0, s>>>(
+                static_cast<unsigned long long*>(buf), nlines, n, sink, seed);
+    } else {
+        ASH_FAIL("unknown probe mode");
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}

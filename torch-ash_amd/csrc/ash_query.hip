@@ -40,6 +40,19 @@ constexpr int kXcds = 8;
 constexpr int64_t kMaxLdsCells = 2048;  // 2048 * 8 * 3 B = 48 KiB
 constexpr uint32_t kNoRow = 0xFFFFFFFFu;
 constexpr int kLdsPerCu = 160 * 1024;
+// Wavefronts per SIMD the kernels are compiled for: the highest occupancy that
+// needs no register spills (measured: spilling costs more than the extra
+// wavefronts bring).  The one-lane-per-query gather fits 4, the
+// channel-parallel kernels, which hold 8 rows plus the run-merge state per
+// lane, fit 3.
+#ifndef ASH_WAVES_GATHER
+#define ASH_WAVES_GATHER 4
+#endif
+#ifndef ASH_WAVES_WIDE
+#define ASH_WAVES_WIDE 3
+#endif
+constexpr int kWavesGather = ASH_WAVES_GATHER;
+constexpr int kWavesWide = ASH_WAVES_WIDE;
 
 struct QDev {
     const void* emb;
@@ -55,7 +68,6 @@ struct QDev {
     int64_t M;
     int E;
     int smooth;    // 0 linear, 1 smooth step
-    int lds_lut;   // per-cell tables staged in LDS
     int merge;     // pre-reduce runs of equal rows before the atomics
 };
 
@@ -124,10 +136,11 @@ struct CellLut {
     const uint8_t* c2g;
 };
 
+template <bool LDS>
 __device__ __forceinline__ void cell_neighbor(const QDev& a, const CellLut& lut,
                                               int64_t cell, int c, int& nb_cell,
                                               int& nb_grid) {
-    if (a.lds_lut) {
+    if constexpr (LDS) {
         nb_cell = lut.c2c[cell * 8 + c];
         nb_grid = lut.c2g[cell * 8 + c];
     } else {
@@ -138,12 +151,13 @@ __device__ __forceinline__ void cell_neighbor(const QDev& a, const CellLut& lut,
     }
 }
 
+template <bool LDS>
 __device__ __forceinline__ CellLut stage_cell_lut(const QDev& a,
                                                   unsigned char* smem) {
     CellLut lut;
     lut.c2c = nullptr;
     lut.c2g = nullptr;
-    if (a.lds_lut) {
+    if constexpr (LDS) {
         uint16_t* s_c2c = reinterpret_cast<uint16_t*>(smem);
         uint8_t* s_c2g = smem + a.M * 8 * 2;
         const int64_t n = a.M * 8;
@@ -180,6 +194,7 @@ struct TileWalk {
 
 // Phase 1 for one query: the 8 corner rows (kNoRow in row[0] when the query is
 // masked out, out of range, or misses a neighbour block) and the offsets.
+template <bool LDS>
 __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
                                              int64_t q, uint32_t (&row)[8],
                                              float (&o)[3]) {
@@ -195,20 +210,26 @@ __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
         valid = gi >= 0 && gi < a.B;
         ci = ci < 0 ? 0 : (ci >= a.M ? a.M - 1 : ci);
     }
-    int64_t g0 = -1;
-    if (valid) g0 = a.lut_g[gi * 8];
+    // Block indices are below 2^31 and a missing block is -1, so the low
+    // dword of each int64 table entry carries everything.
+    const int32_t* lut_g32 = reinterpret_cast<const int32_t*>(a.lut_g) + gi * 16;
+    int32_t g0 = -1;
+    if (valid) g0 = lut_g32[0];
+    const uint32_t nblocks = static_cast<uint32_t>(a.B);
+    const uint32_t cells = static_cast<uint32_t>(a.M);
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
         row[c] = 0;
         if (valid) {
             int nb_cell, nb_grid;
-            cell_neighbor(a, lut, ci, c, nb_cell, nb_grid);
-            int64_t g = g0;
-            if (nb_grid != 0) g = a.lut_g[gi * 8 + nb_grid];
-            if (g < 0 || g >= a.B) {
+            cell_neighbor<LDS>(a, lut, ci, c, nb_cell, nb_grid);
+            int32_t g = g0;
+            if (nb_grid != 0) g = lut_g32[nb_grid * 2];
+            if (static_cast<uint32_t>(g) >= nblocks) {
                 valid = false;
             } else {
-                row[c] = static_cast<uint32_t>(g * a.M + nb_cell);
+                row[c] = static_cast<uint32_t>(g) * cells +
+                         static_cast<uint32_t>(nb_cell);
             }
         }
     }
@@ -217,7 +238,7 @@ __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
 
 // Runs phase 1 for the tile and hands every thread the rows / offsets of the
 // query it serves in pass `p` of phase 2.
-template <int LPQ>
+template <int LPQ, bool LDS>
 struct TileStage {
     static constexpr int kPasses = LPQ;
     static constexpr int kQpp = kBlock / LPQ;  // queries per pass
@@ -227,7 +248,7 @@ struct TileStage {
                                                 int64_t tile, Tile* s,
                                                 uint32_t (&row)[8],
                                                 float (&o)[3]) {
-        resolve_rows(a, lut, tile * kBlock + threadIdx.x, row, o);
+        resolve_rows<LDS>(a, lut, tile * kBlock + threadIdx.x, row, o);
         if constexpr (LPQ > 1) {
             __syncthreads();  // previous tile fully consumed
 #pragma unroll
@@ -271,14 +292,15 @@ struct VecOf<double, 1> {
 };
 
 // ------------------------------------------------------------- forward
-template <typename T, int VEC, int LPQ>
-__global__ __launch_bounds__(kBlock) void query_forward_kernel(
+template <typename T, int VEC, int LPQ, bool LDS>
+__global__ __launch_bounds__(kBlock, LPQ == 1 ? kWavesGather : kWavesWide) void
+query_forward_kernel(
         QDev a, T* __restrict__ out) {
     extern __shared__ __align__(16) unsigned char smem[];
     Tile* tile_s = reinterpret_cast<Tile*>(smem);
     const CellLut lut =
-            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
-    using Stage = TileStage<LPQ>;
+            stage_cell_lut<LDS>(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ, LDS>;
     using V = typename VecOf<T, VEC>::type;
     const int ch0 = (threadIdx.x % LPQ) * VEC;
     const bool chv = ch0 < a.E;
@@ -370,15 +392,16 @@ __device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
 // grad_embeddings[row_c, k] += w_c * z[i,k];
 // grad_offsets[i,:] = sum_c (emb[row_c,:] . z[i,:]) * grad w_c
 // (ash/src/grid.cu:177-255).  One lane per channel.
-template <typename T, int LPQ>
-__global__ __launch_bounds__(kBlock) void query_backward_forward_kernel(
+template <typename T, int LPQ, bool LDS>
+__global__ __launch_bounds__(kBlock, kWavesWide) void
+query_backward_forward_kernel(
         QDev a, const T* __restrict__ z, T* __restrict__ grad_emb,
         T* __restrict__ grad_off) {
     extern __shared__ __align__(16) unsigned char smem[];
     Tile* tile_s = reinterpret_cast<Tile*>(smem);
     const CellLut lut =
-            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
-    using Stage = TileStage<LPQ>;
+            stage_cell_lut<LDS>(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ, LDS>;
     const int lane = threadIdx.x & 63;
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
@@ -429,15 +452,16 @@ __global__ __launch_bounds__(kBlock) void query_backward_forward_kernel(
 // -------------------------------------------------- backward of backward
 // d_c = grad w_c . gg_off[i];  grad_embeddings[row_c,k] += d_c * z[i,k];
 // grad_z[i,k] = sum_c d_c * emb[row_c,k]   (ash/src/grid.cu:309-387).
-template <typename T, int LPQ>
-__global__ __launch_bounds__(kBlock) void query_backward_backward_kernel(
+template <typename T, int LPQ, bool LDS>
+__global__ __launch_bounds__(kBlock, kWavesWide) void
+query_backward_backward_kernel(
         QDev a, const T* __restrict__ gg_off, const T* __restrict__ z,
         T* __restrict__ grad_z, T* __restrict__ grad_emb) {
     extern __shared__ __align__(16) unsigned char smem[];
     Tile* tile_s = reinterpret_cast<Tile*>(smem);
     const CellLut lut =
-            stage_cell_lut(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
-    using Stage = TileStage<LPQ>;
+            stage_cell_lut<LDS>(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ, LDS>;
     const int lane = threadIdx.x & 63;
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
@@ -577,7 +601,6 @@ int check_args(const ash_query_args* a, QDev& d) {
     d.M = a->cells_per_grid;
     d.E = static_cast<int>(a->embedding_dim);
     d.smooth = a->interpolation == ASH_INTERP_SMOOTH_STEP ? 1 : 0;
-    d.lds_lut = d.M <= kMaxLdsCells ? 1 : 0;
     d.merge = merge_enabled() ? 1 : 0;
     return 0;
 }
@@ -588,9 +611,11 @@ int pow2_ceil(int v) {
     return p;
 }
 
+bool lut_in_lds(const QDev& d) { return d.M <= kMaxLdsCells; }
+
 size_t smem_bytes(const QDev& d, int lpq) {
     size_t bytes = lpq > 1 ? sizeof(Tile) : 0;
-    if (d.lds_lut) bytes += static_cast<size_t>(d.M) * 8 * 3;
+    if (lut_in_lds(d)) bytes += static_cast<size_t>(d.M) * 8 * 3;
     return bytes;
 }
 
@@ -624,8 +649,13 @@ template <typename T, int VEC, int LPQ>
 int launch_forward(const QDev& d, void* out, hipStream_t s) {
     const size_t smem = smem_bytes(d, LPQ);
     const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
-    query_forward_kernel<T, VEC, LPQ>
-            <<<g, kBlock, smem, s>>>(d, static_cast<T*>(out));
+    if (lut_in_lds(d)) {
+        query_forward_kernel<T, VEC, LPQ, true>
+                <<<g, kBlock, smem, s>>>(d, static_cast<T*>(out));
+    } else {
+        query_forward_kernel<T, VEC, LPQ, false>
+                <<<g, kBlock, smem, s>>>(d, static_cast<T*>(out));
+    }
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -635,9 +665,15 @@ int launch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
                    hipStream_t s) {
     const size_t smem = smem_bytes(d, LPQ);
     const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
-    query_backward_forward_kernel<T, LPQ><<<g, kBlock, smem, s>>>(
-            d, static_cast<const T*>(z), static_cast<T*>(ge),
-            static_cast<T*>(go));
+    if (lut_in_lds(d)) {
+        query_backward_forward_kernel<T, LPQ, true><<<g, kBlock, smem, s>>>(
+                d, static_cast<const T*>(z), static_cast<T*>(ge),
+                static_cast<T*>(go));
+    } else {
+        query_backward_forward_kernel<T, LPQ, false><<<g, kBlock, smem, s>>>(
+                d, static_cast<const T*>(z), static_cast<T*>(ge),
+                static_cast<T*>(go));
+    }
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -647,9 +683,15 @@ int launch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
                    void* ge, hipStream_t s) {
     const size_t smem = smem_bytes(d, LPQ);
     const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
-    query_backward_backward_kernel<T, LPQ><<<g, kBlock, smem, s>>>(
-            d, static_cast<const T*>(gg), static_cast<const T*>(z),
-            static_cast<T*>(gz), static_cast<T*>(ge));
+    if (lut_in_lds(d)) {
+        query_backward_backward_kernel<T, LPQ, true><<<g, kBlock, smem, s>>>(
+                d, static_cast<const T*>(gg), static_cast<const T*>(z),
+                static_cast<T*>(gz), static_cast<T*>(ge));
+    } else {
+        query_backward_backward_kernel<T, LPQ, false><<<g, kBlock, smem, s>>>(
+                d, static_cast<const T*>(gg), static_cast<const T*>(z),
+                static_cast<T*>(gz), static_cast<T*>(ge));
+    }
     ASH_LAUNCH_CHECK();
     return 0;
 }
