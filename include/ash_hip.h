@@ -77,6 +77,21 @@ int ash_map_destroy(ash_map_t* map);
 int ash_map_find(ash_map_t* map, const int32_t* keys, int64_t n,
                  int64_t* indices, uint8_t* masks, void* stream);
 
+/* Replaces the body of `SparseDenseGrid.query` (ash/grid.py:183-199: about ten
+ * elementwise torch launches around one `find`) for a map with 3-d keys.
+ * x float32[n,3] are positions in cell units and G = grid_dim cells per block
+ * edge; per position, in fp32 and without fused multiply-add so that the
+ * result equals the torch expression bit for bit:
+ *   block = floor(x / G), inner = x - block * G, offsets = inner - floor(inner),
+ *   cell_indices = ix + G*iy + G*G*iz with i = (int)inner,
+ *   (grid_indices, masks) = find((int)block).
+ * Right at a block boundary fp32 rounding can take `inner` out of [0, G)
+ * (negative, or exactly G); such positions are moved to the neighbouring
+ * block so that cell indices stay in range.  Every output element is written. */
+int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
+                   int64_t* grid_indices, int64_t* cell_indices, float* offsets,
+                   uint8_t* masks, void* stream);
+
 /* Replaces `HashMap::insert_keys` (ash/src/hashmap_gpu.cuh:211-247).  New keys
  * pop one index each from the heap; duplicates (in the table or within the
  * batch) are ignored.  Keys beyond `capacity` are dropped and counted

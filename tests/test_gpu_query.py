@@ -325,3 +325,34 @@ def test_full_size_forward_properties(gpu_ash):
     assert bool((complete <= masks).all())
     assert float(complete.float().mean()) > 0.7
     assert torch.allclose(yc[complete], torch.ones_like(yc[complete]), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("grid_dim", [1, 3, 8, 16])
+def test_fused_cell_query_equals_elementwise_chain(gpu_ash, grid_dim):
+    """`SparseDenseGrid.query` through the fused kernel against the reference's
+    chain of elementwise torch operations (ash/grid.py:183-199), bit for bit:
+    random positions, integers, block boundaries and the fp32 rounding edge of
+    tiny negative coordinates; gradients flow to the positions."""
+    grid = _make_grid(gpu_ash, grid_dim, 2, 2, seed=grid_dim, holes=5)
+    g = torch.Generator().manual_seed(50 + grid_dim)
+    span = grid_dim * 4.0
+    rand = (torch.rand(20000, 3, generator=g) * 2 - 1) * span
+    ints = torch.randint(-3 * grid_dim, 3 * grid_dim + 1, (2000, 3), generator=g).float()
+    edge = torch.tensor(
+        [[-1e-9, 0.0, 0.0], [-1e-9, -1e-9, -1e-9], [grid_dim - 1e-7, 0.5, 0.5], [-0.0, 0.0, -1e-30],
+         [grid_dim * 1.0, grid_dim * 2.0, -grid_dim * 1.0], [1e-7 - grid_dim, 0.25, 0.75]]
+    )
+    below = torch.nextafter(ints[:500], torch.full_like(ints[:500], -1e9))
+    x = torch.cat([rand, ints, edge, below]).to(DEV)
+    fused = grid.query(x)
+    chain = grid._query_elementwise(x)
+    names = ("grid_indices", "cell_indices", "offsets", "masks")
+    for name, a, b in zip(names, fused, chain):
+        assert a.dtype == b.dtype and a.shape == b.shape, name
+        assert torch.equal(a, b), name
+    assert int(fused[1].max()) < grid_dim**3 and int(fused[1].min()) >= 0
+    assert float(fused[2].min()) >= 0 and float(fused[2].max()) < 1
+    xg = x.clone().requires_grad_(True)
+    off = grid.query(xg)[2]
+    (off * torch.arange(3, device=DEV)).sum().backward()
+    assert torch.equal(xg.grad, torch.arange(3, device=DEV).float().expand_as(xg))

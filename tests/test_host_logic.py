@@ -154,6 +154,26 @@ def test_query_rounding_edge(cpu_ash):
     assert gi[1].item() == k0.item() and ci[1].item() == 0
 
 
+@pytest.mark.parametrize("grid_dim", [1, 3, 8])
+def test_query_decomposition_invariants(cpu_ash, grid_dim):
+    """For every position, also one ulp below block boundaries:
+    block * G + cell + offset reproduces x, cell in [0, G)^3, offset in [0, 1)."""
+    grid = cpu_ash.SparseDenseGrid(3, 4, 1, grid_dim, device=CPU)
+    g = torch.Generator().manual_seed(grid_dim)
+    ints = torch.randint(-40 * grid_dim, 40 * grid_dim + 1, (4000, 3), generator=g).float()
+    below = torch.nextafter(ints, torch.full_like(ints, -1e9))
+    above = torch.nextafter(ints, torch.full_like(ints, 1e9))
+    rand = (torch.rand(4000, 3, generator=g) * 2 - 1) * 40 * grid_dim
+    x = torch.cat([ints, below, above, rand])
+    _, ci, off, _ = grid.query(x)
+    assert int(ci.min()) >= 0 and int(ci.max()) < grid_dim**3
+    assert float(off.min()) >= 0.0 and float(off.max()) < 1.0
+    cells = grid._delinearize_cell_indices(ci).double()
+    within = cells + off.double()
+    block = torch.round((x.double() - within) / grid_dim)
+    assert torch.allclose(block * grid_dim + within, x.double(), rtol=0, atol=1e-4)
+
+
 def test_spatial_init_dilation_and_bounds(cpu_ash):
     """ash/grid.py:121-159,850-852: dilation windows, out-of-box blocks dropped,
     few points with a wide window (more unique blocks than points)."""

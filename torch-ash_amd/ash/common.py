@@ -65,6 +65,10 @@ _SIGNATURES = {
     "ash_map_attach_general": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_destroy": (ctypes.c_int, [_PTR]),
     "ash_map_find": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR, _PTR, _PTR]),
+    "ash_grid_query": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, _PTR, _PTR, _PTR, _PTR, _PTR],
+    ),
     "ash_map_insert_keys": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_insert_needs_scratch": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_I64)]),
     "ash_map_insert": (
@@ -493,6 +497,30 @@ class _HashMap:
                 )
             )
         return indices, masks
+
+    def query_cells(
+        self, x: torch.Tensor, grid_dim: int
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Fused front end of `SparseDenseGrid.query`: positions in cell units ->
+        (grid_indices, cell_indices, offsets, masks) in one kernel."""
+        if x.dim() != 2 or x.shape[1] != 3 or x.dtype != torch.float32:
+            raise RuntimeError("positions must be float32 (N, 3)")
+        if x.device != self._device:
+            raise RuntimeError(f"positions are on {x.device}, the map on {self._device}")
+        x = x.contiguous()
+        n = x.shape[0]
+        grid_indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        cell_indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        offsets = torch.empty((n, 3), dtype=torch.float32, device=self._device)
+        masks = torch.empty(n, dtype=torch.bool, device=self._device)
+        with torch.cuda.device(self._device):
+            self._check(
+                self._lib.ash_grid_query(
+                    self._handle, x.data_ptr(), n, int(grid_dim), grid_indices.data_ptr(),
+                    cell_indices.data_ptr(), offsets.data_ptr(), masks.data_ptr(), self._stream(),
+                )
+            )
+        return grid_indices, cell_indices, offsets, masks
 
     def insert_keys(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)

@@ -22,6 +22,22 @@ backend = _get_c_extension()
 Interpolation = Literal["nearest", "linear", "smooth_step"]
 
 
+class _FusedCellQuery(torch.autograd.Function):
+    """x (cell units) -> (grid_indices, cell_indices, offsets, masks) through the
+    table's fused kernel.  Only `offsets` depends differentiably on x, with unit
+    Jacobian (offsets = x - floor(x) up to block shifts)."""
+
+    @staticmethod
+    def forward(ctx, x, table, grid_dim):
+        grid_indices, cell_indices, offsets, masks = table.query_cells(x, grid_dim)
+        ctx.mark_non_differentiable(grid_indices, cell_indices, masks)
+        return grid_indices, cell_indices, offsets, masks
+
+    @staticmethod
+    def backward(ctx, _grad_grid, _grad_cell, grad_offsets, _grad_masks):
+        return grad_offsets, None, None
+
+
 class SparseDenseGrid(ASHModule):
     """Grid addressed in cell units: position x lies in block floor(x / G) and,
     inside it, in cell floor(x - G * block).
@@ -134,11 +150,26 @@ class SparseDenseGrid(ASHModule):
         Returns grid_indices (N,), cell_indices (N,), offsets (N, 3) in [0, 1),
         masks (N,) = block is active.
         """
+        table = self.engine.backend
+        if hasattr(table, "query_cells") and x.dtype == torch.float32 and len(x) > 0:
+            # one kernel instead of the elementwise chain; same numbers
+            return _FusedCellQuery.apply(x, table, self.grid_dim)
+        return self._query_elementwise(x)
+
+    def _query_elementwise(self, x: torch.Tensor):
+        """`query` as a chain of elementwise torch operations around one find,
+        as the reference writes it; used for inputs the fused kernel does not
+        take (non-fp32 positions, empty batches)."""
         g = self.grid_dim
         x_sparse = (x / g).floor()
         x_dense = x - x_sparse * g
-        # For tiny negative x the subtraction rounds to exactly g in fp32; that
-        # position is cell 0 of the next block, not a cell index out of range.
+        # Two fp32 rounding cases right at a block boundary, where the plain
+        # formula leaves [0, g): x / g rounds up to an integer although x lies
+        # just below the boundary (x_dense < 0), and x - x_sparse * g rounds to
+        # exactly g for tiny negative x.  Both are moved back into range.
+        under = (x_dense < 0).to(x_dense.dtype)
+        x_sparse = x_sparse - under
+        x_dense = x_dense + under * g
         spill = (x_dense >= g).to(x_dense.dtype)
         x_sparse = x_sparse + spill
         x_dense = x_dense - spill * g

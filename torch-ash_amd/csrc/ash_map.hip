@@ -362,6 +362,79 @@ __global__ __launch_bounds__(kBlock) void find_kernel(
     }
 }
 
+// Fused front end of the sparse-dense grid query (ash/grid.py:183-199): splits a
+// position x (cell units) into block / cell / fractional part and looks the
+// block up, in one pass.  The arithmetic is the reference's torch expression
+// evaluated operation by operation in fp32 (no fused multiply-add, so the
+// results equal the elementwise torch formulation bit for bit):
+//   xs = floor(x / G); xd = x - xs * G; off = xd - floor(xd)
+// with two corrections at block boundaries, where fp32 rounding takes xd out
+// of [0, G): xd < 0 (x / G rounded up to an integer) steps back one block,
+// xd == G (tiny negative x) is cell 0 of the next block.
+__global__ __launch_bounds__(kBlock) void grid_query_kernel(
+        MapDev m, const float* __restrict__ x, int64_t n, float g, int gi,
+        int64_t* __restrict__ grid_idx, int64_t* __restrict__ cell_idx,
+        float* __restrict__ off, uint8_t* __restrict__ mask_out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const bool active = i < n;
+    int32_t k[3];
+    float o[3];
+    int64_t cell = 0;
+    int64_t stride = 1;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        const float xv = active ? x[i * 3 + d] : 0.f;
+        float xs = floorf(__fdiv_rn(xv, g));
+        float xd = __fsub_rn(xv, __fmul_rn(xs, g));
+        const float under = xd < 0.f ? 1.f : 0.f;
+        xs = __fsub_rn(xs, under);
+        xd = __fadd_rn(xd, __fmul_rn(under, g));
+        const float spill = xd >= g ? 1.f : 0.f;
+        xs = __fadd_rn(xs, spill);
+        xd = __fsub_rn(xd, __fmul_rn(spill, g));
+        o[d] = __fsub_rn(xd, floorf(xd));
+        k[d] = static_cast<int32_t>(xs);
+        cell += static_cast<int64_t>(static_cast<int32_t>(xd)) * stride;
+        stride *= gi;
+    }
+    uint64_t code;
+    const bool fits = pack_key<3>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+    int32_t res = 0;
+    bool found = false;
+    while (__ballot(pend)) {
+        ProbeResult p;
+        probe_pass(m, code, b, pend, lane, p);
+        if (pend) {
+            if (p.status == kProbeFound) {
+                found = true;
+                res = p.val;
+                pend = false;
+            } else if (p.status == kProbeHasEmpty) {
+                pend = false;
+            } else {
+                b = next_bucket(b, m.nb);
+                if (++steps >= m.nb) pend = false;
+            }
+        }
+    }
+    if (active && !fits) {
+        uint32_t pos;
+        found = gen_find<3>(m, k, res, pos);
+    }
+    if (active) {
+        grid_idx[i] = found ? static_cast<int64_t>(res) : 0;
+        mask_out[i] = found ? 1 : 0;
+        cell_idx[i] = cell;
+        off[i * 3 + 0] = o[0];
+        off[i * 3 + 1] = o[1];
+        off[i * 3 + 2] = o[2];
+    }
+}
+
 struct ValueArgs {
     int n;
     const uint32_t* src[kMaxFusedValues];
@@ -946,6 +1019,27 @@ int ash_map_find(ash_map_t* map, const int32_t* keys, int64_t n,
             find_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys, n, indices, masks);
             break;
     }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
+                   int64_t* grid_indices, int64_t* cell_indices, float* offsets,
+                   uint8_t* masks, void* stream) {
+    if (check_batch(map, x, n)) return 1;
+    if (map->key_dim != 3) ASH_FAIL("grid queries need a map with 3-d keys");
+    if (grid_dim < 1 || grid_dim > 1024) ASH_FAIL("grid_dim must be in 1..1024");
+    if (n == 0) return 0;
+    if (grid_indices == nullptr || cell_indices == nullptr ||
+        offsets == nullptr || masks == nullptr) {
+        ASH_FAIL("null output pointer");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    grid_query_kernel<<<grid_for(n), kBlock, 0,
+                        static_cast<hipStream_t>(stream)>>>(
+            map->d, x, n, static_cast<float>(grid_dim), grid_dim, grid_indices,
+            cell_indices, offsets, masks);
     ASH_LAUNCH_CHECK();
     return 0;
 }

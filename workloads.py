@@ -231,3 +231,105 @@ def ray_queries(
     t = (t * 2 - 1) * band
     x = target.view(-1, 1, 3) + t.unsqueeze(-1) * d.view(-1, 1, 3)
     return x.view(-1, 3).contiguous()
+
+
+# --------------------------------------------------------------------- cfg 5
+class FusionScene:
+    """Configuration 5: synthetic RGB-D stream.  48 random spheres, a pinhole
+    camera (fx = fy = 525, cx = 319.5, cy = 239.5 at 640x480; scaled with the
+    resolution) on a seeded orbit of radius 3 m looking at the origin, depth
+    images (fp32 metres) by analytic ray casting.  Everything is computed on
+    the CPU in float32 so that every backend is fed identical inputs."""
+
+    def __init__(self, num_spheres: int = 48, width: int = 640, height: int = 480, seed: int = 6):
+        g = _gen("cpu", seed)
+        self.width, self.height = width, height
+        sx, sy = width / 640.0, height / 480.0
+        self.intrinsic = torch.tensor(
+            [[525.0 * sx, 0.0, 319.5 * sx], [0.0, 525.0 * sy, 239.5 * sy], [0.0, 0.0, 1.0]]
+        )
+        self.radii = torch.rand(num_spheres, generator=g) * 0.35 + 0.1
+        self.centres = (torch.rand(num_spheres, 3, generator=g) * 2 - 1) * 1.2
+        self.phase = float(torch.rand(1, generator=g)) * 2 * math.pi
+        self.depth_max = 6.0
+
+    def pose(self, frame: int, num_frames: int = 100) -> torch.Tensor:
+        """world-to-camera 4x4 (camera looks along +z at the origin)."""
+        a = self.phase + 2 * math.pi * frame / num_frames
+        eye = torch.tensor([3.0 * math.cos(a), 0.6 * math.sin(2 * a), 3.0 * math.sin(a)])
+        fwd = -eye / eye.norm()
+        right = torch.linalg.cross(torch.tensor([0.0, 1.0, 0.0]), fwd)
+        right = right / right.norm()
+        up = torch.linalg.cross(fwd, right)
+        rot = torch.stack([right, up, fwd])  # rows: camera axes in world coordinates
+        ext = torch.eye(4)
+        ext[:3, :3] = rot
+        ext[:3, 3] = -rot @ eye
+        return ext
+
+    def depth(self, extrinsic: torch.Tensor) -> torch.Tensor:
+        """(H, W) depth along the camera z axis, 0 where no sphere is hit."""
+        v, u = torch.meshgrid(
+            torch.arange(self.height, dtype=torch.float32),
+            torch.arange(self.width, dtype=torch.float32),
+            indexing="ij",
+        )
+        k = self.intrinsic
+        d_cam = torch.stack([(u - k[0, 2]) / k[0, 0], (v - k[1, 2]) / k[1, 1], torch.ones_like(u)], -1)
+        rot, t = extrinsic[:3, :3], extrinsic[:3, 3]
+        origin = -rot.t() @ t
+        d = d_cam.view(-1, 3) @ rot  # camera ray directions in world coordinates
+        oc = origin.view(1, 1, 3) - self.centres.view(1, -1, 3)
+        b = (d.view(-1, 1, 3) * oc).sum(-1)
+        a = (d * d).sum(-1, keepdim=True)
+        c = (oc * oc).sum(-1) - self.radii.view(1, -1) ** 2
+        disc = b * b - a * c
+        s = (-b - disc.clamp_min(0).sqrt()) / a
+        s = torch.where((disc > 0) & (s > 0), s, torch.full_like(s, float("inf")))
+        z = s.min(dim=1)[0]  # parameter along d_cam == depth, since d_cam.z == 1
+        z = torch.where(torch.isfinite(z) & (z < self.depth_max), z, torch.zeros_like(z))
+        return z.view(self.height, self.width)
+
+    def unproject(self, depth: torch.Tensor, extrinsic: torch.Tensor) -> torch.Tensor:
+        """World-space points of the valid depth pixels (N, 3)."""
+        v, u = torch.nonzero(depth > 0, as_tuple=True)
+        z = depth[v, u]
+        k = self.intrinsic
+        cam = torch.stack([(u.float() - k[0, 2]) / k[0, 0] * z, (v.float() - k[1, 2]) / k[1, 1] * z, z], -1)
+        rot, t = extrinsic[:3, :3], extrinsic[:3, 3]
+        return ((cam - t) @ rot).contiguous()
+
+
+def fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc: float, depth_max: float = 6.0):
+    """One fusion step on `grid` (embedding channels: tsdf, weight), following
+    the reference demo (demo/rgbd_fusion.py:200-254 and :76-110): activate the
+    blocks around `points` with a one-block two-sided dilation, project every
+    cell of the touched blocks into the depth image, and update the running
+    weighted mean.  All tensors must live on the grid's device.  Returns the
+    number of touched blocks."""
+    gc, cc, gi, ci = grid.spatial_init_(points, dilation=1, bidirectional=True)
+    if gi.numel() == 0:
+        return 0
+    positions = grid.cell_to_world(gc, cc)
+    xyz = positions @ extrinsic[:3, :3].t() + extrinsic[:3, 3]
+    uvd = xyz @ intrinsic.t()
+    d = uvd[:, 2]
+    h, w = depth.shape
+    u = (uvd[:, 0] / d).round().long()
+    v = (uvd[:, 1] / d).round().long()
+    inside = (d > 0) & (u >= 0) & (v >= 0) & (u < w) & (v < h)
+    reading = torch.zeros_like(d)
+    reading[inside] = depth[v[inside], u[inside]]
+    sdf = reading - d
+    ok = inside & (reading > 0) & (reading < depth_max) & (sdf >= -trunc)
+    sdf = sdf.clamp(max=trunc)
+    weight = ok.float().view(gi.shape[0], ci.shape[1], 1)
+    sdf = sdf.view(gi.shape[0], ci.shape[1], 1)
+    with torch.no_grad():
+        cur = grid.embeddings[gi, ci]
+        w_sum, mean = cur[..., 1:2], cur[..., 0:1]
+        w_new = w_sum + weight
+        cur[..., 0:1] = (mean * w_sum + sdf * weight) / (w_new + 1e-6)
+        cur[..., 1:2] = w_new
+        grid.embeddings[gi, ci] = cur
+    return int(gi.shape[0])
