@@ -200,7 +200,10 @@ int ash_query_forward(const ash_query_args* a, void* output, void* stream);
 
 /* Replaces `query_backward_forward` (ash/src/grid.cu:177-307).
  * z scalar[N, E]; grad_embeddings scalar[B, M, E] (zero-filled here, then
- * accumulated); grad_offsets scalar[N, 3] (every row written). */
+ * accumulated); grad_offsets scalar[N, 3] (every row written).  One of the two
+ * outputs may be NULL: it is then not computed (for grad_embeddings that saves
+ * the dense zero fill and all atomics), which is what an autograd caller wants
+ * when only one gradient was requested. */
 int ash_query_backward_forward(const ash_query_args* a, const void* z,
                                void* grad_embeddings, void* grad_offsets,
                                void* stream);
@@ -210,7 +213,8 @@ int ash_query_backward_forward(const ash_query_args* a, const void* z,
  * (every row written) and grad_embeddings scalar[B,M,E] (zero-filled here).
  * As in the reference the incoming grad_grad_embeddings is not used and the
  * offsets gradient is identically zero (ash/src/grid.cu:417-426); the caller
- * produces that zero tensor itself. */
+ * produces that zero tensor itself.  One of grad_z / grad_embeddings may be
+ * NULL and is then not computed. */
 int ash_query_backward_backward(const ash_query_args* a,
                                 const void* grad_grad_offsets, const void* z,
                                 void* grad_z, void* grad_embeddings,

@@ -356,3 +356,49 @@ def test_fused_cell_query_equals_elementwise_chain(gpu_ash, grid_dim):
     off = grid.query(xg)[2]
     (off * torch.arange(3, device=DEV)).sum().backward()
     assert torch.equal(xg.grad, torch.arange(3, device=DEV).float().expand_as(xg))
+
+
+def test_optional_gradient_outputs(gpu_ash, oracle):
+    """Each backward entry point may skip one of its outputs; what it still
+    returns must equal the full call, and autograd asks only for what it needs
+    (autograd.grad w.r.t. positions alone never builds the dense embedding
+    gradient)."""
+    grid = _make_grid(gpu_ash, 4, 4, 1, seed=61)
+    x = _queries(4, 1, 5000, seed=62)
+    ops = _operands(grid, x)
+    backend = gpu_ash.grid_query.backend
+    gen = torch.Generator().manual_seed(63)
+    z = (torch.rand(5000, 4, generator=gen) - 0.5).to(DEV)
+    u = (torch.rand(5000, 3, generator=gen) - 0.5).to(DEV)
+    ge, go = backend.query_backward_forward(z, *ops, 4, "smooth_step")
+    ge1, none1 = backend.query_backward_forward(z, *ops, 4, "smooth_step", need_offsets=False)
+    none2, go2 = backend.query_backward_forward(z, *ops, 4, "smooth_step", need_embeddings=False)
+    assert none1 is None and none2 is None
+    assert torch.allclose(ge1, ge, rtol=RTOL32, atol=8 * ATOL32) and torch.equal(go2, go)
+    gz, ge_b, _ = backend.query_backward_backward(None, u, z, *ops, 4, "smooth_step")
+    gz1, n1, _ = backend.query_backward_backward(None, u, z, *ops, 4, "smooth_step", need_embeddings=False)
+    n2, ge_b2, _ = backend.query_backward_backward(None, u, z, *ops, 4, "smooth_step", need_z=False)
+    assert n1 is None and n2 is None
+    assert torch.equal(gz1, gz) and torch.allclose(ge_b2, ge_b, rtol=RTOL32, atol=8 * ATOL32)
+    with pytest.raises(RuntimeError, match="at least one"):
+        backend.query_backward_forward(
+            z, *ops, 4, "smooth_step", need_embeddings=False, need_offsets=False
+        )
+
+    calls = []
+    real = backend.query_backward_forward
+
+    def spy(*args, **kwargs):
+        calls.append(kwargs)
+        return real(*args, **kwargs)
+
+    backend.query_backward_forward = spy
+    try:
+        xq = x.clone().requires_grad_(True)
+        feats, _ = grid(xq, "smooth_step")
+        (gx,) = torch.autograd.grad(feats.sum(), xq, create_graph=True)
+        assert calls == [{"need_embeddings": False, "need_offsets": True}]
+        (gx.norm(dim=-1) - 1).abs().mean().backward()
+        assert grid.embeddings.grad is not None
+    finally:
+        del backend.query_backward_forward

@@ -256,7 +256,12 @@ class _Backend:
         lut_cell_nb2grid_nb,
         grid_dim,
         interpolation,
-    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        need_embeddings: bool = True,
+        need_offsets: bool = True,
+    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """(grad_embeddings, grad_offsets); an output that is not needed is
+        None and its work (for grad_embeddings: dense zero fill + atomics) is
+        skipped."""
         args, held, dev = self._query_args(
             embeddings,
             offsets,
@@ -269,15 +274,19 @@ class _Backend:
             interpolation,
         )
         z = _as_like(z, embeddings, (args.num_queries, args.embedding_dim), "z")
-        grad_embeddings = torch.empty_like(held[0])
-        grad_offsets = torch.empty((args.num_queries, 3), dtype=embeddings.dtype, device=dev)
+        grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
+        grad_offsets = (
+            torch.empty((args.num_queries, 3), dtype=embeddings.dtype, device=dev)
+            if need_offsets
+            else None
+        )
         with torch.cuda.device(dev):
             self.check(
                 self.lib.ash_query_backward_forward(
                     ctypes.byref(args),
                     z.data_ptr(),
-                    grad_embeddings.data_ptr(),
-                    grad_offsets.data_ptr(),
+                    grad_embeddings.data_ptr() if need_embeddings else None,
+                    grad_offsets.data_ptr() if need_offsets else None,
                     _stream_of(dev),
                 )
             )
@@ -298,7 +307,11 @@ class _Backend:
         lut_cell_nb2grid_nb,
         grid_dim,
         interpolation,
-    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        need_z: bool = True,
+        need_embeddings: bool = True,
+    ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor]:
+        """(grad_z, grad_embeddings, zero grad_offsets); outputs that are not
+        needed are None and their work is skipped."""
         args, held, dev = self._query_args(
             embeddings,
             offsets,
@@ -313,16 +326,16 @@ class _Backend:
         n, e = args.num_queries, args.embedding_dim
         z = _as_like(z, embeddings, (n, e), "z")
         gg_off = _as_like(grad_grad_offsets, embeddings, (n, 3), "grad_grad_offsets")
-        grad_z = torch.empty((n, e), dtype=embeddings.dtype, device=dev)
-        grad_embeddings = torch.empty_like(held[0])
+        grad_z = torch.empty((n, e), dtype=embeddings.dtype, device=dev) if need_z else None
+        grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
         with torch.cuda.device(dev):
             self.check(
                 self.lib.ash_query_backward_backward(
                     ctypes.byref(args),
                     gg_off.data_ptr(),
                     z.data_ptr(),
-                    grad_z.data_ptr(),
-                    grad_embeddings.data_ptr(),
+                    grad_z.data_ptr() if need_z else None,
+                    grad_embeddings.data_ptr() if need_embeddings else None,
                     _stream_of(dev),
                 )
             )

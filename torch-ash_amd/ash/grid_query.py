@@ -14,6 +14,21 @@ backend = _get_c_extension()
 _N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
 
 
+def _grad_requested(ctx, index: int) -> bool:
+    """Whether the running backward pass will consume the gradient of input
+    `index`.  `ctx.needs_input_grad` only says that the input requires grad;
+    in `autograd.grad(y, x)` the engine additionally knows which graph nodes it
+    is going to execute, and the node behind an input it will not execute (the
+    dense embeddings parameter, typically) needs no gradient from us."""
+    if not ctx.needs_input_grad[index]:
+        return False
+    try:
+        node = ctx.next_functions[index][0]
+        return node is not None and torch._C._will_engine_execute_node(node)
+    except Exception:  # outside an engine pass, or an older torch: be conservative
+        return True
+
+
 class SparseDenseGridQuery(torch.autograd.Function):
     """y[i] = sum over the 8 cell corners c of w_c(offsets[i]) * embeddings[row_c(i)].
 
@@ -56,8 +71,20 @@ class SparseDenseGridQuery(torch.autograd.Function):
     def backward(ctx, z: torch.Tensor):
         """Delegates to SparseDenseGridQueryBackward so that this step is itself
         differentiable (needed for gradient-norm losses)."""
+        need_embeddings, need_offsets = _grad_requested(ctx, 0), _grad_requested(ctx, 1)
+        if not (need_embeddings or need_offsets):
+            return (None,) * (2 + _N_TABLE_ARGS)
+        # The reference always produces both gradients (ash/grid_query.py:104-116);
+        # the dense embedding gradient (zero fill + atomics over the whole
+        # parameter) is skipped when nobody asked for it, e.g. in
+        # autograd.grad(y, x, create_graph=True).
         grad_embeddings, grad_offsets = SparseDenseGridQueryBackward.apply(
-            z.contiguous(), *ctx.saved_tensors, ctx.grid_dim, ctx.interpolation
+            z.contiguous(),
+            *ctx.saved_tensors,
+            ctx.grid_dim,
+            ctx.interpolation,
+            need_embeddings,
+            need_offsets,
         )
         return (grad_embeddings, grad_offsets) + (None,) * _N_TABLE_ARGS
 
@@ -85,7 +112,12 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
         lut_cell_nb2grid_nb,
         grid_dim,
         interpolation,
+        need_grad_embeddings: bool = True,
+        need_grad_offsets: bool = True,
     ):
+        """With both `need_*` flags at their default this is the reference's
+        signature and result; an output that is not needed is returned as None
+        and its work is skipped."""
         operands = (
             z,
             embeddings,
@@ -100,7 +132,15 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
         ctx.save_for_backward(*operands)
         ctx.grid_dim = grid_dim
         ctx.interpolation = interpolation
-        return backend.query_backward_forward(*operands, grid_dim, interpolation)
+        if need_grad_embeddings and need_grad_offsets:
+            return backend.query_backward_forward(*operands, grid_dim, interpolation)
+        return backend.query_backward_forward(
+            *operands,
+            grid_dim,
+            interpolation,
+            need_embeddings=need_grad_embeddings,
+            need_offsets=need_grad_offsets,
+        )
 
     @staticmethod
     def backward(ctx, grad_grad_embeddings: torch.Tensor, grad_grad_offsets: torch.Tensor):
@@ -113,11 +153,26 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
         ash/src/grid.cu:417-426) the incoming `grad_grad_embeddings` is not used
         and no gradient flows to `offsets` at second order.
         """
-        grad_z, grad_embeddings, _ = backend.query_backward_backward(
-            grad_grad_embeddings,
-            grad_grad_offsets,
-            *ctx.saved_tensors,
-            ctx.grid_dim,
-            ctx.interpolation,
-        )
-        return (grad_z, grad_embeddings) + (None,) * (_N_TABLE_ARGS + 1)
+        need_z, need_embeddings = _grad_requested(ctx, 0), _grad_requested(ctx, 1)
+        n_rest = _N_TABLE_ARGS + 3  # offsets, tables, grid_dim, interpolation, 2 flags
+        if grad_grad_offsets is None or not (need_z or need_embeddings):
+            return (None, None) + (None,) * n_rest
+        if need_z and need_embeddings:
+            grad_z, grad_embeddings, _ = backend.query_backward_backward(
+                grad_grad_embeddings,
+                grad_grad_offsets,
+                *ctx.saved_tensors,
+                ctx.grid_dim,
+                ctx.interpolation,
+            )
+        else:
+            grad_z, grad_embeddings, _ = backend.query_backward_backward(
+                grad_grad_embeddings,
+                grad_grad_offsets,
+                *ctx.saved_tensors,
+                ctx.grid_dim,
+                ctx.interpolation,
+                need_z=need_z,
+                need_embeddings=need_embeddings,
+            )
+        return (grad_z, grad_embeddings) + (None,) * n_rest

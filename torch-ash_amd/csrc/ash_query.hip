@@ -406,6 +406,8 @@ query_backward_forward_kernel(
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const bool want_emb = grad_emb != nullptr;  // either output may be skipped
+    const bool want_off = grad_off != nullptr;
     const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
@@ -421,26 +423,32 @@ query_backward_forward_kernel(
             T e[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                e[c] = on ? emb[static_cast<int64_t>(row[c]) * a.E + ch] : T(0);
+                e[c] = (on && want_off)
+                               ? emb[static_cast<int64_t>(row[c]) * a.E + ch]
+                               : T(0);
             }
             AxisTerms<T> t;
             axis_terms<T, true>(o, a.smooth, t);
             T go[3] = {T(0), T(0), T(0)};
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                const T w = corner_weight<T>(t, c);
-                T gw[3];
-                corner_weight_grad<T>(t, c, gw);
-                accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk,
-                                       lane, a.merge);
-                T dot = e[c] * zk;
+                if (want_emb) {
+                    const T w = corner_weight<T>(t, c);
+                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk,
+                                           lane, a.merge);
+                }
+                if (want_off) {
+                    T gw[3];
+                    corner_weight_grad<T>(t, c, gw);
+                    T dot = e[c] * zk;
 #pragma unroll
-                for (int s = 1; s < LPQ; s <<= 1) dot += __shfl_xor(dot, s);
-                go[0] += dot * gw[0];
-                go[1] += dot * gw[1];
-                go[2] += dot * gw[2];
+                    for (int s = 1; s < LPQ; s <<= 1) dot += __shfl_xor(dot, s);
+                    go[0] += dot * gw[0];
+                    go[1] += dot * gw[1];
+                    go[2] += dot * gw[2];
+                }
             }
-            if (q < a.N && ch == 0) {
+            if (want_off && q < a.N && ch == 0) {
                 grad_off[q * 3 + 0] = valid ? go[0] : T(0);
                 grad_off[q * 3 + 1] = valid ? go[1] : T(0);
                 grad_off[q * 3 + 2] = valid ? go[2] : T(0);
@@ -466,6 +474,8 @@ query_backward_backward_kernel(
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const bool want_z = grad_z != nullptr;  // either output may be skipped
+    const bool want_emb = grad_emb != nullptr;
     const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
@@ -487,7 +497,9 @@ query_backward_backward_kernel(
             T e[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                e[c] = on ? emb[static_cast<int64_t>(row[c]) * a.E + ch] : T(0);
+                e[c] = (on && want_z)
+                               ? emb[static_cast<int64_t>(row[c]) * a.E + ch]
+                               : T(0);
             }
             AxisTerms<T> t;
             axis_terms<T, true>(o, a.smooth, t);
@@ -497,11 +509,15 @@ query_backward_backward_kernel(
                 T gw[3];
                 corner_weight_grad<T>(t, c, gw);
                 const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
-                accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk,
-                                       lane, a.merge);
+                if (want_emb) {
+                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk,
+                                           lane, a.merge);
+                }
                 gz += d * e[c];
             }
-            if (q < a.N && chv) grad_z[q * a.E + ch] = on ? gz : T(0);
+            if (want_z && q < a.N && chv) {
+                grad_z[q * a.E + ch] = on ? gz : T(0);
+            }
         }
     }
 }
@@ -786,13 +802,16 @@ int ash_query_backward_forward(const ash_query_args* a, const void* z,
                                void* stream) {
     QDev d;
     if (check_args(a, d)) return 1;
-    if (grad_embeddings == nullptr) ASH_FAIL("null grad_embeddings pointer");
+    if (grad_embeddings == nullptr && grad_offsets == nullptr) {
+        ASH_FAIL("at least one of grad_embeddings / grad_offsets is required");
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
+    if (grad_embeddings != nullptr &&
+        zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
         return 1;
     }
     if (d.N == 0) return 0;
-    if (z == nullptr || grad_offsets == nullptr) ASH_FAIL("null pointer");
+    if (z == nullptr) ASH_FAIL("null pointer");
     return a->dtype == ASH_F64
                    ? dispatch_bwd_fwd<double>(d, z, grad_embeddings,
                                               grad_offsets, s)
@@ -806,15 +825,16 @@ int ash_query_backward_backward(const ash_query_args* a,
                                 void* stream) {
     QDev d;
     if (check_args(a, d)) return 1;
-    if (grad_embeddings == nullptr) ASH_FAIL("null grad_embeddings pointer");
+    if (grad_embeddings == nullptr && grad_z == nullptr) {
+        ASH_FAIL("at least one of grad_z / grad_embeddings is required");
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
+    if (grad_embeddings != nullptr &&
+        zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
         return 1;
     }
     if (d.N == 0) return 0;
-    if (z == nullptr || grad_grad_offsets == nullptr || grad_z == nullptr) {
-        ASH_FAIL("null pointer");
-    }
+    if (z == nullptr || grad_grad_offsets == nullptr) ASH_FAIL("null pointer");
     return a->dtype == ASH_F64
                    ? dispatch_bwd_bwd<double>(d, grad_grad_offsets, z, grad_z,
                                               grad_embeddings, s)
