@@ -24,6 +24,10 @@
 
 #include "../../include/ash_hip.h"
 
+#ifndef ASH_HEAP_BLOCK
+#define ASH_HEAP_BLOCK 256
+#endif
+
 namespace ash {
 
 static thread_local std::string g_last_error;
@@ -32,6 +36,11 @@ void set_error(const std::string& msg) { g_last_error = msg; }
 namespace {
 
 constexpr int kBlock = 256;
+// Workgroup size of the kernels that advance the heap counter (once per
+// workgroup).  Larger groups mean fewer updates of that single address but
+// make every wavefront wait for the slowest probe of the group; measured on
+// 16 M keys: 256 -> 1.28 ms, 512 -> 1.46 ms, 1024 -> 1.42 ms.
+constexpr int kHeapBlock = ASH_HEAP_BLOCK;
 constexpr int kMaxFusedValues = 4;
 constexpr int kMaxFusedRowDwords = 16;
 constexpr uint32_t kSpinLimit = 1u << 22;
@@ -450,10 +459,10 @@ enum InsertMode {
 };
 
 template <int DIM, int MODE>
-__global__ __launch_bounds__(kBlock) void insert_kernel(
+__global__ __launch_bounds__(kHeapBlock) void insert_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n, ValueArgs va,
         int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kHeapBlock + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const bool active = i < n;
@@ -533,7 +542,7 @@ __global__ __launch_bounds__(kBlock) void insert_kernel(
     if constexpr (MODE == kInsertLoad) {
         if (w) idx = static_cast<int32_t>(given[i]);
     } else {
-        __shared__ int s_cnt[kBlock / 64];
+        __shared__ int s_cnt[kHeapBlock / 64];
         __shared__ int s_base;
         const uint64_t wm = __ballot(w);
         const int nw = __popcll(wm);
@@ -543,7 +552,7 @@ __global__ __launch_bounds__(kBlock) void insert_kernel(
         if (threadIdx.x == 0) {
             int tot = 0;
 #pragma unroll
-            for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+            for (int q = 0; q < kHeapBlock / 64; ++q) tot += s_cnt[q];
             int base = 0;
             if (tot > 0) {
                 base = atomicAdd(m.ctr + kCtrSize, tot);
@@ -600,9 +609,9 @@ __global__ __launch_bounds__(kBlock) void insert_kernel(
 }
 
 template <int DIM>
-__global__ __launch_bounds__(kBlock) void erase_kernel(
+__global__ __launch_bounds__(kHeapBlock) void erase_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kHeapBlock + threadIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const bool active = i < n;
@@ -652,7 +661,7 @@ __global__ __launch_bounds__(kBlock) void erase_kernel(
             }
         }
     }
-    __shared__ int s_cnt[kBlock / 64];
+    __shared__ int s_cnt[kHeapBlock / 64];
     __shared__ int s_base;
     const uint64_t wm = __ballot(won);
     const int nw = __popcll(wm);
@@ -666,7 +675,7 @@ __global__ __launch_bounds__(kBlock) void erase_kernel(
     if (threadIdx.x == 0) {
         int tot = 0;
 #pragma unroll
-        for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+        for (int q = 0; q < kHeapBlock / 64; ++q) tot += s_cnt[q];
         s_base = tot > 0 ? atomicSub(m.ctr + kCtrSize, tot) : 0;
     }
     __syncthreads();
@@ -680,27 +689,47 @@ __global__ __launch_bounds__(kBlock) void erase_kernel(
 
 // items(): thread t reads the 16-byte unit t of the bucket array (two code
 // slots, or index words for the last lanes of a line), four units per thread.
+// Output positions come from one global cursor; atomics on that single address
+// serialise (about 7 ns each across the XCDs), so the workgroup is made as
+// large as possible (1024 threads, one atomic per 4096 units): with 256-thread
+// groups the cursor alone cost more than reading the whole table.
+constexpr int kItemsBlock = 1024;
+constexpr int kItemsUnroll = 4;
+
 template <int DIM>
-__global__ __launch_bounds__(kBlock) void items_kernel(
+__global__ __launch_bounds__(kItemsBlock) void items_kernel(
         MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out,
         int64_t n_expected) {
-    constexpr int kUnroll = 4;
+    constexpr int kUnroll = kItemsUnroll;
+    constexpr int kWaves = kItemsBlock / 64;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int j = lane & (kGroup - 1);
     const bool v0 = (2 * j) < kSlots;
     const bool v1 = (2 * j + 1) < kSlots;
     const uint64_t units = static_cast<uint64_t>(m.nb) * kGroup;
-    const uint64_t t0 = static_cast<uint64_t>(blockIdx.x) * (kBlock * kUnroll) +
-                        threadIdx.x;
+    const uint64_t t0 =
+            static_cast<uint64_t>(blockIdx.x) * (kItemsBlock * kUnroll) +
+            threadIdx.x;
     uint64_t qa[kUnroll], qb[kUnroll];
+    int32_t va[kUnroll], vb[kUnroll];
     bool l0[kUnroll], l1[kUnroll];
     int cnt = 0;
+    // The index of slot s is dword 20+s of the line: for the code lane j (slots
+    // 2j, 2j+1) that is lane 5 + j/2 of the same group, components x,y (j even)
+    // or z,w (j odd).
+    const int vsrc = (lane & ~(kGroup - 1)) + 5 + (j >> 1);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-        const uint64_t t = t0 + static_cast<uint64_t>(u) * kBlock;
+        const uint64_t t = t0 + static_cast<uint64_t>(u) * kItemsBlock;
         uint4 q = make_uint4(~0u, ~0u, ~0u, ~0u);
         if (t < units) q = reinterpret_cast<const uint4*>(m.buckets)[t];
+        const int sx = __shfl(static_cast<int>(q.x), vsrc);
+        const int sy = __shfl(static_cast<int>(q.y), vsrc);
+        const int sz = __shfl(static_cast<int>(q.z), vsrc);
+        const int sw = __shfl(static_cast<int>(q.w), vsrc);
+        va[u] = (j & 1) ? sz : sx;
+        vb[u] = (j & 1) ? sw : sy;
         qa[u] = static_cast<uint64_t>(q.x) | (static_cast<uint64_t>(q.y) << 32);
         qb[u] = static_cast<uint64_t>(q.z) | (static_cast<uint64_t>(q.w) << 32);
         l0[u] = v0 && qa[u] < kTomb;
@@ -714,14 +743,14 @@ __global__ __launch_bounds__(kBlock) void items_kernel(
         const int up = __shfl_up(incl, d);
         if (lane >= d) incl += up;
     }
-    __shared__ int s_cnt[kBlock / 64];
+    __shared__ int s_cnt[kWaves];
     __shared__ int s_base;
     if (lane == 63) s_cnt[wave] = incl;
     __syncthreads();
     if (threadIdx.x == 0) {
         int tot = 0;
 #pragma unroll
-        for (int q = 0; q < kBlock / 64; ++q) tot += s_cnt[q];
+        for (int q = 0; q < kWaves; ++q) tot += s_cnt[q];
         s_base = tot > 0 ? atomicAdd(m.ctr + kCtrCursor, tot) : 0;
     }
     __syncthreads();
@@ -729,20 +758,16 @@ __global__ __launch_bounds__(kBlock) void items_kernel(
     for (int q = 0; q < wave; ++q) pos += s_cnt[q];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-        const uint64_t t = t0 + static_cast<uint64_t>(u) * kBlock;
-        const uint32_t bkt = static_cast<uint32_t>(t / kGroup);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const bool live = h == 0 ? l0[u] : l1[u];
             if (live) {
-                const uint64_t code = h == 0 ? qa[u] : qb[u];
-                const int32_t val = *value_ptr(m, bkt, 2 * j + h);
                 if (pos < n_expected) {
                     int32_t k[DIM];
-                    unpack_key<DIM>(code, k);
+                    unpack_key<DIM>(h == 0 ? qa[u] : qb[u], k);
 #pragma unroll
                     for (int d = 0; d < DIM; ++d) keys_out[pos * DIM + d] = k[d];
-                    idx_out[pos] = val;
+                    idx_out[pos] = h == 0 ? va[u] : vb[u];
                 }
                 ++pos;
             }
@@ -872,22 +897,22 @@ template <int MODE>
 int launch_insert(ash_map* map, const int32_t* keys, int64_t n,
                   const ValueArgs& va, int32_t* assigned, const int64_t* given,
                   hipStream_t s) {
-    const unsigned g = grid_for(n);
+    const unsigned g = grid_for(n, kHeapBlock);
     switch (map->key_dim) {
         case 1:
-            insert_kernel<1, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+            insert_kernel<1, MODE><<<g, kHeapBlock, 0, s>>>(map->d, keys, n, va,
                                                         assigned, given);
             break;
         case 2:
-            insert_kernel<2, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+            insert_kernel<2, MODE><<<g, kHeapBlock, 0, s>>>(map->d, keys, n, va,
                                                         assigned, given);
             break;
         case 3:
-            insert_kernel<3, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+            insert_kernel<3, MODE><<<g, kHeapBlock, 0, s>>>(map->d, keys, n, va,
                                                         assigned, given);
             break;
         default:
-            insert_kernel<4, MODE><<<g, kBlock, 0, s>>>(map->d, keys, n, va,
+            insert_kernel<4, MODE><<<g, kHeapBlock, 0, s>>>(map->d, keys, n, va,
                                                         assigned, given);
             break;
     }
@@ -899,7 +924,7 @@ int check_batch(const ash_map* map, const void* keys, int64_t n) {
     if (check_map(map)) return 1;
     if (n < 0) ASH_FAIL("negative key count");
     if (n > 0 && keys == nullptr) ASH_FAIL("null keys pointer");
-    if (n > (int64_t{1} << 31) - kBlock) ASH_FAIL("too many keys in one call");
+    if (n > (int64_t{1} << 31) - kHeapBlock) ASH_FAIL("too many keys in one call");
     return 0;
 }
 
@@ -1145,19 +1170,19 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const unsigned g = grid_for(n);
+    const unsigned g = grid_for(n, kHeapBlock);
     switch (map->key_dim) {
         case 1:
-            erase_kernel<1><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            erase_kernel<1><<<g, kHeapBlock, 0, s>>>(map->d, keys, n);
             break;
         case 2:
-            erase_kernel<2><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            erase_kernel<2><<<g, kHeapBlock, 0, s>>>(map->d, keys, n);
             break;
         case 3:
-            erase_kernel<3><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            erase_kernel<3><<<g, kHeapBlock, 0, s>>>(map->d, keys, n);
             break;
         default:
-            erase_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys, n);
+            erase_kernel<4><<<g, kHeapBlock, 0, s>>>(map->d, keys, n);
             break;
     }
     ASH_LAUNCH_CHECK();
@@ -1211,22 +1236,22 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrCursor, 0);
     ASH_LAUNCH_CHECK();
     const int64_t units = static_cast<int64_t>(map->d.nb) * kGroup;
-    const unsigned g = grid_for(units, kBlock * 4);
+    const unsigned g = grid_for(units, kItemsBlock * kItemsUnroll);
     switch (map->key_dim) {
         case 1:
-            items_kernel<1><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+            items_kernel<1><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
                                                  n_expected);
             break;
         case 2:
-            items_kernel<2><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+            items_kernel<2><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
                                                  n_expected);
             break;
         case 3:
-            items_kernel<3><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+            items_kernel<3><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
                                                  n_expected);
             break;
         default:
-            items_kernel<4><<<g, kBlock, 0, s>>>(map->d, keys_out, indices_out,
+            items_kernel<4><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
                                                  n_expected);
             break;
     }
