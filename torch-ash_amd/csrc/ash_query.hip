@@ -392,7 +392,8 @@ __device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
 // grad_embeddings[row_c, k] += w_c * z[i,k];
 // grad_offsets[i,:] = sum_c (emb[row_c,:] . z[i,:]) * grad w_c
 // (ash/src/grid.cu:177-255).  One lane per channel.
-template <typename T, int LPQ, bool LDS>
+// OUT: bit 0 = produce grad_embeddings, bit 1 = produce grad_offsets.
+template <typename T, int LPQ, bool LDS, int OUT>
 __global__ __launch_bounds__(kBlock, kWavesWide) void
 query_backward_forward_kernel(
         QDev a, const T* __restrict__ z, T* __restrict__ grad_emb,
@@ -406,8 +407,8 @@ query_backward_forward_kernel(
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
-    const bool want_emb = grad_emb != nullptr;  // either output may be skipped
-    const bool want_off = grad_off != nullptr;
+    constexpr bool want_emb = (OUT & 1) != 0;
+    constexpr bool want_off = (OUT & 2) != 0;
     const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
@@ -432,12 +433,12 @@ query_backward_forward_kernel(
             T go[3] = {T(0), T(0), T(0)};
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
-                if (want_emb) {
+                if constexpr (want_emb) {
                     const T w = corner_weight<T>(t, c);
                     accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk,
                                            lane, a.merge);
                 }
-                if (want_off) {
+                if constexpr (want_off) {
                     T gw[3];
                     corner_weight_grad<T>(t, c, gw);
                     T dot = e[c] * zk;
@@ -460,7 +461,8 @@ query_backward_forward_kernel(
 // -------------------------------------------------- backward of backward
 // d_c = grad w_c . gg_off[i];  grad_embeddings[row_c,k] += d_c * z[i,k];
 // grad_z[i,k] = sum_c d_c * emb[row_c,k]   (ash/src/grid.cu:309-387).
-template <typename T, int LPQ, bool LDS>
+// OUT: bit 0 = produce grad_embeddings, bit 1 = produce grad_z.
+template <typename T, int LPQ, bool LDS, int OUT>
 __global__ __launch_bounds__(kBlock, kWavesWide) void
 query_backward_backward_kernel(
         QDev a, const T* __restrict__ gg_off, const T* __restrict__ z,
@@ -474,8 +476,8 @@ query_backward_backward_kernel(
     const int ch = threadIdx.x % LPQ;
     const bool chv = ch < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
-    const bool want_z = grad_z != nullptr;  // either output may be skipped
-    const bool want_emb = grad_emb != nullptr;
+    constexpr bool want_emb = (OUT & 1) != 0;
+    constexpr bool want_z = (OUT & 2) != 0;
     const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
     TileWalk walk(ntiles);
     for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
@@ -509,7 +511,7 @@ query_backward_backward_kernel(
                 T gw[3];
                 corner_weight_grad<T>(t, c, gw);
                 const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
-                if (want_emb) {
+                if constexpr (want_emb) {
                     accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk,
                                            lane, a.merge);
                 }
@@ -681,15 +683,21 @@ int launch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
                    hipStream_t s) {
     const size_t smem = smem_bytes(d, LPQ);
     const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    const int out = (ge != nullptr ? 1 : 0) | (go != nullptr ? 2 : 0);
+#define ASH_BF(L, O)                                                          \
+    query_backward_forward_kernel<T, LPQ, L, O><<<g, kBlock, smem, s>>>(      \
+            d, static_cast<const T*>(z), static_cast<T*>(ge),                 \
+            static_cast<T*>(go))
     if (lut_in_lds(d)) {
-        query_backward_forward_kernel<T, LPQ, true><<<g, kBlock, smem, s>>>(
-                d, static_cast<const T*>(z), static_cast<T*>(ge),
-                static_cast<T*>(go));
+        if (out == 3) ASH_BF(true, 3);
+        else if (out == 1) ASH_BF(true, 1);
+        else ASH_BF(true, 2);
     } else {
-        query_backward_forward_kernel<T, LPQ, false><<<g, kBlock, smem, s>>>(
-                d, static_cast<const T*>(z), static_cast<T*>(ge),
-                static_cast<T*>(go));
+        if (out == 3) ASH_BF(false, 3);
+        else if (out == 1) ASH_BF(false, 1);
+        else ASH_BF(false, 2);
     }
+#undef ASH_BF
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -699,15 +707,21 @@ int launch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
                    void* ge, hipStream_t s) {
     const size_t smem = smem_bytes(d, LPQ);
     const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    const int out = (ge != nullptr ? 1 : 0) | (gz != nullptr ? 2 : 0);
+#define ASH_BB(L, O)                                                          \
+    query_backward_backward_kernel<T, LPQ, L, O><<<g, kBlock, smem, s>>>(     \
+            d, static_cast<const T*>(gg), static_cast<const T*>(z),           \
+            static_cast<T*>(gz), static_cast<T*>(ge))
     if (lut_in_lds(d)) {
-        query_backward_backward_kernel<T, LPQ, true><<<g, kBlock, smem, s>>>(
-                d, static_cast<const T*>(gg), static_cast<const T*>(z),
-                static_cast<T*>(gz), static_cast<T*>(ge));
+        if (out == 3) ASH_BB(true, 3);
+        else if (out == 1) ASH_BB(true, 1);
+        else ASH_BB(true, 2);
     } else {
-        query_backward_backward_kernel<T, LPQ, false><<<g, kBlock, smem, s>>>(
-                d, static_cast<const T*>(gg), static_cast<const T*>(z),
-                static_cast<T*>(gz), static_cast<T*>(ge));
+        if (out == 3) ASH_BB(false, 3);
+        else if (out == 1) ASH_BB(false, 1);
+        else ASH_BB(false, 2);
     }
+#undef ASH_BB
     ASH_LAUNCH_CHECK();
     return 0;
 }
