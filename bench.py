@@ -48,7 +48,7 @@ MEASURED_TRAFFIC_BYTES = {
     "insert_values": 2_563_000_000 + 1_819_000_000,
     "insert_keys": 2_303_000_000 + 1_564_000_000,
     "find": 2_230_000_000 + 146_000_000,
-    "items": 947_000_000 + 775_000_000,
+    "items": 512_000_000 + 324_000_000,
 }
 
 
