@@ -111,6 +111,30 @@ int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n,
                    int n_values, const void* const* src, void* const* dst,
                    const int64_t* row_bytes, int32_t* assigned, void* stream);
 
+/* Streaming variant of ash_map_insert_keys / ash_map_insert for batches of
+ * the order of the table itself (same reference functions,
+ * ash/src/hashmap_gpu.cuh:211-313, same resulting map): the batch is split by
+ * bucket range in two coalesced passes and each range of 512 buckets is then
+ * built in LDS by one workgroup and written back whole, so no global atomic is
+ * issued per key.  Inputs it cannot place that way (unpackable keys, piles of
+ * duplicates, an exhausted heap) are finished by the per-key kernel inside the
+ * same call.
+ *   ash_map_bulk_workspace_bytes: *bytes = size of the device workspace for
+ *   `n` keys with these value rows, 0 when the path does not apply (fewer than
+ *   4096 keys, rows that need `assigned`, a table of more than 2^25 buckets);
+ *   *worthwhile (optional) = 1 when n is large enough relative to the table
+ *   for the streaming path to be the faster one.
+ *   ash_map_insert_bulk: n_values may be 0 (keys only).  The workspace is
+ *   256-byte aligned, caller-owned and free again when the call's work on
+ *   `stream` has finished. */
+int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
+                                 const int64_t* row_bytes, int64_t* bytes,
+                                 int* worthwhile);
+int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
+                        int n_values, const void* const* src, void* const* dst,
+                        const int64_t* row_bytes, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
 /* Replaces `HashMap::erase` (ash/src/hashmap_gpu.cuh:316-351): found keys are
  * removed and their indices pushed back on the heap; duplicates inside the
  * batch erase once. */

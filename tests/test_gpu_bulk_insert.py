@@ -1,0 +1,159 @@
+"""GPU parity tests of the streaming insert path (ash_map_insert_bulk): forced
+on for every batch that it accepts, it must leave the same map as the oracle and
+as the per-key kernel -- same key set, masks, sizes, heap protocol, and each
+stored key carrying the value rows of ONE of its source rows."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_is_bijection_into, sort_rows
+from test_gpu_hash import _assert_same_map, _oracle_map
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+@pytest.fixture()
+def bulk_ash(gpu_ash, monkeypatch):
+    monkeypatch.setattr(gpu_ash.common, "BULK_INSERT", "always")
+    return gpu_ash
+
+
+def _random_keys(rng, n, dim, span):
+    return torch.from_numpy(rng.integers(-span, span, size=(n, dim)).astype(np.int32))
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 4])
+def test_bulk_keys_with_duplicates_match_oracle(bulk_ash, oracle, dim):
+    capacity = 150_000
+    rng = np.random.default_rng(900 + dim)
+    span = {1: 60_000, 2: 170, 3: 25, 4: 10}[dim]
+    keys = _random_keys(rng, 300_000, dim, span)
+    engine = bulk_ash.ASHEngine(dim, capacity, DEV)
+    omap = _oracle_map(oracle, dim, capacity)
+    engine.backend.insert_keys(keys.to(DEV))
+    omap.insert_keys(keys)
+    probe = _random_keys(rng, 50_000, dim, span + 2)
+    _assert_same_map(engine, omap, probe.to(DEV))
+    # indices of a fresh map are exactly 0 .. size-1 (heap[counter++])
+    _, idx = engine.items()
+    assert torch.equal(torch.sort(idx).values.cpu(), torch.arange(engine.size()))
+    assert engine.backend.status()["dropped"] == 0
+
+
+def test_bulk_into_a_populated_table_with_erases(bulk_ash, oracle):
+    """Second and third bulk batches meet live entries, tombstones and recycled
+    heap entries."""
+    dim, capacity = 3, 400_000
+    rng = np.random.default_rng(910)
+    engine = bulk_ash.ASHEngine(dim, capacity, DEV)
+    omap = _oracle_map(oracle, dim, capacity)
+    first = _random_keys(rng, 250_000, dim, 40)
+    engine.backend.insert_keys(first.to(DEV))
+    omap.insert_keys(first)
+    gone = first[rng.permutation(len(first))[:90_000]]
+    engine.erase(gone.to(DEV))
+    omap.erase(gone)
+    second = torch.cat([_random_keys(rng, 200_000, dim, 45), gone[:20_000]])
+    engine.backend.insert_keys(second.to(DEV))
+    omap.insert_keys(second)
+    probe = _random_keys(rng, 100_000, dim, 47)
+    _assert_same_map(engine, omap, probe.to(DEV))
+    # a small per-key batch and another bulk batch on top
+    third = _random_keys(rng, 3_000, dim, 46)
+    engine.backend.insert_keys(third.to(DEV))
+    omap.insert_keys(third)
+    fourth = _random_keys(rng, 150_000, dim, 46)
+    engine.backend.insert_keys(fourth.to(DEV))
+    omap.insert_keys(fourth)
+    _assert_same_map(engine, omap, probe.to(DEV))
+
+
+@pytest.mark.parametrize("capacity", [1_000, 200_000])
+def test_bulk_values_come_from_one_source_row(bulk_ash, capacity):
+    dim = 3
+    rng = np.random.default_rng(920)
+    n = 180_000
+    span = 4 if capacity == 1_000 else 30
+    keys = _random_keys(rng, n, dim, span).to(DEV)
+    row = torch.arange(n, device=DEV, dtype=torch.float32)
+    values = {
+        "color": torch.stack([row, row + 0.5, 2 * row], dim=1),
+        "depth": row.view(-1, 1).clone(),
+    }
+    hm = bulk_ash.HashMap(dim, {"color": 3, "depth": 1}, capacity, DEV)
+    hm.insert(keys, values)
+    uniq = torch.unique(keys, dim=0)
+    assert hm.size() == len(uniq)
+    idx, masks = hm.engine.find(uniq)
+    assert bool(masks.all())
+    assert_is_bijection_into(idx, capacity)
+    color, depth = hm.color[idx], hm.depth[idx]
+    src = depth[:, 0].long()
+    assert bool((src >= 0).all()) and bool((src < n).all())
+    # both rows come from the same source row, and that row holds this key
+    assert torch.equal(color, values["color"][src])
+    assert torch.equal(keys[src], uniq)
+
+
+def test_bulk_piles_of_duplicates_and_unpackable_keys(bulk_ash, oracle):
+    """Every key far beyond its partition's capacity (spill lists) plus keys
+    that do not fit the packed code (second region)."""
+    dim, capacity = 3, 50_000
+    rng = np.random.default_rng(930)
+    few = _random_keys(rng, 40, dim, 1000)
+    piles = few[rng.integers(0, 40, size=120_000)]
+    spread = _random_keys(rng, 60_000, dim, 18)
+    big = torch.from_numpy(
+        rng.integers(-(2**31), 2**31 - 1, size=(4_000, dim)).astype(np.int32))
+    keys = torch.cat([piles, spread, big, big[:500]])
+    keys = keys[torch.from_numpy(rng.permutation(len(keys)))]
+    engine = bulk_ash.ASHEngine(dim, capacity, DEV)
+    omap = _oracle_map(oracle, dim, capacity)
+    stores = {"v": torch.zeros(capacity, dim, dtype=torch.int32, device=DEV)}
+    engine.insert(keys.to(DEV), {"v": keys.to(DEV)}, stores)
+    omap.insert_keys(keys)
+    probe = torch.cat([keys[:50_000], keys[:20_000] + 1])
+    _assert_same_map(engine, omap, probe.to(DEV))
+    idx, mask = engine.find(keys.to(DEV))
+    assert bool(mask.all()) and torch.equal(stores["v"][idx].cpu(), keys)
+
+
+def test_bulk_overflow_drops_and_stays_usable(bulk_ash):
+    capacity = 30_000
+    engine = bulk_ash.ASHEngine(3, capacity, DEV)
+    g = torch.Generator().manual_seed(940)
+    keys = torch.arange(45_000, dtype=torch.int32).view(-1, 1).tile((1, 3))
+    keys = keys[torch.randperm(len(keys), generator=g)].to(DEV)
+    with pytest.warns(UserWarning, match="exceeds the hash map capacity"):
+        engine.insert_keys(keys)
+    assert engine.size() == capacity
+    idx, mask = engine.find(keys)
+    assert int(mask.sum()) == capacity
+    assert_is_bijection_into(idx[mask], capacity)
+    assert engine.backend.status()["dropped"] == 15_000
+    engine.erase(keys[mask][:9_000])
+    engine.insert_keys(keys[~mask][:9_000])
+    assert engine.size() == capacity
+    assert bool(engine.find(keys[~mask][:9_000])[1].all())
+
+
+def test_bulk_equals_per_key_kernel(gpu_ash, monkeypatch):
+    """The two insert paths on the same input: same key set, same size, and
+    finds agree key by key (indices are free)."""
+    dim, capacity = 3, 1_500_000
+    rng = np.random.default_rng(950)
+    keys = _random_keys(rng, 1_200_000, dim, 70).to(DEV)
+    probe = _random_keys(rng, 300_000, dim, 72).to(DEV)
+    maps = {}
+    for policy in ("always", "never"):
+        monkeypatch.setattr(gpu_ash.common, "BULK_INSERT", policy)
+        engine = gpu_ash.ASHEngine(dim, capacity, DEV)
+        engine.backend.insert_keys(keys)
+        maps[policy] = engine
+    a, b = maps["always"], maps["never"]
+    assert a.size() == b.size() == len(torch.unique(keys, dim=0))
+    assert torch.equal(sort_rows(a.items()[0])[0], sort_rows(b.items()[0])[0])
+    (ia, ma), (ib, mb) = a.find(probe), b.find(probe)
+    assert torch.equal(ma, mb)
+    assert_is_bijection_into(a.items()[1], capacity)

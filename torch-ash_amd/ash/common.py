@@ -85,6 +85,26 @@ _SIGNATURES = {
             _PTR,
         ],
     ),
+    "ash_map_bulk_workspace_bytes": (
+        ctypes.c_int,
+        [_PTR, _I64, ctypes.c_int, ctypes.POINTER(_I64), ctypes.POINTER(_I64),
+         ctypes.POINTER(ctypes.c_int)],
+    ),
+    "ash_map_insert_bulk": (
+        ctypes.c_int,
+        [
+            _PTR,
+            _PTR,
+            _I64,
+            ctypes.c_int,
+            ctypes.POINTER(_PTR),
+            ctypes.POINTER(_PTR),
+            ctypes.POINTER(_I64),
+            _PTR,
+            _I64,
+            _PTR,
+        ],
+    ),
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
     "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
@@ -112,6 +132,12 @@ _SIGNATURES = {
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 _INTERPOLATION = {"linear": 0, "smooth_step": 1}
+
+# Which inserts take the streaming (partition + build in LDS) path of the
+# library instead of the per-key kernel: "auto" = when the library says the
+# batch is large enough relative to the table, "always" = whenever the path
+# applies, "never".
+BULK_INSERT = os.environ.get("ASH_BULK_INSERT", "auto")
 _DTYPE = {torch.float32: 0, torch.float64: 1}
 
 
@@ -535,16 +561,41 @@ class _HashMap:
             )
         return grid_indices, cell_indices, offsets, masks
 
+    def _bulk_workspace(self, n: int, k: int, c_rows) -> Optional[torch.Tensor]:
+        """Workspace for the streaming insert path, or None when this batch goes
+        through the per-key kernel."""
+        if BULK_INSERT == "never":
+            return None
+        nbytes, worthwhile = _I64(0), ctypes.c_int(0)
+        self._check(
+            self._lib.ash_map_bulk_workspace_bytes(
+                self._handle, n, k, c_rows, ctypes.byref(nbytes), ctypes.byref(worthwhile)
+            )
+        )
+        if nbytes.value == 0 or not (worthwhile.value or BULK_INSERT == "always"):
+            return None
+        return torch.empty(nbytes.value, dtype=torch.uint8, device=self._device)
+
     def insert_keys(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)
-        self._make_room(keys.shape[0])
+        n = keys.shape[0]
+        self._make_room(n)
+        workspace = self._bulk_workspace(n, 0, None)
         for _ in range(2):
             with torch.cuda.device(self._device):
-                self._check(
-                    self._lib.ash_map_insert_keys(
-                        self._handle, keys.data_ptr(), keys.shape[0], self._stream()
+                if workspace is not None:
+                    self._check(
+                        self._lib.ash_map_insert_bulk(
+                            self._handle, keys.data_ptr(), n, 0, None, None, None,
+                            workspace.data_ptr(), workspace.numel(), self._stream(),
+                        )
                     )
-                )
+                else:
+                    self._check(
+                        self._lib.ash_map_insert_keys(
+                            self._handle, keys.data_ptr(), n, self._stream()
+                        )
+                    )
             if not self._attach_general_if_needed():
                 break
 
@@ -586,21 +637,30 @@ class _HashMap:
         if self._lib.ash_map_insert_needs_scratch(k, c_rows):
             assigned = torch.empty(n, dtype=torch.int32, device=self._device)
         self._make_room(n)
+        workspace = None if assigned is not None else self._bulk_workspace(n, k, c_rows)
         for _ in range(2):
             with torch.cuda.device(self._device):
-                self._check(
-                    self._lib.ash_map_insert(
-                        self._handle,
-                        keys.data_ptr(),
-                        n,
-                        k,
-                        c_src,
-                        c_dst,
-                        c_rows,
-                        assigned.data_ptr() if assigned is not None else None,
-                        self._stream(),
+                if workspace is not None:
+                    self._check(
+                        self._lib.ash_map_insert_bulk(
+                            self._handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows,
+                            workspace.data_ptr(), workspace.numel(), self._stream(),
+                        )
                     )
-                )
+                else:
+                    self._check(
+                        self._lib.ash_map_insert(
+                            self._handle,
+                            keys.data_ptr(),
+                            n,
+                            k,
+                            c_src,
+                            c_dst,
+                            c_rows,
+                            assigned.data_ptr() if assigned is not None else None,
+                            self._stream(),
+                        )
+                    )
             if not self._attach_general_if_needed():
                 break
 

@@ -20,7 +20,7 @@
 // (ash/src/hashmap_gpu.cuh:211-232,316-336): a new key takes heap[counter++],
 // an erased key stores its index at heap[--counter]; here the counter is
 // advanced once per 256-thread block instead of once per key.
-#include "ash_dev.h"
+#include "ash_table.h"
 
 #include "../../include/ash_hip.h"
 
@@ -41,77 +41,7 @@ constexpr int kBlock = 256;
 // make every wavefront wait for the slowest probe of the group; measured on
 // 16 M keys: 256 -> 1.28 ms, 512 -> 1.46 ms, 1024 -> 1.42 ms.
 constexpr int kHeapBlock = ASH_HEAP_BLOCK;
-constexpr int kMaxFusedValues = 4;
-constexpr int kMaxFusedRowDwords = 16;
 constexpr uint32_t kSpinLimit = 1u << 22;
-
-// ------------------------------------------------------------ key codec
-template <int DIM>
-__device__ __forceinline__ bool pack_key(const int32_t (&k)[DIM],
-                                         uint64_t& code) {
-    if constexpr (DIM == 1) {
-        code = static_cast<uint32_t>(k[0]);
-        return true;
-    } else if constexpr (DIM == 2) {
-        const uint32_t u0 = static_cast<uint32_t>(k[0]) ^ 0x80000000u;
-        const uint32_t u1 = static_cast<uint32_t>(k[1]) ^ 0x80000000u;
-        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 32);
-        return code < kTomb;
-    } else if constexpr (DIM == 3) {
-        const uint32_t u0 = static_cast<uint32_t>(k[0]) + (1u << 20);
-        const uint32_t u1 = static_cast<uint32_t>(k[1]) + (1u << 20);
-        const uint32_t u2 = static_cast<uint32_t>(k[2]) + (1u << 20);
-        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 21) |
-               (static_cast<uint64_t>(u2) << 42);
-        return (u0 | u1 | u2) < (1u << 21);
-    } else {
-        const uint32_t u0 = static_cast<uint32_t>(k[0]) + 32768u;
-        const uint32_t u1 = static_cast<uint32_t>(k[1]) + 32768u;
-        const uint32_t u2 = static_cast<uint32_t>(k[2]) + 32768u;
-        const uint32_t u3 = static_cast<uint32_t>(k[3]) + 32768u;
-        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 16) |
-               (static_cast<uint64_t>(u2) << 32) |
-               (static_cast<uint64_t>(u3) << 48);
-        return (u0 | u1 | u2 | u3) < 65536u && code < kTomb;
-    }
-}
-
-template <int DIM>
-__device__ __forceinline__ void unpack_key(uint64_t code, int32_t (&k)[DIM]) {
-    if constexpr (DIM == 1) {
-        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code));
-    } else if constexpr (DIM == 2) {
-        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code) ^ 0x80000000u);
-        k[1] = static_cast<int32_t>(static_cast<uint32_t>(code >> 32) ^
-                                    0x80000000u);
-    } else if constexpr (DIM == 3) {
-        k[0] = static_cast<int32_t>(code & 0x1FFFFFu) - (1 << 20);
-        k[1] = static_cast<int32_t>((code >> 21) & 0x1FFFFFu) - (1 << 20);
-        k[2] = static_cast<int32_t>((code >> 42) & 0x1FFFFFu) - (1 << 20);
-    } else {
-        k[0] = static_cast<int32_t>(code & 0xFFFFu) - 32768;
-        k[1] = static_cast<int32_t>((code >> 16) & 0xFFFFu) - 32768;
-        k[2] = static_cast<int32_t>((code >> 32) & 0xFFFFu) - 32768;
-        k[3] = static_cast<int32_t>((code >> 48) & 0xFFFFu) - 32768;
-    }
-}
-
-__device__ __forceinline__ uint64_t mix64(uint64_t h) {
-    h ^= h >> 33;
-    h *= 0xff51afd7ed558ccdull;
-    h ^= h >> 33;
-    h *= 0xc4ceb9fe1a85ec53ull;
-    h ^= h >> 33;
-    return h;
-}
-
-__device__ __forceinline__ uint32_t bucket_of(uint64_t code, uint32_t nb) {
-    return __umulhi(static_cast<uint32_t>(mix64(code) >> 32), nb);
-}
-
-__device__ __forceinline__ uint32_t next_bucket(uint32_t b, uint32_t nb) {
-    return (b + 1 == nb) ? 0u : b + 1;
-}
 
 __device__ __forceinline__ uint32_t spread8(uint32_t x) {
     x = (x | (x << 4)) & 0x0F0Fu;
@@ -322,14 +252,6 @@ __device__ int gen_claim(const MapDev& m, const int32_t (&k)[DIM],
 
 // ------------------------------------------------------------- kernels
 template <int DIM>
-__device__ __forceinline__ void load_key(const int32_t* __restrict__ keys,
-                                         int64_t i, bool active,
-                                         int32_t (&k)[DIM]) {
-#pragma unroll
-    for (int d = 0; d < DIM; ++d) k[d] = active ? keys[i * DIM + d] : 0;
-}
-
-template <int DIM>
 __global__ __launch_bounds__(kBlock) void find_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n,
         int64_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out) {
@@ -444,13 +366,6 @@ __global__ __launch_bounds__(kBlock) void grid_query_kernel(
     }
 }
 
-struct ValueArgs {
-    int n;
-    const uint32_t* src[kMaxFusedValues];
-    uint32_t* dst[kMaxFusedValues];
-    int32_t row_dwords[kMaxFusedValues];
-};
-
 enum InsertMode {
     kInsertKeys = 0,    // allocate indices only
     kInsertFused = 1,   // + copy narrow value rows in the same kernel
@@ -458,18 +373,25 @@ enum InsertMode {
     kInsertLoad = 3     // indices are given (state-dict load), heap untouched
 };
 
-template <int DIM, int MODE>
-__global__ __launch_bounds__(kHeapBlock) void insert_kernel(
-        MapDev m, const int32_t* __restrict__ keys, int64_t n, ValueArgs va,
-        int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kHeapBlock + threadIdx.x;
+// One key per thread, every thread of the workgroup calls this together.
+// CODES: `keys` holds packed 64-bit codes instead of int32[DIM] rows.
+template <int DIM, int MODE, bool CODES>
+__device__ __forceinline__ void insert_one(
+        const MapDev& m, const int32_t* __restrict__ keys, int64_t i,
+        bool active, const ValueArgs& va, int32_t* __restrict__ assigned,
+        const int64_t* __restrict__ given) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const bool active = i < n;
-    int32_t k[DIM];
-    load_key<DIM>(keys, i, active, k);
+    int32_t k[DIM] = {};
     uint64_t code;
-    const bool fits = pack_key<DIM>(k, code);
+    bool fits;
+    if constexpr (CODES) {
+        code = active ? reinterpret_cast<const uint64_t*>(keys)[i] : 0ull;
+        fits = true;
+    } else {
+        load_key<DIM>(keys, i, active, k);
+        fits = pack_key<DIM>(k, code);
+    }
     bool pend = active && fits;
     uint32_t b = bucket_of(code, m.nb);
     uint32_t steps = 0;
@@ -605,6 +527,33 @@ __global__ __launch_bounds__(kHeapBlock) void insert_kernel(
     }
     if constexpr (MODE == kInsertAssign) {
         if (active) assigned[i] = idx;
+    }
+}
+
+template <int DIM, int MODE>
+__global__ __launch_bounds__(kHeapBlock) void insert_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n, ValueArgs va,
+        int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kHeapBlock + threadIdx.x;
+    insert_one<DIM, MODE, false>(m, keys, i, i < n, va, assigned, given);
+}
+
+// The same insert over a selection made on the device: thread t of the
+// selection handles row sel[t], t < *nsel.  The grid is fixed; workgroups
+// stride over the selection, which is empty in the common case.
+template <int DIM, int MODE, bool CODES>
+__global__ __launch_bounds__(kHeapBlock) void insert_selected_kernel(
+        MapDev m, const int32_t* __restrict__ keys,
+        const int32_t* __restrict__ sel, const int32_t* __restrict__ nsel,
+        ValueArgs va) {
+    const int64_t total = *nsel;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kHeapBlock;
+         base < total; base += static_cast<int64_t>(gridDim.x) * kHeapBlock) {
+        const int64_t t = base + threadIdx.x;
+        const bool active = t < total;
+        const int64_t i = active ? sel[t] : 0;
+        insert_one<DIM, MODE, CODES>(m, keys, i, active, va, nullptr, nullptr);
+        __syncthreads();
     }
 }
 
@@ -841,23 +790,6 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(
 }
 
 // ---------------------------------------------------------------- host
-struct DeviceGuard {
-    int prev = -1;
-    bool switched = false;
-    hipError_t enter(int device) {
-        hipError_t e = hipGetDevice(&prev);
-        if (e != hipSuccess) return e;
-        if (prev != device) {
-            e = hipSetDevice(device);
-            switched = (e == hipSuccess);
-        }
-        return e;
-    }
-    ~DeviceGuard() {
-        if (switched) (void)hipSetDevice(prev);
-    }
-};
-
 inline unsigned grid_for(int64_t n, int per_block = kBlock) {
     return static_cast<unsigned>((n + per_block - 1) / per_block);
 }
@@ -920,6 +852,40 @@ int launch_insert(ash_map* map, const int32_t* keys, int64_t n,
     return 0;
 }
 
+template <int MODE>
+int launch_selected(ash_map* map, bool codes, const int32_t* keys,
+                    const int32_t* sel, const int32_t* nsel,
+                    const ValueArgs& va, hipStream_t s) {
+    constexpr unsigned g = 512;
+    if (codes) {
+        insert_selected_kernel<1, MODE, true>
+                <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
+    } else {
+        switch (map->key_dim) {
+            case 1:
+                insert_selected_kernel<1, MODE, false>
+                        <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
+                break;
+            case 2:
+                insert_selected_kernel<2, MODE, false>
+                        <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
+                break;
+            case 3:
+                insert_selected_kernel<3, MODE, false>
+                        <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
+                break;
+            default:
+                insert_selected_kernel<4, MODE, false>
+                        <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
+                break;
+        }
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+
 int check_batch(const ash_map* map, const void* keys, int64_t n) {
     if (check_map(map)) return 1;
     if (n < 0) ASH_FAIL("negative key count");
@@ -928,7 +894,16 @@ int check_batch(const ash_map* map, const void* keys, int64_t n) {
     return 0;
 }
 
-}  // namespace
+int insert_selected(ash_map* map, bool codes, const void* keys,
+                    const int32_t* sel, const int32_t* nsel,
+                    const ValueArgs& va, hipStream_t s) {
+    const int32_t* k = static_cast<const int32_t*>(keys);
+    if (va.n > 0) {
+        return launch_selected<kInsertFused>(map, codes, k, sel, nsel, va, s);
+    }
+    return launch_selected<kInsertKeys>(map, codes, k, sel, nsel, va, s);
+}
+
 }  // namespace ash
 
 using namespace ash;

@@ -1,0 +1,127 @@
+// Device-side helpers shared by the table kernels of libash_hip.so: key codec,
+// hash, bucket addressing, the value-row descriptor of a fused insert.
+#pragma once
+
+#include "ash_dev.h"
+
+namespace ash {
+
+constexpr int kMaxFusedValues = 4;
+constexpr int kMaxFusedRowDwords = 16;
+
+// ------------------------------------------------------------ key codec
+template <int DIM>
+__device__ __forceinline__ bool pack_key(const int32_t (&k)[DIM],
+                                         uint64_t& code) {
+    if constexpr (DIM == 1) {
+        code = static_cast<uint32_t>(k[0]);
+        return true;
+    } else if constexpr (DIM == 2) {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) ^ 0x80000000u;
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) ^ 0x80000000u;
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 32);
+        return code < kTomb;
+    } else if constexpr (DIM == 3) {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) + (1u << 20);
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) + (1u << 20);
+        const uint32_t u2 = static_cast<uint32_t>(k[2]) + (1u << 20);
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 21) |
+               (static_cast<uint64_t>(u2) << 42);
+        return (u0 | u1 | u2) < (1u << 21);
+    } else {
+        const uint32_t u0 = static_cast<uint32_t>(k[0]) + 32768u;
+        const uint32_t u1 = static_cast<uint32_t>(k[1]) + 32768u;
+        const uint32_t u2 = static_cast<uint32_t>(k[2]) + 32768u;
+        const uint32_t u3 = static_cast<uint32_t>(k[3]) + 32768u;
+        code = static_cast<uint64_t>(u0) | (static_cast<uint64_t>(u1) << 16) |
+               (static_cast<uint64_t>(u2) << 32) |
+               (static_cast<uint64_t>(u3) << 48);
+        return (u0 | u1 | u2 | u3) < 65536u && code < kTomb;
+    }
+}
+
+template <int DIM>
+__device__ __forceinline__ void unpack_key(uint64_t code, int32_t (&k)[DIM]) {
+    if constexpr (DIM == 1) {
+        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code));
+    } else if constexpr (DIM == 2) {
+        k[0] = static_cast<int32_t>(static_cast<uint32_t>(code) ^ 0x80000000u);
+        k[1] = static_cast<int32_t>(static_cast<uint32_t>(code >> 32) ^
+                                    0x80000000u);
+    } else if constexpr (DIM == 3) {
+        k[0] = static_cast<int32_t>(code & 0x1FFFFFu) - (1 << 20);
+        k[1] = static_cast<int32_t>((code >> 21) & 0x1FFFFFu) - (1 << 20);
+        k[2] = static_cast<int32_t>((code >> 42) & 0x1FFFFFu) - (1 << 20);
+    } else {
+        k[0] = static_cast<int32_t>(code & 0xFFFFu) - 32768;
+        k[1] = static_cast<int32_t>((code >> 16) & 0xFFFFu) - 32768;
+        k[2] = static_cast<int32_t>((code >> 32) & 0xFFFFu) - 32768;
+        k[3] = static_cast<int32_t>((code >> 48) & 0xFFFFu) - 32768;
+    }
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t h) {
+    h ^= h >> 33;
+    h *= 0xff51afd7ed558ccdull;
+    h ^= h >> 33;
+    h *= 0xc4ceb9fe1a85ec53ull;
+    h ^= h >> 33;
+    return h;
+}
+
+__device__ __forceinline__ uint32_t bucket_of(uint64_t code, uint32_t nb) {
+    return __umulhi(static_cast<uint32_t>(mix64(code) >> 32), nb);
+}
+
+__device__ __forceinline__ uint32_t next_bucket(uint32_t b, uint32_t nb) {
+    return (b + 1 == nb) ? 0u : b + 1;
+}
+
+template <int DIM>
+__device__ __forceinline__ void load_key(const int32_t* __restrict__ keys,
+                                         int64_t i, bool active,
+                                         int32_t (&k)[DIM]) {
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) k[d] = active ? keys[i * DIM + d] : 0;
+}
+
+// Value rows copied by a fused insert: row i of src[v] goes to row `index` of
+// dst[v]; rows are row_dwords[v] 32-bit words long.
+struct ValueArgs {
+    int n;
+    const uint32_t* src[kMaxFusedValues];
+    uint32_t* dst[kMaxFusedValues];
+    int32_t row_dwords[kMaxFusedValues];
+};
+
+// ---------------------------------------------------------------- host
+struct DeviceGuard {
+    int prev = -1;
+    bool switched = false;
+    hipError_t enter(int device) {
+        hipError_t e = hipGetDevice(&prev);
+        if (e != hipSuccess) return e;
+        if (prev != device) {
+            e = hipSetDevice(device);
+            switched = (e == hipSuccess);
+        }
+        return e;
+    }
+    ~DeviceGuard() {
+        if (switched) (void)hipSetDevice(prev);
+    }
+};
+
+
+// Inserts the keys selected by `sel[0 .. *nsel)` (both on the device) with the
+// per-key atomic kernel.  `codes` false: `keys` are int32[.., key_dim] rows and
+// sel holds row numbers; true: `keys` are packed 64-bit codes.  The value rows
+// of va.src are addressed by the same selected row number.  Defined in
+// ash_map.hip.
+int insert_selected(ash_map* map, bool codes, const void* keys,
+                    const int32_t* sel, const int32_t* nsel,
+                    const ValueArgs& va, hipStream_t s);
+
+int check_batch(const ash_map* map, const void* keys, int64_t n);
+
+}  // namespace ash
