@@ -49,6 +49,9 @@ MEASURED_TRAFFIC_BYTES = {
     "insert_keys": 2_303_000_000 + 1_564_000_000,
     "find": 2_230_000_000 + 146_000_000,
     "items": 512_000_000 + 324_000_000,
+    # sums over split_keys_kernel, split_records_kernel and build_kernel
+    "insert_values_bulk": 1_285_000_000 + 1_592_000_000,
+    "insert_keys_bulk": 515_000_000 + 786_000_000,
 }
 
 
@@ -199,10 +202,29 @@ def bench_hash(torch, ash, workloads, args, dev):
         if rc != 0:
             raise RuntimeError(lib.ash_last_error().decode())
 
+    # The streaming insert path (what hm.insert takes for a batch of this size
+    # when the library calls it worthwhile) next to the per-key kernel.
+    ws_bytes, worthwhile = ctypes.c_int64(0), ctypes.c_int(0)
+    check(lib.ash_map_bulk_workspace_bytes(
+        handle, n, k, c_rows, ctypes.byref(ws_bytes), ctypes.byref(worthwhile)))
+    bulk = ws_bytes.value > 0
+    api_uses_bulk = bool(bulk and worthwhile.value and ash.common.BULK_INSERT != "never")
+    workspace = torch.empty(max(ws_bytes.value, 256), dtype=torch.uint8, device=dev)
+    t_bulk, t_bulk_keys = EventTimer(torch), EventTimer(torch)
+
     t_clear, t_insert, t_insert_keys, t_find, t_items = (EventTimer(torch) for _ in range(5))
     for it in range(args.warmup + args.steps):
         timed = it >= args.warmup
         run = (lambda timer, fn: timer(fn)) if timed else (lambda timer, fn: fn())
+        if bulk:
+            check(lib.ash_map_clear(handle, stream))
+            run(t_bulk_keys, lambda: check(lib.ash_map_insert_bulk(
+                handle, keys.data_ptr(), n, 0, None, None, None,
+                workspace.data_ptr(), workspace.numel(), stream)))
+            check(lib.ash_map_clear(handle, stream))
+            run(t_bulk, lambda: check(lib.ash_map_insert_bulk(
+                handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows,
+                workspace.data_ptr(), workspace.numel(), stream)))
         run(t_clear, lambda: check(lib.ash_map_clear(handle, stream)))
         run(t_insert_keys, lambda: check(lib.ash_map_insert_keys(handle, keys.data_ptr(), n, stream)))
         check(lib.ash_map_clear(handle, stream))
@@ -222,13 +244,25 @@ def bench_hash(torch, ash, workloads, args, dev):
         "items": roofline_entry("items_kernel<3>", items_bytes(slots, n), t_items.mean_ms()),
         "clear": roofline_entry("fill16+reset_heap", 16 * slots + 4 * args.capacity, t_clear.mean_ms()),
     }
+    if bulk:
+        chain = "split_keys_kernel<3> + split_records_kernel + build_kernel"
+        kernels["insert_values_bulk"] = roofline_entry(
+            chain + " (ash_map_insert_bulk, fused values)",
+            (INSERT_KEY_BYTES + VALUE_ROW_BYTES) * n, t_bulk.mean_ms())
+        kernels["insert_keys_bulk"] = roofline_entry(
+            chain + " (ash_map_insert_bulk, keys)", INSERT_KEY_BYTES * n, t_bulk_keys.mean_ms())
+        for name in ("insert_values_bulk", "insert_keys_bulk"):
+            kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
+            kernels[name]["workspace_bytes"] = ws_bytes.value
+    kernels["api_insert_path"] = "insert_values_bulk" if api_uses_bulk else "insert_values"
     for name in ("insert_values", "insert_keys", "find"):
         kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
     if n == 16_000_000 and args.capacity == 24_000_000:
         for name, traffic in MEASURED_TRAFFIC_BYTES.items():
-            kernels[name]["traffic"] = traffic
-    del hm, w
+            if name in kernels:
+                kernels[name]["traffic"] = traffic
+    del hm, w, workspace
     torch.cuda.empty_cache()
     return ms_per_step, hits, kernels
 
@@ -391,7 +425,7 @@ def main():
     ms_per_step, hits, kernels = bench_hash(torch, ash, workloads, args, dev)
     if not args.no_trilinear:
         kernels.update(bench_trilinear(torch, ash, workloads, args, dev))
-    dominant = max(("insert_values", "find", "items"), key=lambda k: kernels[k]["ms"])
+    dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
     table_bytes = (args.capacity + 5) // 6 * 128
     ceilings = measure_ceilings(torch, ash, dev, table_bytes, 16 << 20)

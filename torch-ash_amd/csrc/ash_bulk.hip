@@ -31,6 +31,8 @@ namespace {
 
 constexpr int kPartShift = 9;
 constexpr int kPartBuckets = 1 << kPartShift;   // buckets per build workgroup
+// Chunk geometry measured on 16 M keys with two value planes (ms per insert):
+// 1024x4 1.03, 1024x2 1.06, 512x4 1.13, 512x8 1.17, 256x8 1.29.
 constexpr int kSplitThreads = 1024;
 constexpr int kSplitKeys = 4;                   // records per thread
 constexpr int kStageDwords = 4;                 // widest row slice staged in LDS
