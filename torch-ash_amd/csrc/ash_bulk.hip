@@ -219,6 +219,25 @@ __device__ __forceinline__ void move_chunk(
         uint64_t* __restrict__ codes_dst, uint32_t cap, DstFirst dst_first,
         Spill spill) {
     const int tid = threadIdx.x;
+    uint32_t regs[kSplitKeys][kStageDwords];
+    auto load_slice = [&](int v, int q0) {
+        const int rd = row_dwords[v];
+        const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
+#pragma unroll
+        for (int k = 0; k < kSplitKeys; ++k) {
+            if (bin[k] >= 0) {
+                const uint32_t* s =
+                        src[v] + (row0 + k * kSplitThreads + tid) * rd + q0;
+#pragma unroll
+                for (int q = 0; q < kStageDwords; ++q) {
+                    if (q < w) regs[k][q] = s[q];
+                }
+            }
+        }
+    };
+    int v = 0, q0 = 0;
+    bool have = n_values > 0;
+    if (have) load_slice(0, 0);
     int sp[kSplitKeys];
 #pragma unroll
     for (int k = 0; k < kSplitKeys; ++k) {
@@ -248,29 +267,40 @@ __device__ __forceinline__ void move_chunk(
             }
         }
     }
-    for (int v = 0; v < n_values; ++v) {
+    // Value rows, one slice of up to kStageDwords words at a time.  The rows of
+    // the next slice are requested while the current one is written out.
+    while (have) {
         const int rd = row_dwords[v];
-        for (int q0 = 0; q0 < rd; q0 += kStageDwords) {
-            const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
-            __syncthreads();
+        const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
+        __syncthreads();
 #pragma unroll
-            for (int k = 0; k < kSplitKeys; ++k) {
-                if (sp[k] >= 0) {
-                    const uint32_t* s = src[v] +
-                            (row0 + k * kSplitThreads + tid) * rd + q0;
-                    for (int q = 0; q < w; ++q) sh.stage[sp[k] * w + q] = s[q];
-                }
-            }
-            __syncthreads();
+        for (int k = 0; k < kSplitKeys; ++k) {
+            if (sp[k] >= 0) {
 #pragma unroll
-            for (int j = 0; j < kSplitKeys; ++j) {
-                if (d[j] >= 0) {
-                    const int s = j * kSplitThreads + tid;
-                    uint32_t* o = dst[v] + d[j] * rd + q0;
-                    for (int q = 0; q < w; ++q) o[q] = sh.stage[s * w + q];
+                for (int q = 0; q < kStageDwords; ++q) {
+                    if (q < w) sh.stage[sp[k] * w + q] = regs[k][q];
                 }
             }
         }
+        int nv = v, nq0 = q0 + kStageDwords;
+        if (nq0 >= rd) {
+            ++nv;
+            nq0 = 0;
+        }
+        const bool nhave = nv < n_values;
+        if (nhave) load_slice(nv, nq0);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kSplitKeys; ++j) {
+            if (d[j] >= 0) {
+                const int s = j * kSplitThreads + tid;
+                uint32_t* o = dst[v] + d[j] * rd + q0;
+                for (int q = 0; q < w; ++q) o[q] = sh.stage[s * w + q];
+            }
+        }
+        v = nv;
+        q0 = nq0;
+        have = nhave;
     }
 }
 
@@ -481,6 +511,26 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
             wrank[k] = __popcll(wm & ((1ull << lane) - 1ull));
             if (lane == 0) s_wcnt[k * (kBuildThreads / 64) + wave] = __popcll(wm);
         }
+        // The first slice of the winners' value rows does not depend on the
+        // indices: it is requested now and travels while the heap counter and
+        // the heap entries are fetched.
+        uint32_t rows[kBuildRecs][kStageDwords];
+        auto load_rows = [&](int v, int q0) {
+            const int rd = va.row_dwords[v];
+            const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
+#pragma unroll
+            for (int k = 0; k < kBuildRecs; ++k) {
+                if (wslot[k] >= 0) {
+                    const uint32_t* s = pl.plane_b[v] +
+                            (bbase + rb + k * kBuildThreads + tid) * rd + q0;
+#pragma unroll
+                    for (int q = 0; q < kStageDwords; ++q) {
+                        if (q < w) rows[k][q] = s[q];
+                    }
+                }
+            }
+        };
+        if (va.n > 0) load_rows(0, 0);
         __syncthreads();
         if (tid == 0) {
             int tot = 0;
@@ -502,28 +552,46 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
             s_base = base;
         }
         __syncthreads();
+        int32_t idx[kBuildRecs];
 #pragma unroll
         for (int k = 0; k < kBuildRecs; ++k) {
+            idx[k] = -1;
             if (wslot[k] < 0) continue;
-            const int r = rb + k * kBuildThreads + tid;
             const int top = s_base + s_wcnt[k * (kBuildThreads / 64) + wave] + wrank[k];
-            const int wlb = wslot[k] >> 4;
-            const int ws = wslot[k] & 15;
             if (top < m.capacity) {
-                const int32_t idx = m.heap[top];
-                tab32[staged(wlb, (kValDword0 + ws) >> 2) * 4 + (ws & 3)] = idx;
-#pragma unroll
-                for (int v = 0; v < kMaxFusedValues; ++v) {
-                    if (v < va.n) {
-                        const int rd = va.row_dwords[v];
-                        copy_row(pl.plane_b[v] + (bbase + r) * rd,
-                                 va.dst[v] + static_cast<int64_t>(idx) * rd, rd);
-                    }
-                }
+                idx[k] = m.heap[top];
             } else {
                 // Heap exhausted: give the slot up again.
+                const int wlb = wslot[k] >> 4;
+                const int ws = wslot[k] & 15;
                 tab64[staged(wlb, ws >> 1) * 2 + (ws & 1)] = kTomb;
                 atomicAdd(m.ctr + kCtrTombs, 1);
+                wslot[k] = -1;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kBuildRecs; ++k) {
+            if (idx[k] >= 0) {
+                const int wlb = wslot[k] >> 4;
+                const int ws = wslot[k] & 15;
+                tab32[staged(wlb, (kValDword0 + ws) >> 2) * 4 + (ws & 3)] = idx[k];
+            }
+        }
+        for (int v = 0; v < va.n; ++v) {
+            const int rd = va.row_dwords[v];
+            for (int q0 = 0; q0 < rd; q0 += kStageDwords) {
+                const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
+                if (v > 0 || q0 > 0) load_rows(v, q0);
+#pragma unroll
+                for (int k = 0; k < kBuildRecs; ++k) {
+                    if (idx[k] >= 0) {
+                        uint32_t* o = va.dst[v] + static_cast<int64_t>(idx[k]) * rd + q0;
+#pragma unroll
+                        for (int q = 0; q < kStageDwords; ++q) {
+                            if (q < w) o[q] = rows[k][q];
+                        }
+                    }
+                }
             }
         }
         __syncthreads();
