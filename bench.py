@@ -1,6 +1,6 @@
 """Benchmark of the two hot paths on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-trilinear] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-trilinear] [--no-fusion] [--no-cpu]
 
 Headline (`value`): configuration 2 of the baseline -- HashMap with values
 {color: fp32[3], depth: fp32[1]}, 16 M distinct voxel keys into capacity 24 M,
@@ -10,11 +10,16 @@ host read-backs), inputs resident in HBM; `value` counts the 32 M keys that
 were inserted or looked up per step.
 
 Beside it, on the same JSON line:
-  roofline      the step's longest kernel, timed alone with HIP events on the
-                stream it runs on (raw C-ABI call, no host read-back inside),
-                priced with the algorithmic bytes per key of that operation;
-  kernels       the same figures for every hash kernel and for the trilinear
-                query kernels of configurations 3 and 4;
+  roofline      the step's longest operation (for an insert of this size the
+                three kernels of the streaming path together), timed alone with
+                HIP events on the stream it runs on (raw C-ABI call, no host
+                read-back inside), priced with the algorithmic bytes per key of
+                that operation;
+  kernels       the same figures for every hash kernel, for the trilinear query
+                kernels of configurations 3 and 4, and the frame rate of the
+                fusion loop of configuration 5;
+  ceilings      what the device delivers for random line reads / updates and
+                for a plain copy, measured in the same run;
   cpu_baseline  the CPU oracle (OpenMP) on a bounded sample of the same
                 workload, on this machine's host cores.
 """
@@ -79,6 +84,7 @@ def parse_args():
     ap.add_argument("--keys", type=int, default=16_000_000, help="distinct keys (configuration 2)")
     ap.add_argument("--capacity", type=int, default=24_000_000)
     ap.add_argument("--no-trilinear", action="store_true", help="skip the trilinear kernel figures")
+    ap.add_argument("--no-fusion", action="store_true", help="skip the configuration 5 figure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-keys", type=int, default=4_000_000, help="CPU baseline sample size")
     ap.add_argument("--calibrate", action="store_true",
@@ -357,6 +363,45 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     return out
 
 
+def bench_fusion(torch, ash, workloads, args, dev, frames=20):
+    """Configuration 5 (secondary figure): depth frames of the synthetic scene
+    fused into an unbounded grid, once with the library's fused activation and
+    integration kernels and once in the reference's formulation (candidate
+    expansion + scratch set, torch expressions around
+    embeddings[grid_indices, cell_indices])."""
+    scene = workloads.FusionScene()
+    intrinsic = scene.intrinsic.to(dev)
+    data = []
+    for f in range(frames):
+        ext = scene.pose(f * (100 // frames))
+        depth = scene.depth(ext)
+        data.append((scene.unproject(depth, ext).to(dev), depth.to(dev), ext.to(dev)))
+    points = sum(d[0].shape[0] for d in data) / frames
+    out = {"frames": frames, "points_per_frame": round(points),
+           "candidate_keys_per_frame": round(points * 27)}
+    for name, fused in (("reference_formulation", False), ("fused", True)):
+        for rep in range(2):  # the first pass warms allocations up
+            grid = ash.UnBoundedSparseDenseGrid(3, 80000, 2, 8, cell_size=0.015, device=dev)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            touched = 0
+            for pts, depth, ext in data:
+                touched += workloads.fuse_frame(grid, pts, depth, intrinsic, ext, trunc=0.04,
+                                                fused=fused)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        out[name] = {
+            "frames_per_s": round(frames / dt, 1),
+            "ms_per_frame": round(dt / frames * 1e3, 3),
+            "Mkeys_per_s": round(points * 27 * frames / dt / 1e6, 1),
+            "active_blocks": grid.engine.size(),
+            "touched_blocks_per_frame": round(touched / frames),
+        }
+        del grid
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(torch, workloads, args):
     """The oracle (OpenMP) on a bounded sample of configuration 2: same
     generator, `--cpu-keys` distinct keys, capacity 1.5x, insert + find + items."""
@@ -425,6 +470,8 @@ def main():
     ms_per_step, hits, kernels = bench_hash(torch, ash, workloads, args, dev)
     if not args.no_trilinear:
         kernels.update(bench_trilinear(torch, ash, workloads, args, dev))
+    if not args.no_fusion:
+        kernels["cfg5_fusion"] = bench_fusion(torch, ash, workloads, args, dev)
     dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
     table_bytes = (args.capacity + 5) // 6 * 128

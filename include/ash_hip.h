@@ -92,6 +92,51 @@ int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
                    int64_t* grid_indices, int64_t* cell_indices, float* offsets,
                    uint8_t* masks, void* stream);
 
+/* Stands for the body of `SparseDenseGrid.spatial_init_` (ash/grid.py:133-152):
+ * for every position `cells[i]` (fp32, cell units) the block
+ * floor(cells[i] / grid_dim) and its neighbours within `dilation` blocks
+ * (offsets -dilation..dilation per axis if `bidirectional`, else 0..dilation)
+ * are inserted as int3 keys.  Blocks with a coordinate outside
+ * [bound_lo, bound_hi] are skipped, and so are all candidates of a position
+ * whose own block is outside (the reference's grids_in_bound, applied before
+ * and after the expansion).  The reference de-duplicates the (2r+1)^3 N
+ * candidate rows through a scratch HashSet; here the candidates are generated
+ * in registers and the table absorbs the duplicates.
+ * Afterwards every touched block (new or already stored) has touched[index] = 1
+ * and its coordinates at coords[3*index..]; both are caller-owned arrays of
+ * `capacity` rows, `touched` zero on entry for the caller to tell this batch's
+ * blocks.  heads_scratch: device temporary of 64 + 3 n int32 (one block per run
+ * of consecutive positions in the same block).  Keys refused for lack of
+ * capacity are counted as by insert_keys. */
+int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
+                      int grid_dim, int dilation, int bidirectional,
+                      int bound_lo, int bound_hi, uint8_t* touched,
+                      int32_t* coords, int32_t* heads_scratch, void* stream);
+
+/* Stands for `project_points_to_rgbd` plus the fusion arithmetic of
+ * `fuse_frame` in the reference's TSDF demo (demo/rgbd_fusion.py:76-110,
+ * 216-254), which are torch expressions around
+ * embeddings[grid_indices, cell_indices]: every cell of the `n_blocks` listed
+ * blocks is projected into the depth image (world = (block * grid_dim + cell)
+ * * cell_size [+ origin], camera = extrinsic * world, pixel = round(K * camera
+ * / z)), and its embedding row is updated in place with the running weighted
+ * mean: channel 0 = truncated signed distance, channels 1..3 = colour when
+ * `color` is given (then embedding_dim >= 5), last channel = weight.
+ * embeddings fp32 [num_embeddings, grid_dim^3, embedding_dim]; grid_indices
+ * int64[n_blocks] rows of it, grid_coords int32[n_blocks,3]; intrinsic 3x3 and
+ * extrinsic 4x4 row-major fp32 ON THE DEVICE; origin: host float[3] or NULL;
+ * depth fp32[height,width] (0 = no reading), color fp32[height,width,3] or
+ * NULL.  Runs on the current device. */
+int ash_grid_integrate_depth(float* embeddings, int64_t num_embeddings,
+                             int grid_dim, int embedding_dim,
+                             const int64_t* grid_indices,
+                             const int32_t* grid_coords, int64_t n_blocks,
+                             float cell_size, const float* origin,
+                             const float* intrinsic, const float* extrinsic,
+                             const float* depth, const float* color, int height,
+                             int width, float trunc, float depth_max,
+                             void* stream);
+
 /* Replaces `HashMap::insert_keys` (ash/src/hashmap_gpu.cuh:211-247).  New keys
  * pop one index each from the heap; duplicates (in the table or within the
  * batch) are ignored.  Keys beyond `capacity` are dropped and counted

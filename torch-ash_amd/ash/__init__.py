@@ -7,6 +7,7 @@ libash_hip.so.
 from .common import DotDict
 from .core import ASHEngine, ASHModule
 from .embedding import HashEmbedding
+from . import fusion
 from .grid import BoundedSparseDenseGrid, SparseDenseGrid, UnBoundedSparseDenseGrid
 from .grid_nns import enumerate_neighbor_coord_offsets
 from .grid_query import SparseDenseGridQuery, SparseDenseGridQueryBackward
@@ -25,4 +26,5 @@ __all__ = [
     "SparseDenseGridQueryBackward",
     "UnBoundedSparseDenseGrid",
     "enumerate_neighbor_coord_offsets",
+    "fusion",
 ]

@@ -69,6 +69,17 @@ _SIGNATURES = {
         ctypes.c_int,
         [_PTR, _PTR, _I64, ctypes.c_int, _PTR, _PTR, _PTR, _PTR, _PTR],
     ),
+    "ash_grid_activate": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         _PTR, _PTR, _PTR, _PTR],
+    ),
+    "ash_grid_integrate_depth": (
+        ctypes.c_int,
+        [_PTR, _I64, ctypes.c_int, ctypes.c_int, _PTR, _PTR, _I64, ctypes.c_float,
+         ctypes.POINTER(ctypes.c_float), _PTR, _PTR, _PTR, _PTR, ctypes.c_int, ctypes.c_int,
+         ctypes.c_float, ctypes.c_float, _PTR],
+    ),
     "ash_map_insert_keys": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_insert_needs_scratch": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_I64)]),
     "ash_map_insert": (
@@ -181,6 +192,60 @@ class _Backend:
         if status != 0:
             msg = self.lib.ash_last_error()
             raise RuntimeError(msg.decode() if msg else "libash_hip call failed")
+
+    # -- depth integration (no pybind counterpart: the reference's demo does
+    #    this with torch expressions, demo/rgbd_fusion.py:76-110,216-254) -----
+    def integrate_depth(
+        self,
+        embeddings: torch.Tensor,
+        grid_indices: torch.Tensor,
+        grid_coords: torch.Tensor,
+        grid_dim: int,
+        cell_size: float,
+        origin: Optional[torch.Tensor],
+        intrinsic: torch.Tensor,
+        extrinsic: torch.Tensor,
+        depth: torch.Tensor,
+        color: Optional[torch.Tensor],
+        trunc: float,
+        depth_max: float,
+    ) -> None:
+        """In-place TSDF update of the cells of the listed blocks."""
+        _require_hip(embeddings, "embeddings")
+        dev = embeddings.device
+        if embeddings.dtype != torch.float32 or not embeddings.is_contiguous():
+            raise RuntimeError("embeddings must be contiguous float32")
+        if embeddings.dim() != 3 or embeddings.shape[1] != grid_dim**3:
+            raise RuntimeError("embeddings must be (num_embeddings, grid_dim^3, embedding_dim)")
+        grid_indices = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
+        grid_coords = grid_coords.reshape(-1, 3).to(dev, torch.int32).contiguous()
+        if grid_coords.shape[0] != grid_indices.shape[0]:
+            raise RuntimeError("one coordinate row per block index is needed")
+        intrinsic = intrinsic.to(dev, torch.float32).contiguous()
+        extrinsic = extrinsic.to(dev, torch.float32).contiguous()
+        if intrinsic.shape != (3, 3) or extrinsic.shape != (4, 4):
+            raise RuntimeError("intrinsic must be 3x3 and extrinsic 4x4")
+        depth = depth.to(dev, torch.float32).contiguous()
+        if depth.dim() != 2:
+            raise RuntimeError("depth must be (H, W)")
+        if color is not None:
+            color = color.to(dev, torch.float32).contiguous()
+            if color.shape != (*depth.shape, 3):
+                raise RuntimeError("color must be (H, W, 3)")
+        c_origin = None
+        if origin is not None:
+            c_origin = (ctypes.c_float * 3)(*[float(v) for v in origin.reshape(-1).tolist()])
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_grid_integrate_depth(
+                    embeddings.data_ptr(), embeddings.shape[0], int(grid_dim), embeddings.shape[2],
+                    grid_indices.data_ptr(), grid_coords.data_ptr(), grid_indices.shape[0],
+                    float(cell_size), c_origin, intrinsic.data_ptr(), extrinsic.data_ptr(),
+                    depth.data_ptr(), color.data_ptr() if color is not None else None,
+                    depth.shape[0], depth.shape[1], float(trunc), float(depth_max),
+                    _stream_of(dev),
+                )
+            )
 
     # -- trilinear queries (ash/src/pybind.cpp:25-29) ---------------------
     def _query_args(
@@ -560,6 +625,49 @@ class _HashMap:
                 )
             )
         return grid_indices, cell_indices, offsets, masks
+
+    def activate_blocks(
+        self,
+        cells: torch.Tensor,
+        grid_dim: int,
+        dilation: int,
+        bidirectional: bool,
+        bound_lo: int,
+        bound_hi: int,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Fused body of `SparseDenseGrid.spatial_init_`: inserts the blocks
+        around the positions `cells` (fp32, cell units) and returns the touched
+        blocks as (grid_coords int32[n,3], grid_indices int64[n])."""
+        if self.key_dim != 3:
+            raise RuntimeError("block activation needs 3-d keys")
+        if cells.dim() != 2 or cells.shape[1] != 3 or cells.dtype != torch.float32:
+            raise RuntimeError("positions must be float32 (N, 3)")
+        if cells.device != self._device:
+            raise RuntimeError(f"positions are on {cells.device}, the map on {self._device}")
+        cells = cells.contiguous()
+        if getattr(self, "_touched", None) is None:
+            self._touched = torch.zeros(self.capacity, dtype=torch.uint8, device=self._device)
+            self._block_coords = torch.zeros(
+                (self.capacity, 3), dtype=torch.int32, device=self._device
+            )
+        self._make_room(cells.shape[0])
+        heads = torch.empty(64 + 3 * cells.shape[0], dtype=torch.int32, device=self._device)
+        for _ in range(2):
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_grid_activate(
+                        self._handle, cells.data_ptr(), cells.shape[0], int(grid_dim),
+                        int(dilation), int(bool(bidirectional)), int(bound_lo), int(bound_hi),
+                        self._touched.data_ptr(), self._block_coords.data_ptr(),
+                        heads.data_ptr(), self._stream(),
+                    )
+                )
+            if not self._attach_general_if_needed():
+                break
+        grid_indices = self._touched.nonzero().view(-1)
+        grid_coords = self._block_coords[grid_indices]
+        self._touched[grid_indices] = 0
+        return grid_coords, grid_indices
 
     def _bulk_workspace(self, n: int, k: int, c_rows) -> Optional[torch.Tensor]:
         """Workspace for the streaming insert path, or None when this batch goes

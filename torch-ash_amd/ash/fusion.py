@@ -1,0 +1,78 @@
+"""TSDF fusion of depth frames into a sparse-dense grid: the per-frame step of
+the reference's demo (demo/rgbd_fusion.py:200-254) on two fused library calls.
+
+The reference activates blocks with `spatial_init_` and then updates
+`embeddings[grid_indices, cell_indices]` through torch expressions
+(`project_points_to_rgbd`, demo/rgbd_fusion.py:76-110, and the running weighted
+mean, :232-254).  Here `spatial_init_` runs as one activation kernel pair and
+the projection + update as one kernel that rewrites the embedding rows in
+place.  Row layout as in the demo: channel 0 signed distance, channels 1..3
+colour (only when a colour image is given), last channel weight.
+"""
+from typing import Optional
+
+import torch
+
+from .common import _get_c_extension
+from .grid import SparseDenseGrid
+
+backend = _get_c_extension()
+
+
+@torch.no_grad()
+def integrate_depth(
+    grid: SparseDenseGrid,
+    grid_coords: torch.Tensor,
+    grid_indices: torch.Tensor,
+    depth: torch.Tensor,
+    intrinsic: torch.Tensor,
+    extrinsic: torch.Tensor,
+    trunc: float,
+    depth_max: float,
+    color: Optional[torch.Tensor] = None,
+) -> None:
+    """Projects every cell of the listed blocks into `depth` (H, W; metres, 0 =
+    no reading) with the pinhole `intrinsic` (3, 3) and the world-to-camera
+    `extrinsic` (4, 4) and folds the truncated signed distance (and `color`
+    (H, W, 3), if given) into the grid's embedding rows."""
+    scale, origin = grid._cell_to_world_affine()
+    backend.integrate_depth(
+        grid.embeddings.data,
+        grid_indices,
+        grid_coords,
+        grid.grid_dim,
+        scale,
+        origin,
+        intrinsic,
+        extrinsic,
+        depth,
+        color,
+        trunc,
+        depth_max,
+    )
+
+
+@torch.no_grad()
+def fuse_frame(
+    grid: SparseDenseGrid,
+    points: torch.Tensor,
+    depth: torch.Tensor,
+    intrinsic: torch.Tensor,
+    extrinsic: torch.Tensor,
+    trunc: float,
+    depth_max: float,
+    color: Optional[torch.Tensor] = None,
+    dilation: int = 1,
+) -> int:
+    """One fusion step: activate the blocks around the unprojected `points`
+    (world coordinates) with a two-sided dilation, then integrate the frame
+    into them.  Returns the number of touched blocks."""
+    grid_coords, _, grid_indices, _ = grid.spatial_init_(
+        points, dilation=dilation, bidirectional=True
+    )
+    if grid_indices.numel() == 0:
+        return 0
+    integrate_depth(
+        grid, grid_coords, grid_indices, depth, intrinsic, extrinsic, trunc, depth_max, color
+    )
+    return int(grid_indices.shape[0])

@@ -101,6 +101,27 @@ class SparseDenseGrid(ASHModule):
         cell_indices (1, M).
         """
         cells = self.transform_world_to_cell(points)
+        table = self.engine.backend
+        if (
+            hasattr(table, "activate_blocks")
+            and self.in_dim == 3
+            and cells.dtype == torch.float32
+            and len(cells) > 0
+        ):
+            # one pass over the positions instead of candidate expansion +
+            # scratch set + insert + find; same set of touched blocks
+            lo, hi = self._block_bounds()
+            dropped_before = self.engine._dropped()
+            unique_coords, grid_indices = table.activate_blocks(
+                cells, self.grid_dim, dilation, bidirectional, lo, hi
+            )
+            self.engine._warn_if_overfull(len(cells), dropped_before)
+            return (
+                unique_coords.view(-1, 1, self.in_dim),
+                self.cell_coords.view(1, -1, self.in_dim),
+                grid_indices.view(-1, 1),
+                self.cell_indices.view(1, -1),
+            )
         block_coords = self.grids_in_bound(torch.floor(cells / self.grid_dim).int())
 
         nb_offsets, _ = enumerate_neighbor_coord_offsets(
@@ -237,6 +258,16 @@ class SparseDenseGrid(ASHModule):
     def grids_in_bound(self, grid_coords: torch.Tensor) -> torch.Tensor:
         """Unbounded by default; the bounded grid filters here."""
         return grid_coords
+
+    def _block_bounds(self) -> Tuple[int, int]:
+        """Inclusive range of block coordinates `grids_in_bound` lets through
+        (all of int32 short of the dilation range when unbounded)."""
+        return -(2**31) + 64, 2**31 - 65
+
+    def _cell_to_world_affine(self) -> Tuple[float, Optional[torch.Tensor]]:
+        """`transform_cell_to_world` as (scale, origin): world = cell * scale
+        [+ origin]."""
+        return 1.0, None
 
     @torch.no_grad()
     def _linearize_cell_coords(self, cell_coords: torch.Tensor) -> torch.Tensor:
@@ -376,6 +407,7 @@ class UnBoundedSparseDenseGrid(SparseDenseGrid):
         self.cell_size = cell_size
         self.transform_world_to_cell = lambda x: x / self.cell_size
         self.transform_cell_to_world = lambda x: x * self.cell_size
+        self._cell_to_world_affine = lambda: (self.cell_size, None)
         self.bbox_min = None
         self.bbox_max = None
 
@@ -429,10 +461,14 @@ class BoundedSparseDenseGrid(SparseDenseGrid):
         self.cell_size = (extent / (sparse_grid_dim * grid_dim - 1)).min().item()
         self.transform_world_to_cell = lambda x: (x - self.bbox_min) / self.cell_size
         self.transform_cell_to_world = lambda x: x * self.cell_size + self.bbox_min
+        self._cell_to_world_affine = lambda: (self.cell_size, self.bbox_min)
 
     def grids_in_bound(self, grid_coords: torch.Tensor) -> torch.Tensor:
         inside = ((grid_coords >= 0) & (grid_coords < self.sparse_grid_dim)).all(dim=-1)
         return grid_coords[inside]
+
+    def _block_bounds(self) -> Tuple[int, int]:
+        return 0, self.sparse_grid_dim - 1
 
     def dense_init_(self):
         """Activates every block of the box."""

@@ -636,9 +636,13 @@ int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
         // MI355X (16 M-slot table): keys only, the streaming path wins from
         // about one key per bucket; with value rows, which travel through both
         // split passes, from about 1.5.
+        // A table below 2^19 buckets has too few partitions to fill the device
+        // in the build pass (a batch that large for it is mostly duplicates,
+        // which the per-key kernel handles without atomics).
         const int64_t nb = static_cast<int64_t>(map->d.nb);
-        const bool big = n_values > 0 ? (n >= (int64_t{1} << 21) && 2 * n >= 3 * nb)
-                                      : (n >= (int64_t{1} << 20) && n >= nb);
+        const bool big = nb >= (int64_t{1} << 19) &&
+                         (n_values > 0 ? (n >= (int64_t{1} << 21) && 2 * n >= 3 * nb)
+                                       : (n >= (int64_t{1} << 20) && n >= nb));
         *worthwhile = (*bytes > 0 && big) ? 1 : 0;
     }
     return 0;

@@ -251,21 +251,19 @@ __device__ int gen_claim(const MapDev& m, const int32_t (&k)[DIM],
 }
 
 // ------------------------------------------------------------- kernels
+// Looks key `k` up; every lane of the wavefront calls this together, lanes
+// with active == false only help.  Returns whether the key is stored and, if
+// so, its index in `res`.
 template <int DIM>
-__global__ __launch_bounds__(kBlock) void find_kernel(
-        MapDev m, const int32_t* __restrict__ keys, int64_t n,
-        int64_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+__device__ __forceinline__ bool find_key(const MapDev& m, const int32_t (&k)[DIM],
+                                         bool active, int32_t& res) {
     const int lane = threadIdx.x & 63;
-    const bool active = i < n;
-    int32_t k[DIM];
-    load_key<DIM>(keys, i, active, k);
     uint64_t code;
     const bool fits = pack_key<DIM>(k, code);
     bool pend = active && fits;
     uint32_t b = bucket_of(code, m.nb);
     uint32_t steps = 0;
-    int32_t res = 0;
+    res = 0;
     bool found = false;
     while (__ballot(pend)) {
         ProbeResult p;
@@ -287,6 +285,19 @@ __global__ __launch_bounds__(kBlock) void find_kernel(
         uint32_t pos;
         found = gen_find<DIM>(m, k, res, pos);
     }
+    return found;
+}
+
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void find_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n,
+        int64_t* __restrict__ idx_out, uint8_t* __restrict__ mask_out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const bool active = i < n;
+    int32_t k[DIM];
+    load_key<DIM>(keys, i, active, k);
+    int32_t res = 0;
+    const bool found = find_key<DIM>(m, k, active, res);
     if (active) {
         idx_out[i] = found ? static_cast<int64_t>(res) : 0;
         mask_out[i] = found ? 1 : 0;
@@ -373,25 +384,15 @@ enum InsertMode {
     kInsertLoad = 3     // indices are given (state-dict load), heap untouched
 };
 
-// One key per thread, every thread of the workgroup calls this together.
-// CODES: `keys` holds packed 64-bit codes instead of int32[DIM] rows.
-template <int DIM, int MODE, bool CODES>
-__device__ __forceinline__ void insert_one(
-        const MapDev& m, const int32_t* __restrict__ keys, int64_t i,
-        bool active, const ValueArgs& va, int32_t* __restrict__ assigned,
-        const int64_t* __restrict__ given) {
+// The insert proper for a key held in registers (`code` is its packed form if
+// `fits`); `i` is the row of the key's value rows / `assigned` / `given` entry.
+template <int DIM, int MODE>
+__device__ __forceinline__ void insert_key(
+        const MapDev& m, const int32_t (&k)[DIM], uint64_t code, bool fits,
+        int64_t i, bool active, const ValueArgs& va,
+        int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    int32_t k[DIM] = {};
-    uint64_t code;
-    bool fits;
-    if constexpr (CODES) {
-        code = active ? reinterpret_cast<const uint64_t*>(keys)[i] : 0ull;
-        fits = true;
-    } else {
-        load_key<DIM>(keys, i, active, k);
-        fits = pack_key<DIM>(k, code);
-    }
     bool pend = active && fits;
     uint32_t b = bucket_of(code, m.nb);
     uint32_t steps = 0;
@@ -530,6 +531,26 @@ __device__ __forceinline__ void insert_one(
     }
 }
 
+// One key per thread, every thread of the workgroup calls this together.
+// CODES: `keys` holds packed 64-bit codes instead of int32[DIM] rows.
+template <int DIM, int MODE, bool CODES>
+__device__ __forceinline__ void insert_one(
+        const MapDev& m, const int32_t* __restrict__ keys, int64_t i,
+        bool active, const ValueArgs& va, int32_t* __restrict__ assigned,
+        const int64_t* __restrict__ given) {
+    int32_t k[DIM] = {};
+    uint64_t code;
+    bool fits;
+    if constexpr (CODES) {
+        code = active ? reinterpret_cast<const uint64_t*>(keys)[i] : 0ull;
+        fits = true;
+    } else {
+        load_key<DIM>(keys, i, active, k);
+        fits = pack_key<DIM>(k, code);
+    }
+    insert_key<DIM, MODE>(m, k, code, fits, i, active, va, assigned, given);
+}
+
 template <int DIM, int MODE>
 __global__ __launch_bounds__(kHeapBlock) void insert_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n, ValueArgs va,
@@ -554,6 +575,119 @@ __global__ __launch_bounds__(kHeapBlock) void insert_selected_kernel(
         const int64_t i = active ? sel[t] : 0;
         insert_one<DIM, MODE, CODES>(m, keys, i, active, va, nullptr, nullptr);
         __syncthreads();
+    }
+}
+
+// Block activation around a batch of positions (ash/grid.py:121-159): the
+// block of every position and its neighbours within the dilation are inserted
+// as int3 keys.  The reference expands every position into (2r+1)^3 candidate
+// rows, de-duplicates them through a scratch hash set and inserts the
+// survivors.  Here positions arrive in image order, so their blocks come in
+// runs: activate_heads_kernel keeps one block per run ("head", one atomic per
+// wavefront to reserve list space), and activate_kernel then handles one
+// (head, neighbour offset) pair per thread, the table absorbing the remaining
+// duplicates.  MARK = false inserts; MARK = true (a second launch, when every
+// index is final) looks the candidates up again, flags their rows in `touched`
+// and records their coordinates, from which the caller lists the touched
+// blocks.
+__device__ __forceinline__ bool block_of_position(
+        const float* __restrict__ cells, int64_t i, float g, int bound_lo,
+        int bound_hi, int32_t (&base)[3]) {
+    bool inside = true;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        base[d] = static_cast<int32_t>(floorf(__fdiv_rn(cells[i * 3 + d], g)));
+        inside = inside && base[d] >= bound_lo && base[d] <= bound_hi;
+    }
+    return inside;
+}
+
+// heads[0] = number of heads (zero on entry), heads[64 + 3 h ..] = block h.
+// One update of the shared counter per 1024 positions.
+constexpr int kHeadsBlock = 1024;
+
+__global__ __launch_bounds__(kHeadsBlock) void activate_heads_kernel(
+        const float* __restrict__ cells, int64_t n, float g, int bound_lo,
+        int bound_hi, int32_t* __restrict__ heads) {
+    __shared__ int s_cnt[kHeadsBlock / 64];
+    __shared__ int s_first;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kHeadsBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    int32_t base[3] = {0, 0, 0};
+    bool lead = false;
+    if (i < n) {
+        lead = block_of_position(cells, i, g, bound_lo, bound_hi, base);
+        if (lead && i > 0) {
+            int32_t prev[3];
+            const bool pin = block_of_position(cells, i - 1, g, bound_lo, bound_hi, prev);
+            lead = !pin || prev[0] != base[0] || prev[1] != base[1] || prev[2] != base[2];
+        }
+    }
+    const uint64_t lm = __ballot(lead);
+    if (lane == 0) s_cnt[wave] = __popcll(lm);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int tot = 0;
+#pragma unroll
+        for (int q = 0; q < kHeadsBlock / 64; ++q) {
+            const int c = s_cnt[q];
+            s_cnt[q] = tot;
+            tot += c;
+        }
+        s_first = tot ? atomicAdd(heads, tot) : 0;
+    }
+    __syncthreads();
+    if (lead) {
+        int32_t* out = heads + 64 +
+                       3 * static_cast<int64_t>(s_first + s_cnt[wave] +
+                                                __popcll(lm & ((1ull << lane) - 1ull)));
+        out[0] = base[0];
+        out[1] = base[1];
+        out[2] = base[2];
+    }
+}
+
+template <bool MARK>
+__global__ __launch_bounds__(kHeapBlock) void activate_kernel(
+        MapDev m, const int32_t* __restrict__ heads, int off_lo, int width,
+        int bound_lo, int bound_hi, uint8_t* __restrict__ touched,
+        int32_t* __restrict__ coords) {
+    const int per_head = width * width * width;
+    const int64_t total = static_cast<int64_t>(heads[0]) * per_head;
+    const ValueArgs none = {};
+    for (int64_t first = static_cast<int64_t>(blockIdx.x) * kHeapBlock; first < total;
+         first += static_cast<int64_t>(gridDim.x) * kHeapBlock) {
+        const int64_t t = first + threadIdx.x;
+        bool ok = t < total;
+        int32_t k[3] = {0, 0, 0};
+        if (ok) {
+            const int64_t h = t / per_head;
+            const int o = static_cast<int>(t - h * per_head);
+            const int32_t* base = heads + 64 + 3 * h;
+            k[0] = base[0] + off_lo + o % width;
+            k[1] = base[1] + off_lo + (o / width) % width;
+            k[2] = base[2] + off_lo + o / (width * width);
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                ok = ok && k[d] >= bound_lo && k[d] <= bound_hi;
+            }
+        }
+        if constexpr (!MARK) {
+            uint64_t code;
+            const bool fits = pack_key<3>(k, code);
+            insert_key<3, kInsertKeys>(m, k, code, fits, 0, ok, none, nullptr, nullptr);
+            __syncthreads();
+        } else {
+            int32_t idx = 0;
+            const bool found = find_key<3>(m, k, ok, idx);
+            if (found && ok) {
+                touched[idx] = 1;
+                coords[static_cast<int64_t>(idx) * 3 + 0] = k[0];
+                coords[static_cast<int64_t>(idx) * 3 + 1] = k[1];
+                coords[static_cast<int64_t>(idx) * 3 + 2] = k[2];
+            }
+        }
     }
 }
 
@@ -1040,6 +1174,42 @@ int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
                         static_cast<hipStream_t>(stream)>>>(
             map->d, x, n, static_cast<float>(grid_dim), grid_dim, grid_indices,
             cell_indices, offsets, masks);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
+                      int grid_dim, int dilation, int bidirectional,
+                      int bound_lo, int bound_hi, uint8_t* touched,
+                      int32_t* coords, int32_t* heads_scratch, void* stream) {
+    if (check_batch(map, cells, n)) return 1;
+    if (map->key_dim != 3) ASH_FAIL("block activation needs a map with 3-d keys");
+    if (grid_dim < 1 || grid_dim > 1024) ASH_FAIL("grid_dim must be in 1..1024");
+    if (dilation < 0 || dilation > 8) ASH_FAIL("dilation must be in 0..8");
+    if (bound_lo > bound_hi) ASH_FAIL("empty block bounds");
+    if (n == 0) return 0;
+    if (touched == nullptr || coords == nullptr || heads_scratch == nullptr) {
+        ASH_FAIL("null output or scratch pointer");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int lo = bidirectional ? -dilation : 0;
+    const int width = dilation - lo + 1;
+    const float g = static_cast<float>(grid_dim);
+    set_counter_kernel<<<1, 64, 0, s>>>(heads_scratch, 0, 0);
+    ASH_LAUNCH_CHECK();
+    activate_heads_kernel<<<grid_for(n, kHeadsBlock), kHeadsBlock, 0, s>>>(
+            cells, n, g, bound_lo, bound_hi, heads_scratch);
+    ASH_LAUNCH_CHECK();
+    int64_t blocks = (n * width * width * width + kHeapBlock - 1) / kHeapBlock;
+    if (blocks > 2048) blocks = 2048;
+    const unsigned gb = static_cast<unsigned>(blocks);
+    activate_kernel<false><<<gb, kHeapBlock, 0, s>>>(
+            map->d, heads_scratch, lo, width, bound_lo, bound_hi, touched, coords);
+    ASH_LAUNCH_CHECK();
+    activate_kernel<true><<<gb, kHeapBlock, 0, s>>>(
+            map->d, heads_scratch, lo, width, bound_lo, bound_hi, touched, coords);
     ASH_LAUNCH_CHECK();
     return 0;
 }

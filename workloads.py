@@ -300,13 +300,19 @@ class FusionScene:
         return ((cam - t) @ rot).contiguous()
 
 
-def fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc: float, depth_max: float = 6.0):
+def fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc: float, depth_max: float = 6.0,
+               fused: bool = False):
     """One fusion step on `grid` (embedding channels: tsdf, weight), following
     the reference demo (demo/rgbd_fusion.py:200-254 and :76-110): activate the
     blocks around `points` with a one-block two-sided dilation, project every
     cell of the touched blocks into the depth image, and update the running
     weighted mean.  All tensors must live on the grid's device.  Returns the
-    number of touched blocks."""
+    number of touched blocks.  `fused` takes the library's integration kernel
+    instead of the torch expressions below (the reference's statement)."""
+    if fused:
+        import ash.fusion
+
+        return ash.fusion.fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc, depth_max)
     gc, cc, gi, ci = grid.spatial_init_(points, dilation=1, bidirectional=True)
     if gi.numel() == 0:
         return 0
