@@ -17,7 +17,7 @@ DEV = torch.device("cuda:0")
 
 def _unfused(gpu_ash, monkeypatch):
     """Makes spatial_init_ take the reference's formulation."""
-    monkeypatch.delattr(gpu_ash.common._HashMap, "activate_blocks")
+    monkeypatch.setattr(gpu_ash.grid, "FUSED_ACTIVATION", False)
 
 
 def _touched(result):

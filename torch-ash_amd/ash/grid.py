@@ -19,6 +19,11 @@ from .hashmap import HashSet
 
 backend = _get_c_extension()
 
+# spatial_init_ through the library's activation kernels (one pass over the
+# positions); False = the reference's formulation: candidate expansion, scratch
+# hash set, insert, find.  Both leave the same map and return the same blocks.
+FUSED_ACTIVATION = True
+
 Interpolation = Literal["nearest", "linear", "smooth_step"]
 
 
@@ -103,7 +108,8 @@ class SparseDenseGrid(ASHModule):
         cells = self.transform_world_to_cell(points)
         table = self.engine.backend
         if (
-            hasattr(table, "activate_blocks")
+            FUSED_ACTIVATION
+            and hasattr(table, "activate_blocks")
             and self.in_dim == 3
             and cells.dtype == torch.float32
             and len(cells) > 0

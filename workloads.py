@@ -313,7 +313,13 @@ def fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc: float, depth_ma
         import ash.fusion
 
         return ash.fusion.fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc, depth_max)
-    gc, cc, gi, ci = grid.spatial_init_(points, dilation=1, bidirectional=True)
+    import ash.grid
+
+    switch, ash.grid.FUSED_ACTIVATION = ash.grid.FUSED_ACTIVATION, False
+    try:
+        gc, cc, gi, ci = grid.spatial_init_(points, dilation=1, bidirectional=True)
+    finally:
+        ash.grid.FUSED_ACTIVATION = switch
     if gi.numel() == 0:
         return 0
     positions = grid.cell_to_world(gc, cc)
