@@ -341,6 +341,9 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     out["cfg4_forward_plus_backward"] = e
     out["cfg4_live_fraction"] = round(n_live / n4, 4)
 
+    if not args.no_cpu:
+        out["cfg4_cpu"] = cpu_trilinear(torch, ops, z, u, 1 << 18)
+
     # module-level training step: value loss + gradient-norm loss
     xq = x.clone().requires_grad_(True)
 
@@ -428,7 +431,7 @@ def cpu_baseline(torch, workloads, args):
         if best is None or t3 - t0 < best[0]:
             best = (t3 - t0, t1 - t0, t2 - t1, t3 - t2)
     total, t_ins, t_find, t_items = best
-    return {
+    out = {
         "value": round(2 * n / total / 1e6, 2),
         "unit": "Mkeys/s",
         "cores": oracle.num_threads(),
@@ -436,6 +439,55 @@ def cpu_baseline(torch, workloads, args):
         "sample": f"configuration 2 generator at {n} keys, capacity {cap}: insert+find+items, best of 2",
         "insert_Mkeys_per_s": round(n / t_ins / 1e6, 2),
         "find_Mkeys_per_s": round(n / t_find / 1e6, 2),
+    }
+    del omap, stores, values, w
+
+    # configuration 1 at full size (HashSet, 1 M inserts with 50 % duplicates
+    # into capacity 2 M, 1 M finds), all threads and one thread
+    w1 = workloads.hashset_uniform_keys(device="cpu")
+    threads = oracle.num_threads()
+    for label, nthreads in (("config1", threads), ("config1_one_thread", 1)):
+        oracle.set_num_threads(nthreads)
+        oset = oracle.HashMap(3, 2_000_000, torch.arange(2_000_000, dtype=torch.int32))
+        t0 = time.perf_counter()
+        oset.insert_keys(w1["insert_keys"])
+        t1 = time.perf_counter()
+        oset.find(w1["query_keys"])
+        t2 = time.perf_counter()
+        out[label] = {
+            "cores": nthreads,
+            "insert_Mkeys_per_s": round(len(w1["insert_keys"]) / (t1 - t0) / 1e6, 2),
+            "find_Mkeys_per_s": round(len(w1["query_keys"]) / (t2 - t1) / 1e6, 2),
+        }
+        del oset
+    oracle.set_num_threads(threads)
+    return out
+
+
+def cpu_trilinear(torch, ops, z, u, n_sample):
+    """The oracle's three query functions on the first `n_sample` queries of
+    configuration 4 (whole rays), all host threads."""
+    import ash_oracle
+
+    oracle = ash_oracle.OracleBackend()
+    emb, off, gi, ci, mk, lut_g, lut_c2c, lut_c2g = ops
+    cops = (emb.cpu(), off[:n_sample].cpu(), gi[:n_sample].cpu(), ci[:n_sample].cpu(),
+            mk[:n_sample].cpu(), lut_g.cpu(), lut_c2c.cpu(), lut_c2g.cpu())
+    zc, uc = z[:n_sample].cpu(), u[:n_sample].cpu()
+    t0 = time.perf_counter()
+    oracle.query_forward(*cops, 8, "smooth_step")
+    t1 = time.perf_counter()
+    oracle.query_backward_forward(zc, *cops, 8, "smooth_step")
+    t2 = time.perf_counter()
+    oracle.query_backward_backward(None, uc, zc, *cops, 8, "smooth_step")
+    t3 = time.perf_counter()
+    return {
+        "cores": oracle.num_threads(),
+        "sample": f"first {n_sample} queries of configuration 4 (E=4); backward passes include the "
+                  "dense zero fill of grad_embeddings",
+        "forward_Mqueries_per_s": round(n_sample / (t1 - t0) / 1e6, 2),
+        "backward_Mqueries_per_s": round(n_sample / (t2 - t1) / 1e6, 2),
+        "double_backward_Mqueries_per_s": round(n_sample / (t3 - t2) / 1e6, 2),
     }
 
 
@@ -509,6 +561,8 @@ def main():
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch, workloads, args)
+        if "cfg4_cpu" in kernels:
+            line["cpu_baseline"]["trilinear"] = kernels.pop("cfg4_cpu")
     print(json.dumps(line))
 
 
