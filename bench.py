@@ -341,6 +341,26 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     out["cfg4_forward_plus_backward"] = e
     out["cfg4_live_fraction"] = round(n_live / n4, 4)
 
+    # the ray sampler that produces such queries (ash/grid.py:322-403)
+    ro, rd = workloads.camera_rays(grid, radii, centres, 32768)
+    extent = float((grid.bbox_max - grid.bbox_min).norm())
+    t_nf, t_rs = EventTimer(torch), EventTimer(torch)
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        box = {}
+        run(t_nf, lambda: box.update(nf=grid.ray_find_near_far(ro, rd, 0.0, extent, 0.01)))
+        run(t_rs, lambda: box.update(rs=grid.ray_sample(ro, rd, *box["nf"], 128)))
+    n_samples = int(box["rs"][0].numel())
+    ms_nf, ms_rs = t_nf.mean_ms(), t_rs.mean_ms()
+    out["cfg4_ray_sampler"] = {
+        "rays": 32768,
+        "samples": n_samples,
+        "ray_find_near_far_ms": round(ms_nf, 4),
+        "ray_sample_ms": round(ms_rs, 4),
+        "Mrays_per_s": round(32768 / (ms_nf + ms_rs) / 1e3, 1),
+        "Msamples_per_s": round(n_samples / (ms_nf + ms_rs) / 1e3, 1),
+    }
+
     if not args.no_cpu:
         out["cfg4_cpu"] = cpu_trilinear(torch, ops, z, u, 1 << 18)
 

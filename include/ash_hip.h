@@ -137,6 +137,30 @@ int ash_grid_integrate_depth(float* embeddings, int64_t num_embeddings,
                              int width, float trunc, float depth_max,
                              void* stream);
 
+/* Replaces `ray_find_near_far` (ash/src/sampler.cu:7-121, pybind.cpp:35): per
+ * ray, march from t_min in steps of half a block while inside the box
+ * [bbox_min, bbox_max] and report the range [near, far] that contains active
+ * blocks; near = -1 when none is met.  Origins / directions fp32[n,3] in cell
+ * units, bbox_min / bbox_max fp32[3] on the device.  `t_step` is accepted and
+ * unused, as in the reference. */
+int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
+                          const float* ray_directions, const float* bbox_min,
+                          const float* bbox_max, int64_t n, float t_min,
+                          float t_max, float t_step, float grid2cell_multiplier,
+                          float* ray_nears, float* ray_fars, void* stream);
+
+/* Replaces the two launches of `ray_sample` (ash/src/sampler.cu:122-294,
+ * pybind.cpp:36-37).  Allocation pass: counts int64[n] receives the number of
+ * samples per ray (prefix and the outputs NULL).  The caller forms the
+ * inclusive prefix sum and allocates; assignment pass: counts NULL, prefix
+ * int64[n], ray_indices int64[total], t_nears / t_fars fp32[total]. */
+int ash_ray_sample(ash_map_t* map, const float* ray_origins,
+                   const float* ray_directions, const float* ray_nears,
+                   const float* ray_fars, int64_t n, int64_t max_samples_per_ray,
+                   float grid2cell_multiplier, int64_t* counts,
+                   const int64_t* prefix, int64_t* ray_indices, float* t_nears,
+                   float* t_fars, void* stream);
+
 /* Replaces `HashMap::insert_keys` (ash/src/hashmap_gpu.cuh:211-247).  New keys
  * pop one index each from the heap; duplicates (in the table or within the
  * batch) are ignored.  Keys beyond `capacity` are dropped and counted

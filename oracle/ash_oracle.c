@@ -38,6 +38,7 @@
  * is what bench.py times as the CPU baseline; with one thread the key loops
  * are strictly sequential and deterministic.
  */
+#include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -562,6 +563,92 @@ int64_t ash_oracle_map_load(ash_oracle_map* m, const int32_t* keys,
 
 DEFINE_QUERY(float, f32)
 DEFINE_QUERY(double, f64)
+
+/* ------------------------------------------------------------------ rays
+ * ash/src/sampler.cu:7-67 and :122-214, one loop iteration per kernel thread.
+ * Positions are `origin + t * direction`; nvcc contracts that expression into
+ * a fused multiply-add, restated with fmaf() so that every implementation
+ * checked against this file rounds alike.  Everything is in cell units; a
+ * block is `grid2cell` cells wide. */
+void ash_oracle_ray_find_near_far(const ash_oracle_map* m, const float* origins,
+                                  const float* directions, const float* bbox_min,
+                                  const float* bbox_max, int64_t n, float t_min,
+                                  float t_max, float grid2cell, float* nears,
+                                  float* fars) {
+    const float cell2grid = (float)(1.0 / grid2cell);
+    const float t_grid_step = (float)(grid2cell * 0.5);
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t i = 0; i < n; ++i) {
+        const float* o = origins + 3 * i;
+        const float* d = directions + 3 * i;
+        float near = -1.f, far = t_max, t = t_min;
+        while (t < t_max) {
+            float x[3];
+            int in_bound = 1;
+            for (int a = 0; a < 3; ++a) {
+                x[a] = fmaf(t, d[a], o[a]);
+                in_bound = in_bound && x[a] >= bbox_min[a] && x[a] <= bbox_max[a];
+            }
+            if (!in_bound) break;
+            int32_t block[3];
+            for (int a = 0; a < 3; ++a) block[a] = (int32_t)floorf(x[a] * cell2grid);
+            if (lookup(m, block) >= 0) {
+                near = near < 0.f ? t : fmaxf(near - t_grid_step, t_min);
+                far = fminf(t + t_grid_step, t_max);
+            }
+            t += t_grid_step;
+        }
+        nears[i] = near;
+        fars[i] = far;
+    }
+}
+
+/* Both passes of ray_sample (ash/src/sampler.cu:122-214): with `counts` the
+ * allocation pass, with `prefix` (inclusive prefix sum of the counts) and the
+ * three output arrays the assignment pass. */
+void ash_oracle_ray_sample(const ash_oracle_map* m, const float* origins,
+                           const float* directions, const float* ray_nears,
+                           const float* ray_fars, int64_t n,
+                           int64_t max_samples_per_ray, float grid2cell,
+                           int64_t* counts, const int64_t* prefix,
+                           int64_t* ray_indices, float* t_nears, float* t_fars) {
+    const float cell2grid = (float)(1.0 / grid2cell);
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t i = 0; i < n; ++i) {
+        const float* o = origins + 3 * i;
+        const float* d = directions + 3 * i;
+        const float ray_near = ray_nears[i], ray_far = ray_fars[i];
+        const float t_step =
+                fmaxf(0.7f, (ray_far - ray_near) / (float)max_samples_per_ray);
+        const float t_grid_step = t_step * grid2cell;
+        float t = ray_near, t_near = ray_near;
+        int64_t local = 0;
+        const int64_t start = prefix ? (i == 0 ? 0 : prefix[i - 1]) : 0;
+        while (t < ray_far) {
+            int32_t block[3];
+            for (int a = 0; a < 3; ++a) {
+                block[a] = (int32_t)floorf(fmaf(t, d[a], o[a]) * cell2grid);
+            }
+            if (lookup(m, block) < 0) {
+                t += t_grid_step;
+            } else {
+                t += t_step;
+                if (prefix) {
+                    ray_indices[start + local] = i;
+                    t_nears[start + local] = t_near;
+                    t_fars[start + local] = t;
+                }
+                t_near = t;
+                ++local;
+            }
+        }
+        if (counts) counts[i] = local;
+    }
+}
 
 int ash_oracle_num_threads(void) {
 #ifdef _OPENMP

@@ -51,6 +51,12 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     lib.ash_oracle_map_items.argtypes = [_PTR, _PTR, _PTR]
     lib.ash_oracle_map_load.restype = _I64
     lib.ash_oracle_map_load.argtypes = [_PTR, _PTR, _PTR, _I64, _PTR]
+    lib.ash_oracle_ray_find_near_far.argtypes = (
+        [_PTR] * 5 + [_I64, ctypes.c_float, ctypes.c_float, ctypes.c_float, _PTR, _PTR]
+    )
+    lib.ash_oracle_ray_sample.argtypes = (
+        [_PTR] * 5 + [_I64, _I64, ctypes.c_float] + [_PTR] * 5
+    )
     lib.ash_oracle_num_threads.restype = ctypes.c_int
     lib.ash_oracle_set_num_threads.argtypes = [ctypes.c_int]
     for sfx in ("f32", "f64"):
@@ -90,6 +96,36 @@ class OracleBackend:
 
     def set_num_threads(self, n: int) -> None:
         self.lib.ash_oracle_set_num_threads(n)
+
+    # -- rays (ash/src/pybind.cpp:35-37) --------------------------------------
+    def ray_find_near_far(self, hashmap, ray_origins, ray_directions, bbox_min, bbox_max,
+                          t_min, t_max, t_step, grid2cell_multiplier):
+        o, d = _cpu(ray_origins, torch.float32), _cpu(ray_directions, torch.float32)
+        lo, hi = _cpu(bbox_min, torch.float32), _cpu(bbox_max, torch.float32)
+        n = o.shape[0]
+        nears, fars = torch.zeros(n), torch.zeros(n)
+        self.lib.ash_oracle_ray_find_near_far(
+            hashmap._h, o.data_ptr(), d.data_ptr(), lo.data_ptr(), hi.data_ptr(), n,
+            float(t_min), float(t_max), float(grid2cell_multiplier), nears.data_ptr(),
+            fars.data_ptr())
+        return nears, fars
+
+    def ray_sample(self, hashmap, ray_origins, ray_directions, ray_nears, ray_fars,
+                   bbox_min, bbox_max, max_samples_per_ray, grid2cell_multiplier):
+        o, d = _cpu(ray_origins, torch.float32), _cpu(ray_directions, torch.float32)
+        nears, fars = _cpu(ray_nears, torch.float32), _cpu(ray_fars, torch.float32)
+        n = o.shape[0]
+        counts = torch.zeros(n, dtype=torch.int64)
+        args = (hashmap._h, o.data_ptr(), d.data_ptr(), nears.data_ptr(), fars.data_ptr(),
+                n, int(max_samples_per_ray), float(grid2cell_multiplier))
+        self.lib.ash_oracle_ray_sample(*args, counts.data_ptr(), None, None, None, None)
+        prefix = torch.cumsum(counts, 0)
+        total = int(prefix[-1]) if n else 0
+        ray_indices = torch.zeros(total, dtype=torch.int64)
+        t_nears, t_fars = torch.zeros(total), torch.zeros(total)
+        self.lib.ash_oracle_ray_sample(*args, None, prefix.data_ptr(), ray_indices.data_ptr(),
+                                       t_nears.data_ptr(), t_fars.data_ptr())
+        return ray_indices, t_nears, t_fars, prefix
 
     # -- queries ------------------------------------------------------------
     @staticmethod

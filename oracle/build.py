@@ -30,7 +30,8 @@ def build(force: bool = False, verbose: bool = True) -> str:
     os.makedirs(OUT_DIR, exist_ok=True)
     gcc = shutil.which("gcc") or "gcc"
     tmp = OUT + ".tmp"
-    cmd = [gcc, "-O2", "-std=gnu11", "-fopenmp", "-fPIC", "-shared", "-Wall", SRC, "-o", tmp]
+    cmd = [gcc, "-O2", "-std=gnu11", "-ffp-contract=off", "-fopenmp", "-fPIC", "-shared", "-Wall", SRC,
+           "-o", tmp, "-lm"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

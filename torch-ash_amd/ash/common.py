@@ -80,6 +80,16 @@ _SIGNATURES = {
          ctypes.POINTER(ctypes.c_float), _PTR, _PTR, _PTR, _PTR, ctypes.c_int, ctypes.c_int,
          ctypes.c_float, ctypes.c_float, _PTR],
     ),
+    "ash_ray_find_near_far": (
+        ctypes.c_int,
+        [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+         ctypes.c_float, _PTR, _PTR, _PTR],
+    ),
+    "ash_ray_sample": (
+        ctypes.c_int,
+        [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, ctypes.c_float, _PTR, _PTR, _PTR, _PTR, _PTR,
+         _PTR],
+    ),
     "ash_map_insert_keys": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_insert_needs_scratch": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_I64)]),
     "ash_map_insert": (
@@ -192,6 +202,76 @@ class _Backend:
         if status != 0:
             msg = self.lib.ash_last_error()
             raise RuntimeError(msg.decode() if msg else "libash_hip call failed")
+
+    # -- rays (ash/src/pybind.cpp:35-37) ----------------------------------
+    @staticmethod
+    def _rays(hashmap, ray_origins, ray_directions):
+        dev = hashmap.device()
+        o = ray_origins.to(dev, torch.float32).contiguous()
+        d = ray_directions.to(dev, torch.float32).contiguous()
+        if o.dim() != 2 or o.shape[1] != 3 or d.shape != o.shape:
+            raise RuntimeError("ray origins and directions must both be (N, 3)")
+        return dev, o, d
+
+    def ray_find_near_far(
+        self, hashmap, ray_origins, ray_directions, bbox_min, bbox_max, t_min, t_max, t_step,
+        grid2cell_multiplier,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Per ray, the parameter range that contains active blocks (cell
+        units); near = -1 where the ray meets none."""
+        dev, o, d = self._rays(hashmap, ray_origins, ray_directions)
+        lo = bbox_min.to(dev, torch.float32).contiguous()
+        hi = bbox_max.to(dev, torch.float32).contiguous()
+        n = o.shape[0]
+        nears = torch.zeros(n, dtype=torch.float32, device=dev)
+        fars = torch.zeros(n, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_ray_find_near_far(
+                    hashmap._handle, o.data_ptr(), d.data_ptr(), lo.data_ptr(), hi.data_ptr(), n,
+                    float(t_min), float(t_max), float(t_step), float(grid2cell_multiplier),
+                    nears.data_ptr(), fars.data_ptr(), _stream_of(dev),
+                )
+            )
+        return nears, fars
+
+    def ray_sample(
+        self, hashmap, ray_origins, ray_directions, ray_nears, ray_fars, bbox_min, bbox_max,
+        max_samples_per_ray, grid2cell_multiplier,
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """(ray_indices int64[M], t_nears fp32[M], t_fars fp32[M], inclusive
+        prefix sum of the per-ray sample counts int64[N])."""
+        dev, o, d = self._rays(hashmap, ray_origins, ray_directions)
+        n = o.shape[0]
+
+        def per_ray(t):
+            if not torch.is_tensor(t):
+                return torch.full((n,), float(t), dtype=torch.float32, device=dev)
+            return t.to(dev, torch.float32).expand(n).contiguous()
+
+        nears, fars = per_ray(ray_nears), per_ray(ray_fars)
+        counts = torch.zeros(n, dtype=torch.int64, device=dev)
+        fixed = (hashmap._handle, o.data_ptr(), d.data_ptr(), nears.data_ptr(), fars.data_ptr(), n,
+                 int(max_samples_per_ray), float(grid2cell_multiplier))
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_ray_sample(*fixed, counts.data_ptr(), None, None, None, None,
+                                        _stream_of(dev))
+            )
+        prefix = torch.cumsum(counts, 0)
+        total = int(prefix[-1]) if n else 0
+        ray_indices = torch.zeros(total, dtype=torch.int64, device=dev)
+        t_nears = torch.zeros(total, dtype=torch.float32, device=dev)
+        t_fars = torch.zeros(total, dtype=torch.float32, device=dev)
+        if total:
+            with torch.cuda.device(dev):
+                self.check(
+                    self.lib.ash_ray_sample(
+                        *fixed, None, prefix.data_ptr(), ray_indices.data_ptr(),
+                        t_nears.data_ptr(), t_fars.data_ptr(), _stream_of(dev),
+                    )
+                )
+        return ray_indices, t_nears, t_fars, prefix
 
     # -- depth integration (no pybind counterpart: the reference's demo does
     #    this with torch expressions, demo/rgbd_fusion.py:76-110,216-254) -----

@@ -308,11 +308,56 @@ class SparseDenseGrid(ASHModule):
         return self.transform_cell_to_world((active_coords[pick].float() + inside) * self.grid_dim)
 
     # Native kernels of the reference that are not part of the query path.
-    def ray_sample(self, *args, **kwargs):
-        raise NotImplementedError("ray_sample is not provided by this build")
+    @torch.no_grad()
+    def ray_sample(
+        self,
+        rays_o: torch.Tensor,
+        rays_d: torch.Tensor,
+        rays_near,
+        rays_far,
+        max_samples_per_ray: int,
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """Samples along rays inside active blocks (ash/grid.py:322-377).
 
-    def ray_find_near_far(self, *args, **kwargs):
-        raise NotImplementedError("ray_find_near_far is not provided by this build")
+        rays_o, rays_d (N, 3) world coordinates; rays_near / rays_far per-ray
+        ranges (tensors as returned by `ray_find_near_far`, or numbers).
+        Returns ray_indices (M,), t_near (M,), t_far (M,) in world units and
+        the inclusive prefix sum of the per-ray sample counts (N,).  Sample
+        positions are rays_o[ray_indices] + (t_near + t_far) / 2 *
+        rays_d[ray_indices]."""
+        bbox_min, bbox_max = self.get_bbox()
+        ray_indices, t_nears, t_fars, ray_prefix_sum = backend.ray_sample(
+            self.engine.backend,
+            self.transform_world_to_cell(rays_o),
+            rays_d,
+            rays_near / self.cell_size,
+            rays_far / self.cell_size,
+            self.transform_world_to_cell(bbox_min),
+            self.transform_world_to_cell(bbox_max),
+            max_samples_per_ray,
+            float(self.grid_dim),
+        )
+        return (ray_indices, t_nears * self.cell_size, t_fars * self.cell_size, ray_prefix_sum)
+
+    @torch.no_grad()
+    def ray_find_near_far(
+        self, rays_o: torch.Tensor, rays_d: torch.Tensor, t_min: float, t_max: float, t_step: float
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Per-ray range that contains active blocks (ash/grid.py:379-403), in
+        world units; near is negative where a ray meets no active block."""
+        bbox_min, bbox_max = self.get_bbox()
+        ray_nears, ray_fars = backend.ray_find_near_far(
+            self.engine.backend,
+            self.transform_world_to_cell(rays_o),
+            rays_d,
+            self.transform_world_to_cell(bbox_min),
+            self.transform_world_to_cell(bbox_max),
+            t_min / self.cell_size,
+            t_max / self.cell_size,
+            t_step / self.cell_size,
+            float(self.grid_dim),
+        )
+        return (ray_nears * self.cell_size, ray_fars * self.cell_size)
 
     def gaussian_filter_(self, *args, **kwargs):
         raise NotImplementedError("gaussian_filter_ is not provided by this build")

@@ -691,6 +691,122 @@ __global__ __launch_bounds__(kHeapBlock) void activate_kernel(
     }
 }
 
+// --------------------------------------------------------------------- rays
+// ash/src/sampler.cu:7-67 and :122-214.  One lane marches one ray; the table
+// lookups of a wavefront's 64 rays are done together (find_key), so the loops
+// run while any lane of the wavefront still has steps to take.  Positions are
+// origin + t * direction as a fused multiply-add (what nvcc makes of the
+// reference's expression); everything is in cell units and a block is
+// `grid2cell` cells wide.
+__device__ __forceinline__ void ray_block(const float (&o)[3], const float (&d)[3],
+                                          float t, float cell2grid,
+                                          int32_t (&block)[3], float (&x)[3]) {
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        x[a] = fmaf(t, d[a], o[a]);
+        block[a] = static_cast<int32_t>(floorf(__fmul_rn(x[a], cell2grid)));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
+        MapDev m, const float* __restrict__ origins,
+        const float* __restrict__ directions, const float* __restrict__ bbox_min,
+        const float* __restrict__ bbox_max, int64_t n, float t_min, float t_max,
+        float grid2cell, float* __restrict__ nears, float* __restrict__ fars) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const bool active = i < n;
+    const float cell2grid = static_cast<float>(1.0 / grid2cell);
+    const float t_grid_step = static_cast<float>(grid2cell * 0.5);
+    float o[3], d[3], lo[3], hi[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        o[a] = active ? origins[i * 3 + a] : 0.f;
+        d[a] = active ? directions[i * 3 + a] : 0.f;
+        lo[a] = bbox_min[a];
+        hi[a] = bbox_max[a];
+    }
+    float near = -1.f, far = t_max, t = t_min;
+    bool live = active && t < t_max;
+    while (__ballot(live)) {
+        int32_t block[3];
+        float x[3];
+        ray_block(o, d, t, cell2grid, block, x);
+        if (live) {
+            bool in_bound = true;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                in_bound = in_bound && x[a] >= lo[a] && x[a] <= hi[a];
+            }
+            if (!in_bound) live = false;
+        }
+        int32_t idx;
+        const bool found = find_key<3>(m, block, live, idx);
+        if (live) {
+            if (found) {
+                near = near < 0.f ? t : fmaxf(near - t_grid_step, t_min);
+                far = fminf(t + t_grid_step, t_max);
+            }
+            t += t_grid_step;
+            live = t < t_max;
+        }
+    }
+    if (active) {
+        nears[i] = near;
+        fars[i] = far;
+    }
+}
+
+// counts != nullptr: allocation pass; otherwise the assignment pass, which
+// writes the samples of ray i at prefix[i - 1] .. prefix[i].
+__global__ __launch_bounds__(kBlock) void ray_sample_kernel(
+        MapDev m, const float* __restrict__ origins,
+        const float* __restrict__ directions, const float* __restrict__ ray_nears,
+        const float* __restrict__ ray_fars, int64_t n, float max_samples,
+        float grid2cell, int64_t* __restrict__ counts,
+        const int64_t* __restrict__ prefix, int64_t* __restrict__ ray_indices,
+        float* __restrict__ t_nears, float* __restrict__ t_fars) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const bool active = i < n;
+    const float cell2grid = static_cast<float>(1.0 / grid2cell);
+    float o[3], d[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        o[a] = active ? origins[i * 3 + a] : 0.f;
+        d[a] = active ? directions[i * 3 + a] : 0.f;
+    }
+    const float ray_near = active ? ray_nears[i] : 0.f;
+    const float ray_far = active ? ray_fars[i] : 0.f;
+    const float t_step = fmaxf(0.7f, __fdiv_rn(ray_far - ray_near, max_samples));
+    const float t_grid_step = __fmul_rn(t_step, grid2cell);
+    const int64_t start = (counts == nullptr && active && i > 0) ? prefix[i - 1] : 0;
+    float t = ray_near, t_near = ray_near;
+    int64_t local = 0;
+    bool live = active && t < ray_far;
+    while (__ballot(live)) {
+        int32_t block[3];
+        float x[3];
+        ray_block(o, d, t, cell2grid, block, x);
+        int32_t idx;
+        const bool found = find_key<3>(m, block, live, idx);
+        if (live) {
+            if (!found) {
+                t += t_grid_step;
+            } else {
+                t += t_step;
+                if (counts == nullptr) {
+                    ray_indices[start + local] = i;
+                    t_nears[start + local] = t_near;
+                    t_fars[start + local] = t;
+                }
+                t_near = t;
+                ++local;
+            }
+            live = t < ray_far;
+        }
+    }
+    if (active && counts != nullptr) counts[i] = local;
+}
+
 template <int DIM>
 __global__ __launch_bounds__(kHeapBlock) void erase_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n) {
@@ -1210,6 +1326,63 @@ int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
     ASH_LAUNCH_CHECK();
     activate_kernel<true><<<gb, kHeapBlock, 0, s>>>(
             map->d, heads_scratch, lo, width, bound_lo, bound_hi, touched, coords);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
+                          const float* ray_directions, const float* bbox_min,
+                          const float* bbox_max, int64_t n, float t_min,
+                          float t_max, float t_step, float grid2cell_multiplier,
+                          float* ray_nears, float* ray_fars, void* stream) {
+    (void)t_step;  // unused by the reference as well (ash/src/sampler.cu:21)
+    if (check_batch(map, ray_origins, n)) return 1;
+    if (map->key_dim != 3) {
+        ASH_FAIL("hashmap is not a GPU hashmap of type <int, 3>, ray sample not supported");
+    }
+    if (!(grid2cell_multiplier > 0.f)) ASH_FAIL("grid2cell_multiplier must be positive");
+    if (n == 0) return 0;
+    if (ray_directions == nullptr || bbox_min == nullptr || bbox_max == nullptr ||
+        ray_nears == nullptr || ray_fars == nullptr) {
+        ASH_FAIL("null pointer in ray_find_near_far");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    ray_near_far_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+            map->d, ray_origins, ray_directions, bbox_min, bbox_max, n, t_min,
+            t_max, grid2cell_multiplier, ray_nears, ray_fars);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_ray_sample(ash_map_t* map, const float* ray_origins,
+                   const float* ray_directions, const float* ray_nears,
+                   const float* ray_fars, int64_t n, int64_t max_samples_per_ray,
+                   float grid2cell_multiplier, int64_t* counts,
+                   const int64_t* prefix, int64_t* ray_indices, float* t_nears,
+                   float* t_fars, void* stream) {
+    if (check_batch(map, ray_origins, n)) return 1;
+    if (map->key_dim != 3) {
+        ASH_FAIL("hashmap is not a GPU hashmap of type <int, 3>, ray sample not supported");
+    }
+    if (!(grid2cell_multiplier > 0.f)) ASH_FAIL("grid2cell_multiplier must be positive");
+    if (max_samples_per_ray < 1) ASH_FAIL("max_samples_per_ray must be positive");
+    if (n == 0) return 0;
+    if (ray_directions == nullptr || ray_nears == nullptr || ray_fars == nullptr) {
+        ASH_FAIL("null pointer in ray_sample");
+    }
+    const bool assign = prefix != nullptr && ray_indices != nullptr &&
+                        t_nears != nullptr && t_fars != nullptr;
+    if ((counts != nullptr) == assign) {
+        ASH_FAIL("ray_sample: pass either counts (allocation pass) or prefix and "
+                 "the three outputs (assignment pass)");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    ray_sample_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+            map->d, ray_origins, ray_directions, ray_nears, ray_fars, n,
+            static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
+            prefix, ray_indices, t_nears, t_fars);
     ASH_LAUNCH_CHECK();
     return 0;
 }

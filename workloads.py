@@ -233,6 +233,20 @@ def ray_queries(
     return x.view(-1, 3).contiguous()
 
 
+def camera_rays(grid, radii, centres, num_rays: int = 32768, seed: int = 5):
+    """Rays for the sampler (world coordinates): origins inside the grid's box,
+    each aimed at a random point of a sphere surface.  Returns (origins,
+    unit directions)."""
+    device = grid.device
+    g = _gen(device, seed)
+    target = _surface_points(radii.to(device), centres.to(device), num_rays, g)
+    lo, hi = grid.get_bbox()
+    origin = lo + (hi - lo) * (0.05 + 0.9 * torch.rand(num_rays, 3, generator=g, device=device))
+    d = target - origin
+    d = d / d.norm(dim=1, keepdim=True).clamp_min(1e-12)
+    return origin.contiguous(), d.contiguous()
+
+
 # --------------------------------------------------------------------- cfg 5
 class FusionScene:
     """Configuration 5: synthetic RGB-D stream.  48 random spheres, a pinhole
