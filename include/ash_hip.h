@@ -313,6 +313,27 @@ int ash_query_backward_backward(const ash_query_args* a,
                                 void* grad_z, void* grad_embeddings,
                                 void* stream);
 
+/* Replaces `convolution_forward` (ash/src/grid.cu:948-1043, pybind.cpp:33).
+ * inputs / outputs scalar[num_embeddings, cells_per_grid, embedding_dim];
+ * weights scalar[num_cell_nbs, embedding_dim] (one weight per window tap and
+ * channel); masks bool[>= num_grids * cells_per_grid]; grid_indices
+ * int64[num_grids] (rows of the listed blocks), cell_indices
+ * int64[cells_per_grid]; the three neighbour tables as for the queries but over
+ * the convolution window: lut_grid_nb2grid_idx int64[num_embeddings,
+ * num_grid_nbs], lut_cell_nb2cell_idx / lut_cell_nb2grid_nb
+ * int64[cells_per_grid, num_cell_nbs].  `outputs` is zero-filled here; rows of
+ * blocks that are not listed stay zero. */
+int ash_convolution_forward(const void* inputs, const void* weights,
+                            const uint8_t* masks, const int64_t* grid_indices,
+                            const int64_t* cell_indices,
+                            const int64_t* lut_grid_nb2grid_idx,
+                            const int64_t* lut_cell_nb2cell_idx,
+                            const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                            int64_t num_grids, int64_t num_embeddings,
+                            int64_t cells_per_grid, int64_t embedding_dim,
+                            int64_t num_cell_nbs, int64_t num_grid_nbs,
+                            int32_t dtype, void* stream);
+
 /* -------------------------------------------------------------- diagnostics */
 
 /* Measures the device's random-access ceilings that bound the table kernels

@@ -564,6 +564,35 @@ int64_t ash_oracle_map_load(ash_oracle_map* m, const int32_t* keys,
 DEFINE_QUERY(float, f32)
 DEFINE_QUERY(double, f64)
 
+/* ----------------------------------------------------------- convolution
+ * ash/src/grid.cu:951-1006: taps accumulated in table order, one fused
+ * multiply-add per tap and channel (nvcc's contraction of `sum += in * w`). */
+#define ASH_ORACLE_CONVOLUTION(NAME, T, FMA)                                   \
+    void NAME(const T* in, const T* w, const uint8_t* masks,                  \
+              const int64_t* grid_indices, const int64_t* cell_indices,       \
+              const int64_t* lut_g, const int64_t* lut_c2c,                   \
+              const int64_t* lut_c2g, T* out, int64_t n_grids, int64_t B,     \
+              int64_t M, int64_t E, int64_t K, int64_t GN) {                  \
+        memset(out, 0, (size_t)(B * M * E) * sizeof(T));                      \
+        _Pragma("omp parallel for schedule(static)")                          \
+        for (int64_t i = 0; i < n_grids * M; ++i) {                           \
+            if (!masks[i]) continue;                                          \
+            const int64_t g = grid_indices[i / M];                            \
+            const int64_t c = cell_indices[i % M];                            \
+            T* o = out + (g * M + c) * E;                                     \
+            for (int64_t k = 0; k < K; ++k) {                                 \
+                const int64_t gi = lut_g[g * GN + lut_c2g[c * K + k]];        \
+                if (gi < 0) continue;                                         \
+                const T* row = in + (gi * M + lut_c2c[c * K + k]) * E;        \
+                for (int64_t e = 0; e < E; ++e) {                             \
+                    o[e] = FMA(row[e], w[k * E + e], o[e]);                   \
+                }                                                             \
+            }                                                                 \
+        }                                                                     \
+    }
+ASH_ORACLE_CONVOLUTION(ash_oracle_convolution_forward_f32, float, fmaf)
+ASH_ORACLE_CONVOLUTION(ash_oracle_convolution_forward_f64, double, fma)
+
 /* ------------------------------------------------------------------ rays
  * ash/src/sampler.cu:7-67 and :122-214, one loop iteration per kernel thread.
  * Positions are `origin + t * direction`; nvcc contracts that expression into

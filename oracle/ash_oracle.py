@@ -51,6 +51,8 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     lib.ash_oracle_map_items.argtypes = [_PTR, _PTR, _PTR]
     lib.ash_oracle_map_load.restype = _I64
     lib.ash_oracle_map_load.argtypes = [_PTR, _PTR, _PTR, _I64, _PTR]
+    for sfx in ("f32", "f64"):
+        getattr(lib, f"ash_oracle_convolution_forward_{sfx}").argtypes = [_PTR] * 9 + [_I64] * 6
     lib.ash_oracle_ray_find_near_far.argtypes = (
         [_PTR] * 5 + [_I64, ctypes.c_float, ctypes.c_float, ctypes.c_float, _PTR, _PTR]
     )
@@ -96,6 +98,22 @@ class OracleBackend:
 
     def set_num_threads(self, n: int) -> None:
         self.lib.ash_oracle_set_num_threads(n)
+
+    # -- sparse convolution (ash/src/pybind.cpp:33) ---------------------------
+    def convolution_forward(self, inputs, weights, masks, grid_indices, cell_indices,
+                            lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb,
+                            grid_dim):
+        x = _cpu(inputs)
+        b, m, e = x.shape
+        w = _cpu(weights, x.dtype)
+        held = [x, w, _cpu(masks, torch.bool).view(-1), _cpu(grid_indices, torch.int64).view(-1),
+                _cpu(cell_indices, torch.int64).view(-1), _cpu(lut_grid_nb2grid_idx, torch.int64),
+                _cpu(lut_cell_nb2cell_idx, torch.int64), _cpu(lut_cell_nb2grid_nb, torch.int64)]
+        out = torch.empty_like(x)
+        fn = getattr(self.lib, f"ash_oracle_convolution_forward_{_SUFFIX[x.dtype]}")
+        fn(*[t.data_ptr() for t in held], out.data_ptr(), held[3].numel(), b, m, e,
+           held[6].shape[1], held[5].shape[1])
+        return out
 
     # -- rays (ash/src/pybind.cpp:35-37) --------------------------------------
     def ray_find_near_far(self, hashmap, ray_origins, ray_directions, bbox_min, bbox_max,

@@ -139,6 +139,10 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_int, _PTR, _I64, _I64, _PTR, ctypes.c_uint64, _PTR],
     ),
+    "ash_convolution_forward": (
+        ctypes.c_int,
+        [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR],
+    ),
     "ash_query_forward": (ctypes.c_int, [ctypes.POINTER(_QueryArgs), _PTR, _PTR]),
     "ash_query_backward_forward": (
         ctypes.c_int,
@@ -202,6 +206,47 @@ class _Backend:
         if status != 0:
             msg = self.lib.ash_last_error()
             raise RuntimeError(msg.decode() if msg else "libash_hip call failed")
+
+    # -- sparse convolution (ash/src/pybind.cpp:33) -------------------------
+    def convolution_forward(
+        self, inputs, weights, masks, grid_indices, cell_indices, lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, grid_dim,
+    ) -> torch.Tensor:
+        """outputs[row] = sum over window taps k of inputs[row of neighbour k] *
+        weights[k], per channel; same shape as `inputs`, zero rows for blocks
+        that are not listed."""
+        _require_hip(inputs, "inputs")
+        dev = inputs.device
+        if inputs.dtype not in _DTYPE or inputs.dim() != 3 or not inputs.is_contiguous():
+            raise RuntimeError("inputs must be contiguous float32/float64 (B, M, E)")
+        b, m, e = inputs.shape
+        weights = weights.to(dev, inputs.dtype).contiguous()
+        lut_g = lut_grid_nb2grid_idx.to(dev, torch.int64).contiguous()
+        lut_c2c = lut_cell_nb2cell_idx.to(dev, torch.int64).contiguous()
+        lut_c2g = lut_cell_nb2grid_nb.to(dev, torch.int64).contiguous()
+        k = lut_c2c.shape[1]
+        if weights.shape != (k, e):
+            raise RuntimeError(f"weights must be ({k}, {e}), got {tuple(weights.shape)}")
+        if lut_c2c.shape != (m, k) or lut_c2g.shape != (m, k) or lut_g.shape[0] != b:
+            raise RuntimeError("neighbour tables do not match the inputs")
+        gi = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
+        ci = cell_indices.reshape(-1).to(dev, torch.int64).contiguous()
+        if ci.numel() != m:
+            raise RuntimeError("cell_indices must list every cell of a block")
+        masks = masks.to(dev, torch.bool).contiguous()
+        if masks.numel() < gi.numel() * m:
+            raise RuntimeError("masks must cover every listed cell")
+        outputs = torch.empty_like(inputs)
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_convolution_forward(
+                    inputs.data_ptr(), weights.data_ptr(), masks.data_ptr(), gi.data_ptr(),
+                    ci.data_ptr(), lut_g.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(),
+                    outputs.data_ptr(), gi.numel(), b, m, e, k, lut_g.shape[1],
+                    _DTYPE[inputs.dtype], _stream_of(dev),
+                )
+            )
+        return outputs
 
     # -- rays (ash/src/pybind.cpp:35-37) ----------------------------------
     @staticmethod

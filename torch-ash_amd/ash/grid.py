@@ -359,11 +359,60 @@ class SparseDenseGrid(ASHModule):
         )
         return (ray_nears * self.cell_size, ray_fars * self.cell_size)
 
-    def gaussian_filter_(self, *args, **kwargs):
-        raise NotImplementedError("gaussian_filter_ is not provided by this build")
+    @torch.no_grad()
+    def gaussian_filter_(self, size: int, sigma: float) -> None:
+        """Smooths the embeddings in place with a size^3 Gaussian window
+        (ash/grid.py:435-476): per-axis weights are the normal probability mass
+        of `size` equal bins over [-sigma, sigma], normalised, and the window is
+        their outer product, the same for every channel."""
+        assert size % 2 == 1, "size must be odd"
+        import numpy as np
+        import scipy.stats as st
 
-    def convolution(self, *args, **kwargs):
-        raise NotImplementedError("convolution is not provided by this build")
+        edges = np.linspace(-sigma, sigma, size + 1)
+        axis = np.diff(st.norm.cdf(edges))
+        window = np.outer(axis, np.outer(axis, axis)).reshape((size, size, size))
+        window = torch.from_numpy(window / window.sum()).float()
+        channels = self.embeddings.shape[-1]
+        weights = window.view(size, size, size, 1).repeat(1, 1, 1, channels)
+        weights = weights.to(self.embeddings.device)
+        self.embeddings.copy_(self.convolution(self.embeddings, weights))
+
+    def convolution(self, inputs: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+        """Per-channel sparse convolution over the active cells
+        (ash/grid.py:478-520).  inputs (num_embeddings, cells_per_grid, C) laid
+        out like the embeddings; weights (2R+1, 2R+1, 2R+1, C), first axis =
+        slowest neighbour offset; neighbours in missing blocks count as zero.
+        Forward only, like the reference."""
+        assert inputs.is_contiguous()
+        assert inputs.shape[:2] == self.embeddings.shape[:2]
+        assert weights.is_contiguous()
+        assert len(weights.shape) == 4
+        assert weights.shape[0] % 2 == 1
+        radius = weights.shape[0] // 2
+        for d in range(3):
+            assert weights.shape[d] == 2 * radius + 1
+        assert weights.shape[3] == inputs.shape[-1]
+        assert weights.device == inputs.device
+
+        lut_cell_nb2grid_nb, lut_cell_nb2cell_idx = self.construct_cell_neighbor_lut(
+            radius, bidirectional=True
+        )
+        grid_radius = (radius + self.grid_dim - 1) // self.grid_dim
+        _, lut_grid_nb2grid_idx = self.construct_grid_neighbor_lut(grid_radius, bidirectional=True)
+        _, _, grid_indices, cell_indices = self.items()
+        num_cell_nbs = lut_cell_nb2grid_nb.shape[1]
+        return backend.convolution_forward(
+            inputs,
+            weights.view(num_cell_nbs, weights.shape[-1]),
+            torch.ones(inputs.shape[:2], dtype=torch.bool, device=inputs.device),
+            grid_indices,
+            cell_indices,
+            lut_grid_nb2grid_idx,
+            lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb,
+            self.grid_dim,
+        )
 
     def marching_cubes(self, *args, **kwargs):
         raise NotImplementedError("marching_cubes is not provided by this build")

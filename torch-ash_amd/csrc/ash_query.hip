@@ -524,6 +524,52 @@ query_backward_backward_kernel(
     }
 }
 
+// Sparse convolution forward (ash/src/grid.cu:948-1043): for every cell of the
+// listed blocks, out[row] = sum over the K window taps k of
+// in[row of neighbour k] * w[k], channel by channel, taps whose block is
+// missing skipped.  One lane per (cell, channel): a wavefront reads whole rows
+// of neighbouring cells, and the taps are accumulated in the reference's order
+// with one fused multiply-add each (what nvcc makes of `sum += in * w`).
+struct ConvDev {
+    const void* in;
+    const void* w;
+    const uint8_t* masks;
+    const int64_t* grid_indices;
+    const int64_t* cell_indices;
+    const int64_t* lut_g;     // [B, GN]
+    const int64_t* lut_c2c;   // [M, K]
+    const int64_t* lut_c2g;   // [M, K]
+    void* out;
+    int64_t n_grids, B, M, E, K, GN;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void convolution_forward_kernel(ConvDev a) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t item = t / a.E;
+    const int e = static_cast<int>(t - item * a.E);
+    if (item >= a.n_grids * a.M || !a.masks[item]) return;
+    const int64_t g = a.grid_indices[item / a.M];
+    const int64_t c = a.cell_indices[item % a.M];
+    if (g < 0 || g >= a.B || c < 0 || c >= a.M) return;
+    const T* in = static_cast<const T*>(a.in);
+    const T* w = static_cast<const T*>(a.w);
+    const int64_t* nb_g = a.lut_g + g * a.GN;
+    const int64_t* nb_c = a.lut_c2c + c * a.K;
+    const int64_t* nb_n = a.lut_c2g + c * a.K;
+    T sum = T(0);
+    for (int64_t k = 0; k < a.K; ++k) {
+        const int64_t gn = nb_n[k];
+        if (gn < 0 || gn >= a.GN) continue;
+        const int64_t gi = nb_g[gn];
+        if (gi < 0 || gi >= a.B) continue;
+        const int64_t ci = nb_c[k];
+        if (ci < 0 || ci >= a.M) continue;
+        sum = fma(in[(gi * a.M + ci) * a.E + e], w[k * a.E + e], sum);
+    }
+    static_cast<T*>(a.out)[(g * a.M + c) * a.E + e] = sum;
+}
+
 __global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p,
                                                         int64_t n16) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
@@ -854,6 +900,65 @@ int ash_query_backward_backward(const ash_query_args* a,
                                               grad_embeddings, s)
                    : dispatch_bwd_bwd<float>(d, grad_grad_offsets, z, grad_z,
                                              grad_embeddings, s);
+}
+
+int ash_convolution_forward(const void* inputs, const void* weights,
+                            const uint8_t* masks, const int64_t* grid_indices,
+                            const int64_t* cell_indices,
+                            const int64_t* lut_grid_nb2grid_idx,
+                            const int64_t* lut_cell_nb2cell_idx,
+                            const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                            int64_t num_grids, int64_t num_embeddings,
+                            int64_t cells_per_grid, int64_t embedding_dim,
+                            int64_t num_cell_nbs, int64_t num_grid_nbs,
+                            int32_t dtype, void* stream) {
+    if (dtype != ASH_F32 && dtype != ASH_F64) ASH_FAIL("unknown dtype");
+    if (num_grids < 0 || num_embeddings < 1 || cells_per_grid < 1 ||
+        embedding_dim < 1 || num_cell_nbs < 1 || num_grid_nbs < 1) {
+        ASH_FAIL("convolution_forward: bad sizes");
+    }
+    if (inputs == nullptr || weights == nullptr || outputs == nullptr ||
+        lut_grid_nb2grid_idx == nullptr || lut_cell_nb2cell_idx == nullptr ||
+        lut_cell_nb2grid_nb == nullptr) {
+        ASH_FAIL("null pointer in convolution_forward");
+    }
+    if (num_grids > 0 && (masks == nullptr || grid_indices == nullptr ||
+                          cell_indices == nullptr)) {
+        ASH_FAIL("null pointer in convolution_forward");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t scalar = dtype == ASH_F32 ? 4 : 8;
+    // rows of blocks that are not listed stay zero (at::zeros_like, grid.cu:1010)
+    if (zero_fill(outputs, num_embeddings * cells_per_grid * embedding_dim * scalar, s)) {
+        return 1;
+    }
+    if (num_grids == 0) return 0;
+    ConvDev a;
+    a.in = inputs;
+    a.w = weights;
+    a.masks = masks;
+    a.grid_indices = grid_indices;
+    a.cell_indices = cell_indices;
+    a.lut_g = lut_grid_nb2grid_idx;
+    a.lut_c2c = lut_cell_nb2cell_idx;
+    a.lut_c2g = lut_cell_nb2grid_nb;
+    a.out = outputs;
+    a.n_grids = num_grids;
+    a.B = num_embeddings;
+    a.M = cells_per_grid;
+    a.E = embedding_dim;
+    a.K = num_cell_nbs;
+    a.GN = num_grid_nbs;
+    const int64_t threads = num_grids * cells_per_grid * embedding_dim;
+    const int64_t blocks = (threads + kBlock - 1) / kBlock;
+    if (blocks > 0x7FFFFFFFll) ASH_FAIL("convolution_forward: too many cells in one call");
+    if (dtype == ASH_F32) {
+        convolution_forward_kernel<float><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
+    } else {
+        convolution_forward_kernel<double><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
 }
 
 }  // extern "C"
