@@ -300,7 +300,23 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         e = roofline_entry(f"query_forward_kernel<f32,E16> {interp}", alg, t.mean_ms())
         e["Mqueries_per_s"] = round(n3 / e["ms"] / 1e3, 1)
         out[f"cfg3_forward_{interp}"] = e
-    del grid, ops, x
+
+    # sparse convolution over the same grid (3^3 window, per channel): every
+    # row is read once per tap through the caches; the algorithmic figure
+    # counts one read and one write of each active row
+    weights = torch.rand(3, 3, 3, 16, device=dev)
+    t = EventTimer(torch)
+    for it in range(3):
+        if it == 0:
+            grid.convolution(grid.embeddings.detach(), weights)
+        else:
+            t(lambda: grid.convolution(grid.embeddings.detach(), weights))
+    cells = grid.engine.size() * 512
+    e = roofline_entry("convolution_cell_kernel<f32,16> 27 taps (incl. table construction)",
+                       2 * 64 * cells, t.mean_ms())
+    e["Gcells_per_s"] = round(cells / e["ms"] / 1e6, 2)
+    out["cfg3_convolution"] = e
+    del grid, ops, x, weights
     torch.cuda.empty_cache()
 
     # configuration 4

@@ -543,6 +543,100 @@ struct ConvDev {
     int64_t n_grids, B, M, E, K, GN;
 };
 
+// One lane per cell with all channels of the row in registers (EC >= E, a
+// power of two up to 16): consecutive lanes are consecutive cells, so a tap
+// reads a contiguous run of rows, and the table entries are fetched once per
+// cell instead of once per channel.  `vec4`: fp32 rows of a multiple of four
+// channels on 16-byte aligned buffers are moved as float4.
+template <typename T, int EC>
+__global__ __launch_bounds__(kBlock) void convolution_cell_kernel(ConvDev a, int vec4) {
+    const int64_t item = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (item >= a.n_grids * a.M || !a.masks[item]) return;
+    const int64_t g = a.grid_indices[item / a.M];
+    const int64_t c = a.cell_indices[item % a.M];
+    if (g < 0 || g >= a.B || c < 0 || c >= a.M) return;
+    const T* in = static_cast<const T*>(a.in);
+    const T* w = static_cast<const T*>(a.w);
+    const int64_t* nb_g = a.lut_g + g * a.GN;
+    const int64_t* nb_c = a.lut_c2c + c * a.K;
+    const int64_t* nb_n = a.lut_c2g + c * a.K;
+    const int E = static_cast<int>(a.E);
+    T acc[EC];
+#pragma unroll
+    for (int e = 0; e < EC; ++e) acc[e] = T(0);
+    for (int64_t k = 0; k < a.K; ++k) {
+        const int64_t gn = nb_n[k];
+        if (gn < 0 || gn >= a.GN) continue;
+        const int64_t gi = nb_g[gn];
+        if (gi < 0 || gi >= a.B) continue;
+        const int64_t ci = nb_c[k];
+        if (ci < 0 || ci >= a.M) continue;
+        const T* row = in + (gi * a.M + ci) * E;
+        const T* wk = w + k * E;
+        if constexpr (sizeof(T) == 4 && EC >= 4) {
+            if (vec4) {
+#pragma unroll
+                for (int q = 0; q < EC / 4; ++q) {
+                    if (4 * q < E) {
+                        const float4 r = reinterpret_cast<const float4*>(row)[q];
+                        acc[4 * q + 0] = fmaf(r.x, wk[4 * q + 0], acc[4 * q + 0]);
+                        acc[4 * q + 1] = fmaf(r.y, wk[4 * q + 1], acc[4 * q + 1]);
+                        acc[4 * q + 2] = fmaf(r.z, wk[4 * q + 2], acc[4 * q + 2]);
+                        acc[4 * q + 3] = fmaf(r.w, wk[4 * q + 3], acc[4 * q + 3]);
+                    }
+                }
+                continue;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < EC; ++e) {
+            if (e < E) acc[e] = fma(row[e], wk[e], acc[e]);
+        }
+    }
+    T* o = static_cast<T*>(a.out) + (g * a.M + c) * E;
+    if constexpr (sizeof(T) == 4 && EC >= 4) {
+        if (vec4) {
+#pragma unroll
+            for (int q = 0; q < EC / 4; ++q) {
+                if (4 * q < E) {
+                    reinterpret_cast<float4*>(o)[q] = make_float4(
+                            acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+                }
+            }
+            return;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < EC; ++e) {
+        if (e < E) o[e] = acc[e];
+    }
+}
+
+template <typename T>
+int launch_convolution_cells(const ConvDev& a, hipStream_t s) {
+    const int64_t threads = a.n_grids * a.M;
+    const int64_t blocks = (threads + kBlock - 1) / kBlock;
+    if (blocks > 0x7FFFFFFFll) ASH_FAIL("convolution_forward: too many cells in one call");
+    const unsigned gb = static_cast<unsigned>(blocks);
+    const uintptr_t align = reinterpret_cast<uintptr_t>(a.in) | reinterpret_cast<uintptr_t>(a.out);
+    const int vec4 = (sizeof(T) == 4 && a.E % 4 == 0 && align % 16 == 0) ? 1 : 0;
+    if (a.E <= 1) {
+        convolution_cell_kernel<T, 1><<<gb, kBlock, 0, s>>>(a, vec4);
+    } else if (a.E <= 2) {
+        convolution_cell_kernel<T, 2><<<gb, kBlock, 0, s>>>(a, vec4);
+    } else if (a.E <= 4) {
+        convolution_cell_kernel<T, 4><<<gb, kBlock, 0, s>>>(a, vec4);
+    } else if (a.E <= 8) {
+        convolution_cell_kernel<T, 8><<<gb, kBlock, 0, s>>>(a, vec4);
+    } else {
+        convolution_cell_kernel<T, 16><<<gb, kBlock, 0, s>>>(a, vec4);
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+// Wider rows than the reference supports (its accumulator holds 16 channels):
+// one lane per (cell, channel).
 template <typename T>
 __global__ __launch_bounds__(kBlock) void convolution_forward_kernel(ConvDev a) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
@@ -949,6 +1043,10 @@ int ash_convolution_forward(const void* inputs, const void* weights,
     a.E = embedding_dim;
     a.K = num_cell_nbs;
     a.GN = num_grid_nbs;
+    if (embedding_dim <= 16) {
+        return dtype == ASH_F32 ? launch_convolution_cells<float>(a, s)
+                                : launch_convolution_cells<double>(a, s);
+    }
     const int64_t threads = num_grids * cells_per_grid * embedding_dim;
     const int64_t blocks = (threads + kBlock - 1) / kBlock;
     if (blocks > 0x7FFFFFFFll) ASH_FAIL("convolution_forward: too many cells in one call");
