@@ -334,6 +334,27 @@ int ash_convolution_forward(const void* inputs, const void* weights,
                             int64_t num_cell_nbs, int64_t num_grid_nbs,
                             int32_t dtype, void* stream);
 
+/* Replaces one launch of `isosurface_extraction` (ash/src/grid.cu:453-602,
+ * pybind.cpp:30), which the reference runs twice: to count, then to fill.
+ * sdfs / weights scalar[num_embeddings, cells_per_grid]; grid_indices
+ * int64[num_grids]; grid_coords_table int32[num_embeddings, 3]; cell_coords_table
+ * int32[cells_per_grid, 3]; the three 8-entry neighbour tables of the queries.
+ * `counter` (device int32) is reset and receives the number of surface points;
+ * with positions == NULL nothing else is written, otherwise positions
+ * fp32[count, 3] (cell units, any order) is filled -- it must hold the count a
+ * previous call reported. */
+int ash_isosurface_extraction(const void* sdfs, const void* weights,
+                              const int64_t* grid_indices,
+                              const int32_t* grid_coords_table,
+                              const int64_t* lut_grid_nb2grid_idx,
+                              const int32_t* cell_coords_table,
+                              const int64_t* lut_cell_nb2cell_idx,
+                              const int64_t* lut_cell_nb2grid_nb,
+                              int64_t num_grids, int64_t num_embeddings,
+                              int64_t cells_per_grid, int grid_dim,
+                              float iso_value, float weight_thr, int32_t dtype,
+                              int32_t* counter, float* positions, void* stream);
+
 /* -------------------------------------------------------------- diagnostics */
 
 /* Measures the device's random-access ceilings that bound the table kernels

@@ -564,6 +564,46 @@ int64_t ash_oracle_map_load(ash_oracle_map* m, const int32_t* keys,
 DEFINE_QUERY(float, f32)
 DEFINE_QUERY(double, f64)
 
+/* ------------------------------------------------------- iso-surface points
+ * ash/src/grid.cu:453-531, cells in launch order.  Returns the number of
+ * points; positions (may be NULL) receives them in that order. */
+#define ASH_ORACLE_ISOSURFACE(NAME, T)                                        \
+    int64_t NAME(const T* sdfs, const T* weights, const int64_t* grid_indices, \
+                 const int32_t* grid_coords, const int64_t* lut_g,            \
+                 const int32_t* cell_coords, const int64_t* lut_c2c,          \
+                 const int64_t* lut_c2g, int64_t n_grids, int64_t M, int g,   \
+                 float iso, float weight_thr, float* positions) {             \
+        int64_t count = 0;                                                    \
+        for (int64_t i = 0; i < n_grids * M; ++i) {                           \
+            const int64_t gi = grid_indices[i / M];                           \
+            const int64_t c = i % M;                                          \
+            if (weights[gi * M + c] < weight_thr) continue;                   \
+            const T self = sdfs[gi * M + c] - iso;                            \
+            for (int d = 0; d < 3; ++d) {                                     \
+                const int nb = 1 << d;                                        \
+                const int64_t ng = lut_g[gi * 8 + lut_c2g[c * 8 + nb]];       \
+                if (ng == -1) break;                                          \
+                const int64_t nc = lut_c2c[c * 8 + nb];                       \
+                const T other = sdfs[ng * M + nc] - iso;                      \
+                if (self * other < 0 && weights[ng * M + nc] >= weight_thr) { \
+                    if (positions) {                                          \
+                        const float ratio = (float)(self / (self - other));   \
+                        for (int a = 0; a < 3; ++a) {                         \
+                            positions[count * 3 + a] =                        \
+                                    (float)(grid_coords[gi * 3 + a] * g +     \
+                                            cell_coords[c * 3 + a]) +         \
+                                    (a == d ? ratio : 0.f);                   \
+                        }                                                     \
+                    }                                                         \
+                    ++count;                                                  \
+                }                                                             \
+            }                                                                 \
+        }                                                                     \
+        return count;                                                         \
+    }
+ASH_ORACLE_ISOSURFACE(ash_oracle_isosurface_f32, float)
+ASH_ORACLE_ISOSURFACE(ash_oracle_isosurface_f64, double)
+
 /* ----------------------------------------------------------- convolution
  * ash/src/grid.cu:951-1006: taps accumulated in table order, one fused
  * multiply-add per tap and channel (nvcc's contraction of `sum += in * w`). */

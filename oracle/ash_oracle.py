@@ -53,6 +53,9 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
     lib.ash_oracle_map_load.argtypes = [_PTR, _PTR, _PTR, _I64, _PTR]
     for sfx in ("f32", "f64"):
         getattr(lib, f"ash_oracle_convolution_forward_{sfx}").argtypes = [_PTR] * 9 + [_I64] * 6
+        iso = getattr(lib, f"ash_oracle_isosurface_{sfx}")
+        iso.restype = _I64
+        iso.argtypes = [_PTR] * 8 + [_I64, _I64, ctypes.c_int, ctypes.c_float, ctypes.c_float, _PTR]
     lib.ash_oracle_ray_find_near_far.argtypes = (
         [_PTR] * 5 + [_I64, ctypes.c_float, ctypes.c_float, ctypes.c_float, _PTR, _PTR]
     )
@@ -98,6 +101,26 @@ class OracleBackend:
 
     def set_num_threads(self, n: int) -> None:
         self.lib.ash_oracle_set_num_threads(n)
+
+    # -- iso-surface points (ash/src/pybind.cpp:30) ---------------------------
+    def isosurface_extraction(self, sdfs, weights, grid_indices, grid_coords_table,
+                              lut_grid_nb2grid_idx, cell_coords_table, lut_cell_nb2cell_idx,
+                              lut_cell_nb2grid_nb, grid_dim, iso_value, weight_thr):
+        x = _cpu(sdfs)
+        b, m = x.shape[0], x.shape[1]
+        x = x.reshape(b, m).contiguous()
+        held = [x, _cpu(weights, x.dtype).reshape(b, m).contiguous(),
+                _cpu(grid_indices, torch.int64).view(-1), _cpu(grid_coords_table, torch.int32),
+                _cpu(lut_grid_nb2grid_idx, torch.int64), _cpu(cell_coords_table, torch.int32),
+                _cpu(lut_cell_nb2cell_idx, torch.int64), _cpu(lut_cell_nb2grid_nb, torch.int64)]
+        fn = getattr(self.lib, f"ash_oracle_isosurface_{_SUFFIX[x.dtype]}")
+        args = [t.data_ptr() for t in held] + [held[2].numel(), m, int(grid_dim),
+                                               float(iso_value), float(weight_thr)]
+        count = fn(*args, None)
+        positions = torch.zeros((count, 3), dtype=torch.float32)
+        if count:
+            fn(*args, positions.data_ptr())
+        return positions
 
     # -- sparse convolution (ash/src/pybind.cpp:33) ---------------------------
     def convolution_forward(self, inputs, weights, masks, grid_indices, cell_indices,

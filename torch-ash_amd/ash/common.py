@@ -139,6 +139,11 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_int, _PTR, _I64, _I64, _PTR, ctypes.c_uint64, _PTR],
     ),
+    "ash_isosurface_extraction": (
+        ctypes.c_int,
+        [_PTR] * 8 + [_I64] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int32,
+                                    _PTR, _PTR, _PTR],
+    ),
     "ash_convolution_forward": (
         ctypes.c_int,
         [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR],
@@ -206,6 +211,52 @@ class _Backend:
         if status != 0:
             msg = self.lib.ash_last_error()
             raise RuntimeError(msg.decode() if msg else "libash_hip call failed")
+
+    # -- iso-surface points (ash/src/pybind.cpp:30) --------------------------
+    def isosurface_extraction(
+        self, sdfs, weights, grid_indices, grid_coords_table, lut_grid_nb2grid_idx,
+        cell_coords_table, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, grid_dim, iso_value,
+        weight_thr,
+    ) -> torch.Tensor:
+        """Zero crossings of `sdfs - iso_value` on the +x/+y/+z edges of the
+        listed blocks' cells, (P, 3) float32 in cell units, in no particular
+        order."""
+        _require_hip(sdfs, "sdfs")
+        dev = sdfs.device
+        if sdfs.dtype not in _DTYPE:
+            raise RuntimeError("sdfs must be float32 or float64")
+        b, m = sdfs.shape[0], sdfs.shape[1]
+        sdfs = sdfs.reshape(b, m).contiguous()
+        weights = weights.to(dev, sdfs.dtype).reshape(b, m).contiguous()
+        gi = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
+        gc = grid_coords_table.to(dev, torch.int32).contiguous()
+        cc = cell_coords_table.to(dev, torch.int32).contiguous()
+        lut_g = lut_grid_nb2grid_idx.to(dev, torch.int64).contiguous()
+        lut_c2c = lut_cell_nb2cell_idx.to(dev, torch.int64).contiguous()
+        lut_c2g = lut_cell_nb2grid_nb.to(dev, torch.int64).contiguous()
+        if gc.shape != (b, 3) or cc.shape != (m, 3) or lut_g.shape != (b, 8):
+            raise RuntimeError("coordinate / neighbour tables do not match the grid")
+        if lut_c2c.shape != (m, 8) or lut_c2g.shape != (m, 8):
+            raise RuntimeError("cell neighbour tables must be (cells_per_grid, 8)")
+        counter = torch.zeros(1, dtype=torch.int32, device=dev)
+
+        def launch(positions):
+            with torch.cuda.device(dev):
+                self.check(
+                    self.lib.ash_isosurface_extraction(
+                        sdfs.data_ptr(), weights.data_ptr(), gi.data_ptr(), gc.data_ptr(),
+                        lut_g.data_ptr(), cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(),
+                        gi.numel(), b, m, int(grid_dim), float(iso_value), float(weight_thr),
+                        _DTYPE[sdfs.dtype], counter.data_ptr(),
+                        positions.data_ptr() if positions is not None else None, _stream_of(dev),
+                    )
+                )
+
+        launch(None)
+        positions = torch.zeros((int(counter.item()), 3), dtype=torch.float32, device=dev)
+        if positions.shape[0]:
+            launch(positions)
+        return positions
 
     # -- sparse convolution (ash/src/pybind.cpp:33) -------------------------
     def convolution_forward(

@@ -414,8 +414,62 @@ class SparseDenseGrid(ASHModule):
             self.grid_dim,
         )
 
-    def marching_cubes(self, *args, **kwargs):
-        raise NotImplementedError("marching_cubes is not provided by this build")
+    @torch.no_grad()
+    def isosurface_points(
+        self, tsdfs: torch.Tensor, weights: torch.Tensor, iso_value: float = 0.0,
+        weight_thr: float = 1.0,
+    ) -> torch.Tensor:
+        """World positions (P, 3) where `tsdfs` crosses `iso_value` on the cell
+        edges of the active blocks, both end points weighing at least
+        `weight_thr`: the `vertices_only` branch of the reference's
+        `marching_cubes` (ash/grid.py:628-678) without its open3d packaging.
+        tsdfs, weights: (num_embeddings, cells_per_grid[, 1])."""
+        if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
+            self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+        _, grid_indices = self.engine.items()
+        vertices = backend.isosurface_extraction(
+            tsdfs,
+            weights,
+            grid_indices,
+            self.grid_coords,
+            self.lut_grid_nb2grid_idx,
+            self.cell_coords,
+            self.lut_cell_nb2cell_idx,
+            self.lut_cell_nb2grid_nb,
+            self.grid_dim,
+            iso_value,
+            weight_thr,
+        )
+        return self.transform_cell_to_world(vertices)
+
+    def marching_cubes(
+        self, tsdfs, weights, color_fn=None, normal_fn=None, iso_value: float = 0.0,
+        weight_thr: float = 1.0, vertices_only: bool = False,
+    ):
+        """Surface extraction (ash/grid.py:628-711).  Only `vertices_only=True`
+        is provided: it returns an open3d point cloud like the reference when
+        open3d is importable, otherwise a dict of tensors with the same fields
+        (positions, colors, normals); None when there are no points.  The
+        triangle mesh needs the marching-cubes case tables and is not built."""
+        if not vertices_only:
+            raise NotImplementedError("marching_cubes triangles are not provided by this build")
+        positions = self.isosurface_points(tsdfs, weights, iso_value, weight_thr)
+        if len(positions) == 0:
+            return None
+        fields = {"positions": positions}
+        if color_fn is not None:
+            fields["colors"] = color_fn(positions)
+        if normal_fn is not None:
+            fields["normals"] = normal_fn(positions)
+        try:
+            import open3d as o3d
+        except ImportError:
+            return fields
+        pcd = o3d.t.geometry.PointCloud(positions.detach().cpu().numpy())
+        for name in ("colors", "normals"):
+            if name in fields:
+                pcd.point[name] = fields[name].detach().cpu().numpy()
+        return pcd
 
     # ------------------------------------------------------ neighbour tables
     @torch.no_grad()
