@@ -312,7 +312,7 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         else:
             t(lambda: grid.convolution(grid.embeddings.detach(), weights))
     cells = grid.engine.size() * 512
-    e = roofline_entry("convolution_cell_kernel<f32,16> 27 taps (incl. table construction)",
+    e = roofline_entry("convolution_block_kernel<f32,16> 27 taps (incl. table construction)",
                        2 * 64 * cells, t.mean_ms())
     e["Gcells_per_s"] = round(cells / e["ms"] / 1e6, 2)
     out["cfg3_convolution"] = e

@@ -88,3 +88,19 @@ def test_gaussian_filter_device_equals_oracle_backend(gpu_ash, oracle, monkeypat
         on_cpu = run(torch.device("cpu"))
     assert torch.equal(on_device, on_cpu)
     assert not torch.equal(on_device, field)
+
+
+def test_few_blocks_take_the_per_cell_kernel(gpu_ash, oracle):
+    """Fewer than 64 listed blocks: the launch that maps one lane to one cell
+    (also with a row width that is not a multiple of four, and one above 16)."""
+    for channels in (3, 8, 20):
+        grid, _, _ = workloads.build_grid(gpu_ash, 48, min(channels, 16), 8, 16, device=DEV)
+        g = torch.Generator().manual_seed(840 + channels)
+        inputs = torch.randn(*grid.embeddings.shape[:2], channels, generator=g).to(DEV)
+        weights = torch.randn(3, 3, 3, channels, generator=g).to(DEV)
+        out = grid.convolution(inputs, weights)
+        c2g, c2c, g2g, gi, ci = _tables(grid, 1)
+        masks = torch.ones(inputs.shape[:2], dtype=torch.bool)
+        ref = oracle.convolution_forward(inputs, weights.view(27, channels), masks, gi, ci,
+                                         g2g, c2c, c2g, 8)
+        assert torch.equal(out.cpu(), ref)

@@ -727,6 +727,7 @@ class _HashMap:
         """After an insert/load: keys that need the second region are counted by
         the kernel; attach the region once and let the caller re-issue."""
         st = self.status()
+        self._status_after_insert = st
         if st["dropped"] > 0 or st["tombstones"] > 0:
             self._maybe_tombstones = True
         if st["exotic_pending"] == 0:
@@ -757,6 +758,12 @@ class _HashMap:
             "exotic_pending": out[3],
             "load_duplicates": out[4],
         }
+
+    def status_after_insert(self) -> Dict[str, int]:
+        """The counters as read back at the end of the latest insert (every
+        insert reads them once); saves the caller a second read-back."""
+        st = getattr(self, "_status_after_insert", None)
+        return st if st is not None else self.status()
 
     def size(self) -> int:
         n = _I64(0)
@@ -951,6 +958,7 @@ class _HashMap:
     def erase(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)
         self._maybe_tombstones = True
+        self._status_after_insert = None
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_erase(
@@ -962,6 +970,7 @@ class _HashMap:
         with torch.cuda.device(self._device):
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
         self._maybe_tombstones = False
+        self._status_after_insert = None
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
         n = self.size()

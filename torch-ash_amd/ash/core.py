@@ -106,7 +106,8 @@ class ASHEngine(nn.Module):
         """The reference notices an overflow by comparing sizes before and after
         (ash/core.py:203-211); here the table refuses the surplus keys and
         counts them, and the same warning is raised from that count."""
-        status = self.backend.status()
+        read = getattr(self.backend, "status_after_insert", self.backend.status)
+        status = read()
         dropped = status["dropped"] - dropped_before
         self._dropped_seen = status["dropped"]
         if dropped > 0:

@@ -612,6 +612,140 @@ __global__ __launch_bounds__(kBlock) void convolution_cell_kernel(ConvDev a, int
     }
 }
 
+// The same per-cell accumulation with one persistent workgroup per block of
+// cells at a time: the block's own rows are staged in LDS (for a 3^3 window
+// about four taps in five stay inside the block) and the two per-cell tables
+// are kept in LDS in compact form (uint16 cell, uint8 block offset) for the
+// whole launch, when they fit.  Taps, order and arithmetic are unchanged.
+constexpr int kConvThreads = 512;
+unsigned persistent_grid(int64_t ntiles, size_t smem);
+
+template <typename T, int EC>
+__global__ __launch_bounds__(kConvThreads) void convolution_block_kernel(
+        ConvDev a, int vec4, int lut_lds, int rows_lds) {
+    extern __shared__ __align__(16) unsigned char conv_smem[];
+    const int tid = threadIdx.x;
+    const int E = static_cast<int>(a.E);
+    const int M = static_cast<int>(a.M);
+    const int K = static_cast<int>(a.K);
+    T* rows = reinterpret_cast<T*>(conv_smem);
+    const size_t rows_bytes =
+            rows_lds ? (static_cast<size_t>(M) * E * sizeof(T) + 15) / 16 * 16 : 0;
+    uint16_t* cc = reinterpret_cast<uint16_t*>(conv_smem + rows_bytes);
+    uint8_t* cg = reinterpret_cast<uint8_t*>(cc + static_cast<size_t>(M) * K);
+    if (lut_lds) {
+        for (int t = tid; t < M * K; t += kConvThreads) {
+            const int64_t ci = a.lut_c2c[t];
+            const int64_t gn = a.lut_c2g[t];
+            cc[t] = (ci >= 0 && ci < M) ? static_cast<uint16_t>(ci) : 0xFFFFu;
+            cg[t] = (gn >= 0 && gn < a.GN) ? static_cast<uint8_t>(gn) : 0xFFu;
+        }
+    }
+    const T* in = static_cast<const T*>(a.in);
+    const T* w = static_cast<const T*>(a.w);
+    for (int64_t blk = blockIdx.x; blk < a.n_grids; blk += gridDim.x) {
+        const int64_t g = a.grid_indices[blk];
+        const bool g_ok = g >= 0 && g < a.B;
+        __syncthreads();
+        if (rows_lds && g_ok) {
+            const T* src = in + g * a.M * E;
+            if (vec4) {
+                for (int t = tid; t < M * E / 4; t += kConvThreads) {
+                    reinterpret_cast<float4*>(rows)[t] = reinterpret_cast<const float4*>(src)[t];
+                }
+            } else {
+                for (int t = tid; t < M * E; t += kConvThreads) rows[t] = src[t];
+            }
+        }
+        __syncthreads();
+        if (!g_ok) continue;
+        const int64_t* nb_g = a.lut_g + g * a.GN;
+        for (int c_i = tid; c_i < M; c_i += kConvThreads) {
+            if (!a.masks[blk * a.M + c_i]) continue;
+            const int64_t c = a.cell_indices[c_i];
+            if (c < 0 || c >= a.M) continue;
+            T acc[EC];
+#pragma unroll
+            for (int e = 0; e < EC; ++e) acc[e] = T(0);
+            for (int k = 0; k < K; ++k) {
+                int64_t gn, ci;
+                if (lut_lds) {
+                    const uint16_t ci16 = cc[c * K + k];
+                    const uint8_t gn8 = cg[c * K + k];
+                    if (ci16 == 0xFFFFu || gn8 == 0xFFu) continue;
+                    ci = ci16;
+                    gn = gn8;
+                } else {
+                    gn = a.lut_c2g[c * K + k];
+                    ci = a.lut_c2c[c * K + k];
+                    if (gn < 0 || gn >= a.GN || ci < 0 || ci >= a.M) continue;
+                }
+                const int64_t gi = nb_g[gn];
+                if (gi < 0 || gi >= a.B) continue;
+                const T* row = (rows_lds && gi == g) ? rows + ci * E
+                                                     : in + (gi * a.M + ci) * E;
+                const T* wk = w + static_cast<int64_t>(k) * E;
+                if constexpr (sizeof(T) == 4 && EC >= 4) {
+                    if (vec4) {
+#pragma unroll
+                        for (int q = 0; q < EC / 4; ++q) {
+                            if (4 * q < E) {
+                                const float4 r = reinterpret_cast<const float4*>(row)[q];
+                                acc[4 * q + 0] = fmaf(r.x, wk[4 * q + 0], acc[4 * q + 0]);
+                                acc[4 * q + 1] = fmaf(r.y, wk[4 * q + 1], acc[4 * q + 1]);
+                                acc[4 * q + 2] = fmaf(r.z, wk[4 * q + 2], acc[4 * q + 2]);
+                                acc[4 * q + 3] = fmaf(r.w, wk[4 * q + 3], acc[4 * q + 3]);
+                            }
+                        }
+                        continue;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < EC; ++e) {
+                    if (e < E) acc[e] = fma(row[e], wk[e], acc[e]);
+                }
+            }
+            T* o = static_cast<T*>(a.out) + (g * a.M + c) * E;
+            bool stored = false;
+            if constexpr (sizeof(T) == 4 && EC >= 4) {
+                if (vec4) {
+#pragma unroll
+                    for (int q = 0; q < EC / 4; ++q) {
+                        if (4 * q < E) {
+                            reinterpret_cast<float4*>(o)[q] = make_float4(
+                                    acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]);
+                        }
+                    }
+                    stored = true;
+                }
+            }
+            if (!stored) {
+#pragma unroll
+                for (int e = 0; e < EC; ++e) {
+                    if (e < E) o[e] = acc[e];
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int EC>
+int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
+    const size_t rows_bytes = (static_cast<size_t>(a.M) * a.E * sizeof(T) + 15) / 16 * 16;
+    const size_t lut_bytes = static_cast<size_t>(a.M) * a.K * 3;
+    const int rows_lds = rows_bytes <= 64 * 1024 ? 1 : 0;
+    const int lut_lds = (lut_bytes <= 48 * 1024 && a.M < 0xFFFF && a.GN < 0xFF) ? 1 : 0;
+    const size_t smem = (rows_lds ? rows_bytes : 0) + (lut_lds ? lut_bytes : 0) + 16;
+    auto kernel = convolution_block_kernel<T, EC>;
+    ASH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                static_cast<int>(smem)));
+    unsigned g = persistent_grid(a.n_grids, smem);
+    kernel<<<g, kConvThreads, smem, s>>>(a, vec4, lut_lds, rows_lds);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
 template <typename T>
 int launch_convolution_cells(const ConvDev& a, hipStream_t s) {
     const int64_t threads = a.n_grids * a.M;
@@ -620,6 +754,14 @@ int launch_convolution_cells(const ConvDev& a, hipStream_t s) {
     const unsigned gb = static_cast<unsigned>(blocks);
     const uintptr_t align = reinterpret_cast<uintptr_t>(a.in) | reinterpret_cast<uintptr_t>(a.out);
     const int vec4 = (sizeof(T) == 4 && a.E % 4 == 0 && align % 16 == 0) ? 1 : 0;
+    if (a.n_grids >= 64 && a.M <= 4096) {
+        // enough blocks to keep persistent workgroups busy
+        if (a.E <= 1) return launch_convolution_block<T, 1>(a, vec4, s);
+        if (a.E <= 2) return launch_convolution_block<T, 2>(a, vec4, s);
+        if (a.E <= 4) return launch_convolution_block<T, 4>(a, vec4, s);
+        if (a.E <= 8) return launch_convolution_block<T, 8>(a, vec4, s);
+        return launch_convolution_block<T, 16>(a, vec4, s);
+    }
     if (a.E <= 1) {
         convolution_cell_kernel<T, 1><<<gb, kBlock, 0, s>>>(a, vec4);
     } else if (a.E <= 2) {
