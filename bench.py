@@ -273,6 +273,42 @@ def bench_hash(torch, ash, workloads, args, dev):
     return ms_per_step, hits, kernels
 
 
+def bench_config1(torch, ash, workloads, dev, reps=5):
+    """Configuration 1 on the device (the configuration the CPU baseline also
+    runs at full size): HashSet, 1 M inserts with 50 % duplicates into
+    capacity 2 M, then 1 M finds; kernel times through the raw C ABI."""
+    w = workloads.hashset_uniform_keys(device=dev)
+    hs = ash.HashSet(3, 2_000_000, dev)
+    backend = hs.engine.backend
+    lib, handle = backend._lib, backend._handle
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    keys, queries = w["insert_keys"], w["query_keys"]
+    n_ins, n_q = keys.shape[0], queries.shape[0]
+    idx = torch.empty(n_q, dtype=torch.int64, device=dev)
+    msk = torch.empty(n_q, dtype=torch.bool, device=dev)
+    t_ins, t_find = EventTimer(torch), EventTimer(torch)
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        assert lib.ash_map_clear(handle, stream) == 0
+        run(t_ins, lambda: lib.ash_map_insert_keys(handle, keys.data_ptr(), n_ins, stream))
+        run(t_find, lambda: lib.ash_map_find(handle, queries.data_ptr(), n_q, idx.data_ptr(),
+                                             msk.data_ptr(), stream))
+    ms_i, ms_f = t_ins.mean_ms(), t_find.mean_ms()
+    unique = hs.size()
+    # 38 B per input key: 12 + 16 for every key, 16 + 4 more for the unique half
+    out = {
+        "insert_keys": roofline_entry("insert_kernel<3,keys> 1 M keys, 50 % duplicates",
+                                      28 * n_ins + 20 * unique, ms_i),
+        "find": roofline_entry("find_kernel<3> 1 M queries", FIND_BYTES * n_q, ms_f),
+        "unique_keys": unique,
+        "hits": int(msk.sum()),
+    }
+    out["insert_keys"]["Mkeys_per_s"] = round(n_ins / ms_i / 1e3, 1)
+    out["find"]["Mkeys_per_s"] = round(n_q / ms_f / 1e3, 1)
+    del hs, w
+    return out
+
+
 def bench_trilinear(torch, ash, workloads, args, dev):
     """Kernel figures of configurations 3 (E=16 forward) and 4 (E=4 forward,
     backward, double backward) plus the module-level autograd step of
@@ -558,6 +594,7 @@ def main():
     ms_per_step, hits, kernels = bench_hash(torch, ash, workloads, args, dev)
     if not args.no_trilinear:
         kernels.update(bench_trilinear(torch, ash, workloads, args, dev))
+    kernels["cfg1_hashset"] = bench_config1(torch, ash, workloads, dev)
     if not args.no_fusion:
         kernels["cfg5_fusion"] = bench_fusion(torch, ash, workloads, args, dev)
     dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
