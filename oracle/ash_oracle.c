@@ -697,7 +697,11 @@ void ash_oracle_ray_sample(const ash_oracle_map* m, const float* origins,
         float t = ray_near, t_near = ray_near;
         int64_t local = 0;
         const int64_t start = prefix ? (i == 0 ? 0 : prefix[i - 1]) : 0;
-        while (t < ray_far) {
+        int moving = 1;
+        /* stops as well when a step no longer advances t (range far beyond
+         * fp32 resolution), where the reference would not return */
+        while (t < ray_far && moving) {
+            const float before = t;
             int32_t block[3];
             for (int a = 0; a < 3; ++a) {
                 block[a] = (int32_t)floorf(fmaf(t, d[a], o[a]) * cell2grid);
@@ -714,6 +718,7 @@ void ash_oracle_ray_sample(const ash_oracle_map* m, const float* origins,
                 t_near = t;
                 ++local;
             }
+            moving = t > before;
         }
         if (counts) counts[i] = local;
     }

@@ -107,3 +107,23 @@ def test_grid_methods_follow_the_reference_wrappers(gpu_ash):
     # intervals that bridge a skipped gap
     assert float(masks.float().mean()) > 0.6
     assert math.isclose(float(tn.min()), float(near[hit].min()), rel_tol=0, abs_tol=grid.cell_size * 8)
+
+
+def test_ranges_beyond_fp32_resolution_end(gpu_ash, oracle):
+    """A sampling range so far out that a step no longer changes t must end
+    (the reference would not return); near/far refuses such a range."""
+    engine, omap, blocks, g = _scene(gpu_ash, oracle, n_blocks=500, seed=730)
+    backend = gpu_ash.grid.backend
+    o = torch.tensor([[10.0, 10.0, 10.0]] * 3)
+    d = torch.tensor([[1.0, 0.0, 0.0]] * 3)
+    lo, hi = torch.zeros(3), torch.full((3,), 512.0)
+    nears = torch.tensor([1.0e9, 0.0, 3.0e7])
+    fars = torch.tensor([2.0e9, 40.0, 3.0e7 + 64])
+    got = backend.ray_sample(engine.backend, o.to(DEV), d.to(DEV), nears.to(DEV), fars.to(DEV),
+                             lo.to(DEV), hi.to(DEV), 10**9, 8.0)
+    ref = oracle.ray_sample(omap, o, d, nears, fars, lo, hi, 10**9, 8.0)
+    for a, b in zip(got, ref):
+        assert torch.equal(a.cpu(), b)
+    with pytest.raises(RuntimeError, match="step is too small"):
+        backend.ray_find_near_far(engine.backend, o.to(DEV), d.to(DEV), lo.to(DEV), hi.to(DEV),
+                                  0.0, 1.0e12, 1.0, 8.0)

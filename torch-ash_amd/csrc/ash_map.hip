@@ -708,49 +708,59 @@ __device__ __forceinline__ void ray_block(const float (&o)[3], const float (&d)[
     }
 }
 
+// One wavefront per ray: the march of ray_find_near_far visits the parameters
+// t_0 = t_min, t_{k+1} = t_k + step regardless of what it finds, so lane l of
+// round r takes step 64 r + l (its t by the same chain of additions), the 64
+// lookups go out together, and the near / far recurrence is then replayed over
+// the hits in step order.  The march ends at the first step that is at or
+// beyond t_max or outside the box, exactly where the sequential loop stops.
 __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
         MapDev m, const float* __restrict__ origins,
         const float* __restrict__ directions, const float* __restrict__ bbox_min,
         const float* __restrict__ bbox_max, int64_t n, float t_min, float t_max,
         float grid2cell, float* __restrict__ nears, float* __restrict__ fars) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    const bool active = i < n;
+    const int lane = threadIdx.x & 63;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
+    if (i >= n) return;  // whole wavefronts leave together
     const float cell2grid = static_cast<float>(1.0 / grid2cell);
     const float t_grid_step = static_cast<float>(grid2cell * 0.5);
     float o[3], d[3], lo[3], hi[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-        o[a] = active ? origins[i * 3 + a] : 0.f;
-        d[a] = active ? directions[i * 3 + a] : 0.f;
+        o[a] = origins[i * 3 + a];
+        d[a] = directions[i * 3 + a];
         lo[a] = bbox_min[a];
         hi[a] = bbox_max[a];
     }
-    float near = -1.f, far = t_max, t = t_min;
-    bool live = active && t < t_max;
-    while (__ballot(live)) {
+    float t = t_min;
+    for (int j = 0; j < 63; ++j) {
+        if (j < lane) t += t_grid_step;
+    }
+    float near = -1.f, far = t_max;
+    for (;;) {
         int32_t block[3];
         float x[3];
         ray_block(o, d, t, cell2grid, block, x);
-        if (live) {
-            bool in_bound = true;
+        bool go = t < t_max;
 #pragma unroll
-            for (int a = 0; a < 3; ++a) {
-                in_bound = in_bound && x[a] >= lo[a] && x[a] <= hi[a];
-            }
-            if (!in_bound) live = false;
-        }
+        for (int a = 0; a < 3; ++a) go = go && x[a] >= lo[a] && x[a] <= hi[a];
+        const uint64_t stop = __ballot(!go);
+        const int first_stop = stop ? __builtin_ctzll(stop) : 64;
+        const bool active = lane < first_stop;
         int32_t idx;
-        const bool found = find_key<3>(m, block, live, idx);
-        if (live) {
-            if (found) {
-                near = near < 0.f ? t : fmaxf(near - t_grid_step, t_min);
-                far = fminf(t + t_grid_step, t_max);
-            }
-            t += t_grid_step;
-            live = t < t_max;
+        const bool found = find_key<3>(m, block, active, idx);
+        uint64_t hits = __ballot(found && active);
+        while (hits) {
+            const int l = __builtin_ctzll(hits);
+            const float t_hit = __shfl(t, l);
+            near = near < 0.f ? t_hit : fmaxf(near - t_grid_step, t_min);
+            far = fminf(t_hit + t_grid_step, t_max);
+            hits &= hits - 1;
         }
+        if (first_stop < 64) break;
+        for (int j = 0; j < 64; ++j) t += t_grid_step;
     }
-    if (active) {
+    if (lane == 0) {
         nears[i] = near;
         fars[i] = far;
     }
@@ -789,6 +799,7 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         int32_t idx;
         const bool found = find_key<3>(m, block, live, idx);
         if (live) {
+            const float before = t;
             if (!found) {
                 t += t_grid_step;
             } else {
@@ -801,7 +812,9 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
                 t_near = t;
                 ++local;
             }
-            live = t < ray_far;
+            // a step that no longer advances t (range far beyond fp32
+            // resolution) would never end; the reference has no such guard
+            live = t < ray_far && t > before;
         }
     }
     if (active && counts != nullptr) counts[i] = local;
@@ -1348,7 +1361,16 @@ int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
     }
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    ray_near_far_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+    // every step must advance t (else the march never ends), and their number
+    // must stay finite
+    const float half_block = static_cast<float>(grid2cell_multiplier * 0.5);
+    if (t_min < t_max) {
+        if (!(t_max + half_block > t_max) ||
+            !((static_cast<double>(t_max) - t_min) / half_block < 1e8)) {
+            ASH_FAIL("ray_find_near_far: the step is too small for this range");
+        }
+    }
+    ray_near_far_kernel<<<grid_for(n, kBlock / 64), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
             map->d, ray_origins, ray_directions, bbox_min, bbox_max, n, t_min,
             t_max, grid2cell_multiplier, ray_nears, ray_fars);
     ASH_LAUNCH_CHECK();
