@@ -218,7 +218,8 @@ def bench_hash(torch, ash, workloads, args, dev):
     workspace = torch.empty(max(ws_bytes.value, 256), dtype=torch.uint8, device=dev)
     t_bulk, t_bulk_keys = EventTimer(torch), EventTimer(torch)
 
-    t_clear, t_insert, t_insert_keys, t_find, t_items = (EventTimer(torch) for _ in range(5))
+    t_clear, t_insert, t_insert_keys, t_find, t_items, t_erase = (
+        EventTimer(torch) for _ in range(6))
     for it in range(args.warmup + args.steps):
         timed = it >= args.warmup
         run = (lambda timer, fn: timer(fn)) if timed else (lambda timer, fn: fn())
@@ -240,7 +241,9 @@ def bench_hash(torch, ash, workloads, args, dev):
             handle, queries.data_ptr(), n, idx_out.data_ptr(), mask_out.data_ptr(), stream)))
         run(t_items, lambda: check(lib.ash_map_items(
             handle, items_keys.data_ptr(), items_idx.data_ptr(), n, stream)))
+        run(t_erase, lambda: check(lib.ash_map_erase(handle, keys.data_ptr(), n, stream)))
     assert int(mask_out.sum()) == hits
+    assert backend.size() == 0
     slots = (backend._table.numel() - 256) // 128 * 10
     kernels = {
         "insert_values": roofline_entry(
@@ -249,6 +252,8 @@ def bench_hash(torch, ash, workloads, args, dev):
         "find": roofline_entry("find_kernel<3>", FIND_BYTES * n, t_find.mean_ms()),
         "items": roofline_entry("items_kernel<3>", items_bytes(slots, n), t_items.mean_ms()),
         "clear": roofline_entry("fill16+reset_heap", 16 * slots + 4 * args.capacity, t_clear.mean_ms()),
+        "erase": roofline_entry("erase_kernel<3> (every key stored)", INSERT_KEY_BYTES * n,
+                                t_erase.mean_ms()),
     }
     if bulk:
         chain = "split_keys_kernel<3> + split_records_kernel + build_kernel"
@@ -261,7 +266,7 @@ def bench_hash(torch, ash, workloads, args, dev):
             kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
             kernels[name]["workspace_bytes"] = ws_bytes.value
     kernels["api_insert_path"] = "insert_values_bulk" if api_uses_bulk else "insert_values"
-    for name in ("insert_values", "insert_keys", "find"):
+    for name in ("insert_values", "insert_keys", "find", "erase"):
         kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
     if n == 16_000_000 and args.capacity == 24_000_000:

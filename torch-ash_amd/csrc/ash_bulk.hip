@@ -73,13 +73,11 @@ inline int64_t align256(int64_t x) { return (x + 255) & ~int64_t{255}; }
 int64_t make_plan(const ash_map* map, int64_t n, int n_values,
                   const int64_t* row_bytes, char* ws, BulkPlan& pl) {
     if (n < kMinKeys || n_values < 0 || n_values > kMaxFusedValues) return 0;
-    int64_t row_dwords = 0;
     for (int v = 0; v < n_values; ++v) {
         if (row_bytes[v] <= 0 || row_bytes[v] % 4 != 0 ||
             row_bytes[v] > kMaxFusedRowDwords * 4) {
             return 0;
         }
-        row_dwords += row_bytes[v] / 4;
     }
     const int64_t nb = map->d.nb;
     const int64_t parts = (nb + kPartBuckets - 1) >> kPartShift;
@@ -132,7 +130,6 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
     pl.spill_keys = reinterpret_cast<int32_t*>(take(n * 4));
     pl.spill_a = reinterpret_cast<int32_t*>(take(n * 4));
     pl.spill_b = reinterpret_cast<int32_t*>(take(n * 4));
-    (void)row_dwords;
     return off;
 }
 
