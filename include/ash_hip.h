@@ -355,6 +355,46 @@ int ash_isosurface_extraction(const void* sdfs, const void* weights,
                               float iso_value, float weight_thr, int32_t dtype,
                               int32_t* counter, float* positions, void* stream);
 
+/* Replace `marching_cubes` (ash/src/grid.cu:606-946, pybind.cpp:31), which the
+ * reference runs as four launches around two host read-backs, by two calls
+ * around one read-back.  Tables and fields as for ash_isosurface_extraction.
+ *
+ * classify: a listed cell takes part when it and the seven cells at its other
+ * corners (entries 1..7 of the 8-entry neighbour tables) exist and weigh at
+ * least weight_thr.  cases uint8[num_embeddings * cells_per_grid] receives its
+ * case (bit c set when corner c is below iso_value; 0 = no surface) and
+ * edge_slots uint32[num_embeddings * cells_per_grid] the flags of the +x/+y/+z
+ * edges that carry a vertex; both need no initialisation, the entries of the
+ * listed rows are cleared here, and every row that the neighbour table reaches
+ * from a listed row must be listed too.  counters int32[4] (device):
+ * [0] = triangles, [1] = vertices, [2], [3] = cursors of extract.
+ *
+ * extract: after the caller has read counters[0..1] and allocated positions
+ * fp32[n_vertices, 3] (cell units) and triangles int32[n_triangles, 3] (vertex
+ * ids, normals pointing from below iso_value to above it).  Vertex and triangle
+ * order follow the order in which workgroups finish, as in the reference.
+ * At most 2^29 - 1 vertices. */
+int ash_marching_cubes_classify(const void* sdfs, const void* weights,
+                                const int64_t* grid_indices,
+                                const int64_t* lut_grid_nb2grid_idx,
+                                const int64_t* lut_cell_nb2cell_idx,
+                                const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                                int64_t num_embeddings, int64_t cells_per_grid,
+                                float iso_value, float weight_thr, int32_t dtype,
+                                uint8_t* cases, uint32_t* edge_slots, int32_t* counters,
+                                void* stream);
+int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
+                               const int32_t* grid_coords_table,
+                               const int64_t* lut_grid_nb2grid_idx,
+                               const int32_t* cell_coords_table,
+                               const int64_t* lut_cell_nb2cell_idx,
+                               const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                               int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
+                               float iso_value, int32_t dtype, const uint8_t* cases,
+                               uint32_t* edge_slots, int32_t* counters, int64_t n_vertices,
+                               int64_t n_triangles, float* positions, int32_t* triangles,
+                               void* stream);
+
 /* -------------------------------------------------------------- diagnostics */
 
 /* Measures the device's random-access ceilings that bound the table kernels

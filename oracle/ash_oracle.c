@@ -604,6 +604,98 @@ DEFINE_QUERY(double, f64)
 ASH_ORACLE_ISOSURFACE(ash_oracle_isosurface_f32, float)
 ASH_ORACLE_ISOSURFACE(ash_oracle_isosurface_f64, double)
 
+/* ---------------------------------------------------------- marching cubes
+ * ash/src/grid.cu:606-946 in launch order: case per cell and placeholders on
+ * the owning cells of crossed edges (:606-703), vertex ids and positions
+ * (:705-774), triangles (:776-842).  Corner c of a cell is entry c of the
+ * 8-entry neighbour tables and bit c of the case (the reference reaches the
+ * same cells through its own corner numbering, grid.cu:646-666); edge
+ * e = 4 * axis + j starts at the corner made by inserting a zero bit at
+ * position `axis` into j.  `table` holds, per case, up to five triangles as
+ * edge triples in output order, -1 padded to 16.  `case_ws` int32[B * M] and
+ * `edge_ws` int32[B * M * 3] are work arrays.  positions / triangles may be
+ * NULL to count only; counts[0] = vertices, counts[1] = triangles. */
+static int mc_low_corner(int e) {
+    const int axis = e >> 2, j = e & 3;
+    return (j & ((1 << axis) - 1)) | ((j >> axis) << (axis + 1));
+}
+
+#define ASH_ORACLE_MARCHING_CUBES(NAME, T)                                     \
+    void NAME(const T* sdfs, const T* weights, const int64_t* grid_indices,    \
+              const int32_t* grid_coords, const int64_t* lut_g,                \
+              const int32_t* cell_coords, const int64_t* lut_c2c,              \
+              const int64_t* lut_c2g, int64_t n_grids, int64_t B, int64_t M,   \
+              int g, float iso, float weight_thr, const int8_t* table,         \
+              int32_t* case_ws, int32_t* edge_ws, int64_t* counts,             \
+              float* positions, int32_t* triangles) {                          \
+        memset(case_ws, 0, sizeof(int32_t) * (size_t)(B * M));                 \
+        memset(edge_ws, 0, sizeof(int32_t) * (size_t)(B * M * 3));             \
+        for (int64_t i = 0; i < n_grids * M; ++i) {                            \
+            const int64_t gi = grid_indices[i / M];                            \
+            const int64_t c = i % M;                                           \
+            if (weights[gi * M + c] < weight_thr) continue;                    \
+            int code = 0, valid = 1;                                           \
+            int64_t at[8];                                                     \
+            for (int k = 0; k < 8 && valid; ++k) {                             \
+                const int64_t ng = lut_g[gi * 8 + lut_c2g[c * 8 + k]];         \
+                if (ng == -1) { valid = 0; break; }                            \
+                at[k] = ng * M + lut_c2c[c * 8 + k];                           \
+                if (weights[at[k]] < weight_thr) { valid = 0; break; }         \
+                code |= ((sdfs[at[k]] - iso) < 0) << k;                        \
+            }                                                                  \
+            if (!valid || code == 0 || code == 255) continue;                  \
+            case_ws[gi * M + c] = code;                                        \
+            for (int e = 0; e < 12; ++e) {                                     \
+                const int lo = mc_low_corner(e), hi = lo | (1 << (e >> 2));    \
+                if (((code >> lo) ^ (code >> hi)) & 1) {                       \
+                    edge_ws[at[lo] * 3 + (e >> 2)] = -1;                       \
+                }                                                              \
+            }                                                                  \
+        }                                                                      \
+        int64_t nv = 0, nt = 0;                                                \
+        for (int64_t i = 0; i < n_grids * M; ++i) {                            \
+            const int64_t gi = grid_indices[i / M];                            \
+            const int64_t c = i % M;                                           \
+            const T self = sdfs[gi * M + c] - iso;                             \
+            for (int d = 0; d < 3; ++d) {                                      \
+                if (edge_ws[(gi * M + c) * 3 + d] != -1) continue;             \
+                const int64_t ng = lut_g[gi * 8 + lut_c2g[c * 8 + (1 << d)]];  \
+                const int64_t nc = lut_c2c[c * 8 + (1 << d)];                  \
+                const T other = sdfs[ng * M + nc] - iso;                       \
+                if (positions) {                                               \
+                    const float ratio = (float)(self / (self - other));        \
+                    for (int a = 0; a < 3; ++a) {                              \
+                        positions[nv * 3 + a] =                                \
+                                (float)(grid_coords[gi * 3 + a] * g +          \
+                                        cell_coords[c * 3 + a]) +              \
+                                (a == d ? ratio : 0.f);                        \
+                    }                                                          \
+                }                                                              \
+                edge_ws[(gi * M + c) * 3 + d] = (int32_t)nv++;                 \
+            }                                                                  \
+        }                                                                      \
+        for (int64_t i = 0; i < n_grids * M; ++i) {                            \
+            const int64_t gi = grid_indices[i / M];                            \
+            const int64_t c = i % M;                                           \
+            const int code = case_ws[gi * M + c];                              \
+            if (code == 0) continue;                                           \
+            for (int t = 0; t < 15 && table[code * 16 + t] != -1; t += 3) {    \
+                for (int v = 0; v < 3 && triangles; ++v) {                     \
+                    const int e = table[code * 16 + t + v];                    \
+                    const int lo = mc_low_corner(e);                           \
+                    const int64_t ng = lut_g[gi * 8 + lut_c2g[c * 8 + lo]];    \
+                    const int64_t nc = lut_c2c[c * 8 + lo];                    \
+                    triangles[nt * 3 + v] = edge_ws[(ng * M + nc) * 3 + (e >> 2)]; \
+                }                                                              \
+                ++nt;                                                          \
+            }                                                                  \
+        }                                                                      \
+        counts[0] = nv;                                                        \
+        counts[1] = nt;                                                        \
+    }
+ASH_ORACLE_MARCHING_CUBES(ash_oracle_marching_cubes_f32, float)
+ASH_ORACLE_MARCHING_CUBES(ash_oracle_marching_cubes_f64, double)
+
 /* ----------------------------------------------------------- convolution
  * ash/src/grid.cu:951-1006: taps accumulated in table order, one fused
  * multiply-add per tap and channel (nvcc's contraction of `sum += in * w`). */

@@ -56,6 +56,9 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
         iso = getattr(lib, f"ash_oracle_isosurface_{sfx}")
         iso.restype = _I64
         iso.argtypes = [_PTR] * 8 + [_I64, _I64, ctypes.c_int, ctypes.c_float, ctypes.c_float, _PTR]
+        getattr(lib, f"ash_oracle_marching_cubes_{sfx}").argtypes = (
+            [_PTR] * 8 + [_I64] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_float] + [_PTR] * 6
+        )
     lib.ash_oracle_ray_find_near_far.argtypes = (
         [_PTR] * 5 + [_I64, ctypes.c_float, ctypes.c_float, ctypes.c_float, _PTR, _PTR]
     )
@@ -75,6 +78,24 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
             [_PTR] * 12 + [_I64, _I64, _I64, _I64, ctypes.c_int]
         )
     return lib
+
+
+_MC_TABLE = None
+
+
+def _mc_table():
+    """The 256 x 16 case table of the library's generator script."""
+    global _MC_TABLE
+    if _MC_TABLE is None:
+        import importlib.util
+
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), os.pardir,
+                            "torch-ash_amd", "csrc", "gen_mc_table.py")
+        spec = importlib.util.spec_from_file_location("gen_mc_table", path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        _MC_TABLE = mod.build_table()
+    return _MC_TABLE
 
 
 def _cpu(t: torch.Tensor, dtype=None) -> torch.Tensor:
@@ -121,6 +142,35 @@ class OracleBackend:
         if count:
             fn(*args, positions.data_ptr())
         return positions
+
+    # -- marching cubes (ash/src/pybind.cpp:31) -------------------------------
+    def marching_cubes(self, sdfs, weights, grid_indices, grid_coords_table,
+                       lut_grid_nb2grid_idx, cell_coords_table, lut_cell_nb2cell_idx,
+                       lut_cell_nb2grid_nb, grid_dim, iso_value, weight_thr):
+        """(triangles int32 (T, 3), vertices float32 (V, 3)), cells in launch
+        order.  The case table comes from the library's generator, whose
+        output the tests pin on their own."""
+        x = _cpu(sdfs)
+        b, m = x.shape[0], x.shape[1]
+        x = x.reshape(b, m).contiguous()
+        held = [x, _cpu(weights, x.dtype).reshape(b, m).contiguous(),
+                _cpu(grid_indices, torch.int64).view(-1), _cpu(grid_coords_table, torch.int32),
+                _cpu(lut_grid_nb2grid_idx, torch.int64), _cpu(cell_coords_table, torch.int32),
+                _cpu(lut_cell_nb2cell_idx, torch.int64), _cpu(lut_cell_nb2grid_nb, torch.int64)]
+        table = torch.tensor(_mc_table(), dtype=torch.int8).contiguous()
+        case_ws = torch.empty(b * m, dtype=torch.int32)
+        edge_ws = torch.empty(b * m * 3, dtype=torch.int32)
+        counts = torch.zeros(2, dtype=torch.int64)
+        fn = getattr(self.lib, f"ash_oracle_marching_cubes_{_SUFFIX[x.dtype]}")
+        args = [t.data_ptr() for t in held] + [
+            held[2].numel(), b, m, int(grid_dim), float(iso_value), float(weight_thr),
+            table.data_ptr(), case_ws.data_ptr(), edge_ws.data_ptr(), counts.data_ptr()]
+        fn(*args, None, None)
+        vertices = torch.zeros((int(counts[0]), 3), dtype=torch.float32)
+        triangles = torch.zeros((int(counts[1]), 3), dtype=torch.int32)
+        if int(counts[0]):
+            fn(*args, vertices.data_ptr(), triangles.data_ptr())
+        return triangles, vertices
 
     # -- sparse convolution (ash/src/pybind.cpp:33) ---------------------------
     def convolution_forward(self, inputs, weights, masks, grid_indices, cell_indices,

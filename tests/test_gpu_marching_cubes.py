@@ -1,0 +1,121 @@
+"""GPU parity tests of marching cubes (ash_marching_cubes_classify / _extract)
+against the oracle.  Vertex and triangle numbering follow the scheduling on
+both sides, so meshes are compared as sets: the vertex positions bit for bit,
+and the triangles as triples of positions in the smallest of their three
+rotations (which keeps the orientation)."""
+import numpy as np
+import pytest
+import torch
+
+import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def _sorted_rows(x):
+    x = x.detach().cpu().numpy()
+    return x[np.lexsort(x.T[::-1])]
+
+
+def _lex_min(a, b):
+    """Row-wise lexicographic minimum of two (T, 9) arrays."""
+    differ = a != b
+    first = differ.argmax(axis=1)
+    rows = np.arange(len(a))
+    take_b = differ.any(axis=1) & (b[rows, first] < a[rows, first])
+    return np.where(take_b[:, None], b, a)
+
+
+def _triangle_set(tri, pts):
+    """(T, 9) float32: corner positions of every triangle in the smallest of
+    its three rotations (which keeps the orientation), rows sorted."""
+    p = pts.detach().cpu()[tri.detach().cpu().long()].numpy()      # (T, 3, 3)
+    rot = [np.concatenate([p[:, k:], p[:, :k]], axis=1).reshape(-1, 9) for k in range(3)]
+    return _sorted_rows(torch.from_numpy(_lex_min(_lex_min(rot[0], rot[1]), rot[2])))
+
+
+def _scene(gpu_ash, dtype, seed):
+    grid, radii, centres = workloads.build_grid(gpu_ash, 3000, 1, 8, 64, device=DEV)
+    keys, idx = grid.engine.items()
+    cells = keys.view(-1, 1, 3) * 8 + grid.cell_coords.view(1, -1, 3)
+    world = grid.transform_cell_to_world(cells.float())  # (n, M, 3)
+    dist = (world.unsqueeze(2) - centres.to(DEV).view(1, 1, -1, 3)).norm(dim=-1) - radii.to(DEV)
+    sdf = torch.zeros(grid.embeddings.shape[:2], dtype=dtype, device=DEV)
+    sdf[idx] = dist.min(dim=2)[0].to(dtype)
+    g = torch.Generator().manual_seed(seed)
+    weights = torch.zeros_like(sdf)
+    weights[idx] = (torch.rand(len(idx), 512, generator=g) * 8).to(DEV, dtype)
+    return grid, idx, sdf, weights
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("iso,thr", [(0.0, 1.0), (0.004, 0.25)])
+def test_mesh_matches_oracle(gpu_ash, oracle, dtype, iso, thr):
+    grid, idx, sdf, weights = _scene(gpu_ash, dtype, 840)
+    args = (idx, grid.grid_coords, grid.lut_grid_nb2grid_idx, grid.cell_coords,
+            grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, 8, iso, thr)
+    tri, pts = gpu_ash.grid.backend.marching_cubes(sdf, weights, *args)
+    tri_ref, pts_ref = oracle.marching_cubes(sdf, weights, *args)
+    assert tri.dtype == torch.int32 and pts.dtype == torch.float32
+    assert pts.shape == pts_ref.shape and tri.shape == tri_ref.shape and len(tri_ref) > 5000
+    assert int(tri.min()) == 0 and int(tri.max()) == len(pts) - 1
+    assert np.array_equal(_sorted_rows(pts), _sorted_rows(pts_ref))
+    assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))
+    # a second extraction on the same inputs gives the same mesh
+    tri2, pts2 = gpu_ash.grid.backend.marching_cubes(sdf, weights, *args)
+    assert np.array_equal(_triangle_set(tri2, pts2), _triangle_set(tri_ref, pts_ref))
+
+
+def test_random_field_matches_oracle(gpu_ash, oracle):
+    """Every case of the table, on a field without structure."""
+    grid, idx, sdf, weights = _scene(gpu_ash, torch.float32, 841)
+    g = torch.Generator().manual_seed(842)
+    sdf[idx] = (torch.rand(len(idx), 512, generator=g) - 0.5).to(DEV)
+    # a part of the blocks only: the rows that the neighbour table reaches from
+    # a listed row must be listed as well, so take the closure of a fifth
+    closure = idx[: len(idx) // 5]
+    while True:
+        lut = grid.lut_grid_nb2grid_idx[closure].view(-1)
+        grown = torch.unique(torch.cat([closure, lut[lut >= 0]]))
+        if len(grown) == len(closure):
+            break
+        closure = grown
+    args = (closure, grid.grid_coords, grid.lut_grid_nb2grid_idx, grid.cell_coords,
+            grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, 8, 0.0, 0.5)
+    tri, pts = gpu_ash.grid.backend.marching_cubes(sdf, weights, *args)
+    tri_ref, pts_ref = oracle.marching_cubes(sdf, weights, *args)
+    assert len(tri_ref) > 100_000 and tri.shape == tri_ref.shape
+    assert np.array_equal(_sorted_rows(pts), _sorted_rows(pts_ref))
+    assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))
+
+
+def test_sphere_mesh_through_the_grid_method(gpu_ash):
+    """One large sphere well inside a dense set of blocks, at full device
+    size: closed, oriented, Euler characteristic 2, the sphere's volume."""
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, 20 ** 3, 1, grid_dim=8, sparse_grid_dim=20, bbox_min=torch.zeros(3),
+        bbox_max=torch.ones(3), device=DEV)
+    grid.dense_init_()
+    keys, idx = grid.engine.items()
+    cells = (keys.view(-1, 1, 3) * 8 + grid.cell_coords.view(1, -1, 3)).float()
+    centre, radius = torch.tensor([80.3, 79.1, 81.7], device=DEV), 61.4
+    sdf = torch.zeros(grid.embeddings.shape[:2], device=DEV)
+    sdf[idx] = (cells - centre).norm(dim=-1) - radius
+    tri, pts = grid.surface_mesh(sdf, torch.ones_like(sdf))
+    assert len(tri) > 100_000
+    v, f = len(pts), len(tri)
+    t = tri.long()
+    edges = torch.cat([t[:, [0, 1]], t[:, [1, 2]], t[:, [2, 0]]])
+    code = edges[:, 0] * v + edges[:, 1]
+    assert len(torch.unique(code)) == len(code)                       # each directed edge once
+    back = edges[:, 1] * v + edges[:, 0]
+    assert torch.equal(torch.sort(code)[0], torch.sort(back)[0])      # and its reverse once
+    assert v - len(code) // 2 + f == 2
+    p = pts.double()[t] / grid.cell_size
+    vol = float((p[:, 0] * torch.cross(p[:, 1], p[:, 2], dim=1)).sum() / 6)
+    assert abs(vol / (4 / 3 * np.pi * radius ** 3) - 1) < 2e-3
+    out = grid.marching_cubes(sdf, torch.ones_like(sdf), None, normal_fn=lambda x: x * 0 + 1.0)
+    if isinstance(out, dict):
+        assert out["triangles"].shape == tri.shape and out["normals"].shape == pts.shape
+    assert grid.marching_cubes(sdf, torch.zeros_like(sdf), None, None) is None

@@ -208,8 +208,6 @@ def test_unbounded_grid_bbox_and_sampling(cpu_ash):
     pts = grid.uniform_sample(500)
     feats, masks = grid(pts, "linear")
     assert masks.all() and feats.shape == (500, 2)
-    with pytest.raises(NotImplementedError):
-        grid.marching_cubes(None, None)  # the triangle mesh is not provided
 
 
 @pytest.mark.parametrize("embedding_dim,grid_dim", [(2, 1), (1, 2), (4, 4)])

@@ -148,6 +148,15 @@ _SIGNATURES = {
         ctypes.c_int,
         [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR],
     ),
+    "ash_marching_cubes_classify": (
+        ctypes.c_int,
+        [_PTR] * 6 + [_I64] * 3 + [ctypes.c_float, ctypes.c_float, ctypes.c_int32] + [_PTR] * 4,
+    ),
+    "ash_marching_cubes_extract": (
+        ctypes.c_int,
+        [_PTR] * 7 + [_I64] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_int32]
+        + [_PTR] * 3 + [_I64] * 2 + [_PTR] * 3,
+    ),
     "ash_query_forward": (ctypes.c_int, [ctypes.POINTER(_QueryArgs), _PTR, _PTR]),
     "ash_query_backward_forward": (
         ctypes.c_int,
@@ -257,6 +266,61 @@ class _Backend:
         if positions.shape[0]:
             launch(positions)
         return positions
+
+    # -- marching cubes (ash/src/pybind.cpp:31) ------------------------------
+    def marching_cubes(
+        self, sdfs, weights, grid_indices, grid_coords_table, lut_grid_nb2grid_idx,
+        cell_coords_table, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, grid_dim, iso_value,
+        weight_thr,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Triangle mesh of the surface `sdfs == iso_value` over the listed
+        blocks: (triangles int32 (T, 3), vertices float32 (V, 3) in cell units).
+        A cell contributes when its eight corners exist and weigh at least
+        `weight_thr`.  Vertex and triangle order vary from run to run."""
+        _require_hip(sdfs, "sdfs")
+        dev = sdfs.device
+        if sdfs.dtype not in _DTYPE:
+            raise RuntimeError("sdfs must be float32 or float64")
+        b, m = sdfs.shape[0], sdfs.shape[1]
+        sdfs = sdfs.reshape(b, m).contiguous()
+        weights = weights.to(dev, sdfs.dtype).reshape(b, m).contiguous()
+        gi = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
+        gc = grid_coords_table.to(dev, torch.int32).contiguous()
+        cc = cell_coords_table.to(dev, torch.int32).contiguous()
+        lut_g = lut_grid_nb2grid_idx.to(dev, torch.int64).contiguous()
+        lut_c2c = lut_cell_nb2cell_idx.to(dev, torch.int64).contiguous()
+        lut_c2g = lut_cell_nb2grid_nb.to(dev, torch.int64).contiguous()
+        if gc.shape != (b, 3) or cc.shape != (m, 3) or lut_g.shape != (b, 8):
+            raise RuntimeError("coordinate / neighbour tables do not match the grid")
+        if lut_c2c.shape != (m, 8) or lut_c2g.shape != (m, 8):
+            raise RuntimeError("cell neighbour tables must be (cells_per_grid, 8)")
+        cases = torch.empty(b * m, dtype=torch.uint8, device=dev)
+        slots = torch.empty(b * m, dtype=torch.int32, device=dev)
+        counters = torch.zeros(4, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_marching_cubes_classify(
+                    sdfs.data_ptr(), weights.data_ptr(), gi.data_ptr(), lut_g.data_ptr(),
+                    lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
+                    float(iso_value), float(weight_thr), _DTYPE[sdfs.dtype],
+                    cases.data_ptr(), slots.data_ptr(), counters.data_ptr(), _stream_of(dev),
+                )
+            )
+            n_triangles, n_vertices = counters[:2].tolist()
+            triangles = torch.empty((n_triangles, 3), dtype=torch.int32, device=dev)
+            vertices = torch.empty((n_vertices, 3), dtype=torch.float32, device=dev)
+            if n_vertices:
+                self.check(
+                    self.lib.ash_marching_cubes_extract(
+                        sdfs.data_ptr(), gi.data_ptr(), gc.data_ptr(), lut_g.data_ptr(),
+                        cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
+                        int(grid_dim), float(iso_value), _DTYPE[sdfs.dtype], cases.data_ptr(),
+                        slots.data_ptr(), counters.data_ptr(), n_vertices, n_triangles,
+                        vertices.data_ptr(), triangles.data_ptr() if n_triangles else None,
+                        _stream_of(dev),
+                    )
+                )
+        return triangles, vertices
 
     # -- sparse convolution (ash/src/pybind.cpp:33) -------------------------
     def convolution_forward(

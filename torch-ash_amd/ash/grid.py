@@ -442,21 +442,52 @@ class SparseDenseGrid(ASHModule):
         )
         return self.transform_cell_to_world(vertices)
 
+    def surface_mesh(
+        self, tsdfs: torch.Tensor, weights: torch.Tensor, iso_value: float = 0.0,
+        weight_thr: float = 1.0,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """Marching cubes over the active blocks: (triangles int32 (T, 3), world
+        positions (V, 3)) -- the mesh branch of the reference's `marching_cubes`
+        (ash/grid.py:680-711) without its open3d packaging.  A cell contributes
+        when all eight of its corners exist and weigh at least `weight_thr`;
+        triangle normals point towards larger `tsdfs`."""
+        if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
+            self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+        _, grid_indices = self.engine.items()
+        triangles, vertices = backend.marching_cubes(
+            tsdfs,
+            weights,
+            grid_indices,
+            self.grid_coords,
+            self.lut_grid_nb2grid_idx,
+            self.cell_coords,
+            self.lut_cell_nb2cell_idx,
+            self.lut_cell_nb2grid_nb,
+            self.grid_dim,
+            iso_value,
+            weight_thr,
+        )
+        return triangles, self.transform_cell_to_world(vertices)
+
     def marching_cubes(
         self, tsdfs, weights, color_fn=None, normal_fn=None, iso_value: float = 0.0,
         weight_thr: float = 1.0, vertices_only: bool = False,
     ):
-        """Surface extraction (ash/grid.py:628-711).  Only `vertices_only=True`
-        is provided: it returns an open3d point cloud like the reference when
-        open3d is importable, otherwise a dict of tensors with the same fields
-        (positions, colors, normals); None when there are no points.  The
-        triangle mesh needs the marching-cubes case tables and is not built."""
-        if not vertices_only:
-            raise NotImplementedError("marching_cubes triangles are not provided by this build")
-        positions = self.isosurface_points(tsdfs, weights, iso_value, weight_thr)
+        """Surface extraction (ash/grid.py:628-711): a point cloud of the edge
+        crossings (`vertices_only=True`) or a triangle mesh.  Returns the open3d
+        geometry of the reference when open3d is importable, otherwise a dict of
+        tensors with the same fields (positions, [triangles,] colors, normals);
+        None when there are no points."""
+        triangles = None
+        if vertices_only:
+            positions = self.isosurface_points(tsdfs, weights, iso_value, weight_thr)
+        else:
+            triangles, positions = self.surface_mesh(tsdfs, weights, iso_value, weight_thr)
         if len(positions) == 0:
             return None
         fields = {"positions": positions}
+        if triangles is not None:
+            fields["triangles"] = triangles
         if color_fn is not None:
             fields["colors"] = color_fn(positions)
         if normal_fn is not None:
@@ -465,11 +496,18 @@ class SparseDenseGrid(ASHModule):
             import open3d as o3d
         except ImportError:
             return fields
-        pcd = o3d.t.geometry.PointCloud(positions.detach().cpu().numpy())
+        if triangles is None:
+            geometry = o3d.t.geometry.PointCloud(positions.detach().cpu().numpy())
+            attributes = geometry.point
+        else:
+            geometry = o3d.t.geometry.TriangleMesh(
+                positions.detach().cpu().numpy(), triangles.detach().cpu().numpy()
+            )
+            attributes = geometry.vertex
         for name in ("colors", "normals"):
             if name in fields:
-                pcd.point[name] = fields[name].detach().cpu().numpy()
-        return pcd
+                attributes[name] = fields[name].detach().cpu().numpy()
+        return geometry
 
     # ------------------------------------------------------ neighbour tables
     @torch.no_grad()
