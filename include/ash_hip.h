@@ -366,22 +366,25 @@ int ash_isosurface_extraction(const void* sdfs, const void* weights,
  * edge_slots uint32[num_embeddings * cells_per_grid] the flags of the +x/+y/+z
  * edges that carry a vertex; both need no initialisation, the entries of the
  * listed rows are cleared here, and every row that the neighbour table reaches
- * from a listed row must be listed too.  counters int32[4] (device):
- * [0] = triangles, [1] = vertices, [2], [3] = cursors of extract.
+ * from a listed row must be listed too.  workspace (device int32, as many as
+ * ash_marching_cubes_workspace_ints returns, no initialisation): [0] =
+ * triangles, [1] = vertices, the rest is carried to extract.
  *
- * extract: after the caller has read counters[0..1] and allocated positions
+ * extract: after the caller has read workspace[0..1] and allocated positions
  * fp32[n_vertices, 3] (cell units) and triangles int32[n_triangles, 3] (vertex
- * ids, normals pointing from below iso_value to above it).  Vertex and triangle
- * order follow the order in which workgroups finish, as in the reference.
- * At most 2^29 - 1 vertices. */
+ * ids, normals pointing from below iso_value to above it).  Vertices and
+ * triangles come in the order of the listing, the same on every run.  May be
+ * repeated after one classify.  At most 2^29 - 1 vertices. */
+int64_t ash_marching_cubes_workspace_ints(int64_t num_grids, int64_t cells_per_grid);
 int ash_marching_cubes_classify(const void* sdfs, const void* weights,
                                 const int64_t* grid_indices,
                                 const int64_t* lut_grid_nb2grid_idx,
+                                const int32_t* cell_coords_table,
                                 const int64_t* lut_cell_nb2cell_idx,
                                 const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
-                                int64_t num_embeddings, int64_t cells_per_grid,
+                                int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
                                 float iso_value, float weight_thr, int32_t dtype,
-                                uint8_t* cases, uint32_t* edge_slots, int32_t* counters,
+                                uint8_t* cases, uint32_t* edge_slots, int32_t* workspace,
                                 void* stream);
 int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
                                const int32_t* grid_coords_table,
@@ -391,7 +394,7 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
                                const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
                                int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
                                float iso_value, int32_t dtype, const uint8_t* cases,
-                               uint32_t* edge_slots, int32_t* counters, int64_t n_vertices,
+                               uint32_t* edge_slots, int32_t* workspace, int64_t n_vertices,
                                int64_t n_triangles, float* positions, int32_t* triangles,
                                void* stream);
 

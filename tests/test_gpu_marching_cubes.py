@@ -119,3 +119,30 @@ def test_sphere_mesh_through_the_grid_method(gpu_ash):
     if isinstance(out, dict):
         assert out["triangles"].shape == tri.shape and out["normals"].shape == pts.shape
     assert grid.marching_cubes(sdf, torch.zeros_like(sdf), None, None) is None
+
+
+@pytest.mark.parametrize("grid_dim", [1, 2, 3, 5, 16, 20])
+def test_block_sizes_match_oracle(gpu_ash, oracle, grid_dim):
+    """Block edges from one cell (every corner in another block) over sizes whose
+    cell count is no multiple of the kernels' chunking to edges beyond the
+    LDS-tiled path, with missing blocks and light cells."""
+    s = max(3, min(12, 40 // grid_dim))
+    g = torch.Generator().manual_seed(850 + grid_dim)
+    blocks = torch.stack(torch.meshgrid(*[torch.arange(s)] * 3, indexing="ij"), -1).view(-1, 3)
+    blocks = blocks[torch.rand(len(blocks), generator=g) < 0.85]
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, len(blocks) + 7, 1, grid_dim=grid_dim, sparse_grid_dim=s, bbox_min=torch.zeros(3),
+        bbox_max=torch.ones(3), device=DEV)
+    grid.engine.insert_keys(blocks.int().to(DEV))
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    _, idx = grid.engine.items()
+    shape = grid.embeddings.shape[:2]
+    sdf = (torch.rand(shape, generator=g) - 0.45).to(DEV)
+    weights = (torch.rand(shape, generator=g) * 10).to(DEV)
+    args = (idx, grid.grid_coords, grid.lut_grid_nb2grid_idx, grid.cell_coords,
+            grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, grid_dim, 0.02, 0.4)
+    tri, pts = gpu_ash.grid.backend.marching_cubes(sdf, weights, *args)
+    tri_ref, pts_ref = oracle.marching_cubes(sdf, weights, *args)
+    assert len(tri_ref) > 300 and tri.shape == tri_ref.shape and pts.shape == pts_ref.shape
+    assert np.array_equal(_sorted_rows(pts), _sorted_rows(pts_ref))
+    assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))

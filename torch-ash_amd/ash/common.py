@@ -148,9 +148,11 @@ _SIGNATURES = {
         ctypes.c_int,
         [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR],
     ),
+    "ash_marching_cubes_workspace_ints": (ctypes.c_int64, [_I64, _I64]),
     "ash_marching_cubes_classify": (
         ctypes.c_int,
-        [_PTR] * 6 + [_I64] * 3 + [ctypes.c_float, ctypes.c_float, ctypes.c_int32] + [_PTR] * 4,
+        [_PTR] * 7 + [_I64] * 3
+        + [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int32] + [_PTR] * 4,
     ),
     "ash_marching_cubes_extract": (
         ctypes.c_int,
@@ -276,7 +278,7 @@ class _Backend:
         """Triangle mesh of the surface `sdfs == iso_value` over the listed
         blocks: (triangles int32 (T, 3), vertices float32 (V, 3) in cell units).
         A cell contributes when its eight corners exist and weigh at least
-        `weight_thr`.  Vertex and triangle order vary from run to run."""
+        `weight_thr`.  Vertices and triangles follow the order of `grid_indices`."""
         _require_hip(sdfs, "sdfs")
         dev = sdfs.device
         if sdfs.dtype not in _DTYPE:
@@ -296,13 +298,15 @@ class _Backend:
             raise RuntimeError("cell neighbour tables must be (cells_per_grid, 8)")
         cases = torch.empty(b * m, dtype=torch.uint8, device=dev)
         slots = torch.empty(b * m, dtype=torch.int32, device=dev)
-        counters = torch.zeros(4, dtype=torch.int32, device=dev)
+        counters = torch.empty(
+            self.lib.ash_marching_cubes_workspace_ints(gi.numel(), m), dtype=torch.int32, device=dev
+        )
         with torch.cuda.device(dev):
             self.check(
                 self.lib.ash_marching_cubes_classify(
                     sdfs.data_ptr(), weights.data_ptr(), gi.data_ptr(), lut_g.data_ptr(),
-                    lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
-                    float(iso_value), float(weight_thr), _DTYPE[sdfs.dtype],
+                    cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
+                    int(grid_dim), float(iso_value), float(weight_thr), _DTYPE[sdfs.dtype],
                     cases.data_ptr(), slots.data_ptr(), counters.data_ptr(), _stream_of(dev),
                 )
             )

@@ -205,6 +205,13 @@ def header_text() -> str:
         lines.append("    " + ", ".join(str(v) for v in counts[i : i + 32]) + ",")
     lines.append("};")
     lines.append("")
+    lines.append("// The rows again, four bits per entry (15 = none), entry i in bits 4i..4i+3.")
+    lines.append("__device__ const uint64_t kMcPackedRows[256] = {")
+    packed = [sum(((v if v >= 0 else 15) << (4 * i)) for i, v in enumerate(row)) for row in table]
+    for i in range(0, 256, 4):
+        lines.append("    " + ", ".join(f"0x{v:016x}ull" for v in packed[i : i + 4]) + ",")
+    lines.append("};")
+    lines.append("")
     lines.append("}  // namespace ash")
     return "\n".join(lines) + "\n"
 
