@@ -334,30 +334,47 @@ int ash_convolution_forward(const void* inputs, const void* weights,
                             int64_t num_cell_nbs, int64_t num_grid_nbs,
                             int32_t dtype, void* stream);
 
-/* Replaces one launch of `isosurface_extraction` (ash/src/grid.cu:453-602,
- * pybind.cpp:30), which the reference runs twice: to count, then to fill.
- * sdfs / weights scalar[num_embeddings, cells_per_grid]; grid_indices
- * int64[num_grids]; grid_coords_table int32[num_embeddings, 3]; cell_coords_table
- * int32[cells_per_grid, 3]; the three 8-entry neighbour tables of the queries.
- * `counter` (device int32) is reset and receives the number of surface points;
- * with positions == NULL nothing else is written, otherwise positions
- * fp32[count, 3] (cell units, any order) is filled -- it must hold the count a
- * previous call reported. */
-int ash_isosurface_extraction(const void* sdfs, const void* weights,
-                              const int64_t* grid_indices,
-                              const int32_t* grid_coords_table,
-                              const int64_t* lut_grid_nb2grid_idx,
-                              const int32_t* cell_coords_table,
-                              const int64_t* lut_cell_nb2cell_idx,
-                              const int64_t* lut_cell_nb2grid_nb,
-                              int64_t num_grids, int64_t num_embeddings,
-                              int64_t cells_per_grid, int grid_dim,
-                              float iso_value, float weight_thr, int32_t dtype,
-                              int32_t* counter, float* positions, void* stream);
+/* Replace the two launches of `isosurface_extraction` (ash/src/grid.cu:453-602,
+ * pybind.cpp:30; the reference counts, allocates and runs the same kernel again
+ * to fill).  sdfs / weights scalar[num_embeddings, cells_per_grid];
+ * grid_indices int64[num_grids]; grid_coords_table int32[num_embeddings, 3];
+ * cell_coords_table int32[cells_per_grid, 3]; the three 8-entry neighbour
+ * tables of the queries.
+ *
+ * classify: flags uint8[num_embeddings * cells_per_grid] (no initialisation)
+ * receives, for every cell of the listed rows, bit d set when the field crosses
+ * iso_value on the cell's +x/+y/+z edge (d = 0, 1, 2) and both ends weigh at
+ * least weight_thr; a missing neighbour block ends a cell's scan as in the
+ * reference.  workspace (device int32, as many as
+ * ash_isosurface_workspace_ints returns, no initialisation): [0] = number of
+ * points, the rest is carried to the second call.
+ *
+ * points: after the caller has read workspace[0] and allocated positions
+ * fp32[n_points, 3] (cell units); the points come in the order of the listing,
+ * the same on every run. */
+int64_t ash_isosurface_workspace_ints(int64_t num_grids, int64_t cells_per_grid);
+int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t* grid_indices,
+                            const int64_t* lut_grid_nb2grid_idx,
+                            const int32_t* cell_coords_table,
+                            const int64_t* lut_cell_nb2cell_idx,
+                            const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                            int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
+                            float iso_value, float weight_thr, int32_t dtype, uint8_t* flags,
+                            int32_t* workspace, void* stream);
+int ash_isosurface_points(const void* sdfs, const int64_t* grid_indices,
+                          const int32_t* grid_coords_table,
+                          const int64_t* lut_grid_nb2grid_idx,
+                          const int32_t* cell_coords_table,
+                          const int64_t* lut_cell_nb2cell_idx,
+                          const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                          int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
+                          float iso_value, int32_t dtype, const uint8_t* flags,
+                          const int32_t* workspace, int64_t n_points, float* positions,
+                          void* stream);
 
 /* Replace `marching_cubes` (ash/src/grid.cu:606-946, pybind.cpp:31), which the
  * reference runs as four launches around two host read-backs, by two calls
- * around one read-back.  Tables and fields as for ash_isosurface_extraction.
+ * around one read-back.  Tables and fields as for ash_isosurface_classify.
  *
  * classify: a listed cell takes part when it and the seven cells at its other
  * corners (entries 1..7 of the 8-entry neighbour tables) exist and weigh at

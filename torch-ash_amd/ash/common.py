@@ -139,10 +139,16 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.c_int, _PTR, _I64, _I64, _PTR, ctypes.c_uint64, _PTR],
     ),
-    "ash_isosurface_extraction": (
+    "ash_isosurface_workspace_ints": (ctypes.c_int64, [_I64, _I64]),
+    "ash_isosurface_classify": (
         ctypes.c_int,
-        [_PTR] * 8 + [_I64] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int32,
-                                    _PTR, _PTR, _PTR],
+        [_PTR] * 7 + [_I64] * 3
+        + [ctypes.c_int, ctypes.c_float, ctypes.c_float, ctypes.c_int32] + [_PTR] * 3,
+    ),
+    "ash_isosurface_points": (
+        ctypes.c_int,
+        [_PTR] * 7 + [_I64] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_int32]
+        + [_PTR] * 2 + [_I64] + [_PTR] * 2,
     ),
     "ash_convolution_forward": (
         ctypes.c_int,
@@ -230,8 +236,8 @@ class _Backend:
         weight_thr,
     ) -> torch.Tensor:
         """Zero crossings of `sdfs - iso_value` on the +x/+y/+z edges of the
-        listed blocks' cells, (P, 3) float32 in cell units, in no particular
-        order."""
+        listed blocks' cells, (P, 3) float32 in cell units, in the order of the
+        listing."""
         _require_hip(sdfs, "sdfs")
         dev = sdfs.device
         if sdfs.dtype not in _DTYPE:
@@ -249,24 +255,30 @@ class _Backend:
             raise RuntimeError("coordinate / neighbour tables do not match the grid")
         if lut_c2c.shape != (m, 8) or lut_c2g.shape != (m, 8):
             raise RuntimeError("cell neighbour tables must be (cells_per_grid, 8)")
-        counter = torch.zeros(1, dtype=torch.int32, device=dev)
-
-        def launch(positions):
-            with torch.cuda.device(dev):
+        flags = torch.empty(b * m, dtype=torch.uint8, device=dev)
+        workspace = torch.empty(
+            self.lib.ash_isosurface_workspace_ints(gi.numel(), m), dtype=torch.int32, device=dev
+        )
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_isosurface_classify(
+                    sdfs.data_ptr(), weights.data_ptr(), gi.data_ptr(), lut_g.data_ptr(),
+                    cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
+                    int(grid_dim), float(iso_value), float(weight_thr), _DTYPE[sdfs.dtype],
+                    flags.data_ptr(), workspace.data_ptr(), _stream_of(dev),
+                )
+            )
+            n_points = int(workspace[0].item())
+            positions = torch.empty((n_points, 3), dtype=torch.float32, device=dev)
+            if n_points:
                 self.check(
-                    self.lib.ash_isosurface_extraction(
-                        sdfs.data_ptr(), weights.data_ptr(), gi.data_ptr(), gc.data_ptr(),
-                        lut_g.data_ptr(), cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(),
-                        gi.numel(), b, m, int(grid_dim), float(iso_value), float(weight_thr),
-                        _DTYPE[sdfs.dtype], counter.data_ptr(),
-                        positions.data_ptr() if positions is not None else None, _stream_of(dev),
+                    self.lib.ash_isosurface_points(
+                        sdfs.data_ptr(), gi.data_ptr(), gc.data_ptr(), lut_g.data_ptr(),
+                        cc.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(), gi.numel(), b, m,
+                        int(grid_dim), float(iso_value), _DTYPE[sdfs.dtype], flags.data_ptr(),
+                        workspace.data_ptr(), n_points, positions.data_ptr(), _stream_of(dev),
                     )
                 )
-
-        launch(None)
-        positions = torch.zeros((int(counter.item()), 3), dtype=torch.float32, device=dev)
-        if positions.shape[0]:
-            launch(positions)
         return positions
 
     # -- marching cubes (ash/src/pybind.cpp:31) ------------------------------

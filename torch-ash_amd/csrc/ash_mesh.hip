@@ -249,19 +249,14 @@ constexpr int kSrcOwn = 8;              // source "the block itself"
 
 __host__ __device__ inline int tile_cells(int g) { return (g + 1) * (g + 1) * (g + 1); }
 
-template <typename T>
-__global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a) {
-    extern __shared__ __align__(16) uint8_t lds[];
-    __shared__ int64_t s_nb[kSrcOwn + 1];
-    const T* sdfs = static_cast<const T*>(a.sdfs);
-    const T* weights = static_cast<const T*>(a.weights);
+// s_src[t]: where tile cell t comes from, source << 12 | cell (source 0..7 =
+// entry of the block's neighbour row, kSrcOwn = the block itself); s_pos[c]:
+// tile index of the block's cell c.
+__device__ __forceinline__ void build_tile_map(const McDev& a, uint16_t* s_src, uint16_t* s_pos) {
     const int G = a.g;
     const int W = G + 1;
     const int M = static_cast<int>(a.M);
     const int W3 = tile_cells(G);
-    uint16_t* s_src = reinterpret_cast<uint16_t*>(lds);   // [W3] source << 12 | cell
-    uint16_t* s_pos = s_src + W3;                          // [M]  tile index of a cell
-    uint8_t* tile = reinterpret_cast<uint8_t*>(s_pos + M); // [W3]
     const int lane = threadIdx.x;
     const int off[3] = {1, W, W * W};
     for (int t = lane; t < W3; t += kTileThreads) s_src[t] = kSrcNone;
@@ -287,21 +282,49 @@ __global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a)
                     static_cast<uint16_t>((gn << 12) | ci);
         }
     }
+}
+
+// Row of listed block b (lane kSrcOwn) and of its neighbours (lanes 0..7); -1
+// where there is none.
+__device__ __forceinline__ int64_t fetch_block_rows(const McDev& a, int64_t b) {
+    const int lane = threadIdx.x;
+    if (b >= a.n_grids || lane > kSrcOwn) return -1;
+    const int64_t g = a.grid_indices[b];
+    if (g < 0 || g >= a.B) return -1;
+    if (lane == kSrcOwn) return g;
+    const int64_t r = a.lut_g[g * 8 + lane];
+    return (r >= 0 && r < a.B) ? r : -1;
+}
+
+// Index in the per-cell arrays of tile cell t, -1 if it does not exist.
+__device__ __forceinline__ int64_t tile_source(const McDev& a, const uint16_t* s_src,
+                                               const int64_t* s_nb, int t) {
+    const int src = s_src[t];
+    const int from = src >> 12;
+    if (from > kSrcOwn || s_nb[from] < 0) return -1;
+    return s_nb[from] * a.M + (src & 0xFFF);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ int64_t s_nb[kSrcOwn + 1];
+    const T* sdfs = static_cast<const T*>(a.sdfs);
+    const T* weights = static_cast<const T*>(a.weights);
+    const int W = a.g + 1;
+    const int M = static_cast<int>(a.M);
+    const int W3 = tile_cells(a.g);
+    uint16_t* s_src = reinterpret_cast<uint16_t*>(lds);   // [W3]
+    uint16_t* s_pos = s_src + W3;                          // [M]
+    uint8_t* tile = reinterpret_cast<uint8_t*>(s_pos + M); // [W3]
+    const int lane = threadIdx.x;
+    build_tile_map(a, s_src, s_pos);
     int64_t blk = blockIdx.x;
-    // rows of the block (lane 8) and of its neighbours (lanes 0..7)
-    auto fetch_rows = [&](int64_t b) -> int64_t {
-        if (b >= a.n_grids || lane > kSrcOwn) return -1;
-        const int64_t g = a.grid_indices[b];
-        if (g < 0 || g >= a.B) return -1;
-        if (lane == kSrcOwn) return g;
-        const int64_t r = a.lut_g[g * 8 + lane];
-        return (r >= 0 && r < a.B) ? r : -1;
-    };
-    int64_t row = fetch_rows(blk);
+    int64_t row = fetch_block_rows(a, blk);
     for (; blk < a.n_grids; blk += gridDim.x) {
         __syncthreads();  // set-up done; previous block's tile and rows read
         if (lane <= kSrcOwn) s_nb[lane] = row;
-        row = fetch_rows(blk + gridDim.x);
+        row = fetch_block_rows(a, blk + gridDim.x);
         __syncthreads();
         const int64_t g = s_nb[kSrcOwn];
         if (g < 0) continue;  // the same for the whole wavefront
@@ -311,12 +334,7 @@ __global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a)
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int t = t0 + k * kTileThreads + lane;
-                at[k] = -1;
-                if (t < W3) {
-                    const int src = s_src[t];
-                    const int from = src >> 12;
-                    if (from <= kSrcOwn && s_nb[from] >= 0) at[k] = s_nb[from] * a.M + (src & 0xFFF);
-                }
+                at[k] = t < W3 ? tile_source(a, s_src, s_nb, t) : -1;
                 w[k] = at[k] >= 0 ? weights[at[k]] : T(0);
                 v[k] = at[k] >= 0 ? sdfs[at[k]] : T(0);
             }
@@ -450,16 +468,18 @@ __global__ __launch_bounds__(kBlock) void mc_count_kernel(McDev a) {
     }
 }
 
-// Turns the per-chunk counts into running sums (one workgroup; every thread
-// takes a contiguous share of the chunks) and stores the totals.
+// Turns `arrays` (1 or 2) consecutive arrays of per-chunk counts into running
+// sums (one workgroup; every thread takes a contiguous share of the chunks) and
+// stores their totals in ws[slot0] / ws[slot1].
 constexpr int kScanThreads = 1024;
 
-__global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int64_t chunks) {
+__global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int64_t chunks,
+                                                              int arrays, int slot0, int slot1) {
     __shared__ int64_t s_sum[kScanThreads];
     const int64_t share = (chunks + kScanThreads - 1) / kScanThreads;
     const int64_t lo = share * threadIdx.x < chunks ? share * threadIdx.x : chunks;
     const int64_t hi = lo + share < chunks ? lo + share : chunks;
-    for (int which = 0; which < 2; ++which) {
+    for (int which = 0; which < arrays; ++which) {
         int32_t* counts = ws + kMcHeader + which * chunks;
         int64_t mine = 0;
         for (int64_t i = lo; i < hi; ++i) mine += counts[i];
@@ -480,9 +500,39 @@ __global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int6
         }
         if (threadIdx.x == kScanThreads - 1) {
             const int64_t total = s_sum[threadIdx.x];
-            ws[which == 0 ? kMcVertices32 : kMcTriangles32] =
+            ws[which == 0 ? slot0 : slot1] =
                     static_cast<int32_t>(total < 0x7FFFFFFF ? total : 0x7FFFFFFF);
         }
+    }
+}
+
+// The zero crossings on the flagged +x/+y/+z edges (bits of f) of cell c of row
+// g, linear between the two ends of an edge, to positions[out...]
+// (ash/src/grid.cu:510-527 and :748-771).
+template <typename T>
+__device__ __forceinline__ void write_edge_points(const McDev& a, int64_t g, int64_t c,
+                                                  int64_t own, int f, int64_t out) {
+    const T* sdfs = static_cast<const T*>(a.sdfs);
+    const T self = sdfs[own] - static_cast<T>(a.iso);
+    float base[3];
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        base[d] = static_cast<float>(a.grid_coords[g * 3 + d] * a.g + a.cell_coords[c * 3 + d]);
+    }
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        if (!(f & (1 << d))) continue;
+        int64_t gi, ci;
+        float ratio = 0.f;
+        if (corner_cell(a, g, c, 1 << d, gi, ci)) {
+            const T other = sdfs[gi * a.M + ci] - static_cast<T>(a.iso);
+            ratio = static_cast<float>(self / (self - other));
+        }
+        float* p = a.positions + out * 3;
+        p[0] = base[0] + (d == 0 ? ratio : 0.f);
+        p[1] = base[1] + (d == 1 ? ratio : 0.f);
+        p[2] = base[2] + (d == 2 ? ratio : 0.f);
+        ++out;
     }
 }
 
@@ -493,7 +543,6 @@ template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
     __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
     __shared__ int32_t s_id[kChunk];      // id of its first vertex
-    const T* sdfs = static_cast<const T*>(a.sdfs);
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint64_t flags = 0;   // 3 bits per own cell
@@ -537,28 +586,7 @@ __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
             int64_t out = s_id[q];
             a.slots[own] = static_cast<uint32_t>(f) | (static_cast<uint32_t>(out) << 3);
             if (out + __popc(f) > a.n_vertices) continue;  // never with the counts of classify
-            const T self = sdfs[own] - static_cast<T>(a.iso);
-            float base[3];
-#pragma unroll
-            for (int d = 0; d < 3; ++d) {
-                base[d] = static_cast<float>(a.grid_coords[g * 3 + d] * a.g +
-                                             a.cell_coords[c * 3 + d]);
-            }
-#pragma unroll
-            for (int d = 0; d < 3; ++d) {
-                if (!(f & (1 << d))) continue;
-                int64_t gi, ci;
-                float ratio = 0.f;
-                if (corner_cell(a, g, c, 1 << d, gi, ci)) {
-                    const T other = sdfs[gi * a.M + ci] - static_cast<T>(a.iso);
-                    ratio = static_cast<float>(self / (self - other));
-                }
-                float* p = a.positions + out * 3;
-                p[0] = base[0] + (d == 0 ? ratio : 0.f);
-                p[1] = base[1] + (d == 1 ? ratio : 0.f);
-                p[2] = base[2] + (d == 2 ? ratio : 0.f);
-                ++out;
-            }
+            write_edge_points<T>(a, g, c, own, f, out);
         }
     }
 }
@@ -649,6 +677,180 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Iso-surface points (ash/src/grid.cu:453-602): every listed cell that weighs
+// enough looks at its +x, +y, +z neighbours; where the field changes sign
+// against a neighbour that weighs enough as well, the zero crossing on that
+// edge is a point.  As in the reference a missing neighbour block ends the
+// cell's scan, later axes included, and "changes sign" is `self * other < 0`
+// evaluated in the field's type.  The reference runs its kernel twice (count,
+// fill) with one atomic per point; here the first call leaves the three
+// crossing flags of every cell in `cases` and per-chunk counts in the
+// workspace, the second writes the points from the chunks' offsets.
+template <typename T>
+__device__ __forceinline__ int crossing_flags(T self, const T* diff, const uint8_t* state,
+                                              int p, const int* off) {
+    int f = 0;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        const int q = p + off[d];
+        const int st = state[q];
+        if (!(st & 2)) break;
+        if (self * diff[q] < T(0) && (st & 1)) f |= 1 << d;
+    }
+    return f;
+}
+
+// One wavefront per block: field minus iso value of the (G+1)^3 corner cells
+// in LDS, state bit 0 = weighs enough, bit 1 = exists.
+template <typename T>
+__global__ __launch_bounds__(kTileThreads) void iso_classify_tile_kernel(McDev a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    __shared__ int64_t s_nb[kSrcOwn + 1];
+    const T* sdfs = static_cast<const T*>(a.sdfs);
+    const T* weights = static_cast<const T*>(a.weights);
+    const int W = a.g + 1;
+    const int M = static_cast<int>(a.M);
+    const int W3 = tile_cells(a.g);
+    T* diff = reinterpret_cast<T*>(lds);                       // [W3]
+    uint16_t* s_src = reinterpret_cast<uint16_t*>(diff + W3);  // [W3]
+    uint16_t* s_pos = s_src + W3;                              // [M]
+    uint8_t* state = reinterpret_cast<uint8_t*>(s_pos + M);    // [W3]
+    const int lane = threadIdx.x;
+    const int off[3] = {1, W, W * W};
+    build_tile_map(a, s_src, s_pos);
+    int64_t blk = blockIdx.x;
+    int64_t row = fetch_block_rows(a, blk);
+    for (; blk < a.n_grids; blk += gridDim.x) {
+        __syncthreads();  // set-up done; previous block's tile and rows read
+        if (lane <= kSrcOwn) s_nb[lane] = row;
+        row = fetch_block_rows(a, blk + gridDim.x);
+        __syncthreads();
+        const int64_t g = s_nb[kSrcOwn];
+        if (g < 0) continue;  // the same for the whole wavefront
+        for (int t0 = 0; t0 < W3; t0 += 4 * kTileThreads) {
+            int64_t at[4];
+            T w[4], v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int t = t0 + k * kTileThreads + lane;
+                at[k] = t < W3 ? tile_source(a, s_src, s_nb, t) : -1;
+                w[k] = at[k] >= 0 ? weights[at[k]] : T(0);
+                v[k] = at[k] >= 0 ? sdfs[at[k]] : T(0);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int t = t0 + k * kTileThreads + lane;
+                if (t < W3) {
+                    diff[t] = v[k] - static_cast<T>(a.iso);
+                    state[t] = at[k] < 0 ? 0 : (2 | (w[k] >= static_cast<T>(a.weight_thr) ? 1 : 0));
+                }
+            }
+        }
+        __syncthreads();
+        for (int c = lane; c < M; c += kTileThreads) {
+            const int p = s_pos[c];
+            a.cases[g * a.M + c] = static_cast<uint8_t>(
+                    (state[p] & 1) ? crossing_flags<T>(diff[p], diff, state, p, off) : 0);
+        }
+    }
+}
+
+// The same through the tables, for blocks that do not fit the tile.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void iso_classify_cell_kernel(McDev a) {
+    const T* sdfs = static_cast<const T*>(a.sdfs);
+    const T* weights = static_cast<const T*>(a.weights);
+    const int64_t cells = a.n_grids * a.M;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    for (int64_t item = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; item < cells;
+         item += stride) {
+        const int64_t g = a.grid_indices[item / a.M];
+        const int64_t c = item % a.M;
+        if (g < 0 || g >= a.B) continue;
+        int f = 0;
+        if (weights[g * a.M + c] >= static_cast<T>(a.weight_thr)) {
+            const T self = sdfs[g * a.M + c] - static_cast<T>(a.iso);
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                int64_t gi, ci;
+                if (!corner_cell(a, g, c, 1 << d, gi, ci)) break;
+                const T other = sdfs[gi * a.M + ci] - static_cast<T>(a.iso);
+                if (self * other < T(0) && weights[gi * a.M + ci] >= static_cast<T>(a.weight_thr)) {
+                    f |= 1 << d;
+                }
+            }
+        }
+        a.cases[g * a.M + c] = static_cast<uint8_t>(f);
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void iso_count_kernel(McDev a) {
+    const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
+    for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
+        int n = 0;
+        for_own_groups<VEC>(a, ch, [&](int, uint32_t, int64_t at) {
+            if constexpr (VEC == 4) {
+                n += __popc(*reinterpret_cast<const uint32_t*>(a.cases + at) & 0x07070707u);
+            } else {
+                n += __popc(a.cases[at] & 7u);
+            }
+        });
+        int total;
+        block_exclusive(n, total);
+        if (threadIdx.x == 0) a.counters[kMcHeader + ch] = total;
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void iso_points_kernel(McDev a) {
+    __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
+    __shared__ int32_t s_id[kChunk];      // its first point
+    const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
+    for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
+        uint64_t flags = 0;   // 3 bits per own cell
+        int part[kPerThread / VEC] = {};   // per group: listed cells | points << 16
+        for_own_groups<VEC>(a, ch, [&](int j, uint32_t, int64_t at) {
+            uint32_t w;
+            if constexpr (VEC == 4) {
+                w = *reinterpret_cast<const uint32_t*>(a.cases + at);
+            } else {
+                w = a.cases[at];
+            }
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const uint32_t f = (w >> (8 * k)) & 7u;
+                flags |= static_cast<uint64_t>(f) << (3 * (j * VEC + k));
+                part[j] += (f != 0u) + (__popc(f) << 16);
+            }
+        });
+        const int total = chunk_exclusive(part);
+        const int first = a.counters[kMcHeader + ch];
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+            const int f = static_cast<int>(flags >> (3 * j)) & 7;
+            if (f) {
+                int& at = part[j / VEC];
+                s_cell[at & 0xFFFF] =
+                        static_cast<uint16_t>((own_group_offset<VEC>(j / VEC) + j % VEC) | (f << 12));
+                s_id[at & 0xFFFF] = first + (at >> 16);
+                at += 1 + (__popc(f) << 16);
+            }
+        }
+        __syncthreads();
+        const int listed = total & 0xFFFF;
+        for (int q = threadIdx.x; q < listed; q += kBlock) {
+            const int f = s_cell[q] >> 12;
+            int64_t g, c;
+            const int64_t own = cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c);
+            const int64_t out = s_id[q];
+            if (out + __popc(f) > a.n_vertices) continue;  // never with the count of classify
+            write_edge_points<T>(a, g, c, own, f, out);
+        }
+    }
+}
+
 // Groups of four cells can be moved as one word of cases and one 16-byte
 // vector of slots when blocks hold a multiple of four cells and both arrays
 // are aligned accordingly.
@@ -666,17 +868,17 @@ int fill_common(McDev& a, const void* sdfs, const int64_t* grid_indices,
                 const int32_t* cell_coords, const int64_t* lut_g, const int64_t* lut_c2c,
                 const int64_t* lut_c2g, int64_t num_grids, int64_t num_embeddings,
                 int64_t cells_per_grid, int grid_dim, float iso_value, int32_t dtype,
-                uint8_t* cases, uint32_t* slots, int32_t* counters) {
+                uint8_t* cases, uint32_t* slots, bool with_slots, int32_t* counters) {
     if (dtype != ASH_F32 && dtype != ASH_F64) ASH_FAIL("unknown dtype");
     if (num_grids < 0 || num_embeddings < 1 || cells_per_grid < 1 || grid_dim < 1) {
-        ASH_FAIL("marching_cubes: bad sizes");
+        ASH_FAIL("surface extraction: bad sizes");
     }
-    if (counters == nullptr) ASH_FAIL("marching_cubes: null counters");
+    if (counters == nullptr) ASH_FAIL("surface extraction: null workspace");
     if (num_grids > 0 &&
         (sdfs == nullptr || grid_indices == nullptr || cell_coords == nullptr ||
          lut_g == nullptr || lut_c2c == nullptr || lut_c2g == nullptr || cases == nullptr ||
-         slots == nullptr)) {
-        ASH_FAIL("null pointer in marching_cubes");
+         (with_slots && slots == nullptr))) {
+        ASH_FAIL("null pointer in surface extraction");
     }
     if (cells_per_grid > (int64_t{1} << 24) || num_grids > (int64_t{1} << 40) / cells_per_grid) {
         ASH_FAIL("marching_cubes: too many cells in one call");
@@ -724,7 +926,7 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     McDev a = {};
     if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
                     lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
-                    cells_per_grid, grid_dim, iso_value, dtype, cases, edge_slots, counters)) {
+                    cells_per_grid, grid_dim, iso_value, dtype, cases, edge_slots, true, counters)) {
         return 1;
     }
     if (num_grids > 0 && weights == nullptr) ASH_FAIL("null pointer in marching_cubes");
@@ -765,7 +967,8 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
         mc_count_kernel<1><<<by_chunk, kBlock, 0, s>>>(a);
     }
     ASH_LAUNCH_CHECK();
-    mc_scan_kernel<<<1, kScanThreads, 0, s>>>(counters, (cells + kChunk - 1) / kChunk);
+    mc_scan_kernel<<<1, kScanThreads, 0, s>>>(counters, (cells + kChunk - 1) / kChunk, 2,
+                                              kMcVertices32, kMcTriangles32);
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -785,7 +988,7 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
     if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
                     lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
                     cells_per_grid, grid_dim, iso_value, dtype, const_cast<uint8_t*>(cases),
-                    edge_slots, counters)) {
+                    edge_slots, true, counters)) {
         return 1;
     }
     if (n_vertices < 0 || n_triangles < 0) ASH_FAIL("marching_cubes: negative counts");
@@ -825,6 +1028,109 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
         }
         ASH_LAUNCH_CHECK();
     }
+    return 0;
+}
+
+int64_t ash_isosurface_workspace_ints(int64_t num_grids, int64_t cells_per_grid) {
+    if (num_grids < 0 || cells_per_grid < 1) return kMcHeader;
+    return kMcHeader + (num_grids * cells_per_grid + kChunk - 1) / kChunk;
+}
+
+int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t* grid_indices,
+                            const int64_t* lut_grid_nb2grid_idx,
+                            const int32_t* cell_coords_table,
+                            const int64_t* lut_cell_nb2cell_idx,
+                            const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                            int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
+                            float iso_value, float weight_thr, int32_t dtype, uint8_t* flags,
+                            int32_t* workspace, void* stream) {
+    McDev a = {};
+    if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
+                    lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
+                    cells_per_grid, grid_dim, iso_value, dtype, flags, nullptr, false,
+                    workspace)) {
+        return 1;
+    }
+    if (num_grids > 0 && weights == nullptr) ASH_FAIL("null pointer in isosurface_classify");
+    a.weights = weights;
+    a.weight_thr = weight_thr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t cells = num_grids * cells_per_grid;
+    const int64_t chunks = (cells + kChunk - 1) / kChunk;
+    if (num_grids > 0) {
+        const bool tiled = grid_dim <= kMaxTileG &&
+                           static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
+        if (tiled) {
+            const unsigned by_block =
+                    static_cast<unsigned>(num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid);
+            const size_t cell_bytes = dtype == ASH_F32 ? 4 : 8;
+            const size_t lds = (cell_bytes + 3) * tile_cells(grid_dim) + 2 * cells_per_grid;
+            if (dtype == ASH_F32) {
+                iso_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
+            } else {
+                iso_classify_tile_kernel<double><<<by_block, kTileThreads, lds, s>>>(a);
+            }
+        } else {
+            const unsigned by_cell = persistent_grid((cells + kBlock - 1) / kBlock);
+            if (dtype == ASH_F32) {
+                iso_classify_cell_kernel<float><<<by_cell, kBlock, 0, s>>>(a);
+            } else {
+                iso_classify_cell_kernel<double><<<by_cell, kBlock, 0, s>>>(a);
+            }
+        }
+        ASH_LAUNCH_CHECK();
+        if (a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0) {
+            iso_count_kernel<4><<<persistent_grid(chunks), kBlock, 0, s>>>(a);
+        } else {
+            iso_count_kernel<1><<<persistent_grid(chunks), kBlock, 0, s>>>(a);
+        }
+        ASH_LAUNCH_CHECK();
+    }
+    mc_scan_kernel<<<1, kScanThreads, 0, s>>>(workspace, chunks, 1, 0, 0);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_isosurface_points(const void* sdfs, const int64_t* grid_indices,
+                          const int32_t* grid_coords_table,
+                          const int64_t* lut_grid_nb2grid_idx,
+                          const int32_t* cell_coords_table,
+                          const int64_t* lut_cell_nb2cell_idx,
+                          const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
+                          int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
+                          float iso_value, int32_t dtype, const uint8_t* flags,
+                          const int32_t* workspace, int64_t n_points, float* positions,
+                          void* stream) {
+    McDev a = {};
+    if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
+                    lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
+                    cells_per_grid, grid_dim, iso_value, dtype, const_cast<uint8_t*>(flags),
+                    nullptr, false, const_cast<int32_t*>(workspace))) {
+        return 1;
+    }
+    if (n_points < 0 || n_points > 0x7FFFFFFFll) ASH_FAIL("isosurface_points: bad point count");
+    if (num_grids == 0 || n_points == 0) return 0;
+    if (grid_coords_table == nullptr || positions == nullptr) {
+        ASH_FAIL("null pointer in isosurface_points");
+    }
+    a.grid_coords = grid_coords_table;
+    a.positions = positions;
+    a.n_vertices = n_points;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned by_chunk = persistent_grid((num_grids * cells_per_grid + kChunk - 1) / kChunk);
+    const bool vec = a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0;
+    if (dtype == ASH_F32) {
+        if (vec) {
+            iso_points_kernel<float, 4><<<by_chunk, kBlock, 0, s>>>(a);
+        } else {
+            iso_points_kernel<float, 1><<<by_chunk, kBlock, 0, s>>>(a);
+        }
+    } else if (vec) {
+        iso_points_kernel<double, 4><<<by_chunk, kBlock, 0, s>>>(a);
+    } else {
+        iso_points_kernel<double, 1><<<by_chunk, kBlock, 0, s>>>(a);
+    }
+    ASH_LAUNCH_CHECK();
     return 0;
 }
 

@@ -806,104 +806,6 @@ __global__ __launch_bounds__(kBlock) void convolution_forward_kernel(ConvDev a) 
     static_cast<T*>(a.out)[(g * a.M + c) * a.E + e] = sum;
 }
 
-// Iso-surface points (ash/src/grid.cu:453-531): every listed cell with enough
-// weight looks at its +x, +y, +z neighbours (entries 1, 2, 4 of the 8-entry
-// tables); where the field changes sign against a neighbour that has enough
-// weight as well, the zero crossing on that edge is a surface point.  As in
-// the reference a missing neighbour block ends the cell's scan, later axes
-// included.  positions == nullptr counts only.  The points of a workgroup are
-// appended with one update of the shared counter.
-struct IsoDev {
-    const void* sdfs;
-    const void* weights;
-    const int64_t* grid_indices;
-    const int32_t* grid_coords;   // [B, 3] by row
-    const int64_t* lut_g;         // [B, 8]
-    const int32_t* cell_coords;   // [M, 3]
-    const int64_t* lut_c2c;       // [M, 8]
-    const int64_t* lut_c2g;       // [M, 8]
-    int32_t* counter;
-    float* positions;
-    int64_t n_grids, B, M;
-    float iso, weight_thr;
-    int g;
-};
-
-template <typename T>
-__global__ __launch_bounds__(kBlock) void isosurface_points_kernel(IsoDev a) {
-    __shared__ int s_cnt[kBlock / 64];
-    __shared__ int s_first;
-    const int64_t item = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const T* sdfs = static_cast<const T*>(a.sdfs);
-    const T* weights = static_cast<const T*>(a.weights);
-    int found = 0;          // bit d: crossing on the +d edge
-    float ratio[3] = {0.f, 0.f, 0.f};
-    int64_t g = 0;
-    int64_t c = 0;
-    if (item < a.n_grids * a.M) {
-        g = a.grid_indices[item / a.M];
-        c = item % a.M;
-        if (g >= 0 && g < a.B && weights[g * a.M + c] >= static_cast<T>(a.weight_thr)) {
-            const T self = sdfs[g * a.M + c] - static_cast<T>(a.iso);
-#pragma unroll
-            for (int d = 0; d < 3; ++d) {
-                const int nb = 1 << d;
-                const int64_t gn = a.lut_c2g[c * 8 + nb];
-                const int64_t gi = (gn >= 0 && gn < 8) ? a.lut_g[g * 8 + gn] : -1;
-                if (gi < 0 || gi >= a.B) break;
-                const int64_t ci = a.lut_c2c[c * 8 + nb];
-                const T other = sdfs[gi * a.M + ci] - static_cast<T>(a.iso);
-                if (self * other < T(0) && weights[gi * a.M + ci] >= static_cast<T>(a.weight_thr)) {
-                    found |= 1 << d;
-                    ratio[d] = static_cast<float>(self / (self - other));
-                }
-            }
-        }
-    }
-    const int mine = __popc(found);
-    // exclusive prefix of `mine` over the workgroup
-    int incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d);
-        if (lane >= d) incl += up;
-    }
-    if (lane == 63) s_cnt[wave] = incl;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int tot = 0;
-#pragma unroll
-        for (int q = 0; q < kBlock / 64; ++q) {
-            const int v = s_cnt[q];
-            s_cnt[q] = tot;
-            tot += v;
-        }
-        s_first = tot ? atomicAdd(a.counter, tot) : 0;
-    }
-    __syncthreads();
-    if (a.positions == nullptr || mine == 0) return;
-    int64_t out = static_cast<int64_t>(s_first) + s_cnt[wave] + incl - mine;
-    float base[3];
-#pragma unroll
-    for (int d = 0; d < 3; ++d) {
-        base[d] = static_cast<float>(a.grid_coords[g * 3 + d] * a.g + a.cell_coords[c * 3 + d]);
-    }
-#pragma unroll
-    for (int d = 0; d < 3; ++d) {
-        if (found & (1 << d)) {
-            float* p = a.positions + out * 3;
-            p[0] = base[0] + (d == 0 ? ratio[d] : 0.f);
-            p[1] = base[1] + (d == 1 ? ratio[d] : 0.f);
-            p[2] = base[2] + (d == 2 ? ratio[d] : 0.f);
-            ++out;
-        }
-    }
-}
-
-__global__ void zero_counter_kernel(int32_t* p) { *p = 0; }
-
 __global__ __launch_bounds__(kBlock) void zero16_kernel(uint4* __restrict__ p,
                                                         int64_t n16) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
@@ -1294,60 +1196,6 @@ int ash_convolution_forward(const void* inputs, const void* weights,
         convolution_forward_kernel<float><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
     } else {
         convolution_forward_kernel<double><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
-    }
-    ASH_LAUNCH_CHECK();
-    return 0;
-}
-
-int ash_isosurface_extraction(const void* sdfs, const void* weights,
-                              const int64_t* grid_indices,
-                              const int32_t* grid_coords_table,
-                              const int64_t* lut_grid_nb2grid_idx,
-                              const int32_t* cell_coords_table,
-                              const int64_t* lut_cell_nb2cell_idx,
-                              const int64_t* lut_cell_nb2grid_nb,
-                              int64_t num_grids, int64_t num_embeddings,
-                              int64_t cells_per_grid, int grid_dim,
-                              float iso_value, float weight_thr, int32_t dtype,
-                              int32_t* counter, float* positions, void* stream) {
-    if (dtype != ASH_F32 && dtype != ASH_F64) ASH_FAIL("unknown dtype");
-    if (num_grids < 0 || num_embeddings < 1 || cells_per_grid < 1 || grid_dim < 1) {
-        ASH_FAIL("isosurface_extraction: bad sizes");
-    }
-    if (counter == nullptr) ASH_FAIL("isosurface_extraction: null counter");
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    zero_counter_kernel<<<1, 1, 0, s>>>(counter);
-    ASH_LAUNCH_CHECK();
-    if (num_grids == 0) return 0;
-    if (sdfs == nullptr || weights == nullptr || grid_indices == nullptr ||
-        grid_coords_table == nullptr || lut_grid_nb2grid_idx == nullptr ||
-        cell_coords_table == nullptr || lut_cell_nb2cell_idx == nullptr ||
-        lut_cell_nb2grid_nb == nullptr) {
-        ASH_FAIL("null pointer in isosurface_extraction");
-    }
-    IsoDev a;
-    a.sdfs = sdfs;
-    a.weights = weights;
-    a.grid_indices = grid_indices;
-    a.grid_coords = grid_coords_table;
-    a.lut_g = lut_grid_nb2grid_idx;
-    a.cell_coords = cell_coords_table;
-    a.lut_c2c = lut_cell_nb2cell_idx;
-    a.lut_c2g = lut_cell_nb2grid_nb;
-    a.counter = counter;
-    a.positions = positions;
-    a.n_grids = num_grids;
-    a.B = num_embeddings;
-    a.M = cells_per_grid;
-    a.iso = iso_value;
-    a.weight_thr = weight_thr;
-    a.g = grid_dim;
-    const int64_t blocks = (num_grids * cells_per_grid + kBlock - 1) / kBlock;
-    if (blocks > 0x7FFFFFFFll) ASH_FAIL("isosurface_extraction: too many cells in one call");
-    if (dtype == ASH_F32) {
-        isosurface_points_kernel<float><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
-    } else {
-        isosurface_points_kernel<double><<<static_cast<unsigned>(blocks), kBlock, 0, s>>>(a);
     }
     ASH_LAUNCH_CHECK();
     return 0;
