@@ -418,6 +418,29 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         "Msamples_per_s": round(n_samples / (ms_nf + ms_rs) / 1e3, 1),
     }
 
+    # surface extraction over the same blocks (ash/grid.py:628-711): the
+    # algorithmic figure counts one read of field and weight per cell and one
+    # write of every vertex and triangle
+    field = workloads.sphere_distance_field(grid, radii, centres)
+    ones = torch.ones_like(field)
+    t_mesh, t_pts = EventTimer(torch), EventTimer(torch)
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        run(t_mesh, lambda: box.update(mesh=grid.surface_mesh(field, ones)))
+        run(t_pts, lambda: box.update(pts=grid.isosurface_points(field, ones)))
+    cells = grid.engine.size() * 512
+    n_tri, n_vtx, n_pts = len(box["mesh"][0]), len(box["mesh"][1]), len(box["pts"])
+    e = roofline_entry("marching cubes: classify + extract (6 kernels, one read-back)",
+                       8 * cells + 12 * (n_tri + n_vtx), t_mesh.mean_ms())
+    e.update(cells=cells, vertices=n_vtx, triangles=n_tri,
+             Gcells_per_s=round(cells / e["ms"] / 1e6, 2))
+    out["cfg4_surface_mesh"] = e
+    e = roofline_entry("iso-surface points: classify + points (4 kernels, one read-back)",
+                       8 * cells + 12 * n_pts, t_pts.mean_ms())
+    e.update(cells=cells, points=n_pts, Gcells_per_s=round(cells / e["ms"] / 1e6, 2))
+    out["cfg4_isosurface_points"] = e
+    del field, ones, box
+
     if not args.no_cpu:
         out["cfg4_cpu"] = cpu_trilinear(torch, ops, z, u, 1 << 18)
 

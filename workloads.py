@@ -179,6 +179,28 @@ def build_grid(
     return grid, radii, centres
 
 
+def sphere_distance_field(grid, radii, centres) -> torch.Tensor:
+    """Signed distance to the union of the scene's spheres at every cell of the
+    grid's active blocks, (num_embeddings, cells_per_grid) in world units; zero
+    in rows of inactive blocks.  The field the surface extraction of the demos
+    runs on after fusion."""
+    dev = grid.embeddings.device
+    keys, idx = grid.engine.items()
+    field = torch.zeros(grid.embeddings.shape[:2], device=dev)
+    cell_coords = grid.cell_coords.view(1, -1, 3)
+    centres, radii = centres.to(dev), radii.to(dev)
+    for s in range(0, len(idx), 16384):
+        cells = (keys[s : s + 16384].view(-1, 1, 3) * grid.grid_dim + cell_coords).float()
+        world = grid.transform_cell_to_world(cells)
+        best = None
+        for c in range(0, len(centres), 8):
+            d = (world.unsqueeze(2) - centres[c : c + 8].view(1, 1, -1, 3)).norm(dim=-1)
+            d = (d - radii[c : c + 8]).min(dim=2)[0]
+            best = d if best is None else torch.minimum(best, d)
+        field[idx[s : s + 16384]] = best
+    return field
+
+
 def uniform_queries(
     grid, num_inside: int = 4_000_000, empty_fraction: float = 0.1, seed: int = 4
 ) -> torch.Tensor:
