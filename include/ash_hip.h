@@ -161,6 +161,22 @@ int ash_ray_sample(ash_map_t* map, const float* ray_origins,
                    const int64_t* prefix, int64_t* ray_indices, float* t_nears,
                    float* t_fars, void* stream);
 
+/* The same result with one march instead of two (no counterpart in the
+ * reference, whose second launch repeats the march of the first).  staged:
+ * the allocation pass, which also keeps the first `stride` samples of every ray
+ * in stage fp32[n * stride * 2] (8-byte aligned).  compact: the assignment
+ * pass as a copy out of `stage`; valid when no ray has more than `stride`
+ * samples (counts tells; max_samples_per_ray + 2 always suffices), otherwise
+ * run the assignment pass of ash_ray_sample. */
+int ash_ray_sample_staged(ash_map_t* map, const float* ray_origins,
+                          const float* ray_directions, const float* ray_nears,
+                          const float* ray_fars, int64_t n, int64_t max_samples_per_ray,
+                          float grid2cell_multiplier, int64_t* counts, float* stage,
+                          int64_t stride, void* stream);
+int ash_ray_sample_compact(const int64_t* counts, const int64_t* prefix, const float* stage,
+                           int64_t stride, int64_t n, int64_t* ray_indices, float* t_nears,
+                           float* t_fars, void* stream);
+
 /* Replaces `HashMap::insert_keys` (ash/src/hashmap_gpu.cuh:211-247).  New keys
  * pop one index each from the heap; duplicates (in the table or within the
  * batch) are ignored.  Keys beyond `capacity` are dropped and counted

@@ -60,6 +60,29 @@ def test_near_far_and_samples_match_oracle(gpu_ash, oracle, n):
             assert ref[0].numel() > 10 * n
 
 
+@pytest.mark.parametrize("mode", ["two_marches", "stage_overflow"])
+def test_sample_paths_agree(gpu_ash, oracle, monkeypatch, mode):
+    """ray_sample keeps the samples of its allocation pass and copies them; the
+    reference's second march remains for staging areas that would be too large
+    and for rays with more samples than the staging stride."""
+    engine, omap, blocks, g = _scene(gpu_ash, oracle)
+    backend = gpu_ash.grid.backend
+    extent = 64 * 8.0
+    o, d = _rays(g, 3000, extent, blocks)
+    lo, hi = torch.zeros(3, device=DEV), torch.full((3,), extent, device=DEV)
+    near, far = backend.ray_find_near_far(engine.backend, o.to(DEV), d.to(DEV), lo, hi,
+                                          0.5, 700.0, 1.0, 8.0)
+    staged = backend.ray_sample(engine.backend, o.to(DEV), d.to(DEV), near, far, lo, hi, 64, 8.0)
+    if mode == "two_marches":
+        monkeypatch.setattr(gpu_ash.common, "RAY_STAGE_LIMIT", 0)
+    else:
+        monkeypatch.setattr(gpu_ash.common, "RAY_STAGE_EXTRA", -60)   # stride 4
+    other = backend.ray_sample(engine.backend, o.to(DEV), d.to(DEV), near, far, lo, hi, 64, 8.0)
+    assert staged[0].numel() > 20_000 and int(torch.diff(staged[3]).max()) > 4
+    for a, b in zip(staged, other):
+        assert torch.equal(a, b)
+
+
 def test_samples_start_inside_active_blocks(gpu_ash, oracle):
     """Property at a larger size: every interval starts in an active block,
     intervals of a ray are ordered, counts agree with the prefix sum."""

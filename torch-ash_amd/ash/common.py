@@ -90,6 +90,11 @@ _SIGNATURES = {
         [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, _I64, ctypes.c_float, _PTR, _PTR, _PTR, _PTR, _PTR,
          _PTR],
     ),
+    "ash_ray_sample_staged": (
+        ctypes.c_int,
+        [_PTR] * 5 + [_I64, _I64, ctypes.c_float, _PTR, _PTR, _I64, _PTR],
+    ),
+    "ash_ray_sample_compact": (ctypes.c_int, [_PTR] * 3 + [_I64, _I64] + [_PTR] * 4),
     "ash_map_insert_keys": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_insert_needs_scratch": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_I64)]),
     "ash_map_insert": (
@@ -179,6 +184,13 @@ _SIGNATURES = {
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 _INTERPOLATION = {"linear": 0, "smooth_step": 1}
+
+# Largest number of staged sample slots (rays x stride, 8 bytes each) for which
+# ray_sample keeps the samples of its allocation pass; beyond it the march is
+# run twice as in the reference.
+RAY_STAGE_LIMIT = 1 << 30
+# Staged slots per ray beyond max_samples_per_ray.
+RAY_STAGE_EXTRA = 2
 
 # Which inserts take the streaming (partition + build in LDS) path of the
 # library instead of the per-key kernel: "auto" = when the library says the
@@ -429,24 +441,50 @@ class _Backend:
         counts = torch.zeros(n, dtype=torch.int64, device=dev)
         fixed = (hashmap._handle, o.data_ptr(), d.data_ptr(), nears.data_ptr(), fars.data_ptr(), n,
                  int(max_samples_per_ray), float(grid2cell_multiplier))
-        with torch.cuda.device(dev):
-            self.check(
-                self.lib.ash_ray_sample(*fixed, counts.data_ptr(), None, None, None, None,
-                                        _stream_of(dev))
-            )
-        prefix = torch.cumsum(counts, 0)
-        total = int(prefix[-1]) if n else 0
-        ray_indices = torch.zeros(total, dtype=torch.int64, device=dev)
-        t_nears = torch.zeros(total, dtype=torch.float32, device=dev)
-        t_fars = torch.zeros(total, dtype=torch.float32, device=dev)
-        if total:
+        # One march: the allocation pass keeps its samples, the assignment pass
+        # copies them.  A ray takes at most max_samples steps of its own size
+        # (+ rounding), so the staging stride below is never exceeded; the
+        # two-march path of the reference remains for the case that it is.
+        stride = max(1, int(max_samples_per_ray) + RAY_STAGE_EXTRA)
+        staged = n * stride <= RAY_STAGE_LIMIT
+        if staged:
+            stage = torch.empty((n, stride, 2), dtype=torch.float32, device=dev)
             with torch.cuda.device(dev):
                 self.check(
-                    self.lib.ash_ray_sample(
-                        *fixed, None, prefix.data_ptr(), ray_indices.data_ptr(),
-                        t_nears.data_ptr(), t_fars.data_ptr(), _stream_of(dev),
-                    )
+                    self.lib.ash_ray_sample_staged(*fixed, counts.data_ptr(), stage.data_ptr(),
+                                                   stride, _stream_of(dev))
                 )
+        else:
+            with torch.cuda.device(dev):
+                self.check(
+                    self.lib.ash_ray_sample(*fixed, counts.data_ptr(), None, None, None, None,
+                                            _stream_of(dev))
+                )
+        prefix = torch.cumsum(counts, 0)
+        if n:
+            total, most = torch.stack([prefix[-1], counts.max()]).tolist()
+        else:
+            total, most = 0, 0
+        ray_indices = torch.empty(total, dtype=torch.int64, device=dev)
+        t_nears = torch.empty(total, dtype=torch.float32, device=dev)
+        t_fars = torch.empty(total, dtype=torch.float32, device=dev)
+        if total:
+            with torch.cuda.device(dev):
+                if staged and most <= stride:
+                    self.check(
+                        self.lib.ash_ray_sample_compact(
+                            counts.data_ptr(), prefix.data_ptr(), stage.data_ptr(), stride, n,
+                            ray_indices.data_ptr(), t_nears.data_ptr(), t_fars.data_ptr(),
+                            _stream_of(dev),
+                        )
+                    )
+                else:
+                    self.check(
+                        self.lib.ash_ray_sample(
+                            *fixed, None, prefix.data_ptr(), ray_indices.data_ptr(),
+                            t_nears.data_ptr(), t_fars.data_ptr(), _stream_of(dev),
+                        )
+                    )
         return ray_indices, t_nears, t_fars, prefix
 
     # -- depth integration (no pybind counterpart: the reference's demo does

@@ -767,14 +767,18 @@ __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
 }
 
 // counts != nullptr: allocation pass; otherwise the assignment pass, which
-// writes the samples of ray i at prefix[i - 1] .. prefix[i].
+// writes the samples of ray i at prefix[i - 1] .. prefix[i].  An allocation
+// pass with `stage` also keeps the first `stride` samples of ray i as pairs
+// (t_near, t_far) at stage[2 * (i * stride + k)], so that the assignment pass
+// can be a copy instead of a second march.
 __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         MapDev m, const float* __restrict__ origins,
         const float* __restrict__ directions, const float* __restrict__ ray_nears,
         const float* __restrict__ ray_fars, int64_t n, float max_samples,
         float grid2cell, int64_t* __restrict__ counts,
         const int64_t* __restrict__ prefix, int64_t* __restrict__ ray_indices,
-        float* __restrict__ t_nears, float* __restrict__ t_fars) {
+        float* __restrict__ t_nears, float* __restrict__ t_fars,
+        float2* __restrict__ stage, int64_t stride) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     const bool active = i < n;
     const float cell2grid = static_cast<float>(1.0 / grid2cell);
@@ -808,6 +812,8 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
                     ray_indices[start + local] = i;
                     t_nears[start + local] = t_near;
                     t_fars[start + local] = t;
+                } else if (stage != nullptr && local < stride) {
+                    stage[i * stride + local] = make_float2(t_near, t);
                 }
                 t_near = t;
                 ++local;
@@ -818,6 +824,24 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         }
     }
     if (active && counts != nullptr) counts[i] = local;
+}
+
+// Assignment pass from the staged samples: one thread per staged slot.
+__global__ __launch_bounds__(kBlock) void ray_compact_kernel(
+        const int64_t* __restrict__ counts, const int64_t* __restrict__ prefix,
+        const float2* __restrict__ stage, int64_t stride, int64_t n,
+        int64_t* __restrict__ ray_indices, float* __restrict__ t_nears,
+        float* __restrict__ t_fars) {
+    const int64_t slot = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (slot >= n * stride) return;
+    const int64_t i = slot / stride;
+    const int64_t k = slot - i * stride;
+    if (k >= counts[i]) return;
+    const int64_t out = (i > 0 ? prefix[i - 1] : 0) + k;
+    const float2 s = stage[slot];
+    ray_indices[out] = i;
+    t_nears[out] = s.x;
+    t_fars[out] = s.y;
 }
 
 // Workgroup size of erase: the heap counter and the tombstone counter are each
@@ -1419,7 +1443,52 @@ int ash_ray_sample(ash_map_t* map, const float* ray_origins,
     ray_sample_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
             map->d, ray_origins, ray_directions, ray_nears, ray_fars, n,
             static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
-            prefix, ray_indices, t_nears, t_fars);
+            prefix, ray_indices, t_nears, t_fars, nullptr, 0);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_ray_sample_staged(ash_map_t* map, const float* ray_origins,
+                          const float* ray_directions, const float* ray_nears,
+                          const float* ray_fars, int64_t n, int64_t max_samples_per_ray,
+                          float grid2cell_multiplier, int64_t* counts, float* stage,
+                          int64_t stride, void* stream) {
+    if (check_batch(map, ray_origins, n)) return 1;
+    if (map->key_dim != 3) {
+        ASH_FAIL("hashmap is not a GPU hashmap of type <int, 3>, ray sample not supported");
+    }
+    if (!(grid2cell_multiplier > 0.f)) ASH_FAIL("grid2cell_multiplier must be positive");
+    if (max_samples_per_ray < 1) ASH_FAIL("max_samples_per_ray must be positive");
+    if (stride < 1) ASH_FAIL("ray_sample_staged: stride must be positive");
+    if (n == 0) return 0;
+    if (ray_directions == nullptr || ray_nears == nullptr || ray_fars == nullptr ||
+        counts == nullptr || stage == nullptr) {
+        ASH_FAIL("null pointer in ray_sample_staged");
+    }
+    if (reinterpret_cast<uintptr_t>(stage) % 8 != 0) ASH_FAIL("ray_sample_staged: stage must be 8-byte aligned");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    ray_sample_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+            map->d, ray_origins, ray_directions, ray_nears, ray_fars, n,
+            static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts, nullptr,
+            nullptr, nullptr, nullptr, reinterpret_cast<float2*>(stage), stride);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int ash_ray_sample_compact(const int64_t* counts, const int64_t* prefix, const float* stage,
+                           int64_t stride, int64_t n, int64_t* ray_indices, float* t_nears,
+                           float* t_fars, void* stream) {
+    if (n < 0 || stride < 1) ASH_FAIL("ray_sample_compact: bad sizes");
+    if (n == 0) return 0;
+    if (counts == nullptr || prefix == nullptr || stage == nullptr || ray_indices == nullptr ||
+        t_nears == nullptr || t_fars == nullptr) {
+        ASH_FAIL("null pointer in ray_sample_compact");
+    }
+    if (n > (int64_t{1} << 40) / stride) ASH_FAIL("ray_sample_compact: too many slots");
+    ray_compact_kernel<<<grid_for(n * stride), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+            counts, prefix, reinterpret_cast<const float2*>(stage), stride, n, ray_indices,
+            t_nears, t_fars);
     ASH_LAUNCH_CHECK();
     return 0;
 }
