@@ -104,3 +104,42 @@ def test_few_blocks_take_the_per_cell_kernel(gpu_ash, oracle):
         ref = oracle.convolution_forward(inputs, weights.view(27, channels), masks, gi, ci,
                                          g2g, c2c, c2g, 8)
         assert torch.equal(out.cpu(), ref)
+
+
+def test_tables_in_another_order_take_the_table_path(gpu_ash, oracle):
+    """The tiled kernel assumes the layout the Python layer builds and checks
+    the tables against it; taps listed in another order must give the same
+    result through the tables (weights permuted alike, so the sums differ only
+    in the order of their terms -- and that order is the tables')."""
+    grid, _, _ = workloads.build_grid(gpu_ash, 300, 5, 8, 32, device=DEV)
+    g = torch.Generator().manual_seed(820)
+    inputs = torch.randn(grid.embeddings.shape, generator=g).to(DEV)
+    weights = torch.randn(27, 5, generator=g).to(DEV)
+    c2g, c2c, g2g, gi, ci = _tables(grid, 1)
+    perm = torch.randperm(27, generator=g).to(DEV)
+    masks = torch.ones(inputs.shape[:2], dtype=torch.bool)
+    backend = gpu_ash.grid.backend
+    args = (masks, gi, ci, g2g, c2c[:, perm].contiguous(), c2g[:, perm].contiguous(), 8)
+    out = backend.convolution_forward(inputs, weights[perm].contiguous(), *args)
+    ref = oracle.convolution_forward(inputs, weights[perm].contiguous(), *args)
+    assert torch.equal(out.cpu(), ref)
+    # five channels through the tile: one pass of eight with three idle
+    plain = backend.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g, 8)
+    plain_ref = oracle.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g, 8)
+    assert torch.equal(plain.cpu(), plain_ref)
+    assert torch.allclose(out, plain, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("radius,channels", [(3, 5), (2, 16), (3, 16)])
+def test_wide_windows_and_rows(gpu_ash, oracle, radius, channels):
+    grid, _, _ = workloads.build_grid(gpu_ash, 200, channels, 8, 32, device=DEV)
+    g = torch.Generator().manual_seed(830 + radius)
+    inputs = torch.randn(grid.embeddings.shape, generator=g).to(DEV)
+    size = 2 * radius + 1
+    weights = torch.randn(size**3, channels, generator=g).to(DEV)
+    c2g, c2c, g2g, gi, ci = _tables(grid, radius)
+    masks = (torch.rand(inputs.shape[:2], generator=g) < 0.9)
+    args = (masks, gi, ci.view(-1)[torch.randperm(512, generator=g).to(DEV)], g2g, c2c, c2g, 8)
+    out = gpu_ash.grid.backend.convolution_forward(inputs, weights, *args)
+    ref = oracle.convolution_forward(inputs, weights, *args)
+    assert torch.equal(out.cpu(), ref)

@@ -26,6 +26,8 @@
 // one atomic per run (ray-ordered samples produce long runs).
 #include "ash_dev.h"
 
+#include <type_traits>
+
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
 #include <cstdlib>
@@ -618,7 +620,7 @@ __global__ __launch_bounds__(kBlock) void convolution_cell_kernel(ConvDev a, int
 // are kept in LDS in compact form (uint16 cell, uint8 block offset) for the
 // whole launch, when they fit.  Taps, order and arithmetic are unchanged.
 constexpr int kConvThreads = 512;
-unsigned persistent_grid(int64_t ntiles, size_t smem);
+unsigned persistent_grid(int64_t ntiles, size_t smem, int max_per_cu = 8);
 
 template <typename T, int EC>
 __global__ __launch_bounds__(kConvThreads) void convolution_block_kernel(
@@ -746,6 +748,313 @@ int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
     return 0;
 }
 
+// Cube windows over cubic blocks in the layout the Python layer builds
+// (cell c = x + G y + G^2 z; tap k = (dx + r) + W (dy + r) + W^2 (dz + r) with
+// W = 2 r + 1; neighbour block (bx + 1) + 3 (by + 1) + 9 (bz + 1)): the block's
+// cells together with their halo of r cells, (G + 2r)^3 rows of EC channels,
+// are staged in LDS once per block, and every cell then reads its W^3 taps from
+// there -- in table order, one fused multiply-add per tap and channel, like the
+// other kernels.  Rows of missing blocks are staged as zeros: with finite
+// weights adding 0 * w leaves the accumulator as it is (it starts at +0 and so
+// never is -0), which is what skipping the tap does.  Every workgroup first
+// checks the two per-cell tables against this layout and, should they describe
+// something else, takes its blocks through the tables instead.
+template <typename T, int EC, int WT>
+__global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
+        ConvDev a, int G, int r, int e0, int ec, int vec) {
+    extern __shared__ __align__(16) unsigned char conv_smem[];
+    __shared__ int64_t s_nb[2][28];   // rows of 27 neighbour blocks + the block itself
+    __shared__ int s_bad;
+    const int tid = threadIdx.x;
+    const int E = static_cast<int>(a.E);
+    const int M = static_cast<int>(a.M);
+    const int K = static_cast<int>(a.K);
+    const int W = WT > 0 ? WT : 2 * r + 1;   // WT: window edge known at compile time
+    const int Tn = G + 2 * r;
+    const int T3 = Tn * Tn * Tn;
+    T* tile = reinterpret_cast<T*>(conv_smem);                             // [T3][EC]
+    T* s_w = tile + static_cast<size_t>(T3) * EC;                          // [K][EC]
+    uint32_t* s_src = reinterpret_cast<uint32_t*>(s_w + static_cast<size_t>(K) * EC);  // [T3]
+    const T* in = static_cast<const T*>(a.in);
+    const T* w = static_cast<const T*>(a.w);
+    T* out = static_cast<T*>(a.out);
+
+    if (tid == 0) s_bad = 0;
+    __syncthreads();
+    {
+        int bad = 0;
+        for (int t = tid; t < M * K; t += kConvThreads) {
+            const int c = t / K;
+            const int k = t - c * K;
+            const int x[3] = {c % G, (c / G) % G, c / (G * G)};
+            const int o[3] = {k % W - r, (k / W) % W - r, k / (W * W) - r};
+            int gn = 0, ci = 0, gs = 1, cs = 1;
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                const int t_d = x[d] + o[d];
+                const int b = t_d < 0 ? -1 : (t_d >= G ? 1 : 0);
+                gn += (b + 1) * gs;
+                ci += (t_d - b * G) * cs;
+                gs *= 3;
+                cs *= G;
+            }
+            bad |= a.lut_c2g[t] != gn || a.lut_c2c[t] != ci;
+        }
+        if (bad) s_bad = 1;
+        // where every row of the tile comes from: neighbour block << 12 | cell
+        for (int p = tid; p < T3; p += kConvThreads) {
+            const int tx[3] = {p % Tn - r, (p / Tn) % Tn - r, p / (Tn * Tn) - r};
+            int gn = 0, ci = 0, gs = 1, cs = 1;
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                const int b = tx[d] < 0 ? -1 : (tx[d] >= G ? 1 : 0);
+                gn += (b + 1) * gs;
+                ci += (tx[d] - b * G) * cs;
+                gs *= 3;
+                cs *= G;
+            }
+            s_src[p] = static_cast<uint32_t>((gn << 12) | ci);
+        }
+        for (int t = tid; t < K * EC; t += kConvThreads) {
+            const int k = t / EC;
+            const int q = t - k * EC;
+            s_w[t] = q < ec ? w[k * E + e0 + q] : T(0);
+        }
+    }
+    __syncthreads();
+    const bool by_table = s_bad != 0;
+
+    for (int64_t blk = blockIdx.x; by_table && blk < a.n_grids; blk += gridDim.x) {
+        const int64_t g = a.grid_indices[blk];
+        if (g < 0 || g >= a.B) continue;  // the same for the whole workgroup
+        {
+            const int64_t* nb_g = a.lut_g + g * a.GN;
+            for (int c_i = tid; c_i < M; c_i += kConvThreads) {
+                if (!a.masks[blk * a.M + c_i]) continue;
+                const int64_t c = a.cell_indices[c_i];
+                if (c < 0 || c >= a.M) continue;
+                T acc[EC];
+#pragma unroll
+                for (int q = 0; q < EC; ++q) acc[q] = T(0);
+                for (int k = 0; k < K; ++k) {
+                    const int64_t gn = a.lut_c2g[c * K + k];
+                    if (gn < 0 || gn >= a.GN) continue;
+                    const int64_t gi = nb_g[gn];
+                    if (gi < 0 || gi >= a.B) continue;
+                    const int64_t ci = a.lut_c2c[c * K + k];
+                    if (ci < 0 || ci >= a.M) continue;
+#pragma unroll
+                    for (int q = 0; q < EC; ++q) {
+                        if (q < ec) {
+                            acc[q] = fma(in[(gi * a.M + ci) * E + e0 + q], s_w[k * EC + q], acc[q]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < EC; ++q) {
+                    if (q < ec) out[(g * a.M + c) * E + e0 + q] = acc[q];
+                }
+            }
+        }
+    }
+    if (by_table) return;
+
+    // Blocks through the tile, software-pipelined: while a block is computed
+    // from LDS, the rows of the next block's tile are already on their way
+    // into registers and the row numbers of the block after that are fetched.
+    constexpr int kPre = EC >= 16 ? 2 : (EC >= 8 ? 4 : 6);   // tile rows a thread can hold
+    const bool prefetch = T3 <= kPre * kConvThreads;
+    auto fetch_rows = [&](int64_t b) -> int64_t {  // lanes 0..26 neighbours, 27 the block
+        if (tid > 27 || b >= a.n_grids) return -1;
+        const int64_t g = a.grid_indices[b];
+        if (g < 0 || g >= a.B) return -1;
+        if (tid == 27) return g;
+        const int64_t row = a.lut_g[g * 27 + tid];
+        return (row >= 0 && row < a.B) ? row : -1;
+    };
+    auto load_row = [&](const int64_t* nb, int p, T (&v)[EC]) {
+#pragma unroll
+        for (int q = 0; q < EC; ++q) v[q] = T(0);
+        if (p >= T3) return;
+        const uint32_t src_cell = s_src[p];
+        const int64_t row = nb[src_cell >> 12];
+        if (row < 0) return;
+        const T* src = in + (row * a.M + (src_cell & 0xFFF)) * E + e0;
+        if (vec) {   // EC is a multiple of four here
+#pragma unroll
+            for (int q4 = 0; q4 < (EC + 3) / 4; ++q4) {
+                const float4 f = reinterpret_cast<const float4*>(src)[q4];
+                v[(4 * q4) % EC] = f.x;
+                v[(4 * q4 + 1) % EC] = f.y;
+                v[(4 * q4 + 2) % EC] = f.z;
+                v[(4 * q4 + 3) % EC] = f.w;
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < EC; ++q) {
+                if (q < ec) v[q] = src[q];
+            }
+        }
+    };
+    int64_t blk = blockIdx.x;
+    int buf = 0;
+    int64_t rows_reg = fetch_rows(blk);
+    if (tid <= 27) s_nb[0][tid] = rows_reg;
+    rows_reg = fetch_rows(blk + gridDim.x);
+    __syncthreads();
+    T pre[kPre][EC];
+    if (prefetch) {
+#pragma unroll
+        for (int i = 0; i < kPre; ++i) load_row(s_nb[0], tid + i * kConvThreads, pre[i]);
+    }
+    for (; blk < a.n_grids; blk += gridDim.x, buf ^= 1) {
+        __syncthreads();  // the previous block's tile has been read
+        const int64_t g = s_nb[buf][27];
+        if (prefetch) {
+#pragma unroll
+            for (int i = 0; i < kPre; ++i) {
+                const int p = tid + i * kConvThreads;
+                if (p < T3) {
+#pragma unroll
+                    for (int q = 0; q < EC; ++q) tile[p * EC + q] = pre[i][q];
+                }
+            }
+        } else {
+            for (int p = tid; p < T3; p += kConvThreads) {
+                T v[EC];
+                load_row(s_nb[buf], p, v);
+#pragma unroll
+                for (int q = 0; q < EC; ++q) tile[p * EC + q] = v[q];
+            }
+        }
+        if (tid <= 27) s_nb[buf ^ 1][tid] = rows_reg;
+        __syncthreads();
+        rows_reg = fetch_rows(blk + 2 * static_cast<int64_t>(gridDim.x));
+        if (prefetch && blk + gridDim.x < a.n_grids) {
+#pragma unroll
+            for (int i = 0; i < kPre; ++i) load_row(s_nb[buf ^ 1], tid + i * kConvThreads, pre[i]);
+        }
+        if (g < 0) continue;  // the same for the whole workgroup
+        for (int c_i = tid; c_i < M; c_i += kConvThreads) {
+            if (!a.masks[blk * a.M + c_i]) continue;
+            const int64_t c64 = a.cell_indices[c_i];
+            if (c64 < 0 || c64 >= a.M) continue;
+            const int c = static_cast<int>(c64);
+            // tile index of the tap (-r, -r, -r) of this cell
+            const int base = c % G + Tn * ((c / G) % G) + Tn * Tn * (c / (G * G));
+            T acc[EC];
+#pragma unroll
+            for (int q = 0; q < EC; ++q) acc[q] = T(0);
+            // only the innermost loop is unrolled: a fully unrolled window keeps
+            // hundreds of values in flight and costs the occupancy
+#pragma unroll 1
+            for (int dz = 0; dz < W; ++dz) {
+#pragma unroll 1
+                for (int dy = 0; dy < W; ++dy) {
+                    const T* row = tile + static_cast<size_t>(base + Tn * dy + Tn * Tn * dz) * EC;
+                    const T* wrow = s_w + static_cast<size_t>((dz * W + dy) * W) * EC;
+                    if constexpr (WT > 0) {
+#pragma unroll
+                        for (int dx = 0; dx < WT; ++dx) {
+#pragma unroll
+                            for (int q = 0; q < EC; ++q) {
+                                acc[q] = fma(row[dx * EC + q], wrow[dx * EC + q], acc[q]);
+                            }
+                        }
+                    } else {
+                        for (int dx = 0; dx < W; ++dx) {
+#pragma unroll
+                            for (int q = 0; q < EC; ++q) {
+                                acc[q] = fma(row[dx * EC + q], wrow[dx * EC + q], acc[q]);
+                            }
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < EC; ++q) {
+                if (q < ec) out[(g * a.M + c) * E + e0 + q] = acc[q];
+            }
+        }
+    }
+}
+
+#ifndef ASH_CONV_TILE_MIN_TAPS
+#define ASH_CONV_TILE_MIN_TAPS 27
+#endif
+constexpr int kTileMinTaps = ASH_CONV_TILE_MIN_TAPS;
+#ifndef ASH_CONV_TILE_BYTES
+#define ASH_CONV_TILE_BYTES (64 * 1024)
+#endif
+constexpr size_t kConvTileBytes = ASH_CONV_TILE_BYTES;   // LDS a tile may take
+
+// Largest cube edge G with G^3 == m, or 0.
+inline int cube_edge(int64_t m) {
+    int g = 1;
+    while (static_cast<int64_t>(g) * g * g < m) ++g;
+    return static_cast<int64_t>(g) * g * g == m ? g : 0;
+}
+
+// Takes the tile kernel when the sizes describe a cube window over cubic
+// blocks with 27 neighbour blocks and the tile fits; returns -1 when not.
+template <typename T>
+int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
+    const int G = cube_edge(a.M);
+    const int W = cube_edge(a.K);
+    if (G == 0 || W < 3 || W % 2 == 0 || a.GN != 27 || a.n_grids < 64) return -1;
+    const int r = W / 2;
+    if (r > G || a.M > 4096 || a.M * a.K > (int64_t{1} << 30)) return -1;
+    const int64_t Tn = G + 2 * r;
+    // As many channels per pass as fit: a pass fetches the cache lines of all
+    // channels of a row whatever it uses of them.
+    constexpr int kMaxEc = sizeof(T) == 4 ? 16 : 8;
+    const size_t cell_bytes = static_cast<size_t>(Tn * Tn * Tn) * sizeof(T);
+    int ec_max = kMaxEc;
+    while (ec_max > 1 && cell_bytes * ec_max > kConvTileBytes) ec_max /= 2;
+    if (cell_bytes * ec_max > kConvTileBytes) return -1;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(a.in);
+    for (int e0 = 0; e0 < a.E;) {
+        int width = ec_max;                  // channels of the template instance
+        while (width > 1 && width / 2 >= a.E - e0) width /= 2;
+        const int ec = static_cast<int>(a.E - e0 < width ? a.E - e0 : width);
+        const size_t smem = (cell_bytes + static_cast<size_t>(a.K) * sizeof(T)) * width +
+                            static_cast<size_t>(Tn * Tn * Tn) * 4 + 16;
+        const int vec = (sizeof(T) == 4 && ec == width && width % 4 == 0 && a.E % 4 == 0 &&
+                         e0 % 4 == 0 && align % 16 == 0) ? 1 : 0;
+        const unsigned grid = persistent_grid(a.n_grids, smem + 512, 2048 / kConvThreads);
+        auto launch = [&](auto kernel) -> int {
+            ASH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        static_cast<int>(smem)));
+            kernel<<<grid, kConvThreads, smem, s>>>(a, G, r, e0, ec, vec);
+            ASH_LAUNCH_CHECK();
+            return 0;
+        };
+        auto by_window = [&](auto ec_tag) -> int {
+            constexpr int kEc = decltype(ec_tag)::value;
+            if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3>);
+            if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5>);
+            if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7>);
+            return launch(convolution_tile_kernel<T, kEc, 0>);
+        };
+        int rc = 1;
+        if (width == 16) {
+            if constexpr (kMaxEc >= 16) rc = by_window(std::integral_constant<int, 16>());
+        } else if (width == 8) {
+            rc = by_window(std::integral_constant<int, 8>());
+        } else if (width == 4) {
+            rc = by_window(std::integral_constant<int, 4>());
+        } else if (width == 2) {
+            rc = by_window(std::integral_constant<int, 2>());
+        } else {
+            rc = by_window(std::integral_constant<int, 1>());
+        }
+        if (rc) return 1;
+        e0 += ec;
+    }
+    return 0;
+}
+
 template <typename T>
 int launch_convolution_cells(const ConvDev& a, hipStream_t s) {
     const int64_t threads = a.n_grids * a.M;
@@ -754,6 +1063,10 @@ int launch_convolution_cells(const ConvDev& a, hipStream_t s) {
     const unsigned gb = static_cast<unsigned>(blocks);
     const uintptr_t align = reinterpret_cast<uintptr_t>(a.in) | reinterpret_cast<uintptr_t>(a.out);
     const int vec4 = (sizeof(T) == 4 && a.E % 4 == 0 && align % 16 == 0) ? 1 : 0;
+    if (a.K >= kTileMinTaps) {
+        const int rc = launch_convolution_tile<T>(a, s);
+        if (rc >= 0) return rc;
+    }
     if (a.n_grids >= 64 && a.M <= 4096) {
         // enough blocks to keep persistent workgroups busy
         if (a.E <= 1) return launch_convolution_block<T, 1>(a, vec4, s);
@@ -920,7 +1233,7 @@ size_t smem_bytes(const QDev& d, int lpq) {
 }
 
 // Enough persistent workgroups to fill every CU as far as LDS allows.
-unsigned persistent_grid(int64_t ntiles, size_t smem) {
+unsigned persistent_grid(int64_t ntiles, size_t smem, int max_per_cu) {
     static int cus = 0;
     if (cus == 0) {
         int dev = 0, n = 0;
@@ -933,7 +1246,7 @@ unsigned persistent_grid(int64_t ntiles, size_t smem) {
             cus = 256;
         }
     }
-    int per_cu = 8;
+    int per_cu = max_per_cu;
     if (smem > 0) {
         const int fit = static_cast<int>(kLdsPerCu / smem);
         if (fit < per_cu) per_cu = fit < 1 ? 1 : fit;
