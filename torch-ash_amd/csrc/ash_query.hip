@@ -759,7 +759,7 @@ int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
 // never is -0), which is what skipping the tap does.  Every workgroup first
 // checks the two per-cell tables against this layout and, should they describe
 // something else, takes its blocks through the tables instead.
-template <typename T, int EC, int WT>
+template <typename T, int EC, int WT, bool YB>
 __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         ConvDev a, int G, int r, int e0, int ec, int vec) {
     extern __shared__ __align__(16) unsigned char conv_smem[];
@@ -775,6 +775,11 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
     T* tile = reinterpret_cast<T*>(conv_smem);                             // [T3][EC]
     T* s_w = tile + static_cast<size_t>(T3) * EC;                          // [K][EC]
     uint32_t* s_src = reinterpret_cast<uint32_t*>(s_w + static_cast<size_t>(K) * EC);  // [T3]
+    uint16_t* s_inv = reinterpret_cast<uint16_t*>(s_src + T3);   // [M] position of a cell in cell_indices (YB)
+    // YB keeps one plane per channel (a lane reads runs of one channel along
+    // x), otherwise the channels of a row sit together.
+    auto tile_at = [&](int p, int q) { return YB ? q * T3 + p : p * EC + q; };
+    auto w_at = [&](int k, int q) { return YB ? q * K + k : k * EC + q; };
     const T* in = static_cast<const T*>(a.in);
     const T* w = static_cast<const T*>(a.w);
     T* out = static_cast<T*>(a.out);
@@ -818,7 +823,17 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         for (int t = tid; t < K * EC; t += kConvThreads) {
             const int k = t / EC;
             const int q = t - k * EC;
-            s_w[t] = q < ec ? w[k * E + e0 + q] : T(0);
+            s_w[w_at(k, q)] = q < ec ? w[k * E + e0 + q] : T(0);
+        }
+        if constexpr (YB) {
+            for (int c = tid; c < M; c += kConvThreads) s_inv[c] = 0xFFFFu;
+        }
+    }
+    __syncthreads();
+    if constexpr (YB) {
+        for (int c_i = tid; c_i < M; c_i += kConvThreads) {
+            const int64_t c = a.cell_indices[c_i];
+            if (c >= 0 && c < a.M) s_inv[c] = static_cast<uint16_t>(c_i);
         }
     }
     __syncthreads();
@@ -846,7 +861,7 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
 #pragma unroll
                     for (int q = 0; q < EC; ++q) {
                         if (q < ec) {
-                            acc[q] = fma(in[(gi * a.M + ci) * E + e0 + q], s_w[k * EC + q], acc[q]);
+                            acc[q] = fma(in[(gi * a.M + ci) * E + e0 + q], s_w[w_at(k, q)], acc[q]);
                         }
                     }
                 }
@@ -916,7 +931,7 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                 const int p = tid + i * kConvThreads;
                 if (p < T3) {
 #pragma unroll
-                    for (int q = 0; q < EC; ++q) tile[p * EC + q] = pre[i][q];
+                    for (int q = 0; q < EC; ++q) tile[tile_at(p, q)] = pre[i][q];
                 }
             }
         } else {
@@ -924,7 +939,7 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                 T v[EC];
                 load_row(s_nb[buf], p, v);
 #pragma unroll
-                for (int q = 0; q < EC; ++q) tile[p * EC + q] = v[q];
+                for (int q = 0; q < EC; ++q) tile[tile_at(p, q)] = v[q];
             }
         }
         if (tid <= 27) s_nb[buf ^ 1][tid] = rows_reg;
@@ -935,6 +950,61 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             for (int i = 0; i < kPre; ++i) load_row(s_nb[buf ^ 1], tid + i * kConvThreads, pre[i]);
         }
         if (g < 0) continue;  // the same for the whole workgroup
+        if constexpr (YB) {
+            // One lane = one channel of four cells that follow each other in y.
+            // For every (dz, dy) the W weights of the tap row are read once and
+            // used by all four cells, and the four tile rows they meet stay in
+            // registers from one dy to the next (row dy + j serves cell j), so
+            // that a step costs one new tile row and one weight row for
+            // 4 W fused multiply-adds.  Every cell still sees its taps in table
+            // order: dz, then dy, then dx.
+            const int yq_n = G / 4;
+            const int combos = G * yq_n * G;
+            for (int item = tid; item < combos * EC; item += kConvThreads) {
+                const int q = item / combos;
+                if (q >= ec) continue;
+                const int rem = item - q * combos;
+                const int x = rem % G;
+                const int y0 = 4 * ((rem / G) % yq_n);
+                const int z = rem / (G * yq_n);
+                const T* plane = tile + static_cast<size_t>(q) * T3 + x + Tn * y0 + Tn * Tn * z;
+                const T* wq = s_w + static_cast<size_t>(q) * K;
+                T acc[4] = {T(0), T(0), T(0), T(0)};
+#pragma unroll 1
+                for (int dz = 0; dz < WT; ++dz) {
+                    const T* pz = plane + Tn * Tn * dz;
+                    T win[4][WT > 0 ? WT : 1];
+#pragma unroll
+                    for (int yy = 0; yy < 3; ++yy) {
+#pragma unroll
+                        for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
+                    }
+#pragma unroll
+                    for (int dy = 0; dy < WT; ++dy) {
+#pragma unroll
+                        for (int dx = 0; dx < WT; ++dx) win[(dy + 3) & 3][dx] = pz[Tn * (dy + 3) + dx];
+                        T wr[WT > 0 ? WT : 1];
+#pragma unroll
+                        for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                            for (int dx = 0; dx < WT; ++dx) {
+                                acc[j] = fma(win[(dy + j) & 3][dx], wr[dx], acc[j]);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int c = x + G * (y0 + j) + G * G * z;
+                    const int c_i = s_inv[c];
+                    if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
+                    out[(g * a.M + c) * E + e0 + q] = acc[j];
+                }
+            }
+            continue;
+        }
         for (int c_i = tid; c_i < M; c_i += kConvThreads) {
             if (!a.masks[blk * a.M + c_i]) continue;
             const int64_t c64 = a.cell_indices[c_i];
@@ -987,6 +1057,10 @@ constexpr int kTileMinTaps = ASH_CONV_TILE_MIN_TAPS;
 #define ASH_CONV_TILE_BYTES (64 * 1024)
 #endif
 constexpr size_t kConvTileBytes = ASH_CONV_TILE_BYTES;   // LDS a tile may take
+#ifndef ASH_CONV_ROW_BLOCKING
+#define ASH_CONV_ROW_BLOCKING 1
+#endif
+constexpr bool kConvRowBlocking = ASH_CONV_ROW_BLOCKING != 0;
 
 // Largest cube edge G with G^3 == m, or 0.
 inline int cube_edge(int64_t m) {
@@ -1018,7 +1092,7 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
         while (width > 1 && width / 2 >= a.E - e0) width /= 2;
         const int ec = static_cast<int>(a.E - e0 < width ? a.E - e0 : width);
         const size_t smem = (cell_bytes + static_cast<size_t>(a.K) * sizeof(T)) * width +
-                            static_cast<size_t>(Tn * Tn * Tn) * 4 + 16;
+                            static_cast<size_t>(Tn * Tn * Tn) * 4 + static_cast<size_t>(a.M) * 2 + 16;
         const int vec = (sizeof(T) == 4 && ec == width && width % 4 == 0 && a.E % 4 == 0 &&
                          e0 % 4 == 0 && align % 16 == 0) ? 1 : 0;
         const unsigned grid = persistent_grid(a.n_grids, smem + 512, 2048 / kConvThreads);
@@ -1032,10 +1106,15 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
         };
         auto by_window = [&](auto ec_tag) -> int {
             constexpr int kEc = decltype(ec_tag)::value;
-            if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3>);
-            if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5>);
-            if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7>);
-            return launch(convolution_tile_kernel<T, kEc, 0>);
+            if (G % 4 == 0 && kConvRowBlocking) {
+                if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, true>);
+                if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, true>);
+                if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, true>);
+            }
+            if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, false>);
+            if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, false>);
+            if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, false>);
+            return launch(convolution_tile_kernel<T, kEc, 0, false>);
         };
         int rc = 1;
         if (width == 16) {
