@@ -143,3 +143,49 @@ def test_wide_windows_and_rows(gpu_ash, oracle, radius, channels):
     out = gpu_ash.grid.backend.convolution_forward(inputs, weights, *args)
     ref = oracle.convolution_forward(inputs, weights, *args)
     assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("radius", [1, 3])
+def test_impulse_and_constant_field_on_a_dense_volume(gpu_ash, radius):
+    """Independent of the oracle: on a dense volume an impulse at cell p gives
+    out[p - o_k] = w[k] (tap k reads the cell at offset o_k), and a field of
+    ones gives the sum of the weights, added in table order, at every cell
+    whose window lies inside the volume."""
+    s, g_dim, e = 5, 8, 4
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, s**3, e, grid_dim=g_dim, sparse_grid_dim=s, bbox_min=torch.zeros(3),
+        bbox_max=torch.ones(3), device=DEV)
+    grid.dense_init_()
+    keys, idx = grid.engine.items()
+    size = 2 * radius + 1
+    g = torch.Generator().manual_seed(840 + radius)
+    weights = torch.randn(size, size, size, e, generator=g).to(DEV)
+    n = s * g_dim
+    # dense view of a (B, M, E) tensor: vol[x, y, z, :]
+    cells = (keys.view(-1, 1, 3) * g_dim + grid.cell_coords.view(1, -1, 3)).long()
+
+    def densify(t):
+        vol = torch.zeros(n, n, n, e, device=DEV)
+        vol[cells[..., 0], cells[..., 1], cells[..., 2]] = t[idx]
+        return vol
+
+    p = torch.tensor([17, 22, 19], device=DEV)
+    inputs = torch.zeros(grid.embeddings.shape, device=DEV)
+    block = (keys == (p // g_dim).int()).all(dim=1).nonzero().item()
+    local = p % g_dim
+    inputs[idx[block], local[0] + g_dim * local[1] + g_dim**2 * local[2]] = 1.0
+    vol = densify(grid.convolution(inputs, weights))
+    lo, hi = p - radius, p + radius + 1
+    patch = vol[lo[0]:hi[0], lo[1]:hi[1], lo[2]:hi[2]]
+    # weights[i, j, k] belongs to the offset (k, j, i) - radius: x varies fastest
+    expect = weights.permute(2, 1, 0, 3).flip(0, 1, 2)
+    assert torch.equal(patch, expect)
+    assert int((vol != 0).sum()) == int((expect != 0).sum())
+
+    ones = torch.ones(grid.embeddings.shape, device=DEV)
+    vol = densify(grid.convolution(ones, weights))
+    total = torch.zeros(e)
+    for row in weights.view(-1, e).cpu():
+        total = total + row          # fma(1, w, acc) in table order
+    inner = vol[radius:n - radius, radius:n - radius, radius:n - radius]
+    assert torch.equal(inner.reshape(-1, e).cpu(), total.expand(inner.numel() // e, e))
