@@ -884,6 +884,11 @@ class _HashMap:
         return st if st is not None else self.status()
 
     def size(self) -> int:
+        # every insert / load / activation ends with one read-back of the
+        # counters; until the next erase or clear that read-back still holds
+        st = getattr(self, "_status_after_insert", None)
+        if st is not None:
+            return st["size"]
         n = _I64(0)
         with torch.cuda.device(self._device):
             self._check(self._lib.ash_map_size(self._handle, ctypes.byref(n), self._stream()))
