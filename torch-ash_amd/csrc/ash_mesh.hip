@@ -1058,13 +1058,15 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
     const int64_t cells = num_grids * cells_per_grid;
     const int64_t chunks = (cells + kChunk - 1) / kChunk;
     if (num_grids > 0) {
-        const bool tiled = grid_dim <= kMaxTileG &&
+        const size_t cell_bytes = dtype == ASH_F32 ? 4 : 8;
+        const size_t lds = (cell_bytes + 3) * tile_cells(grid_dim < 64 ? grid_dim : 64) +
+                           2 * static_cast<size_t>(cells_per_grid);
+        // the tile has to fit the 64 KB a launch may take without further ado
+        const bool tiled = grid_dim <= kMaxTileG && lds <= 63 * 1024 &&
                            static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
         if (tiled) {
             const unsigned by_block =
                     static_cast<unsigned>(num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid);
-            const size_t cell_bytes = dtype == ASH_F32 ? 4 : 8;
-            const size_t lds = (cell_bytes + 3) * tile_cells(grid_dim) + 2 * cells_per_grid;
             if (dtype == ASH_F32) {
                 iso_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
             } else {
