@@ -402,3 +402,48 @@ def test_optional_gradient_outputs(gpu_ash, oracle):
         assert grid.embeddings.grad is not None
     finally:
         del backend.query_backward_forward
+
+
+def test_query_and_find_replay_in_a_hip_graph(gpu_ash):
+    """The library allocates nothing, synchronises nowhere on these paths and
+    clears its outputs with kernels, so the query kernels and the table look-up
+    can be captured once and replayed; every replay is checked against the
+    eager result on the inputs of that replay."""
+    grid = _make_grid(gpu_ash, 4, 4, 2, seed=31, holes=6)
+    backend = gpu_ash.grid_query.backend
+    g = torch.Generator().manual_seed(32)
+    x = _queries(4, 2, 20_000, 33)
+    gi, ci, off, mk = grid.query(x.to(DEV))
+    emb = grid.embeddings.detach().clone()
+    z = torch.rand(x.shape[0], 4, generator=g).to(DEV) - 0.5
+    tables = (grid.lut_grid_nb2grid_idx, grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)
+    keys = (torch.randint(-3, 4, (5000, 3), generator=g) ).int().to(DEV)
+
+    def run():
+        out = backend.query_forward(emb, off, gi, ci, mk, *tables, 4, "smooth_step")
+        g_emb, g_off = backend.query_backward_forward(z, emb, off, gi, ci, mk, *tables, 4,
+                                                      "smooth_step")
+        idx, found = grid.engine.find(keys)
+        return out, g_emb, g_off, idx, found
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for trial in range(3):
+        emb.copy_((torch.rand(emb.shape, generator=g) * 2 - 1).to(DEV))
+        z.copy_((torch.rand(z.shape, generator=g) - 0.5).to(DEV))
+        keys.copy_(torch.randint(-3, 4, (5000, 3), generator=g).int().to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = run()
+        torch.cuda.synchronize()
+        assert torch.equal(captured[0], eager[0])
+        assert torch.allclose(captured[1], eager[1], rtol=1e-4, atol=1e-5)   # atomic order
+        assert torch.allclose(captured[2], eager[2], rtol=1e-5, atol=1e-6)
+        assert torch.equal(captured[3], eager[3]) and torch.equal(captured[4], eager[4])
+        assert int(eager[4].sum()) > 100 and float(eager[1].abs().sum()) > 1.0
