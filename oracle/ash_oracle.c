@@ -1,5 +1,6 @@
 /*
- * ash_oracle.c -- CPU restatement of torch-ash's hash map and trilinear query.
+ * ash_oracle.c -- CPU restatement of torch-ash's hash map, trilinear query and
+ * the grid functions around them.
  *
  * TEST INFRASTRUCTURE ONLY.  This file is the checker for the HIP library: it
  * is called from tests/, from __graft_entry__.smoke() and from the
@@ -24,7 +25,19 @@
  *     except through the order of items(), which every caller sorts away.
  *   - the three query kernels of ash/src/grid.cu (:68-132, :177-255, :309-387)
  *     with their interpolation functors (:7-41), in the same operation order
- *     and in the same scalar type.
+ *     and in the same scalar type;
+ *   - the callers either side of those paths: the ray marches of
+ *     ash/src/sampler.cu, the sparse convolution (grid.cu:951-1006), the
+ *     iso-surface point extraction (grid.cu:453-531) and marching cubes
+ *     (grid.cu:606-946), each described at its function below.
+ *
+ * Marching cubes: the 256-row case table of the reference (mc_macros.h) is not
+ * restated here; the functions take a table as an argument, and the tests pass
+ * the one that the library's generator derives from the cube.  That table is
+ * pinned against the reference case by case in the outline, the facing and the
+ * number of triangles of every patch, and by the geometry of the meshes it
+ * gives; how a polygon of more than three corners is cut into triangles is the
+ * generator's choice, so the triangle list is "parity unpinned" beyond that.
  *
  * Where the reference has undefined behaviour (inserting more distinct keys
  * than `capacity` reads past the heap, ash/src/hashmap_gpu.cuh:226-227) the
@@ -32,7 +45,9 @@
  *
  * Parity pins: see tests/test_oracle_*.py (dictionary model, the invariants of
  * the reference's unittests, closed forms, torch.nn.functional.grid_sample,
- * float64 autograd of an independent formula, finite differences).
+ * float64 autograd of an independent formula, finite differences; hand-derived
+ * marches, dense conv3d, spheres / tori / brute-force counts for the surface
+ * functions).
  *
  * With OpenMP (-fopenmp) the loops over keys / queries run in parallel, which
  * is what bench.py times as the CPU baseline; with one thread the key loops
