@@ -189,3 +189,28 @@ def test_impulse_and_constant_field_on_a_dense_volume(gpu_ash, radius):
         total = total + row          # fma(1, w, acc) in table order
     inner = vol[radius:n - radius, radius:n - radius, radius:n - radius]
     assert torch.equal(inner.reshape(-1, e).cpu(), total.expand(inner.numel() // e, e))
+
+
+@pytest.mark.parametrize("grid_dim,radius,channels", [(4, 1, 3), (4, 2, 2), (16, 1, 2), (6, 2, 4),
+                                                      (12, 3, 1)])
+def test_other_block_edges(gpu_ash, oracle, grid_dim, radius, channels):
+    """Block edges that are and are not multiples of four (the latter compute
+    one cell per lane), windows reaching two blocks deep into a small block."""
+    s = 5
+    g = torch.Generator().manual_seed(850 + grid_dim)
+    blocks = torch.stack(torch.meshgrid(*[torch.arange(s)] * 3, indexing="ij"), -1).view(-1, 3)
+    blocks = blocks[torch.rand(len(blocks), generator=g) < 0.8]
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, len(blocks) + 3, channels, grid_dim=grid_dim, sparse_grid_dim=s,
+        bbox_min=torch.zeros(3), bbox_max=torch.ones(3), device=DEV)
+    grid.engine.insert_keys(blocks.int().to(DEV))
+    assert grid.engine.size() >= 64
+    inputs = torch.randn(grid.embeddings.shape, generator=g).to(DEV)
+    size = 2 * radius + 1
+    weights = torch.randn(size**3, channels, generator=g).to(DEV)
+    c2g, c2c, g2g, gi, ci = _tables(grid, radius)
+    masks = torch.ones(inputs.shape[:2], dtype=torch.bool)
+    out = gpu_ash.grid.backend.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g,
+                                                   grid_dim)
+    ref = oracle.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g, grid_dim)
+    assert torch.equal(out.cpu(), ref) and float(ref.abs().max()) > 1.0
