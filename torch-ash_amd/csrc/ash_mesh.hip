@@ -482,7 +482,8 @@ __global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int6
     for (int which = 0; which < arrays; ++which) {
         int32_t* counts = ws + kMcHeader + which * chunks;
         int64_t mine = 0;
-        for (int64_t i = lo; i < hi; ++i) mine += counts[i];
+#pragma unroll 8
+        for (int64_t i = lo; i < hi; ++i) mine += counts[i];   // independent loads
         __syncthreads();
         s_sum[threadIdx.x] = mine;
         __syncthreads();
@@ -493,6 +494,7 @@ __global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int6
             __syncthreads();
         }
         int64_t run = s_sum[threadIdx.x] - mine;
+#pragma unroll 8
         for (int64_t i = lo; i < hi; ++i) {
             const int32_t n = counts[i];
             counts[i] = static_cast<int32_t>(run < 0x7FFFFFFF ? run : 0x7FFFFFFF);
@@ -542,7 +544,7 @@ __device__ __forceinline__ void write_edge_points(const McDev& a, int64_t g, int
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
     __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
-    __shared__ int32_t s_id[kChunk];      // id of its first vertex
+    __shared__ uint16_t s_id[kChunk];     // id of its first vertex, from the chunk's first
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint64_t flags = 0;   // 3 bits per own cell
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
                 int& at = part[j / VEC];
                 s_cell[at & 0xFFFF] =
                         static_cast<uint16_t>((own_group_offset<VEC>(j / VEC) + j % VEC) | (f << 12));
-                s_id[at & 0xFFFF] = first + (at >> 16);
+                s_id[at & 0xFFFF] = static_cast<uint16_t>(at >> 16);
                 at += 1 + (__popc(f) << 16);
             }
         }
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
             const int f = s_cell[q] >> 12;
             int64_t g, c;
             const int64_t own = cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c);
-            int64_t out = s_id[q];
+            int64_t out = static_cast<int64_t>(first) + s_id[q];
             a.slots[own] = static_cast<uint32_t>(f) | (static_cast<uint32_t>(out) << 3);
             if (out + __popc(f) > a.n_vertices) continue;  // never with the counts of classify
             write_edge_points<T>(a, g, c, own, f, out);
@@ -597,7 +599,7 @@ __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
     __shared__ uint32_t s_cell[kChunk];   // cell of the chunk | case << 12
-    __shared__ int32_t s_out[kChunk];     // its first triangle
+    __shared__ uint16_t s_out[kChunk];    // its first triangle, from the chunk's first
     __shared__ McTables tables;
     load_tables(tables);
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
@@ -624,7 +626,7 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
             if (code) {
                 int& at = part[j / VEC];
                 s_cell[at & 0xFFFF] = (own_group_offset<VEC>(j / VEC) + j % VEC) | (code << 12);
-                s_out[at & 0xFFFF] = first + (at >> 16);
+                s_out[at & 0xFFFF] = static_cast<uint16_t>(at >> 16);
                 at += 1 + (tables.count[code] << 16);
             }
         }
@@ -635,8 +637,8 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
             int64_t g, c;
             if (cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c) < 0) continue;
             const int mine = tables.count[code];
-            const int64_t first = s_out[q];
-            if (first + mine > a.n_triangles) continue;  // never with the counts of classify
+            const int64_t first_tri = static_cast<int64_t>(first) + s_out[q];
+            if (first_tri + mine > a.n_triangles) continue;  // never with the counts of classify
             // rows of the cells at the eight corners, then the id on every crossed edge
             int need = 0;   // corners that own a crossed edge
 #pragma unroll
@@ -661,7 +663,7 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
             }
             const uint64_t row = tables.rows[code];
             for (int t = 0; t < mine; ++t) {
-                int32_t* tri = a.triangles + (first + t) * 3;
+                int32_t* tri = a.triangles + (first_tri + t) * 3;
 #pragma unroll
                 for (int v = 0; v < 3; ++v) {
                     const int e = static_cast<int>(row >> (4 * (3 * t + v))) & 15;
@@ -806,7 +808,7 @@ __global__ __launch_bounds__(kBlock) void iso_count_kernel(McDev a) {
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void iso_points_kernel(McDev a) {
     __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
-    __shared__ int32_t s_id[kChunk];      // its first point
+    __shared__ uint16_t s_id[kChunk];     // its first point, from the chunk's first
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint64_t flags = 0;   // 3 bits per own cell
@@ -834,7 +836,7 @@ __global__ __launch_bounds__(kBlock) void iso_points_kernel(McDev a) {
                 int& at = part[j / VEC];
                 s_cell[at & 0xFFFF] =
                         static_cast<uint16_t>((own_group_offset<VEC>(j / VEC) + j % VEC) | (f << 12));
-                s_id[at & 0xFFFF] = first + (at >> 16);
+                s_id[at & 0xFFFF] = static_cast<uint16_t>(at >> 16);
                 at += 1 + (__popc(f) << 16);
             }
         }
@@ -844,7 +846,7 @@ __global__ __launch_bounds__(kBlock) void iso_points_kernel(McDev a) {
             const int f = s_cell[q] >> 12;
             int64_t g, c;
             const int64_t own = cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c);
-            const int64_t out = s_id[q];
+            const int64_t out = static_cast<int64_t>(first) + s_id[q];
             if (out + __popc(f) > a.n_vertices) continue;  // never with the count of classify
             write_edge_points<T>(a, g, c, own, f, out);
         }
