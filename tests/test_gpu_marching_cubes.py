@@ -146,3 +146,36 @@ def test_block_sizes_match_oracle(gpu_ash, oracle, grid_dim):
     assert len(tri_ref) > 300 and tri.shape == tri_ref.shape and pts.shape == pts_ref.shape
     assert np.array_equal(_sorted_rows(pts), _sorted_rows(pts_ref))
     assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))
+
+
+def test_spatial_listing_follows_the_table(gpu_ash):
+    """The Z-order listing of the blocks is kept while the table is unchanged
+    and rebuilt after every call that can change its keys."""
+    from helpers import sort_rows
+
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, 17 ** 3 + 10, 1, grid_dim=2, sparse_grid_dim=20, bbox_min=torch.zeros(3),
+        bbox_max=torch.ones(3), device=DEV)
+    r = torch.arange(17, dtype=torch.int32)
+    blocks = torch.stack(torch.meshgrid(r, r, r, indexing="ij"), -1).view(-1, 3).to(DEV)
+    grid.engine.insert_keys(blocks)
+
+    def same_set(listing):
+        keys, idx = grid.engine.items()
+        a, b = sort_rows(listing[0], listing[1]), sort_rows(keys, idx)
+        return torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+    first = grid._blocks_in_spatial_order()
+    assert same_set(first) and len(first[1]) == 17 ** 3
+    # neighbours in the listing are neighbours in space far more often than in table order
+    step = (first[0][1:] - first[0][:-1]).abs().sum(dim=1).float().mean()
+    table_step = (grid.engine.items()[0][1:] - grid.engine.items()[0][:-1]).abs().sum(dim=1).float().mean()
+    assert float(step) < 0.3 * float(table_step)
+    again = grid._blocks_in_spatial_order()
+    assert again[0] is first[0] and again[1] is first[1]
+    grid.engine.insert_keys(torch.tensor([[18, 18, 18], [19, 0, 3]], dtype=torch.int32, device=DEV))
+    grown = grid._blocks_in_spatial_order()
+    assert len(grown[1]) == 17 ** 3 + 2 and same_set(grown)
+    grid.engine.erase(blocks[:100])
+    shrunk = grid._blocks_in_spatial_order()
+    assert len(shrunk[1]) == 17 ** 3 - 98 and same_set(shrunk)

@@ -780,6 +780,9 @@ class _HashMap:
         self._table = torch.empty(table_bytes.value, dtype=torch.uint8, device=self._device)
         self._general = None
         self._maybe_tombstones = False
+        # counts the calls that may have changed the stored keys; lets callers
+        # keep results derived from the key set (orderings, tables) while it stands
+        self.version = 0
         handle = _PTR()
         with torch.cuda.device(self._device):
             self._check(
@@ -846,6 +849,7 @@ class _HashMap:
         the kernel; attach the region once and let the caller re-issue."""
         st = self.status()
         self._status_after_insert = st
+        self.version += 1
         if st["dropped"] > 0 or st["tombstones"] > 0:
             self._maybe_tombstones = True
         if st["exotic_pending"] == 0:
@@ -1082,6 +1086,7 @@ class _HashMap:
         keys = self._keys(keys)
         self._maybe_tombstones = True
         self._status_after_insert = None
+        self.version += 1
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_erase(
@@ -1094,6 +1099,7 @@ class _HashMap:
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
         self._maybe_tombstones = False
         self._status_after_insert = None
+        self.version += 1
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
         n = self.size()

@@ -1,10 +1,10 @@
 """Sparse-dense grids: a hash map of active blocks, each a dense G^3 array of
 cells carrying an embedding row.
 
-Public names, shapes and semantics follow ash/grid.py:29-863 for what lies on
-the query path (allocation, query, interpolation, enumeration, neighbour
-tables, coordinate transforms).  Ray sampling, filtering and surface extraction
-belong to other native kernels of the reference and are not provided.
+Public names, shapes and semantics follow ash/grid.py:29-863: allocation,
+query, interpolation, enumeration, neighbour tables and coordinate transforms
+on the query path, and around it ray sampling, filtering / convolution and
+surface extraction, each on the library's kernel for it.
 """
 from typing import Literal, Optional, Tuple, Union
 
@@ -23,6 +23,10 @@ backend = _get_c_extension()
 # positions); False = the reference's formulation: candidate expansion, scratch
 # hash set, insert, find.  Both leave the same map and return the same blocks.
 FUSED_ACTIVATION = True
+
+# From this many active blocks on, the functions that walk all blocks list them
+# along a Z-order curve (see SparseDenseGrid._blocks_in_spatial_order).
+SPATIAL_ORDER_MIN_BLOCKS = 4096
 
 Interpolation = Literal["nearest", "linear", "smooth_step"]
 
@@ -235,6 +239,40 @@ class SparseDenseGrid(ASHModule):
         )
         return features, masks
 
+    @torch.no_grad()
+    def _blocks_in_spatial_order(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(grid_coords (n, 3), grid_indices (n,)) of the active blocks along a
+        Z-order curve instead of in table order.  Kernels that walk the listing
+        and read across block faces (surface extraction, convolution) then find
+        the cells of neighbouring blocks in cache; their results do not depend
+        on the order of the listing."""
+        # kept while the table holds the same keys (its shim counts the calls
+        # that may change them)
+        table = self.engine.backend
+        stamp = (id(table), getattr(table, "version", None))
+        cached = getattr(self, "_spatial_order_cache", None)
+        if stamp[1] is not None and cached is not None and cached[0] == stamp:
+            return cached[1], cached[2]
+        keys, indices = self.engine.items()
+        if len(indices) < SPATIAL_ORDER_MIN_BLOCKS:
+            return keys, indices
+
+        def spread(v):  # bit i of v -> bit 3 i
+            v = v & 0x1FFFFF
+            v = (v | (v << 32)) & 0x1F00000000FFFF
+            v = (v | (v << 16)) & 0x1F0000FF0000FF
+            v = (v | (v << 8)) & 0x100F00F00F00F00F
+            v = (v | (v << 4)) & 0x10C30C30C30C30C3
+            v = (v | (v << 2)) & 0x1249249249249249
+            return v
+
+        k = (keys - keys.min(dim=0)[0]).long()
+        code = spread(k[:, 0]) | (spread(k[:, 1]) << 1) | (spread(k[:, 2]) << 2)
+        order = torch.argsort(code)
+        keys, indices = keys[order], indices[order]
+        self._spatial_order_cache = (stamp, keys, indices)
+        return keys, indices
+
     def items(self) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
         """Active blocks in broadcastable form (ash/grid.py:240-266):
         grid_coords (n, 1, 3), cell_coords (1, M, 3), grid_indices (n, 1),
@@ -400,7 +438,8 @@ class SparseDenseGrid(ASHModule):
         )
         grid_radius = (radius + self.grid_dim - 1) // self.grid_dim
         _, lut_grid_nb2grid_idx = self.construct_grid_neighbor_lut(grid_radius, bidirectional=True)
-        _, _, grid_indices, cell_indices = self.items()
+        _, grid_indices = self._blocks_in_spatial_order()
+        cell_indices = self.cell_indices
         num_cell_nbs = lut_cell_nb2grid_nb.shape[1]
         return backend.convolution_forward(
             inputs,
@@ -426,7 +465,7 @@ class SparseDenseGrid(ASHModule):
         tsdfs, weights: (num_embeddings, cells_per_grid[, 1])."""
         if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
             self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
-        _, grid_indices = self.engine.items()
+        _, grid_indices = self._blocks_in_spatial_order()
         vertices = backend.isosurface_extraction(
             tsdfs,
             weights,
@@ -453,7 +492,7 @@ class SparseDenseGrid(ASHModule):
         triangle normals point towards larger `tsdfs`."""
         if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
             self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
-        _, grid_indices = self.engine.items()
+        _, grid_indices = self._blocks_in_spatial_order()
         triangles, vertices = backend.marching_cubes(
             tsdfs,
             weights,

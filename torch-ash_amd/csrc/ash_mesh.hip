@@ -284,11 +284,38 @@ __device__ __forceinline__ void build_tile_map(const McDev& a, uint16_t* s_src, 
     }
 }
 
+// The listing positions a one-wavefront workgroup walks.  Workgroups go to the
+// eight XCDs round robin and every XCD has an L2 of its own, so each XCD takes
+// a contiguous eighth of the listing: with blocks listed in a space-filling
+// order, the cells a block fetches from its neighbours have then mostly just
+// been fetched by a workgroup on the same XCD.
+constexpr int kXcds = 8;
+
+struct BlockWalk {
+    int64_t first, end, step;
+};
+
+__device__ __forceinline__ BlockWalk block_walk(int64_t n) {
+    BlockWalk w;
+    if (gridDim.x % kXcds != 0) {
+        w.first = blockIdx.x;
+        w.end = n;
+        w.step = gridDim.x;
+        return w;
+    }
+    const int64_t share = (n + kXcds - 1) / kXcds;
+    const int64_t xcd = blockIdx.x % kXcds;
+    w.first = xcd * share + blockIdx.x / kXcds;
+    w.end = (xcd + 1) * share < n ? (xcd + 1) * share : n;
+    w.step = gridDim.x / kXcds;
+    return w;
+}
+
 // Row of listed block b (lane kSrcOwn) and of its neighbours (lanes 0..7); -1
-// where there is none.
-__device__ __forceinline__ int64_t fetch_block_rows(const McDev& a, int64_t b) {
+// where there is none or b is past `end`.
+__device__ __forceinline__ int64_t fetch_block_rows(const McDev& a, int64_t b, int64_t end) {
     const int lane = threadIdx.x;
-    if (b >= a.n_grids || lane > kSrcOwn) return -1;
+    if (b >= end || lane > kSrcOwn) return -1;
     const int64_t g = a.grid_indices[b];
     if (g < 0 || g >= a.B) return -1;
     if (lane == kSrcOwn) return g;
@@ -319,12 +346,13 @@ __global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a)
     uint8_t* tile = reinterpret_cast<uint8_t*>(s_pos + M); // [W3]
     const int lane = threadIdx.x;
     build_tile_map(a, s_src, s_pos);
-    int64_t blk = blockIdx.x;
-    int64_t row = fetch_block_rows(a, blk);
-    for (; blk < a.n_grids; blk += gridDim.x) {
+    const BlockWalk walk = block_walk(a.n_grids);
+    int64_t blk = walk.first;
+    int64_t row = fetch_block_rows(a, blk, walk.end);
+    for (; blk < walk.end; blk += walk.step) {
         __syncthreads();  // set-up done; previous block's tile and rows read
         if (lane <= kSrcOwn) s_nb[lane] = row;
-        row = fetch_block_rows(a, blk + gridDim.x);
+        row = fetch_block_rows(a, blk + walk.step, walk.end);
         __syncthreads();
         const int64_t g = s_nb[kSrcOwn];
         if (g < 0) continue;  // the same for the whole wavefront
@@ -721,12 +749,13 @@ __global__ __launch_bounds__(kTileThreads) void iso_classify_tile_kernel(McDev a
     const int lane = threadIdx.x;
     const int off[3] = {1, W, W * W};
     build_tile_map(a, s_src, s_pos);
-    int64_t blk = blockIdx.x;
-    int64_t row = fetch_block_rows(a, blk);
-    for (; blk < a.n_grids; blk += gridDim.x) {
+    const BlockWalk walk = block_walk(a.n_grids);
+    int64_t blk = walk.first;
+    int64_t row = fetch_block_rows(a, blk, walk.end);
+    for (; blk < walk.end; blk += walk.step) {
         __syncthreads();  // set-up done; previous block's tile and rows read
         if (lane <= kSrcOwn) s_nb[lane] = row;
-        row = fetch_block_rows(a, blk + gridDim.x);
+        row = fetch_block_rows(a, blk + walk.step, walk.end);
         __syncthreads();
         const int64_t g = s_nb[kSrcOwn];
         if (g < 0) continue;  // the same for the whole wavefront
@@ -861,6 +890,14 @@ bool vector_access(const McDev& a) {
            reinterpret_cast<uintptr_t>(a.slots) % 16 == 0;
 }
 
+// Workgroups of a one-wavefront-per-block launch: a multiple of the number of
+// XCDs whenever there are that many blocks (see block_walk).
+unsigned tile_grid(int64_t num_grids) {
+    int64_t g = num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid;
+    if (g >= kXcds) g -= g % kXcds;
+    return static_cast<unsigned>(g < 1 ? 1 : g);
+}
+
 unsigned persistent_grid(int64_t work_items) {
     if (work_items < 1) return 1;
     return static_cast<unsigned>(work_items < kMaxGrid ? work_items : kMaxGrid);
@@ -949,8 +986,7 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     const bool tiled = grid_dim <= kMaxTileG &&
                        static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
     if (tiled) {
-        const unsigned by_block =
-                static_cast<unsigned>(num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid);
+        const unsigned by_block = tile_grid(num_grids);
         const size_t lds = static_cast<size_t>(3 * tile_cells(grid_dim)) + 2 * cells_per_grid;
         if (dtype == ASH_F32) {
             mc_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
@@ -1067,8 +1103,7 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
         const bool tiled = grid_dim <= kMaxTileG && lds <= 63 * 1024 &&
                            static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
         if (tiled) {
-            const unsigned by_block =
-                    static_cast<unsigned>(num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid);
+            const unsigned by_block = tile_grid(num_grids);
             if (dtype == ASH_F32) {
                 iso_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
             } else {

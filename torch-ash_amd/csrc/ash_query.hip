@@ -877,10 +877,14 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
     // Blocks through the tile, software-pipelined: while a block is computed
     // from LDS, the rows of the next block's tile are already on their way
     // into registers and the row numbers of the block after that are fetched.
+    // each XCD walks a contiguous eighth of the listing (TileWalk): with blocks
+    // listed along a space-filling curve the halo rows are then mostly in the
+    // XCD's own L2
+    const TileWalk walk(a.n_grids);
     constexpr int kPre = EC >= 16 ? 2 : (EC >= 8 ? 4 : 6);   // tile rows a thread can hold
     const bool prefetch = T3 <= kPre * kConvThreads;
     auto fetch_rows = [&](int64_t b) -> int64_t {  // lanes 0..26 neighbours, 27 the block
-        if (tid > 27 || b >= a.n_grids) return -1;
+        if (tid > 27 || b >= walk.end) return -1;
         const int64_t g = a.grid_indices[b];
         if (g < 0 || g >= a.B) return -1;
         if (tid == 27) return g;
@@ -911,18 +915,18 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             }
         }
     };
-    int64_t blk = blockIdx.x;
+    int64_t blk = walk.next;
     int buf = 0;
     int64_t rows_reg = fetch_rows(blk);
     if (tid <= 27) s_nb[0][tid] = rows_reg;
-    rows_reg = fetch_rows(blk + gridDim.x);
+    rows_reg = fetch_rows(blk + walk.step);
     __syncthreads();
     T pre[kPre][EC];
     if (prefetch) {
 #pragma unroll
         for (int i = 0; i < kPre; ++i) load_row(s_nb[0], tid + i * kConvThreads, pre[i]);
     }
-    for (; blk < a.n_grids; blk += gridDim.x, buf ^= 1) {
+    for (; blk < walk.end; blk += walk.step, buf ^= 1) {
         __syncthreads();  // the previous block's tile has been read
         const int64_t g = s_nb[buf][27];
         if (prefetch) {
@@ -944,8 +948,8 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         }
         if (tid <= 27) s_nb[buf ^ 1][tid] = rows_reg;
         __syncthreads();
-        rows_reg = fetch_rows(blk + 2 * static_cast<int64_t>(gridDim.x));
-        if (prefetch && blk + gridDim.x < a.n_grids) {
+        rows_reg = fetch_rows(blk + 2 * walk.step);
+        if (prefetch && blk + walk.step < walk.end) {
 #pragma unroll
             for (int i = 0; i < kPre; ++i) load_row(s_nb[buf ^ 1], tid + i * kConvThreads, pre[i]);
         }
