@@ -58,7 +58,7 @@ struct McDev {
     const int64_t* lut_c2g;       // [M, 8]
     uint8_t* cases;               // [B * M]
     uint32_t* slots;              // [B * M]
-    int32_t* counters;            // [4]
+    int32_t* counters;            // workspace: totals, then per-chunk counts / running sums
     float* positions;             // [V, 3]
     int32_t* triangles;           // [T, 3]
     int64_t n_grids, B, M;
@@ -960,12 +960,12 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
                                 const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
                                 int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
                                 float iso_value, float weight_thr, int32_t dtype,
-                                uint8_t* cases, uint32_t* edge_slots, int32_t* counters,
+                                uint8_t* cases, uint32_t* edge_slots, int32_t* workspace,
                                 void* stream) {
     McDev a = {};
     if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
                     lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
-                    cells_per_grid, grid_dim, iso_value, dtype, cases, edge_slots, true, counters)) {
+                    cells_per_grid, grid_dim, iso_value, dtype, cases, edge_slots, true, workspace)) {
         return 1;
     }
     if (num_grids > 0 && weights == nullptr) ASH_FAIL("null pointer in marching_cubes");
@@ -1005,7 +1005,7 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
         mc_count_kernel<1><<<by_chunk, kBlock, 0, s>>>(a);
     }
     ASH_LAUNCH_CHECK();
-    mc_scan_kernel<<<1, kScanThreads, 0, s>>>(counters, (cells + kChunk - 1) / kChunk, 2,
+    mc_scan_kernel<<<1, kScanThreads, 0, s>>>(workspace, (cells + kChunk - 1) / kChunk, 2,
                                               kMcVertices32, kMcTriangles32);
     ASH_LAUNCH_CHECK();
     return 0;
@@ -1019,14 +1019,14 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
                                const int64_t* lut_cell_nb2grid_nb, int64_t num_grids,
                                int64_t num_embeddings, int64_t cells_per_grid, int grid_dim,
                                float iso_value, int32_t dtype, const uint8_t* cases,
-                               uint32_t* edge_slots, int32_t* counters, int64_t n_vertices,
+                               uint32_t* edge_slots, int32_t* workspace, int64_t n_vertices,
                                int64_t n_triangles, float* positions, int32_t* triangles,
                                void* stream) {
     McDev a = {};
     if (fill_common(a, sdfs, grid_indices, cell_coords_table, lut_grid_nb2grid_idx,
                     lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, num_grids, num_embeddings,
                     cells_per_grid, grid_dim, iso_value, dtype, const_cast<uint8_t*>(cases),
-                    edge_slots, true, counters)) {
+                    edge_slots, true, workspace)) {
         return 1;
     }
     if (n_vertices < 0 || n_triangles < 0) ASH_FAIL("marching_cubes: negative counts");
