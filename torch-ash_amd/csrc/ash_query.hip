@@ -964,47 +964,97 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             // order: dz, then dy, then dx.
             const int yq_n = G / 4;
             const int combos = G * yq_n * G;
-            for (int item = tid; item < combos * EC; item += kConvThreads) {
-                const int q = item / combos;
-                if (q >= ec) continue;
-                const int rem = item - q * combos;
-                const int x = rem % G;
-                const int y0 = 4 * ((rem / G) % yq_n);
-                const int z = rem / (G * yq_n);
-                const T* plane = tile + static_cast<size_t>(q) * T3 + x + Tn * y0 + Tn * Tn * z;
-                const T* wq = s_w + static_cast<size_t>(q) * K;
-                T acc[4] = {T(0), T(0), T(0), T(0)};
+            // Results go out through LDS when a thread can hold all of its
+            // items' sums until the tile is no longer read: the tile's space
+            // then takes them cell by cell (rows padded by one word against
+            // bank conflicts) and whole output rows are written by consecutive
+            // lanes.  Written one channel per lane straight from the
+            // registers, a row reaches memory as EC separate 4-byte pieces from
+            // different wavefronts, which more than doubles the bytes written.
+            // Pays for its two barriers with full rows of 16 channels only.
+            constexpr int kHold = 4;
+            const bool staged = EC >= 16 && combos * EC <= kHold * kConvThreads;
+            T held[kHold][4];
+#pragma unroll
+            for (int it = 0; it < kHold; ++it) {
+                const int item = tid + it * kConvThreads;
+                if (!staged && it > 0) break;
+                for (int at = item; at < combos * EC; at += staged ? combos * EC : kConvThreads) {
+                    const int q = at / combos;
+                    if (q >= ec) continue;
+                    const int rem = at - q * combos;
+                    const int x = rem % G;
+                    const int y0 = 4 * ((rem / G) % yq_n);
+                    const int z = rem / (G * yq_n);
+                    const T* plane = tile + static_cast<size_t>(q) * T3 + x + Tn * y0 + Tn * Tn * z;
+                    const T* wq = s_w + static_cast<size_t>(q) * K;
+                    T acc[4] = {T(0), T(0), T(0), T(0)};
 #pragma unroll 1
-                for (int dz = 0; dz < WT; ++dz) {
-                    const T* pz = plane + Tn * Tn * dz;
-                    T win[4][WT > 0 ? WT : 1];
+                    for (int dz = 0; dz < WT; ++dz) {
+                        const T* pz = plane + Tn * Tn * dz;
+                        T win[4][WT > 0 ? WT : 1];
 #pragma unroll
-                    for (int yy = 0; yy < 3; ++yy) {
+                        for (int yy = 0; yy < 3; ++yy) {
 #pragma unroll
-                        for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
-                    }
+                            for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
+                        }
 #pragma unroll
-                    for (int dy = 0; dy < WT; ++dy) {
-#pragma unroll
-                        for (int dx = 0; dx < WT; ++dx) win[(dy + 3) & 3][dx] = pz[Tn * (dy + 3) + dx];
-                        T wr[WT > 0 ? WT : 1];
-#pragma unroll
-                        for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
+                        for (int dy = 0; dy < WT; ++dy) {
 #pragma unroll
                             for (int dx = 0; dx < WT; ++dx) {
-                                acc[j] = fma(win[(dy + j) & 3][dx], wr[dx], acc[j]);
+                                win[(dy + 3) & 3][dx] = pz[Tn * (dy + 3) + dx];
+                            }
+                            T wr[WT > 0 ? WT : 1];
+#pragma unroll
+                            for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                                for (int dx = 0; dx < WT; ++dx) {
+                                    acc[j] = fma(win[(dy + j) & 3][dx], wr[dx], acc[j]);
+                                }
                             }
                         }
                     }
-                }
+                    if (staged) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int c = x + G * (y0 + j) + G * G * z;
+                        for (int j = 0; j < 4; ++j) held[it][j] = acc[j];
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int c = x + G * (y0 + j) + G * G * z;
+                            const int c_i = s_inv[c];
+                            if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
+                            out[(g * a.M + c) * E + e0 + q] = acc[j];
+                        }
+                    }
+                }
+            }
+            if (staged) {
+                __syncthreads();  // the tile has been read
+                T* stage = tile;  // [M][EC + 1]
+#pragma unroll
+                for (int it = 0; it < kHold; ++it) {
+                    const int item = tid + it * kConvThreads;
+                    if (item >= combos * EC) continue;
+                    const int q = item / combos;
+                    if (q >= ec) continue;
+                    const int rem = item - q * combos;
+                    const int x = rem % G;
+                    const int y0 = 4 * ((rem / G) % yq_n);
+                    const int z = rem / (G * yq_n);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        stage[(x + G * (y0 + j) + G * G * z) * (EC + 1) + q] = held[it][j];
+                    }
+                }
+                __syncthreads();
+                for (int i = tid; i < M * ec; i += kConvThreads) {
+                    const int c = i / ec;
+                    const int q = i - c * ec;
                     const int c_i = s_inv[c];
                     if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
-                    out[(g * a.M + c) * E + e0 + q] = acc[j];
+                    out[(g * a.M + c) * E + e0 + q] = stage[c * (EC + 1) + q];
                 }
             }
             continue;
