@@ -759,9 +759,10 @@ int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
 // never is -0), which is what skipping the tap does.  Every workgroup first
 // checks the two per-cell tables against this layout and, should they describe
 // something else, takes its blocks through the tables instead.
-template <typename T, int EC, int WT, bool YB>
+template <typename T, int EC, int WT, int NY>
 __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         ConvDev a, int G, int r, int e0, int ec, int vec) {
+    constexpr bool YB = NY > 0;   // NY cells that follow each other in y per lane
     extern __shared__ __align__(16) unsigned char conv_smem[];
     __shared__ int64_t s_nb[2][28];   // rows of 27 neighbour blocks + the block itself
     __shared__ int s_bad;
@@ -955,14 +956,15 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         }
         if (g < 0) continue;  // the same for the whole workgroup
         if constexpr (YB) {
-            // One lane = one channel of four cells that follow each other in y.
+            // One lane = one channel of NY cells that follow each other in y.
             // For every (dz, dy) the W weights of the tap row are read once and
-            // used by all four cells, and the four tile rows they meet stay in
+            // used by all NY cells, and the NY tile rows they meet stay in
             // registers from one dy to the next (row dy + j serves cell j), so
             // that a step costs one new tile row and one weight row for
-            // 4 W fused multiply-adds.  Every cell still sees its taps in table
-            // order: dz, then dy, then dx.
-            const int yq_n = G / 4;
+            // NY * W fused multiply-adds.  Every cell still sees its taps in
+            // table order: dz, then dy, then dx.
+            constexpr int kNy = NY > 0 ? NY : 4;
+            const int yq_n = G / kNy;
             const int combos = G * yq_n * G;
             // Results go out through LDS when a thread can hold all of its
             // items' sums until the tile is no longer read: the tile's space
@@ -974,7 +976,7 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             // Pays for its two barriers with full rows of 16 channels only.
             constexpr int kHold = 4;
             const bool staged = EC >= 16 && combos * EC <= kHold * kConvThreads;
-            T held[kHold][4];
+            T held[kHold][kNy];
 #pragma unroll
             for (int it = 0; it < kHold; ++it) {
                 const int item = tid + it * kConvThreads;
@@ -984,17 +986,19 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                     if (q >= ec) continue;
                     const int rem = at - q * combos;
                     const int x = rem % G;
-                    const int y0 = 4 * ((rem / G) % yq_n);
+                    const int y0 = kNy * ((rem / G) % yq_n);
                     const int z = rem / (G * yq_n);
                     const T* plane = tile + static_cast<size_t>(q) * T3 + x + Tn * y0 + Tn * Tn * z;
                     const T* wq = s_w + static_cast<size_t>(q) * K;
-                    T acc[4] = {T(0), T(0), T(0), T(0)};
+                    T acc[kNy];
+#pragma unroll
+                    for (int j = 0; j < kNy; ++j) acc[j] = T(0);
 #pragma unroll 1
                     for (int dz = 0; dz < WT; ++dz) {
                         const T* pz = plane + Tn * Tn * dz;
-                        T win[4][WT > 0 ? WT : 1];
+                        T win[kNy][WT > 0 ? WT : 1];
 #pragma unroll
-                        for (int yy = 0; yy < 3; ++yy) {
+                        for (int yy = 0; yy < kNy - 1; ++yy) {
 #pragma unroll
                             for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
                         }
@@ -1002,26 +1006,26 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                         for (int dy = 0; dy < WT; ++dy) {
 #pragma unroll
                             for (int dx = 0; dx < WT; ++dx) {
-                                win[(dy + 3) & 3][dx] = pz[Tn * (dy + 3) + dx];
+                                win[(dy + kNy - 1) & (kNy - 1)][dx] = pz[Tn * (dy + kNy - 1) + dx];
                             }
                             T wr[WT > 0 ? WT : 1];
 #pragma unroll
                             for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {
+                            for (int j = 0; j < kNy; ++j) {
 #pragma unroll
                                 for (int dx = 0; dx < WT; ++dx) {
-                                    acc[j] = fma(win[(dy + j) & 3][dx], wr[dx], acc[j]);
+                                    acc[j] = fma(win[(dy + j) & (kNy - 1)][dx], wr[dx], acc[j]);
                                 }
                             }
                         }
                     }
                     if (staged) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) held[it][j] = acc[j];
+                        for (int j = 0; j < kNy; ++j) held[it][j] = acc[j];
                     } else {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
+                        for (int j = 0; j < kNy; ++j) {
                             const int c = x + G * (y0 + j) + G * G * z;
                             const int c_i = s_inv[c];
                             if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
@@ -1041,10 +1045,10 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                     if (q >= ec) continue;
                     const int rem = item - q * combos;
                     const int x = rem % G;
-                    const int y0 = 4 * ((rem / G) % yq_n);
+                    const int y0 = kNy * ((rem / G) % yq_n);
                     const int z = rem / (G * yq_n);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
+                    for (int j = 0; j < kNy; ++j) {
                         stage[(x + G * (y0 + j) + G * G * z) * (EC + 1) + q] = held[it][j];
                     }
                 }
@@ -1115,6 +1119,10 @@ constexpr size_t kConvTileBytes = ASH_CONV_TILE_BYTES;   // LDS a tile may take
 #define ASH_CONV_ROW_BLOCKING 1
 #endif
 constexpr bool kConvRowBlocking = ASH_CONV_ROW_BLOCKING != 0;
+#ifndef ASH_CONV_ROWS8
+#define ASH_CONV_ROWS8 1
+#endif
+constexpr bool kConvRows8 = ASH_CONV_ROWS8 != 0;
 
 // Largest cube edge G with G^3 == m, or 0.
 inline int cube_edge(int64_t m) {
@@ -1137,9 +1145,15 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
     // channels of a row whatever it uses of them.
     constexpr int kMaxEc = sizeof(T) == 4 ? 16 : 8;
     const size_t cell_bytes = static_cast<size_t>(Tn * Tn * Tn) * sizeof(T);
+    // two workgroups per CU (64 KB each) run faster than one with twice the
+    // channels -- except for rows of a cache line or more, where every pass
+    // over a part of the channels fetches the whole rows again (measured on 7^3
+    // windows: E = 8 15.1 vs 16.2 ms, E = 16 39.4 vs 34.2 ms)
+    const size_t budget = a.E * sizeof(T) >= 64 ? kConvTileBytes + kConvTileBytes / 2
+                                                : kConvTileBytes;
     int ec_max = kMaxEc;
-    while (ec_max > 1 && cell_bytes * ec_max > kConvTileBytes) ec_max /= 2;
-    if (cell_bytes * ec_max > kConvTileBytes) return -1;
+    while (ec_max > 1 && cell_bytes * ec_max > budget) ec_max /= 2;
+    if (cell_bytes * ec_max > budget) return -1;
     const uintptr_t align = reinterpret_cast<uintptr_t>(a.in);
     for (int e0 = 0; e0 < a.E;) {
         int width = ec_max;                  // channels of the template instance
@@ -1161,14 +1175,18 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
         auto by_window = [&](auto ec_tag) -> int {
             constexpr int kEc = decltype(ec_tag)::value;
             if (G % 4 == 0 && kConvRowBlocking) {
-                if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, true>);
-                if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, true>);
-                if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, true>);
+                if (G % 8 == 0 && kConvRows8) {
+                    if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, 8>);
+                    if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, 8>);
+                }
+                if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, 4>);
+                if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, 4>);
+                if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, 4>);
             }
-            if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, false>);
-            if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, false>);
-            if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, false>);
-            return launch(convolution_tile_kernel<T, kEc, 0, false>);
+            if (W == 3) return launch(convolution_tile_kernel<T, kEc, 3, 0>);
+            if (W == 5) return launch(convolution_tile_kernel<T, kEc, 5, 0>);
+            if (W == 7) return launch(convolution_tile_kernel<T, kEc, 7, 0>);
+            return launch(convolution_tile_kernel<T, kEc, 0, 0>);
         };
         int rc = 1;
         if (width == 16) {
