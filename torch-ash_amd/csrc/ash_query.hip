@@ -759,6 +759,8 @@ int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
 // never is -0), which is what skipping the tap does.  Every workgroup first
 // checks the two per-cell tables against this layout and, should they describe
 // something else, takes its blocks through the tables instead.
+// EC: channels per pass; WT: window edge when it is 3, 5 or 7, else 0; NY: cells
+// per lane along y (0: one lane = one cell with all EC channels).
 template <typename T, int EC, int WT, int NY>
 __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         ConvDev a, int G, int r, int e0, int ec, int vec) {
