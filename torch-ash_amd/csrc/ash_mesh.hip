@@ -566,27 +566,36 @@ __device__ __forceinline__ void write_edge_points(const McDev& a, int64_t g, int
     }
 }
 
-// Gives the flagged edges of every cell their ids and writes the vertices:
-// the zero crossing of the field along the edge, linear between its two ends
-// (ash/src/grid.cu:748-771).
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
+// Writes the point of every flagged edge: the zero crossing of the field
+// along the edge, linear between its two ends (ash/src/grid.cu:510-527 and
+// :748-771).  SLOTS: the flags are the low bits of the cells' slot words
+// (marching cubes), and every flagged cell's word also receives the id of its
+// first point; otherwise they are the low bits of the cells' bytes in `cases`
+// (iso-surface points).
+template <typename T, int VEC, bool SLOTS>
+__global__ __launch_bounds__(kBlock) void edge_points_kernel(McDev a) {
     __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
-    __shared__ uint16_t s_id[kChunk];     // id of its first vertex, from the chunk's first
+    __shared__ uint16_t s_id[kChunk];     // its first point, from the chunk's first
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint64_t flags = 0;   // 3 bits per own cell
-        int part[kPerThread / VEC] = {};   // per group: listed cells | vertices << 16
+        int part[kPerThread / VEC] = {};   // per group: listed cells | points << 16
         for_own_groups<VEC>(a, ch, [&](int j, uint32_t, int64_t at) {
             uint32_t f[VEC];
-            if constexpr (VEC == 4) {
+            if constexpr (SLOTS && VEC == 4) {
                 const uint4 w = *reinterpret_cast<const uint4*>(a.slots + at);
                 f[0] = w.x & 7u;
                 f[1] = w.y & 7u;
                 f[2] = w.z & 7u;
                 f[3] = w.w & 7u;
-            } else {
+            } else if constexpr (SLOTS) {
                 f[0] = a.slots[at] & 7u;
+            } else if constexpr (VEC == 4) {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(a.cases + at);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) f[k] = (w >> (8 * k)) & 7u;
+            } else {
+                f[0] = a.cases[at] & 7u;
             }
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
@@ -613,8 +622,10 @@ __global__ __launch_bounds__(kBlock) void mc_vertices_kernel(McDev a) {
             const int f = s_cell[q] >> 12;
             int64_t g, c;
             const int64_t own = cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c);
-            int64_t out = static_cast<int64_t>(first) + s_id[q];
-            a.slots[own] = static_cast<uint32_t>(f) | (static_cast<uint32_t>(out) << 3);
+            const int64_t out = static_cast<int64_t>(first) + s_id[q];
+            if constexpr (SLOTS) {
+                a.slots[own] = static_cast<uint32_t>(f) | (static_cast<uint32_t>(out) << 3);
+            }
             if (out + __popc(f) > a.n_vertices) continue;  // never with the counts of classify
             write_edge_points<T>(a, g, c, own, f, out);
         }
@@ -834,54 +845,6 @@ __global__ __launch_bounds__(kBlock) void iso_count_kernel(McDev a) {
     }
 }
 
-template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void iso_points_kernel(McDev a) {
-    __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
-    __shared__ uint16_t s_id[kChunk];     // its first point, from the chunk's first
-    const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
-    for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
-        uint64_t flags = 0;   // 3 bits per own cell
-        int part[kPerThread / VEC] = {};   // per group: listed cells | points << 16
-        for_own_groups<VEC>(a, ch, [&](int j, uint32_t, int64_t at) {
-            uint32_t w;
-            if constexpr (VEC == 4) {
-                w = *reinterpret_cast<const uint32_t*>(a.cases + at);
-            } else {
-                w = a.cases[at];
-            }
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) {
-                const uint32_t f = (w >> (8 * k)) & 7u;
-                flags |= static_cast<uint64_t>(f) << (3 * (j * VEC + k));
-                part[j] += (f != 0u) + (__popc(f) << 16);
-            }
-        });
-        const int total = chunk_exclusive(part);
-        const int first = a.counters[kMcHeader + ch];
-#pragma unroll
-        for (int j = 0; j < kPerThread; ++j) {
-            const int f = static_cast<int>(flags >> (3 * j)) & 7;
-            if (f) {
-                int& at = part[j / VEC];
-                s_cell[at & 0xFFFF] =
-                        static_cast<uint16_t>((own_group_offset<VEC>(j / VEC) + j % VEC) | (f << 12));
-                s_id[at & 0xFFFF] = static_cast<uint16_t>(at >> 16);
-                at += 1 + (__popc(f) << 16);
-            }
-        }
-        __syncthreads();
-        const int listed = total & 0xFFFF;
-        for (int q = threadIdx.x; q < listed; q += kBlock) {
-            const int f = s_cell[q] >> 12;
-            int64_t g, c;
-            const int64_t own = cell_of_chunk(a, ch, s_cell[q] & 0xFFF, g, c);
-            const int64_t out = static_cast<int64_t>(first) + s_id[q];
-            if (out + __popc(f) > a.n_vertices) continue;  // never with the count of classify
-            write_edge_points<T>(a, g, c, own, f, out);
-        }
-    }
-}
-
 // Groups of four cells can be moved as one word of cases and one 16-byte
 // vector of slots when blocks hold a multiple of four cells and both arrays
 // are aligned accordingly.
@@ -1048,14 +1011,14 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
     const bool vec = vector_access(a);
     if (dtype == ASH_F32) {
         if (vec) {
-            mc_vertices_kernel<float, 4><<<by_chunk, kBlock, 0, s>>>(a);
+            edge_points_kernel<float, 4, true><<<by_chunk, kBlock, 0, s>>>(a);
         } else {
-            mc_vertices_kernel<float, 1><<<by_chunk, kBlock, 0, s>>>(a);
+            edge_points_kernel<float, 1, true><<<by_chunk, kBlock, 0, s>>>(a);
         }
     } else if (vec) {
-        mc_vertices_kernel<double, 4><<<by_chunk, kBlock, 0, s>>>(a);
+        edge_points_kernel<double, 4, true><<<by_chunk, kBlock, 0, s>>>(a);
     } else {
-        mc_vertices_kernel<double, 1><<<by_chunk, kBlock, 0, s>>>(a);
+        edge_points_kernel<double, 1, true><<<by_chunk, kBlock, 0, s>>>(a);
     }
     ASH_LAUNCH_CHECK();
     if (n_triangles > 0) {
@@ -1160,14 +1123,14 @@ int ash_isosurface_points(const void* sdfs, const int64_t* grid_indices,
     const bool vec = a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0;
     if (dtype == ASH_F32) {
         if (vec) {
-            iso_points_kernel<float, 4><<<by_chunk, kBlock, 0, s>>>(a);
+            edge_points_kernel<float, 4, false><<<by_chunk, kBlock, 0, s>>>(a);
         } else {
-            iso_points_kernel<float, 1><<<by_chunk, kBlock, 0, s>>>(a);
+            edge_points_kernel<float, 1, false><<<by_chunk, kBlock, 0, s>>>(a);
         }
     } else if (vec) {
-        iso_points_kernel<double, 4><<<by_chunk, kBlock, 0, s>>>(a);
+        edge_points_kernel<double, 4, false><<<by_chunk, kBlock, 0, s>>>(a);
     } else {
-        iso_points_kernel<double, 1><<<by_chunk, kBlock, 0, s>>>(a);
+        edge_points_kernel<double, 1, false><<<by_chunk, kBlock, 0, s>>>(a);
     }
     ASH_LAUNCH_CHECK();
     return 0;
