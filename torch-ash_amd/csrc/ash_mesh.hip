@@ -234,9 +234,9 @@ __device__ __forceinline__ void record_case(const McDev& a, int code, const int6
     }
 }
 
-// One wavefront per block, blocks taken round robin.  tile[] holds, for the
-// (G+1)^3 cells at the corners of the block's cells, bit 0 = exists and weighs
-// enough, bit 1 = below the iso value.  Where each tile cell comes from -- the
+// One wavefront per block, blocks taken along the listing (block_walk below).
+// tile[] holds, for the (G+1)^3 cells at the corners of the block's cells,
+// bit 0 = exists and weighs enough, bit 1 = below the iso value.  Where each tile cell comes from -- the
 // block itself or one of its seven neighbours, and which cell there -- is the
 // same for every block and is worked out once per workgroup from the tables:
 // a cell on a high face of the block names the cells beyond that face.  The
