@@ -288,6 +288,66 @@ __device__ __forceinline__ bool find_key(const MapDev& m, const int32_t (&k)[DIM
     return found;
 }
 
+// The same look-up when the eight lanes of a group all hold the same key (and
+// the same `active`): the group reads the key's bucket once, 16 bytes per lane,
+// instead of taking turns with eight different keys.
+template <int DIM>
+__device__ __forceinline__ bool find_key_shared(const MapDev& m, const int32_t (&k)[DIM],
+                                                bool active, int32_t& res) {
+    const int lane = threadIdx.x & 63;
+    const int j = lane & (kGroup - 1);
+    const int gbase = lane & ~(kGroup - 1);
+    const bool v0 = (2 * j) < kSlots;
+    const bool v1 = (2 * j + 1) < kSlots;
+    uint64_t code;
+    const bool fits = pack_key<DIM>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+    res = 0;
+    bool found = false;
+    while (__ballot(pend)) {
+        uint4 line = make_uint4(0u, 0u, 0u, 0u);
+        if (pend) {
+            line = *(reinterpret_cast<const uint4*>(m.buckets +
+                                                    static_cast<size_t>(b) * kBucketQwords) + j);
+        }
+        const uint64_t qa = static_cast<uint64_t>(line.x) | (static_cast<uint64_t>(line.y) << 32);
+        const uint64_t qb = static_cast<uint64_t>(line.z) | (static_cast<uint64_t>(line.w) << 32);
+        const uint32_t gm0 = static_cast<uint32_t>(__ballot(pend && v0 && qa == code) >> gbase) & 0xFFu;
+        const uint32_t gm1 = static_cast<uint32_t>(__ballot(pend && v1 && qb == code) >> gbase) & 0xFFu;
+        const uint32_t ge0 = static_cast<uint32_t>(__ballot(pend && v0 && qa == kEmpty) >> gbase) & 0xFFu;
+        const uint32_t ge1 = static_cast<uint32_t>(__ballot(pend && v1 && qb == kEmpty) >> gbase) & 0xFFu;
+        int slot = -1;
+        if (gm0) {
+            slot = 2 * __builtin_ctz(gm0);
+        } else if (gm1) {
+            slot = 2 * __builtin_ctz(gm1) + 1;
+        }
+        const int t = kValDword0 + (slot < 0 ? 0 : slot);
+        const int comp = t & 3;
+        const uint32_t sel = comp == 0 ? line.x : comp == 1 ? line.y : comp == 2 ? line.z : line.w;
+        const int32_t val = __shfl(static_cast<int>(sel), gbase + (t >> 2));
+        if (pend) {
+            if (slot >= 0) {
+                found = true;
+                res = val;
+                pend = false;
+            } else if (ge0 | ge1) {
+                pend = false;
+            } else {
+                b = next_bucket(b, m.nb);
+                if (++steps >= m.nb) pend = false;
+            }
+        }
+    }
+    if (active && !fits) {
+        uint32_t pos;
+        found = gen_find<DIM>(m, k, res, pos);
+    }
+    return found;
+}
+
 template <int DIM>
 __global__ __launch_bounds__(kBlock) void find_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n,
@@ -747,8 +807,21 @@ __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
         const uint64_t stop = __ballot(!go);
         const int first_stop = stop ? __builtin_ctzll(stop) : 64;
         const bool active = lane < first_stop;
+        // steps are half a block apart, so neighbouring lanes often stand in
+        // the same block: only the first lane of such a run goes to the table,
+        // the others take its answer
+        bool head = true;
+        {
+            int same = lane > 0;
+#pragma unroll
+            for (int a = 0; a < 3; ++a) same &= __shfl_up(block[a], 1) == block[a];
+            head = !same;
+        }
         int32_t idx;
-        const bool found = find_key<3>(m, block, active, idx);
+        const bool asked = find_key<3>(m, block, active && head, idx);
+        const uint64_t heads = __ballot(head);
+        const int my_head = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));
+        const bool found = __shfl(static_cast<int>(asked), my_head) != 0;
         uint64_t hits = __ballot(found && active);
         while (hits) {
             const int l = __builtin_ctzll(hits);
@@ -771,6 +844,11 @@ __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
 // pass with `stage` also keeps the first `stride` samples of ray i as pairs
 // (t_near, t_far) at stage[2 * (i * stride + k)], so that the assignment pass
 // can be a copy instead of a second march.
+// LPR lanes per ray: 1, or 8 lanes that march the same ray in step and share
+// every look-up (find_key_shared) -- eight times the wavefronts for the same
+// rays, which is what hides the latency of a march that is one dependent
+// look-up after the other.
+template <int LPR>
 __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         MapDev m, const float* __restrict__ origins,
         const float* __restrict__ directions, const float* __restrict__ ray_nears,
@@ -779,7 +857,9 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         const int64_t* __restrict__ prefix, int64_t* __restrict__ ray_indices,
         float* __restrict__ t_nears, float* __restrict__ t_fars,
         float2* __restrict__ stage, int64_t stride) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t gid = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t i = gid / LPR;
+    const bool writer = gid % LPR == 0;   // the lane of a ray that stores its results
     const bool active = i < n;
     const float cell2grid = static_cast<float>(1.0 / grid2cell);
     float o[3], d[3];
@@ -796,34 +876,60 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
     float t = ray_near, t_near = ray_near;
     int64_t local = 0;
     bool live = active && t < ray_far;
-    while (__ballot(live)) {
-        int32_t block[3];
-        float x[3];
-        ray_block(o, d, t, cell2grid, block, x);
-        int32_t idx;
-        const bool found = find_key<3>(m, block, live, idx);
-        if (live) {
-            const float before = t;
-            if (!found) {
-                t += t_grid_step;
-            } else {
-                t += t_step;
-                if (counts == nullptr) {
-                    ray_indices[start + local] = i;
-                    t_nears[start + local] = t_near;
-                    t_fars[start + local] = t;
-                } else if (stage != nullptr && local < stride) {
-                    stage[i * stride + local] = make_float2(t_near, t);
-                }
-                t_near = t;
-                ++local;
+    // One step of the march, given whether the block under t is stored.
+    auto step = [&](bool found) {
+        const float before = t;
+        if (!found) {
+            t += t_grid_step;
+        } else {
+            t += t_step;
+            if (!writer) {
+            } else if (counts == nullptr) {
+                ray_indices[start + local] = i;
+                t_nears[start + local] = t_near;
+                t_fars[start + local] = t;
+            } else if (stage != nullptr && local < stride) {
+                stage[i * stride + local] = make_float2(t_near, t);
             }
-            // a step that no longer advances t (range far beyond fp32
-            // resolution) would never end; the reference has no such guard
-            live = t < ray_far && t > before;
+            t_near = t;
+            ++local;
+        }
+        // a step that no longer advances t (range far beyond fp32
+        // resolution) would never end; the reference has no such guard
+        live = t < ray_far && t > before;
+    };
+    // The reference looks the block under t up at every step.  Samples are a
+    // fraction of a block apart, so consecutive steps mostly ask for the same
+    // block: a lane answers those from its last look-up and the wavefront goes
+    // to the table only when some lane has entered another block -- a dozen
+    // round trips to memory per ray instead of one per step, same answers.
+    int32_t known[3] = {0, 0, 0};
+    bool have = false;
+    bool known_found = false;
+    while (__ballot(live)) {
+        int32_t block[3] = {0, 0, 0};
+        float x[3];
+        bool ask = false;
+        while (live) {
+            ray_block(o, d, t, cell2grid, block, x);
+            if (!have || block[0] != known[0] || block[1] != known[1] || block[2] != known[2]) {
+                ask = true;
+                break;
+            }
+            step(known_found);
+        }
+        int32_t idx;
+        const bool found = LPR == 8 ? find_key_shared<3>(m, block, live && ask, idx)
+                                    : find_key<3>(m, block, live && ask, idx);
+        if (live && ask) {
+#pragma unroll
+            for (int a = 0; a < 3; ++a) known[a] = block[a];
+            known_found = found;
+            have = true;
+            step(found);
         }
     }
-    if (active && counts != nullptr) counts[i] = local;
+    if (active && writer && counts != nullptr) counts[i] = local;
 }
 
 // Assignment pass from the staged samples: one thread per staged slot.
@@ -1103,6 +1209,28 @@ inline unsigned capped_grid(int64_t n) {
     if (g < 1) g = 1;
     return static_cast<unsigned>(g);
 }
+
+// Few rays cannot fill the device with one lane each; up to this many they
+// march with eight lanes per ray.
+constexpr int64_t kRaysPerLaneMin = int64_t{1} << 20;
+
+int launch_ray_sample(ash_map_t* map, const float* origins, const float* directions,
+                      const float* nears, const float* fars, int64_t n, float max_samples,
+                      float grid2cell, int64_t* counts, const int64_t* prefix,
+                      int64_t* ray_indices, float* t_nears, float* t_fars, float2* stage,
+                      int64_t stride, hipStream_t s) {
+    if (n < kRaysPerLaneMin) {
+        ray_sample_kernel<8><<<grid_for(n * 8), kBlock, 0, s>>>(
+                map->d, origins, directions, nears, fars, n, max_samples, grid2cell, counts,
+                prefix, ray_indices, t_nears, t_fars, stage, stride);
+    } else {
+        ray_sample_kernel<1><<<grid_for(n), kBlock, 0, s>>>(
+                map->d, origins, directions, nears, fars, n, max_samples, grid2cell, counts,
+                prefix, ray_indices, t_nears, t_fars, stage, stride);
+    }
+    return 0;
+}
+
 
 int check_map(const ash_map* map) {
     if (map == nullptr) ASH_FAIL("null map handle");
@@ -1440,10 +1568,10 @@ int ash_ray_sample(ash_map_t* map, const float* ray_origins,
     }
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    ray_sample_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
-            map->d, ray_origins, ray_directions, ray_nears, ray_fars, n,
-            static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
-            prefix, ray_indices, t_nears, t_fars, nullptr, 0);
+    launch_ray_sample(map, ray_origins, ray_directions, ray_nears, ray_fars, n,
+                      static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
+                      prefix, ray_indices, t_nears, t_fars, nullptr, 0,
+                      static_cast<hipStream_t>(stream));
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -1468,10 +1596,10 @@ int ash_ray_sample_staged(ash_map_t* map, const float* ray_origins,
     if (reinterpret_cast<uintptr_t>(stage) % 8 != 0) ASH_FAIL("ray_sample_staged: stage must be 8-byte aligned");
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    ray_sample_kernel<<<grid_for(n), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
-            map->d, ray_origins, ray_directions, ray_nears, ray_fars, n,
-            static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts, nullptr,
-            nullptr, nullptr, nullptr, reinterpret_cast<float2*>(stage), stride);
+    launch_ray_sample(map, ray_origins, ray_directions, ray_nears, ray_fars, n,
+                      static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
+                      nullptr, nullptr, nullptr, nullptr, reinterpret_cast<float2*>(stage),
+                      stride, static_cast<hipStream_t>(stream));
     ASH_LAUNCH_CHECK();
     return 0;
 }
