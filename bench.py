@@ -403,6 +403,21 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     out["cfg4_forward_plus_backward"] = e
     out["cfg4_live_fraction"] = round(n_live / n4, 4)
 
+    # the front end that turns positions into the operands above
+    # (ash/grid.py:183-199): 12 B read, 8 + 8 + 12 + 1 B written per position
+    xc = grid.transform_world_to_cell(x).contiguous()
+    t_q = EventTimer(torch)
+    for it in range(2 + reps):
+        if it < 2:
+            grid.query(xc)
+        else:
+            t_q(lambda: grid.query(xc))
+    e = roofline_entry("grid_query_kernel (positions -> block, cell, offset, mask)", 41 * n4,
+                       t_q.mean_ms())
+    e["Mqueries_per_s"] = round(n4 / e["ms"] / 1e3, 1)
+    out["cfg4_grid_query"] = e
+    del xc
+
     # the ray sampler that produces such queries (ash/grid.py:322-403)
     ro, rd = workloads.camera_rays(grid, radii, centres, 32768)
     extent = float((grid.bbox_max - grid.bbox_min).norm())

@@ -60,6 +60,27 @@ def test_near_far_and_samples_match_oracle(gpu_ash, oracle, n):
             assert ref[0].numel() > 10 * n
 
 
+def test_many_rays_match_oracle(gpu_ash, oracle):
+    """Enough rays for the sampler's one-lane-per-ray kernel (the cases above
+    run the variant for few rays)."""
+    engine, omap, blocks, g = _scene(gpu_ash, oracle, seed=705)
+    backend = gpu_ash.grid.backend
+    extent = 64 * 8.0
+    n = 70_000
+    o, d = _rays(g, n, extent, blocks)
+    lo, hi = torch.zeros(3), torch.full((3,), extent)
+    near, far = backend.ray_find_near_far(engine.backend, o.to(DEV), d.to(DEV), lo.to(DEV),
+                                          hi.to(DEV), 0.5, 700.0, 1.0, 8.0)
+    near_ref, far_ref = oracle.ray_find_near_far(omap, o, d, lo, hi, 0.5, 700.0, 1.0, 8.0)
+    assert torch.equal(near.cpu(), near_ref) and torch.equal(far.cpu(), far_ref)
+    got = backend.ray_sample(engine.backend, o.to(DEV), d.to(DEV), near, far, lo.to(DEV),
+                             hi.to(DEV), 48, 8.0)
+    ref = oracle.ray_sample(omap, o, d, near_ref, far_ref, lo, hi, 48, 8.0)
+    assert ref[0].numel() > 10 * n
+    for a, b in zip(got, ref):
+        assert a.dtype == b.dtype and torch.equal(a.cpu(), b)
+
+
 @pytest.mark.parametrize("mode", ["two_marches", "stage_overflow"])
 def test_sample_paths_agree(gpu_ash, oracle, monkeypatch, mode):
     """ray_sample keeps the samples of its allocation pass and copies them; the

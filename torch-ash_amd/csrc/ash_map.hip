@@ -348,6 +348,56 @@ __device__ __forceinline__ bool find_key_shared(const MapDev& m, const int32_t (
     return found;
 }
 
+// The same look-up by one lane on its own: it reads the ten codes of the key's
+// bucket itself (five 16-byte loads of one 128-byte line).  Far fewer vector
+// instructions per wavefront than the cooperative probe, at the price of one
+// line per lane and load instruction; for kernels whose table is small enough
+// to stay in the caches and that are bound by instructions, not by lines.
+template <int DIM>
+__device__ __forceinline__ bool find_key_alone(const MapDev& m, const int32_t (&k)[DIM],
+                                               bool active, int32_t& res) {
+    static_assert(kSlots == 10, "reads the codes as five 16-byte words");
+    uint64_t code;
+    const bool fits = pack_key<DIM>(k, code);
+    bool pend = active && fits;
+    uint32_t b = bucket_of(code, m.nb);
+    uint32_t steps = 0;
+    res = 0;
+    bool found = false;
+    while (pend) {
+        const uint4* line = reinterpret_cast<const uint4*>(
+                m.buckets + static_cast<size_t>(b) * kBucketQwords);
+        uint4 w[5];
+#pragma unroll
+        for (int r = 0; r < 5; ++r) w[r] = line[r];
+        int slot = -1;
+        bool empty = false;
+#pragma unroll
+        for (int r = 4; r >= 0; --r) {
+            const uint64_t qa = static_cast<uint64_t>(w[r].x) | (static_cast<uint64_t>(w[r].y) << 32);
+            const uint64_t qb = static_cast<uint64_t>(w[r].z) | (static_cast<uint64_t>(w[r].w) << 32);
+            empty = empty || qa == kEmpty || qb == kEmpty;
+            if (qb == code) slot = 2 * r + 1;
+            if (qa == code) slot = 2 * r;
+        }
+        if (slot >= 0) {
+            found = true;
+            res = *value_ptr(m, b, slot);
+            pend = false;
+        } else if (empty) {
+            pend = false;
+        } else {
+            b = next_bucket(b, m.nb);
+            if (++steps >= m.nb) pend = false;
+        }
+    }
+    if (active && !fits) {
+        uint32_t pos;
+        found = gen_find<DIM>(m, k, res, pos);
+    }
+    return found;
+}
+
 template <int DIM>
 __global__ __launch_bounds__(kBlock) void find_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n,
@@ -400,33 +450,19 @@ __global__ __launch_bounds__(kBlock) void grid_query_kernel(
         cell += static_cast<int64_t>(static_cast<int32_t>(xd)) * stride;
         stride *= gi;
     }
-    uint64_t code;
-    const bool fits = pack_key<3>(k, code);
-    bool pend = active && fits;
-    uint32_t b = bucket_of(code, m.nb);
-    uint32_t steps = 0;
+    // neighbouring positions (samples along a ray) often stand in the same
+    // block: the first lane of such a run looks the block up, by itself, and
+    // the others take its answer
+    int same = lane > 0;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) same &= __shfl_up(k[d], 1) == k[d];
+    const bool head = !same;
     int32_t res = 0;
-    bool found = false;
-    while (__ballot(pend)) {
-        ProbeResult p;
-        probe_pass(m, code, b, pend, lane, p);
-        if (pend) {
-            if (p.status == kProbeFound) {
-                found = true;
-                res = p.val;
-                pend = false;
-            } else if (p.status == kProbeHasEmpty) {
-                pend = false;
-            } else {
-                b = next_bucket(b, m.nb);
-                if (++steps >= m.nb) pend = false;
-            }
-        }
-    }
-    if (active && !fits) {
-        uint32_t pos;
-        found = gen_find<3>(m, k, res, pos);
-    }
+    const bool asked = find_key_alone<3>(m, k, active && head, res);
+    const uint64_t heads = __ballot(head);
+    const int my_head = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));
+    const bool found = __shfl(static_cast<int>(asked), my_head) != 0;
+    res = __shfl(res, my_head);
     if (active) {
         grid_idx[i] = found ? static_cast<int64_t>(res) : 0;
         mask_out[i] = found ? 1 : 0;
@@ -752,9 +788,7 @@ __global__ __launch_bounds__(kHeapBlock) void activate_kernel(
 }
 
 // --------------------------------------------------------------------- rays
-// ash/src/sampler.cu:7-67 and :122-214.  One lane marches one ray; the table
-// lookups of a wavefront's 64 rays are done together (find_key), so the loops
-// run while any lane of the wavefront still has steps to take.  Positions are
+// ash/src/sampler.cu:7-67 and :122-214.  Positions are
 // origin + t * direction as a fused multiply-add (what nvcc makes of the
 // reference's expression); everything is in cell units and a block is
 // `grid2cell` cells wide.
@@ -818,7 +852,7 @@ __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
             head = !same;
         }
         int32_t idx;
-        const bool asked = find_key<3>(m, block, active && head, idx);
+        const bool asked = find_key_alone<3>(m, block, active && head, idx);
         const uint64_t heads = __ballot(head);
         const int my_head = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));
         const bool found = __shfl(static_cast<int>(asked), my_head) != 0;
@@ -844,10 +878,11 @@ __global__ __launch_bounds__(kBlock) void ray_near_far_kernel(
 // pass with `stage` also keeps the first `stride` samples of ray i as pairs
 // (t_near, t_far) at stage[2 * (i * stride + k)], so that the assignment pass
 // can be a copy instead of a second march.
-// LPR lanes per ray: 1, or 8 lanes that march the same ray in step and share
-// every look-up (find_key_shared) -- eight times the wavefronts for the same
-// rays, which is what hides the latency of a march that is one dependent
-// look-up after the other.
+// LPR lanes per ray: 1 (every lane looks its block up by itself,
+// find_key_alone), or 8 lanes that march the same ray in step and share every
+// look-up (find_key_shared) -- eight times the wavefronts for the same rays,
+// which is what hides the latency of a march that is one dependent look-up
+// after the other when the rays are few.
 template <int LPR>
 __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         MapDev m, const float* __restrict__ origins,
@@ -920,7 +955,7 @@ __global__ __launch_bounds__(kBlock) void ray_sample_kernel(
         }
         int32_t idx;
         const bool found = LPR == 8 ? find_key_shared<3>(m, block, live && ask, idx)
-                                    : find_key<3>(m, block, live && ask, idx);
+                                    : find_key_alone<3>(m, block, live && ask, idx);
         if (live && ask) {
 #pragma unroll
             for (int a = 0; a < 3; ++a) known[a] = block[a];
@@ -1210,9 +1245,10 @@ inline unsigned capped_grid(int64_t n) {
     return static_cast<unsigned>(g);
 }
 
-// Few rays cannot fill the device with one lane each; up to this many they
-// march with eight lanes per ray.
-constexpr int64_t kRaysPerLaneMin = int64_t{1} << 20;
+// Few rays cannot fill the device with one lane each; below this many they
+// march with eight lanes per ray (32 768 rays: 110 against 120 us; from 65 536
+// rays on one lane per ray is the faster one, 1.6x at half a million).
+constexpr int64_t kRaysPerLaneMin = int64_t{1} << 16;
 
 int launch_ray_sample(ash_map_t* map, const float* origins, const float* directions,
                       const float* nears, const float* fars, int64_t n, float max_samples,
