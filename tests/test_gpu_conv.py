@@ -130,7 +130,7 @@ def test_tables_in_another_order_take_the_table_path(gpu_ash, oracle):
     assert torch.allclose(out, plain, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("radius,channels", [(3, 5), (2, 16), (3, 16)])
+@pytest.mark.parametrize("radius,channels", [(3, 5), (2, 16), (3, 16), (1, 8), (1, 6), (1, 12), (2, 8)])
 def test_wide_windows_and_rows(gpu_ash, oracle, radius, channels):
     grid, _, _ = workloads.build_grid(gpu_ash, 200, channels, 8, 32, device=DEV)
     g = torch.Generator().manual_seed(830 + radius)

@@ -1649,7 +1649,7 @@ int ash_ray_sample_compact(const int64_t* counts, const int64_t* prefix, const f
         t_nears == nullptr || t_fars == nullptr) {
         ASH_FAIL("null pointer in ray_sample_compact");
     }
-    if (n > (int64_t{1} << 40) / stride) ASH_FAIL("ray_sample_compact: too many slots");
+    if (n > ((int64_t{1} << 32) - kBlock) / stride) ASH_FAIL("ray_sample_compact: too many slots");
     ray_compact_kernel<<<grid_for(n * stride), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
             counts, prefix, reinterpret_cast<const float2*>(stage), stride, n, ray_indices,
             t_nears, t_fars);

@@ -761,9 +761,12 @@ int launch_convolution_block(const ConvDev& a, int vec4, hipStream_t s) {
 // something else, takes its blocks through the tables instead.
 // EC: channels per pass; WT: window edge when it is 3, 5 or 7, else 0; NY: cells
 // per lane along y (0: one lane = one cell with all EC channels).
+// The second launch bound asks for four wavefronts per SIMD (two workgroups
+// per CU, at most 128 registers) for all but the widest instances, which need
+// more registers than that for their window.
 template <typename T, int EC, int WT, int NY>
-__global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
-        ConvDev a, int G, int r, int e0, int ec, int vec) {
+__global__ __launch_bounds__(kConvThreads, (EC >= 16 && NY >= 8) ? 2 : 4) void convolution_tile_kernel(
+        ConvDev a, int G, int r, int e0, int ec, int vec, int Tz) {
     constexpr bool YB = NY > 0;   // NY cells that follow each other in y per lane
     extern __shared__ __align__(16) unsigned char conv_smem[];
     __shared__ int64_t s_nb[2][28];   // rows of 27 neighbour blocks + the block itself
@@ -775,13 +778,22 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
     const int W = WT > 0 ? WT : 2 * r + 1;   // WT: window edge known at compile time
     const int Tn = G + 2 * r;
     const int T3 = Tn * Tn * Tn;
-    T* tile = reinterpret_cast<T*>(conv_smem);                             // [T3][EC]
-    T* s_w = tile + static_cast<size_t>(T3) * EC;                          // [K][EC]
+    // Tz: words from one z layer of a channel's plane to the next, Tn * Tn or
+    // a little more (YB): the lanes of a wavefront read G words along x at
+    // NY * Tn words from one group of lanes to the next in y and Tz in z, and
+    // the host pads Tz so that the groups served together fall on different
+    // LDS banks.
+    const int Ts = Tz * Tn;        // words of one channel's plane
+    const int zpad = Tz - Tn * Tn;
+    T* tile = reinterpret_cast<T*>(conv_smem);                             // [Ts][EC]
+    T* s_w = tile + static_cast<size_t>(Ts) * EC;                          // [K][EC]
     uint32_t* s_src = reinterpret_cast<uint32_t*>(s_w + static_cast<size_t>(K) * EC);  // [T3]
     uint16_t* s_inv = reinterpret_cast<uint16_t*>(s_src + T3);   // [M] position of a cell in cell_indices (YB)
     // YB keeps one plane per channel (a lane reads runs of one channel along
-    // x), otherwise the channels of a row sit together.
-    auto tile_at = [&](int p, int q) { return YB ? q * T3 + p : p * EC + q; };
+    // x), otherwise the channels of a row sit together.  p counts the rows of
+    // the tile without the padding.
+    auto plane_at = [&](int p) { return p + zpad * (p / (Tn * Tn)); };
+    auto tile_at = [&](int p, int q) { return YB ? q * Ts + plane_at(p) : p * EC + q; };
     auto w_at = [&](int k, int q) { return YB ? q * K + k : k * EC + q; };
     const T* in = static_cast<const T*>(a.in);
     const T* w = static_cast<const T*>(a.w);
@@ -809,7 +821,8 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             bad |= a.lut_c2g[t] != gn || a.lut_c2c[t] != ci;
         }
         if (bad) s_bad = 1;
-        // where every row of the tile comes from: neighbour block << 12 | cell
+        // where every row of the tile comes from and where it goes:
+        // place in the tile << 17 | neighbour block << 12 | cell
         for (int p = tid; p < T3; p += kConvThreads) {
             const int tx[3] = {p % Tn - r, (p / Tn) % Tn - r, p / (Tn * Tn) - r};
             int gn = 0, ci = 0, gs = 1, cs = 1;
@@ -821,7 +834,7 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
                 gs *= 3;
                 cs *= G;
             }
-            s_src[p] = static_cast<uint32_t>((gn << 12) | ci);
+            s_src[p] = (static_cast<uint32_t>(tile_at(p, 0)) << 17) | static_cast<uint32_t>((gn << 12) | ci);
         }
         for (int t = tid; t < K * EC; t += kConvThreads) {
             const int k = t / EC;
@@ -894,14 +907,19 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         const int64_t row = a.lut_g[g * 27 + tid];
         return (row >= 0 && row < a.B) ? row : -1;
     };
-    auto load_row = [&](const int64_t* nb, int p, T (&v)[EC]) {
+    // src_cell: an entry of s_src, or kNoRow for a thread without a row
+    constexpr uint32_t kNoRow = 0xFFFFFFFFu;
+    const T* in_e0 = in + e0;
+    const uint32_t block_words = static_cast<uint32_t>(M * E);   // <= 4096 * 16
+    auto load_row = [&](const int64_t* nb, uint32_t src_cell, T (&v)[EC]) {
 #pragma unroll
         for (int q = 0; q < EC; ++q) v[q] = T(0);
-        if (p >= T3) return;
-        const uint32_t src_cell = s_src[p];
-        const int64_t row = nb[src_cell >> 12];
+        if (src_cell == kNoRow) return;
+        const int64_t row = nb[(src_cell >> 12) & 31];
         if (row < 0) return;
-        const T* src = in + (row * a.M + (src_cell & 0xFFF)) * E + e0;
+        // row < B < 2^31: one 32 x 32 -> 64 bit product
+        const T* src = in_e0 + (static_cast<uint64_t>(static_cast<uint32_t>(row)) * block_words +
+                                (src_cell & 0xFFF) * static_cast<uint32_t>(E));
         if (vec) {   // EC is a multiple of four here
 #pragma unroll
             for (int q4 = 0; q4 < (EC + 3) / 4; ++q4) {
@@ -918,16 +936,89 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
             }
         }
     };
+    // One lane = one channel of NY cells that follow each other in y.  For
+    // every (dz, dy) the W weights of the tap row are read once and used by all
+    // NY cells, and the NY tile rows they meet stay in registers from one dy to
+    // the next (row dy + j serves cell j), so that a step costs one new tile
+    // row and one weight row for NY * W fused multiply-adds.  Every cell still
+    // sees its taps in table order: dz, then dy, then dx.
+    constexpr int kNy = NY > 0 ? NY : 4;
+    const int yq_n = G / kNy;
+    const int combos = G * yq_n * G;
+    auto window_sums = [&](const T* plane, const T* wq, T (&acc)[kNy]) {
+#pragma unroll
+        for (int j = 0; j < kNy; ++j) acc[j] = T(0);
+#pragma unroll 1
+        for (int dz = 0; dz < WT; ++dz) {
+            const T* pz = plane + Tz * dz;
+            T win[kNy][WT > 0 ? WT : 1];
+#pragma unroll
+            for (int yy = 0; yy < kNy - 1; ++yy) {
+#pragma unroll
+                for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
+            }
+#pragma unroll
+            for (int dy = 0; dy < WT; ++dy) {
+#pragma unroll
+                for (int dx = 0; dx < WT; ++dx) {
+                    win[(dy + kNy - 1) & (kNy - 1)][dx] = pz[Tn * (dy + kNy - 1) + dx];
+                }
+                T wr[WT > 0 ? WT : 1];
+#pragma unroll
+                for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
+#pragma unroll
+                for (int j = 0; j < kNy; ++j) {
+#pragma unroll
+                    for (int dx = 0; dx < WT; ++dx) {
+                        acc[j] = fma(win[(dy + j) & (kNy - 1)][dx], wr[dx], acc[j]);
+                    }
+                }
+            }
+        }
+    };
+    // Results go out through LDS when a thread can hold all of its items' sums
+    // until the tile is no longer read: the tile's space then takes them cell
+    // by cell (rows padded by one word against bank conflicts) and whole output
+    // rows are written by consecutive lanes.  Written one channel per lane
+    // straight from the registers, a row reaches memory as EC separate 4-byte
+    // pieces from different wavefronts, which more than doubles the bytes
+    // written.  Pays for its two barriers with full rows of 16 channels and
+    // with 3^3 windows; the wider windows of narrower rows need the registers
+    // that would hold the results for their window.
+    constexpr int kHold = 4;
+    const bool staged = YB && (EC >= 16 || (WT == 3 && EC >= 4)) && combos * EC <= kHold * kConvThreads;
+    T held[kHold][kNy];
+    // staged: combos divides the workgroup size, so the items of a thread are
+    // the same cells in channels task_q, task_q + task_qstep, ...
+    const int task_qstep = staged ? kConvThreads / combos : 0;
+    const int task_q = staged ? tid / combos : EC;
+    int task_plane = 0, task_cell = 0;
+    if (staged) {
+        const int rem = tid - task_q * combos;
+        const int x = rem % G;
+        const int y0 = kNy * ((rem / G) % yq_n);
+        const int z = rem / (G * yq_n);
+        task_plane = x + Tn * y0 + Tz * z;
+        task_cell = (x + G * y0 + G * G * z) * (EC + 1);
+    }
     int64_t blk = walk.next;
     int buf = 0;
     int64_t rows_reg = fetch_rows(blk);
     if (tid <= 27) s_nb[0][tid] = rows_reg;
     rows_reg = fetch_rows(blk + walk.step);
     __syncthreads();
+    // what does not change from block to block is read once: the source and the
+    // place in the tile of the rows this thread stages
     T pre[kPre][EC];
+    uint32_t pre_src[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+        const int p = tid + i * kConvThreads;
+        pre_src[i] = (prefetch && p < T3) ? s_src[p] : kNoRow;
+    }
     if (prefetch) {
 #pragma unroll
-        for (int i = 0; i < kPre; ++i) load_row(s_nb[0], tid + i * kConvThreads, pre[i]);
+        for (int i = 0; i < kPre; ++i) load_row(s_nb[0], pre_src[i], pre[i]);
     }
     for (; blk < walk.end; blk += walk.step, buf ^= 1) {
         __syncthreads();  // the previous block's tile has been read
@@ -935,18 +1026,20 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         if (prefetch) {
 #pragma unroll
             for (int i = 0; i < kPre; ++i) {
-                const int p = tid + i * kConvThreads;
-                if (p < T3) {
+                if (pre_src[i] != kNoRow) {
+                    T* at = tile + (pre_src[i] >> 17);
 #pragma unroll
-                    for (int q = 0; q < EC; ++q) tile[tile_at(p, q)] = pre[i][q];
+                    for (int q = 0; q < EC; ++q) at[YB ? q * Ts : q] = pre[i][q];
                 }
             }
         } else {
             for (int p = tid; p < T3; p += kConvThreads) {
                 T v[EC];
-                load_row(s_nb[buf], p, v);
+                const uint32_t src_cell = s_src[p];
+                load_row(s_nb[buf], src_cell, v);
+                T* at = tile + (src_cell >> 17);
 #pragma unroll
-                for (int q = 0; q < EC; ++q) tile[tile_at(p, q)] = v[q];
+                for (int q = 0; q < EC; ++q) at[YB ? q * Ts : q] = v[q];
             }
         }
         if (tid <= 27) s_nb[buf ^ 1][tid] = rows_reg;
@@ -954,113 +1047,71 @@ __global__ __launch_bounds__(kConvThreads) void convolution_tile_kernel(
         rows_reg = fetch_rows(blk + 2 * walk.step);
         if (prefetch && blk + walk.step < walk.end) {
 #pragma unroll
-            for (int i = 0; i < kPre; ++i) load_row(s_nb[buf ^ 1], tid + i * kConvThreads, pre[i]);
+            for (int i = 0; i < kPre; ++i) load_row(s_nb[buf ^ 1], pre_src[i], pre[i]);
         }
         if (g < 0) continue;  // the same for the whole workgroup
         if constexpr (YB) {
-            // One lane = one channel of NY cells that follow each other in y.
-            // For every (dz, dy) the W weights of the tap row are read once and
-            // used by all NY cells, and the NY tile rows they meet stay in
-            // registers from one dy to the next (row dy + j serves cell j), so
-            // that a step costs one new tile row and one weight row for
-            // NY * W fused multiply-adds.  Every cell still sees its taps in
-            // table order: dz, then dy, then dx.
-            constexpr int kNy = NY > 0 ? NY : 4;
-            const int yq_n = G / kNy;
-            const int combos = G * yq_n * G;
-            // Results go out through LDS when a thread can hold all of its
-            // items' sums until the tile is no longer read: the tile's space
-            // then takes them cell by cell (rows padded by one word against
-            // bank conflicts) and whole output rows are written by consecutive
-            // lanes.  Written one channel per lane straight from the
-            // registers, a row reaches memory as EC separate 4-byte pieces from
-            // different wavefronts, which more than doubles the bytes written.
-            // Pays for its two barriers with full rows of 16 channels only.
-            constexpr int kHold = 4;
-            const bool staged = EC >= 16 && combos * EC <= kHold * kConvThreads;
-            T held[kHold][kNy];
+            if (staged) {
 #pragma unroll
-            for (int it = 0; it < kHold; ++it) {
-                const int item = tid + it * kConvThreads;
-                if (!staged && it > 0) break;
-                for (int at = item; at < combos * EC; at += staged ? combos * EC : kConvThreads) {
+                for (int it = 0; it < kHold; ++it) {
+                    const int q = task_q + it * task_qstep;
+                    if (q < ec) window_sums(tile + q * Ts + task_plane, s_w + q * K, held[it]);
+                }
+                __syncthreads();  // the tile has been read
+                T* stage = tile;  // [M][EC + 1]
+#pragma unroll
+                for (int it = 0; it < kHold; ++it) {
+                    const int q = task_q + it * task_qstep;
+                    if (q >= ec) continue;
+#pragma unroll
+                    for (int j = 0; j < kNy; ++j) {
+                        stage[task_cell + q + j * G * (EC + 1)] = held[it][j];
+                    }
+                }
+                __syncthreads();
+                T* out_g = out + static_cast<uint64_t>(static_cast<uint32_t>(g)) * block_words + e0;
+                const uint8_t* mask_b = reinterpret_cast<const uint8_t*>(a.masks) + blk * a.M;
+                if (vec && ec == EC) {   // whole rows, 16 bytes per lane
+                    if constexpr (sizeof(T) == 4 && EC % 4 == 0) {
+                        constexpr int kQ = EC / 4;
+                        for (int i = tid; i < M * kQ; i += kConvThreads) {
+                            const int c = i / kQ;
+                            const int q4 = i - c * kQ;
+                            const int c_i = s_inv[c];
+                            if (c_i == 0xFFFF || !mask_b[c_i]) continue;
+                            const T* sp = stage + c * (EC + 1) + 4 * q4;
+                            reinterpret_cast<float4*>(out_g + static_cast<uint32_t>(c) * E)[q4] =
+                                    make_float4(sp[0], sp[1], sp[2], sp[3]);
+                        }
+                    }
+                } else {
+                    for (int i = tid; i < M * ec; i += kConvThreads) {
+                        const int c = i / ec;
+                        const int q = i - c * ec;
+                        const int c_i = s_inv[c];
+                        if (c_i == 0xFFFF || !mask_b[c_i]) continue;
+                        out_g[static_cast<uint32_t>(c) * E + q] = stage[c * (EC + 1) + q];
+                    }
+                }
+            } else {
+#pragma unroll 1
+                for (int at = tid; at < combos * EC; at += kConvThreads) {
                     const int q = at / combos;
                     if (q >= ec) continue;
                     const int rem = at - q * combos;
                     const int x = rem % G;
                     const int y0 = kNy * ((rem / G) % yq_n);
                     const int z = rem / (G * yq_n);
-                    const T* plane = tile + static_cast<size_t>(q) * T3 + x + Tn * y0 + Tn * Tn * z;
-                    const T* wq = s_w + static_cast<size_t>(q) * K;
                     T acc[kNy];
-#pragma unroll
-                    for (int j = 0; j < kNy; ++j) acc[j] = T(0);
-#pragma unroll 1
-                    for (int dz = 0; dz < WT; ++dz) {
-                        const T* pz = plane + Tn * Tn * dz;
-                        T win[kNy][WT > 0 ? WT : 1];
-#pragma unroll
-                        for (int yy = 0; yy < kNy - 1; ++yy) {
-#pragma unroll
-                            for (int dx = 0; dx < WT; ++dx) win[yy][dx] = pz[Tn * yy + dx];
-                        }
-#pragma unroll
-                        for (int dy = 0; dy < WT; ++dy) {
-#pragma unroll
-                            for (int dx = 0; dx < WT; ++dx) {
-                                win[(dy + kNy - 1) & (kNy - 1)][dx] = pz[Tn * (dy + kNy - 1) + dx];
-                            }
-                            T wr[WT > 0 ? WT : 1];
-#pragma unroll
-                            for (int dx = 0; dx < WT; ++dx) wr[dx] = wq[(dz * WT + dy) * WT + dx];
-#pragma unroll
-                            for (int j = 0; j < kNy; ++j) {
-#pragma unroll
-                                for (int dx = 0; dx < WT; ++dx) {
-                                    acc[j] = fma(win[(dy + j) & (kNy - 1)][dx], wr[dx], acc[j]);
-                                }
-                            }
-                        }
-                    }
-                    if (staged) {
-#pragma unroll
-                        for (int j = 0; j < kNy; ++j) held[it][j] = acc[j];
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < kNy; ++j) {
-                            const int c = x + G * (y0 + j) + G * G * z;
-                            const int c_i = s_inv[c];
-                            if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
-                            out[(g * a.M + c) * E + e0 + q] = acc[j];
-                        }
-                    }
-                }
-            }
-            if (staged) {
-                __syncthreads();  // the tile has been read
-                T* stage = tile;  // [M][EC + 1]
-#pragma unroll
-                for (int it = 0; it < kHold; ++it) {
-                    const int item = tid + it * kConvThreads;
-                    if (item >= combos * EC) continue;
-                    const int q = item / combos;
-                    if (q >= ec) continue;
-                    const int rem = item - q * combos;
-                    const int x = rem % G;
-                    const int y0 = kNy * ((rem / G) % yq_n);
-                    const int z = rem / (G * yq_n);
+                    window_sums(tile + static_cast<size_t>(q) * Ts + x + Tn * y0 + Tz * z,
+                                s_w + static_cast<size_t>(q) * K, acc);
 #pragma unroll
                     for (int j = 0; j < kNy; ++j) {
-                        stage[(x + G * (y0 + j) + G * G * z) * (EC + 1) + q] = held[it][j];
+                        const int c = x + G * (y0 + j) + G * G * z;
+                        const int c_i = s_inv[c];
+                        if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
+                        out[(g * a.M + c) * E + e0 + q] = acc[j];
                     }
-                }
-                __syncthreads();
-                for (int i = tid; i < M * ec; i += kConvThreads) {
-                    const int c = i / ec;
-                    const int q = i - c * ec;
-                    const int c_i = s_inv[c];
-                    if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
-                    out[(g * a.M + c) * E + e0 + q] = stage[c * (EC + 1) + q];
                 }
             }
             continue;
@@ -1143,16 +1194,35 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
     const int r = W / 2;
     if (r > G || a.M > 4096 || a.M * a.K > (int64_t{1} << 30)) return -1;
     const int64_t Tn = G + 2 * r;
+    // cells per lane along y, as by_window below picks the instance
+    const bool windowed = W == 3 || W == 5 || W == 7;
+    const int ny = !(windowed && G % 4 == 0 && kConvRowBlocking) ? 0
+                   : (G % 8 == 0 && kConvRows8 && W != 3) ? 8 : 4;
+    // Words between the z layers of a channel's plane.  With blocks of 8^3 a
+    // wavefront's lanes read 8 words along x per group, groups ny * Tn words
+    // apart in y (four cells per lane) and one layer apart in z; the layers are
+    // padded so that the four groups of every 32 lanes meet different banks.
+    int64_t Tz = Tn * Tn;
+    if (G == 8 && ny > 0 && sizeof(T) == 4) {
+        const int a_y = static_cast<int>((4 * Tn) % 32);   // 8, 16 or 24
+        int best = 32;
+        for (int target : {8, 16, 24}) {
+            const bool ok = ny == 8 ? target != 16 : (a_y == 16 ? target != 16 : target == 16);
+            const int pad = static_cast<int>(((target - Tz) % 32 + 32) % 32);
+            if (ok && pad < best) best = pad;
+        }
+        Tz += best;
+    }
     // As many channels per pass as fit: a pass fetches the cache lines of all
     // channels of a row whatever it uses of them.
     constexpr int kMaxEc = sizeof(T) == 4 ? 16 : 8;
-    const size_t cell_bytes = static_cast<size_t>(Tn * Tn * Tn) * sizeof(T);
+    const size_t cell_bytes = static_cast<size_t>(Tz * Tn) * sizeof(T);
     // two workgroups per CU (64 KB each) run faster than one with twice the
     // channels -- except for rows of a cache line or more, where every pass
-    // over a part of the channels fetches the whole rows again (measured on 7^3
-    // windows: E = 8 15.1 vs 16.2 ms, E = 16 39.4 vs 34.2 ms)
-    const size_t budget = a.E * sizeof(T) >= 64 ? kConvTileBytes + kConvTileBytes / 2
-                                                : kConvTileBytes;
+    // over a part of the channels fetches the whole rows again: those may take
+    // most of a CU's LDS for one workgroup (measured with 16 channels: 5^3
+    // window in one pass 13.1 ms, in two passes of eight channels 15.5 ms)
+    const size_t budget = a.E * sizeof(T) >= 64 ? 2 * kConvTileBytes : kConvTileBytes;
     int ec_max = kMaxEc;
     while (ec_max > 1 && cell_bytes * ec_max > budget) ec_max /= 2;
     if (cell_bytes * ec_max > budget) return -1;
@@ -1170,7 +1240,7 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
             ASH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                         hipFuncAttributeMaxDynamicSharedMemorySize,
                                         static_cast<int>(smem)));
-            kernel<<<grid, kConvThreads, smem, s>>>(a, G, r, e0, ec, vec);
+            kernel<<<grid, kConvThreads, smem, s>>>(a, G, r, e0, ec, vec, static_cast<int>(Tz));
             ASH_LAUNCH_CHECK();
             return 0;
         };
