@@ -324,12 +324,14 @@ __device__ __forceinline__ int64_t fetch_block_rows(const McDev& a, int64_t b, i
 }
 
 // Index in the per-cell arrays of tile cell t, -1 if it does not exist.
-__device__ __forceinline__ int64_t tile_source(const McDev& a, const uint16_t* s_src,
-                                               const int64_t* s_nb, int t) {
+// s_nb[s]: index of the first cell of source block s (its row times the cells
+// per block, multiplied once per block instead of once per tile cell), -1 if
+// there is no such block.
+__device__ __forceinline__ int64_t tile_source(const uint16_t* s_src, const int64_t* s_nb, int t) {
     const int src = s_src[t];
     const int from = src >> 12;
     if (from > kSrcOwn || s_nb[from] < 0) return -1;
-    return s_nb[from] * a.M + (src & 0xFFF);
+    return s_nb[from] + (src & 0xFFF);
 }
 
 template <typename T>
@@ -341,28 +343,28 @@ __global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a)
     const int W = a.g + 1;
     const int M = static_cast<int>(a.M);
     const int W3 = tile_cells(a.g);
-    uint16_t* s_src = reinterpret_cast<uint16_t*>(lds);   // [W3]
-    uint16_t* s_pos = s_src + W3;                          // [M]
-    uint8_t* tile = reinterpret_cast<uint8_t*>(s_pos + M); // [W3]
+    uint32_t* s_list = reinterpret_cast<uint32_t*>(lds);        // [2 * 64] cells the surface crosses
+    uint16_t* s_src = reinterpret_cast<uint16_t*>(s_list + 2 * kTileThreads);  // [W3]
+    uint16_t* s_pos = s_src + W3;                               // [M]
+    uint8_t* tile = reinterpret_cast<uint8_t*>(s_pos + M);      // [W3]
     const int lane = threadIdx.x;
     build_tile_map(a, s_src, s_pos);
     const BlockWalk walk = block_walk(a.n_grids);
     int64_t blk = walk.first;
     int64_t row = fetch_block_rows(a, blk, walk.end);
     for (; blk < walk.end; blk += walk.step) {
-        __syncthreads();  // set-up done; previous block's tile and rows read
-        if (lane <= kSrcOwn) s_nb[lane] = row;
+        __syncthreads();  // set-up done; previous block's tile, rows and list read
+        if (lane <= kSrcOwn) s_nb[lane] = row < 0 ? -1 : row * a.M;
         row = fetch_block_rows(a, blk + walk.step, walk.end);
         __syncthreads();
-        const int64_t g = s_nb[kSrcOwn];
-        if (g < 0) continue;  // the same for the whole wavefront
+        if (s_nb[kSrcOwn] < 0) continue;  // the same for the whole wavefront
         for (int t0 = 0; t0 < W3; t0 += 4 * kTileThreads) {
             int64_t at[4];
             T w[4], v[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int t = t0 + k * kTileThreads + lane;
-                at[k] = t < W3 ? tile_source(a, s_src, s_nb, t) : -1;
+                at[k] = t < W3 ? tile_source(s_src, s_nb, t) : -1;
                 w[k] = at[k] >= 0 ? weights[at[k]] : T(0);
                 v[k] = at[k] >= 0 ? sdfs[at[k]] : T(0);
             }
@@ -377,29 +379,56 @@ __global__ __launch_bounds__(kTileThreads) void mc_classify_tile_kernel(McDev a)
             }
         }
         __syncthreads();
-        for (int c = lane; c < M; c += kTileThreads) {
-            const int p = s_pos[c];
+        // The cells the surface crosses are few (a twentieth in a block at the
+        // surface): they are listed first, cell | case << 12, and then handled
+        // by consecutive lanes, instead of by the odd lane of every 64 cells.
+        // The list holds two rounds of cells and is worked off when a third
+        // might not fit.
+        int listed = 0;
+        auto work_off = [&]() {
+            __syncthreads();
+            for (int i = lane; i < listed; i += kTileThreads) {
+                const int p = s_pos[s_list[i] & 0xFFF];
+                const int code = static_cast<int>(s_list[i] >> 12);
+                int64_t at[8];
+                bool usable = true;
+#pragma unroll
+                for (int nb = 0; nb < 8; ++nb) {
+                    // every corner has a source and a row, or `ok` would be clear
+                    const int src = s_src[p + (nb & 1) + ((nb >> 1) & 1) * W + (nb >> 2) * W * W];
+                    const int from = src >> 12;
+                    usable = usable && from <= kSrcOwn;
+                    at[nb] = s_nb[from <= kSrcOwn ? from : kSrcOwn] + (src & 0xFFF);
+                }
+                if (usable) record_case(a, code, at);
+            }
+            __syncthreads();
+            listed = 0;
+        };
+        for (int c0 = 0; c0 < M; c0 += kTileThreads) {
+            const int c = c0 + lane;
             int code = 0;
-            int ok = 1;
+            int ok = 0;
+            if (c < M) {
+                const int p = s_pos[c];
+                ok = 1;
 #pragma unroll
-            for (int nb = 0; nb < 8; ++nb) {
-                const int v = tile[p + (nb & 1) + ((nb >> 1) & 1) * W + (nb >> 2) * W * W];
-                ok &= v;
-                code |= (v >> 1) << nb;
+                for (int nb = 0; nb < 8; ++nb) {
+                    const int v = tile[p + (nb & 1) + ((nb >> 1) & 1) * W + (nb >> 2) * W * W];
+                    ok &= v;
+                    code |= (v >> 1) << nb;
+                }
             }
-            if (!ok || code == 0 || code == 255) continue;
-            int64_t at[8];
-            bool usable = true;
-#pragma unroll
-            for (int nb = 0; nb < 8; ++nb) {
-                // every corner has a source and a row, or `ok` would be clear
-                const int src = s_src[p + (nb & 1) + ((nb >> 1) & 1) * W + (nb >> 2) * W * W];
-                const int from = src >> 12;
-                usable = usable && from <= kSrcOwn;
-                at[nb] = s_nb[from <= kSrcOwn ? from : kSrcOwn] * a.M + (src & 0xFFF);
+            const bool crossed = ok && code != 0 && code != 255;
+            const uint64_t m = __ballot(crossed);
+            if (crossed) {
+                s_list[listed + __popcll(m & ((1ull << lane) - 1ull))] =
+                        static_cast<uint32_t>(c) | (static_cast<uint32_t>(code) << 12);
             }
-            if (usable) record_case(a, code, at);
+            listed += __popcll(m);
+            if (listed > kTileThreads) work_off();   // the same for the whole wavefront
         }
+        work_off();
     }
 }
 
@@ -765,10 +794,10 @@ __global__ __launch_bounds__(kTileThreads) void iso_classify_tile_kernel(McDev a
     int64_t row = fetch_block_rows(a, blk, walk.end);
     for (; blk < walk.end; blk += walk.step) {
         __syncthreads();  // set-up done; previous block's tile and rows read
-        if (lane <= kSrcOwn) s_nb[lane] = row;
+        if (lane <= kSrcOwn) s_nb[lane] = row < 0 ? -1 : row * a.M;
         row = fetch_block_rows(a, blk + walk.step, walk.end);
         __syncthreads();
-        const int64_t g = s_nb[kSrcOwn];
+        const int64_t g = s_nb[kSrcOwn];  // first cell of the block
         if (g < 0) continue;  // the same for the whole wavefront
         for (int t0 = 0; t0 < W3; t0 += 4 * kTileThreads) {
             int64_t at[4];
@@ -776,7 +805,7 @@ __global__ __launch_bounds__(kTileThreads) void iso_classify_tile_kernel(McDev a
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int t = t0 + k * kTileThreads + lane;
-                at[k] = t < W3 ? tile_source(a, s_src, s_nb, t) : -1;
+                at[k] = t < W3 ? tile_source(s_src, s_nb, t) : -1;
                 w[k] = at[k] >= 0 ? weights[at[k]] : T(0);
                 v[k] = at[k] >= 0 ? sdfs[at[k]] : T(0);
             }
@@ -792,7 +821,7 @@ __global__ __launch_bounds__(kTileThreads) void iso_classify_tile_kernel(McDev a
         __syncthreads();
         for (int c = lane; c < M; c += kTileThreads) {
             const int p = s_pos[c];
-            a.cases[g * a.M + c] = static_cast<uint8_t>(
+            a.cases[g + c] = static_cast<uint8_t>(
                     (state[p] & 1) ? crossing_flags<T>(diff[p], diff, state, p, off) : 0);
         }
     }
@@ -855,8 +884,16 @@ bool vector_access(const McDev& a) {
 
 // Workgroups of a one-wavefront-per-block launch: a multiple of the number of
 // XCDs whenever there are that many blocks (see block_walk).
-unsigned tile_grid(int64_t num_grids) {
-    int64_t g = num_grids < kTileMaxGrid ? num_grids : kTileMaxGrid;
+// No more of them than the device holds at once (256 CUs with 160 KB of LDS
+// and 32 wavefronts each): workgroups that had to wait for a free CU would
+// start on their share of the blocks when the others are done with theirs.
+unsigned tile_grid(int64_t num_grids, size_t lds_bytes) {
+    const size_t per_group = (lds_bytes + 128 + 1023) / 1024 * 1024;  // + static, allocation unit
+    int64_t per_cu = static_cast<int64_t>(160 * 1024 / per_group);
+    if (per_cu > 32) per_cu = 32;
+    if (per_cu < 1) per_cu = 1;
+    const int64_t resident = per_cu * 256 < kTileMaxGrid ? per_cu * 256 : kTileMaxGrid;
+    int64_t g = num_grids < resident ? num_grids : resident;
     if (g >= kXcds) g -= g % kXcds;
     return static_cast<unsigned>(g < 1 ? 1 : g);
 }
@@ -949,8 +986,9 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     const bool tiled = grid_dim <= kMaxTileG &&
                        static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
     if (tiled) {
-        const unsigned by_block = tile_grid(num_grids);
-        const size_t lds = static_cast<size_t>(3 * tile_cells(grid_dim)) + 2 * cells_per_grid;
+        const size_t lds = static_cast<size_t>(3 * tile_cells(grid_dim)) + 2 * cells_per_grid +
+                           8 * kTileThreads;
+        const unsigned by_block = tile_grid(num_grids, lds);
         if (dtype == ASH_F32) {
             mc_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
         } else {
@@ -1066,7 +1104,7 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
         const bool tiled = grid_dim <= kMaxTileG && lds <= 63 * 1024 &&
                            static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
         if (tiled) {
-            const unsigned by_block = tile_grid(num_grids);
+            const unsigned by_block = tile_grid(num_grids, lds);
             if (dtype == ASH_F32) {
                 iso_classify_tile_kernel<float><<<by_block, kTileThreads, lds, s>>>(a);
             } else {
