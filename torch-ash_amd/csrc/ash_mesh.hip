@@ -40,7 +40,7 @@ constexpr int kBlock = 256;
 constexpr int kPerThread = 16;
 constexpr int kChunk = kBlock * kPerThread;   // cells per reservation
 constexpr int kMaxTileG = 16;                 // block edge handled by the LDS tile
-constexpr int kMaxGrid = 4096;                // workgroups of a persistent launch
+constexpr int kMaxGrid = 65536;               // workgroups of a chunk launch: one per chunk up to here (8192: 5 % slower, 4096: 10 %)
 constexpr int64_t kMaxVertices = int64_t{1} << 29;  // ids live in 29 bits
 
 // Layout of the int32 workspace: totals, then per chunk of kChunk cells the
@@ -898,7 +898,7 @@ unsigned tile_grid(int64_t num_grids, size_t lds_bytes) {
     return static_cast<unsigned>(g < 1 ? 1 : g);
 }
 
-unsigned persistent_grid(int64_t work_items) {
+unsigned chunk_grid(int64_t work_items) {
     if (work_items < 1) return 1;
     return static_cast<unsigned>(work_items < kMaxGrid ? work_items : kMaxGrid);
 }
@@ -973,8 +973,8 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     a.weight_thr = weight_thr;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cells = num_grids * cells_per_grid;
-    const unsigned by_cell = persistent_grid((cells + kBlock - 1) / kBlock);
-    const unsigned by_chunk = persistent_grid((cells + kChunk - 1) / kChunk);
+    const unsigned by_cell = chunk_grid((cells + kBlock - 1) / kBlock);
+    const unsigned by_chunk = chunk_grid((cells + kChunk - 1) / kChunk);
     const bool vec = vector_access(a);
     if (vec) {
         mc_clear_kernel<4><<<by_chunk, kBlock, 0, s>>>(a);
@@ -1045,7 +1045,7 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
     a.n_triangles = n_triangles;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cells = num_grids * cells_per_grid;
-    const unsigned by_chunk = persistent_grid((cells + kChunk - 1) / kChunk);
+    const unsigned by_chunk = chunk_grid((cells + kChunk - 1) / kChunk);
     const bool vec = vector_access(a);
     if (dtype == ASH_F32) {
         if (vec) {
@@ -1111,7 +1111,7 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
                 iso_classify_tile_kernel<double><<<by_block, kTileThreads, lds, s>>>(a);
             }
         } else {
-            const unsigned by_cell = persistent_grid((cells + kBlock - 1) / kBlock);
+            const unsigned by_cell = chunk_grid((cells + kBlock - 1) / kBlock);
             if (dtype == ASH_F32) {
                 iso_classify_cell_kernel<float><<<by_cell, kBlock, 0, s>>>(a);
             } else {
@@ -1120,9 +1120,9 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
         }
         ASH_LAUNCH_CHECK();
         if (a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0) {
-            iso_count_kernel<4><<<persistent_grid(chunks), kBlock, 0, s>>>(a);
+            iso_count_kernel<4><<<chunk_grid(chunks), kBlock, 0, s>>>(a);
         } else {
-            iso_count_kernel<1><<<persistent_grid(chunks), kBlock, 0, s>>>(a);
+            iso_count_kernel<1><<<chunk_grid(chunks), kBlock, 0, s>>>(a);
         }
         ASH_LAUNCH_CHECK();
     }
@@ -1157,7 +1157,7 @@ int ash_isosurface_points(const void* sdfs, const int64_t* grid_indices,
     a.positions = positions;
     a.n_vertices = n_points;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const unsigned by_chunk = persistent_grid((num_grids * cells_per_grid + kChunk - 1) / kChunk);
+    const unsigned by_chunk = chunk_grid((num_grids * cells_per_grid + kChunk - 1) / kChunk);
     const bool vec = a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0;
     if (dtype == ASH_F32) {
         if (vec) {
