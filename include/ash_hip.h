@@ -329,6 +329,21 @@ int ash_query_backward_backward(const ash_query_args* a,
                                 void* grad_z, void* grad_embeddings,
                                 void* stream);
 
+/* The two gradient calls above with grad_embeddings added to instead of
+ * zero-filled: the caller passes a gradient that already holds the other
+ * contributions to the same embeddings (it must not be NULL).  No counterpart
+ * in the reference, which zero-fills a new dense tensor in every call and
+ * leaves the sum of two such tensors to autograd: a training step with a value
+ * loss and a gradient-norm loss then pays two dense fills and one dense add
+ * that this variant saves. */
+int ash_query_backward_forward_accumulate(const ash_query_args* a, const void* z,
+                                          void* grad_embeddings, void* grad_offsets,
+                                          void* stream);
+int ash_query_backward_backward_accumulate(const ash_query_args* a,
+                                           const void* grad_grad_offsets, const void* z,
+                                           void* grad_z, void* grad_embeddings,
+                                           void* stream);
+
 /* Replaces `convolution_forward` (ash/src/grid.cu:948-1043, pybind.cpp:33).
  * inputs / outputs scalar[num_embeddings, cells_per_grid, embedding_dim];
  * weights scalar[num_cell_nbs, embedding_dim] (one weight per window tap and

@@ -256,7 +256,7 @@ class OracleBackend:
     def query_backward_forward(
         self, z, embeddings, offsets, grid_indices, cell_indices, masks,
         lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb,
-        grid_dim, interpolation, need_embeddings=True, need_offsets=True,
+        grid_dim, interpolation, need_embeddings=True, need_offsets=True, accumulate_into=None,
     ) -> Tuple[torch.Tensor, torch.Tensor]:
         if interpolation not in _INTERP:
             raise RuntimeError(f"Unknown interpolation functor: {interpolation}")
@@ -275,13 +275,16 @@ class OracleBackend:
             z.data_ptr(), *[t.data_ptr() for t in held], grad_emb.data_ptr(),
             grad_off.data_ptr(), n, b, m, e, _INTERP[interpolation],
         )
+        if accumulate_into is not None:
+            accumulate_into.add_(grad_emb.to(accumulate_into.device))
+            grad_emb = accumulate_into
         return (grad_emb if need_embeddings else None), (grad_off if need_offsets else None)
 
     def query_backward_backward(
         self, grad_grad_embeddings, grad_grad_offsets, z, embeddings, offsets,
         grid_indices, cell_indices, masks, lut_grid_nb2grid_idx,
         lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, grid_dim, interpolation,
-        need_z=True, need_embeddings=True,
+        need_z=True, need_embeddings=True, accumulate_into=None,
     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         if interpolation not in _INTERP:
             raise RuntimeError(f"Unknown interpolation functor: {interpolation}")
@@ -301,6 +304,9 @@ class OracleBackend:
             gg_off.data_ptr(), z.data_ptr(), *[t.data_ptr() for t in held],
             grad_z.data_ptr(), grad_emb.data_ptr(), n, b, m, e, _INTERP[interpolation],
         )
+        if accumulate_into is not None:
+            accumulate_into.add_(grad_emb.to(accumulate_into.device))
+            grad_emb = accumulate_into
         return (
             grad_z if need_z else None,
             grad_emb if need_embeddings else None,

@@ -269,6 +269,99 @@ def test_eikonal_training_step_matches_autograd(gpu_ash, interpolation):
     assert torch.allclose(got, ref, rtol=1e-4, atol=1e-6), (got - ref).abs().max()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_accumulating_gradient_calls(gpu_ash, oracle, dtype):
+    """ash_query_backward_forward_accumulate / _backward_accumulate add to the
+    tensor they are given what the plain calls return (checked against the
+    oracle's gradient on top of a random start), write the other output as
+    usual, and refuse a tensor that is not like the embeddings."""
+    grid = _make_grid(gpu_ash, 4, 3, 1, dtype=dtype, seed=51, holes=2)
+    x = _queries(4, 1, 5000, seed=52, margin=1.0)
+    ops = _operands(grid, x)
+    backend = gpu_ash.grid_query.backend
+    g = torch.Generator().manual_seed(53)
+    n = x.shape[0]
+    z = (torch.rand(n, 3, generator=g, dtype=dtype) - 0.5).to(DEV)
+    u = (torch.rand(n, 3, generator=g, dtype=dtype) - 0.5).to(DEV)
+    start = (torch.rand(ops[0].shape, generator=g, dtype=dtype) - 0.5).to(DEV)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-12, atol=1e-12)
+
+    ref_emb, ref_off = oracle.query_backward_forward(z.cpu(), *_to_cpu(ops), 4, "smooth_step")
+    acc = start.clone()
+    got_emb, got_off = backend.query_backward_forward(z, *ops, 4, "smooth_step", accumulate_into=acc)
+    assert got_emb is acc
+    assert torch.allclose(acc.cpu(), start.cpu() + ref_emb, **tol)
+    assert torch.allclose(got_off.cpu(), ref_off, **tol)
+    acc = start.clone()
+    _, none_off = backend.query_backward_forward(z, *ops, 4, "smooth_step", need_offsets=False,
+                                                 accumulate_into=acc)
+    assert none_off is None and torch.allclose(acc.cpu(), start.cpu() + ref_emb, **tol)
+
+    ref_z, ref_emb2, _ = oracle.query_backward_backward(None, u.cpu(), z.cpu(), *_to_cpu(ops), 4, "smooth_step")
+    acc = start.clone()
+    got_z, got_emb2, _ = backend.query_backward_backward(None, u, z, *ops, 4, "smooth_step",
+                                                         accumulate_into=acc)
+    assert got_emb2 is acc
+    assert torch.allclose(acc.cpu(), start.cpu() + ref_emb2, **tol)
+    assert torch.allclose(got_z.cpu(), ref_z, **tol)
+
+    with pytest.raises(RuntimeError, match="accumulate_into"):
+        backend.query_backward_forward(z, *ops, 4, "smooth_step", accumulate_into=start[:-1])
+    with pytest.raises(RuntimeError, match="accumulate_into"):
+        backend.query_backward_backward(None, u, z, *ops, 4, "smooth_step",
+                                        accumulate_into=start.to(torch.float16))
+
+
+def test_training_step_shares_one_dense_gradient(gpu_ash):
+    """In a pass that reaches the embeddings through the first- and the
+    second-order backward, the second node adds to the first one's gradient
+    (ash_query_backward_*_accumulate) instead of filling a dense tensor of its
+    own: same .grad as two separate passes, one accumulating call per pass,
+    also on a second pass into an existing .grad."""
+    grid = _make_grid(gpu_ash, 4, 4, 2, seed=41, holes=5)
+    x = _queries(4, 2, 20_000, seed=42)
+    backend = gpu_ash.grid_query.backend
+    shared_calls = []
+    reals = {name: getattr(backend, name)
+             for name in ("query_backward_forward", "query_backward_backward")}
+
+    def spy(name):
+        def call(*args, **kwargs):
+            if kwargs.get("accumulate_into") is not None:
+                shared_calls.append(name)
+            return reals[name](*args, **kwargs)
+        return call
+
+    def losses():
+        xq = x.clone().requires_grad_(True)
+        feats, _ = grid(xq, "smooth_step")
+        (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+        return (feats[:, 1:] ** 2).mean(), (gx.norm(dim=-1) - 1).abs().mean()
+
+    for name in reals:
+        setattr(backend, name, spy(name))
+    try:
+        expected = torch.zeros_like(grid.embeddings)
+        for which in (0, 1):
+            grid.embeddings.grad = None
+            losses()[which].backward()
+            expected += grid.embeddings.grad
+        assert shared_calls == []
+        grid.embeddings.grad = None
+        value, eikonal = losses()
+        (value + eikonal).backward()
+        assert len(shared_calls) == 1
+        # atomically accumulated sums of a few terms each: order-dependent rounding only
+        assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-4, atol=1e-7)
+        value, eikonal = losses()
+        (value + eikonal).backward()
+        assert len(shared_calls) == 2
+        assert torch.allclose(grid.embeddings.grad, 2 * expected, rtol=1e-4, atol=2e-7)
+    finally:
+        for name in reals:
+            delattr(backend, name)
+
+
 def _config_grid(gpu_ash, embedding_dim, num_blocks=3000, sparse=64):
     return workloads.build_grid(
         gpu_ash, num_blocks, embedding_dim, grid_dim=8, sparse_grid_dim=sparse, device=DEV

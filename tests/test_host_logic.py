@@ -239,6 +239,91 @@ def test_grid_gradcheck_through_autograd_functions(cpu_ash, embedding_dim, grid_
     assert torch.equal(a, b)
 
 
+def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
+    """A value loss plus a gradient-norm loss reach the embeddings through the
+    first- and the second-order backward in one pass: the second node adds to
+    the first node's gradient instead of producing a dense tensor of its own,
+    and the result is what separate passes give -- also with another user of
+    the embeddings in the loss, on a second pass into an existing .grad, and
+    not at all while a graph of the backward is being recorded."""
+    torch.manual_seed(7)
+    g_dim = 2
+    grid = cpu_ash.SparseDenseGrid(3, 8, 3, g_dim, device=CPU)
+    r = torch.arange(0, 2, dtype=torch.int)
+    grid.spatial_init_(g_dim * torch.stack(torch.meshgrid(r, r, r, indexing="ij"), -1).view(-1, 3), dilation=0)
+    grid.construct_grid_neighbor_lut_(1, False)
+    with torch.no_grad():
+        grid.embeddings.copy_(torch.rand(grid.embeddings.shape) * 2 - 1)
+    x = (torch.randint(high=g_dim * 2 - 1, size=(50, 3)) + torch.rand(50, 3).clamp(0.05, 0.95))
+
+    shared_calls = []
+    for name in ("query_backward_forward", "query_backward_backward"):
+        real = getattr(oracle, name)
+
+        def spy(*args, _real=real, _name=name, **kwargs):
+            if kwargs.get("accumulate_into") is not None:
+                shared_calls.append(_name)
+            return _real(*args, **kwargs)
+
+        monkeypatch.setattr(oracle, name, spy, raising=False)
+
+    def losses(xq):
+        feats, _ = grid(xq, "smooth_step")
+        (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+        return (feats[:, 1:] ** 2).mean(), (gx.norm(dim=-1) - 1).abs().mean()
+
+    def separate():
+        total = torch.zeros_like(grid.embeddings)
+        for which in (0, 1):
+            grid.embeddings.grad = None
+            losses(x.clone().requires_grad_(True))[which].backward()
+            total += grid.embeddings.grad
+        return total
+
+    expected = separate()
+    assert shared_calls == []          # one producer per pass: nothing to share
+
+    grid.embeddings.grad = None
+    value, eikonal = losses(x.clone().requires_grad_(True))
+    (value + eikonal).backward()
+    assert len(shared_calls) == 1
+    assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
+
+    # a second pass adds to the existing .grad
+    value, eikonal = losses(x.clone().requires_grad_(True))
+    (value + eikonal).backward()
+    assert len(shared_calls) == 2
+    assert torch.allclose(grid.embeddings.grad, 2 * expected, rtol=1e-5, atol=1e-6)
+
+    # a regulariser is a third contribution; whether autograd sums it into the
+    # shared tensor or into a new one (which ends the sharing), the total holds
+    grid.embeddings.grad = None
+    value, eikonal = losses(x.clone().requires_grad_(True))
+    (value + eikonal + 0.5 * (grid.embeddings ** 2).sum()).backward()
+    want = expected + grid.embeddings.detach()
+    assert torch.allclose(grid.embeddings.grad, want, rtol=1e-5, atol=1e-6)
+
+    # while a graph of the backward pass is recorded nothing is shared
+    before = len(shared_calls)
+    grid.embeddings.grad = None
+    value, eikonal = losses(x.clone().requires_grad_(True))
+    (got,) = torch.autograd.grad(value + eikonal, grid.embeddings, create_graph=True)
+    assert len(shared_calls) == before
+    assert torch.allclose(got.detach(), expected, rtol=1e-5, atol=1e-7)
+
+    # two different leaves over the same storage are two consumers
+    grid.embeddings.grad = None
+    alias = grid.embeddings.detach().requires_grad_(True)
+    tables = (grid.lut_grid_nb2grid_idx, grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, g_dim)
+    gi, ci, off, masks = grid.query(x)
+    before = len(shared_calls)
+    a = cpu_ash.SparseDenseGridQuery.apply(grid.embeddings, off, gi, ci, masks, *tables)
+    b = cpu_ash.SparseDenseGridQuery.apply(alias, off, gi, ci, masks, *tables)
+    (a.sum() + 2 * b.sum()).backward()
+    assert len(shared_calls) == before
+    assert torch.allclose(alias.grad, 2 * grid.embeddings.grad)
+
+
 # ---------------------------------------------- engine / set / map / embedding
 @pytest.mark.parametrize("dim", [1, 2, 3, 4])
 def test_engine_state_dict_layout_and_round_trip(cpu_ash, dim, tmp_path):

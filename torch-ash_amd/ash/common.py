@@ -179,6 +179,14 @@ _SIGNATURES = {
         ctypes.c_int,
         [ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR, _PTR],
     ),
+    "ash_query_backward_forward_accumulate": (
+        ctypes.c_int,
+        [ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR],
+    ),
+    "ash_query_backward_backward_accumulate": (
+        ctypes.c_int,
+        [ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR, _PTR],
+    ),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -643,10 +651,13 @@ class _Backend:
         interpolation,
         need_embeddings: bool = True,
         need_offsets: bool = True,
+        accumulate_into: Optional[torch.Tensor] = None,
     ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
         """(grad_embeddings, grad_offsets); an output that is not needed is
         None and its work (for grad_embeddings: dense zero fill + atomics) is
-        skipped."""
+        skipped.  With `accumulate_into` (a gradient of the embeddings' shape
+        that already holds other contributions) the embedding gradient is added
+        to that tensor, which is also what is returned."""
         args, held, dev = self._query_args(
             embeddings,
             offsets,
@@ -659,7 +670,13 @@ class _Backend:
             interpolation,
         )
         z = _as_like(z, embeddings, (args.num_queries, args.embedding_dim), "z")
-        grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
+        entry = self.lib.ash_query_backward_forward
+        if accumulate_into is not None:
+            need_embeddings = True
+            grad_embeddings = _accumulator(accumulate_into, held[0])
+            entry = self.lib.ash_query_backward_forward_accumulate
+        else:
+            grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
         grad_offsets = (
             torch.empty((args.num_queries, 3), dtype=embeddings.dtype, device=dev)
             if need_offsets
@@ -667,7 +684,7 @@ class _Backend:
         )
         with torch.cuda.device(dev):
             self.check(
-                self.lib.ash_query_backward_forward(
+                entry(
                     ctypes.byref(args),
                     z.data_ptr(),
                     grad_embeddings.data_ptr() if need_embeddings else None,
@@ -694,9 +711,11 @@ class _Backend:
         interpolation,
         need_z: bool = True,
         need_embeddings: bool = True,
+        accumulate_into: Optional[torch.Tensor] = None,
     ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor]:
         """(grad_z, grad_embeddings, zero grad_offsets); outputs that are not
-        needed are None and their work is skipped."""
+        needed are None and their work is skipped.  `accumulate_into` as for
+        query_backward_forward."""
         args, held, dev = self._query_args(
             embeddings,
             offsets,
@@ -712,10 +731,16 @@ class _Backend:
         z = _as_like(z, embeddings, (n, e), "z")
         gg_off = _as_like(grad_grad_offsets, embeddings, (n, 3), "grad_grad_offsets")
         grad_z = torch.empty((n, e), dtype=embeddings.dtype, device=dev) if need_z else None
-        grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
+        entry = self.lib.ash_query_backward_backward
+        if accumulate_into is not None:
+            need_embeddings = True
+            grad_embeddings = _accumulator(accumulate_into, held[0])
+            entry = self.lib.ash_query_backward_backward_accumulate
+        else:
+            grad_embeddings = torch.empty_like(held[0]) if need_embeddings else None
         with torch.cuda.device(dev):
             self.check(
-                self.lib.ash_query_backward_backward(
+                entry(
                     ctypes.byref(args),
                     gg_off.data_ptr(),
                     z.data_ptr(),
@@ -727,6 +752,18 @@ class _Backend:
         # the offsets second-order term is not produced (ash/src/grid.cu:417-418)
         grad_offsets = torch.zeros((n, 3), dtype=embeddings.dtype, device=dev)
         return grad_z, grad_embeddings, grad_offsets
+
+
+def _accumulator(t: torch.Tensor, embeddings: torch.Tensor) -> torch.Tensor:
+    """Checks that `t` can take a gradient of `embeddings` in place."""
+    if (
+        t.shape != embeddings.shape
+        or t.dtype != embeddings.dtype
+        or t.device != embeddings.device
+        or not t.is_contiguous()
+    ):
+        raise RuntimeError("accumulate_into must be a contiguous tensor like the embeddings")
+    return t
 
 
 def _numel(shape) -> int:

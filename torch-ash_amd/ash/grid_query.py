@@ -3,6 +3,7 @@ backward.  Two chained Functions with the same operands and return
 conventions as the reference (ash/grid_query.py:10-283); each one is a single
 call into the HIP library.
 """
+import weakref
 from typing import Literal
 
 import torch
@@ -12,6 +13,52 @@ from .common import _get_c_extension
 backend = _get_c_extension()
 
 _N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
+
+# One backward pass can reach the same embeddings through several nodes: a
+# training step with a value loss and a gradient-norm loss runs both the first-
+# and the second-order backward, and each would zero-fill a dense gradient of the
+# whole parameter and leave the sum of the two to autograd (two fills and an add
+# over the parameter: about a third of such a step).  Instead, the first node of
+# a pass that produces the gradient for a consumer remembers it here, and a
+# later node of the same pass adds its contribution to that tensor in place and
+# returns no gradient of its own.
+#   consumer (graph node, input number) -> (graph task id, weak reference)
+# Only passes without create_graph share (an in-place change would be invisible
+# to a graph recorded over the first gradient); the tensor is only referenced
+# weakly, so autograd can still adopt it as .grad without a copy, and a tensor
+# that autograd has already replaced by a sum is gone and not written to.
+_shared_gradients = {}
+_SHARED_MAX = 8
+
+
+def _pass_id() -> int:
+    if torch.is_grad_enabled():
+        return -1
+    try:
+        return torch._C._current_graph_task_id()
+    except Exception:  # older torch
+        return -1
+
+
+def _shared_gradient(consumer):
+    """The gradient another node of the running pass already produced for
+    `consumer`, or None."""
+    task = _pass_id()
+    if task < 0 or consumer is None or consumer[0] is None:
+        return None
+    entry = _shared_gradients.get(consumer)
+    if entry is None or entry[0] != task:
+        return None
+    return entry[1]()
+
+
+def _share_gradient(consumer, gradient) -> None:
+    task = _pass_id()
+    if task < 0 or gradient is None or consumer is None or consumer[0] is None:
+        return
+    if len(_shared_gradients) >= _SHARED_MAX:
+        _shared_gradients.clear()
+    _shared_gradients[consumer] = (task, weakref.ref(gradient))
 
 
 def _grad_requested(ctx, index: int) -> bool:
@@ -78,6 +125,20 @@ class SparseDenseGridQuery(torch.autograd.Function):
         # the dense embedding gradient (zero fill + atomics over the whole
         # parameter) is skipped when nobody asked for it, e.g. in
         # autograd.grad(y, x, create_graph=True).
+        consumer = ctx.next_functions[0] if need_embeddings else None
+        shared = _shared_gradient(consumer)
+        if shared is not None:
+            # no graph is being recorded: the library is called directly
+            _, grad_offsets = backend.query_backward_forward(
+                z.contiguous(),
+                *ctx.saved_tensors,
+                ctx.grid_dim,
+                ctx.interpolation,
+                need_embeddings=True,
+                need_offsets=need_offsets,
+                accumulate_into=shared,
+            )
+            return (None, grad_offsets) + (None,) * _N_TABLE_ARGS
         grad_embeddings, grad_offsets = SparseDenseGridQueryBackward.apply(
             z.contiguous(),
             *ctx.saved_tensors,
@@ -86,6 +147,7 @@ class SparseDenseGridQuery(torch.autograd.Function):
             need_embeddings,
             need_offsets,
         )
+        _share_gradient(consumer, grad_embeddings)
         return (grad_embeddings, grad_offsets) + (None,) * _N_TABLE_ARGS
 
 
@@ -157,6 +219,20 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
         n_rest = _N_TABLE_ARGS + 3  # offsets, tables, grid_dim, interpolation, 2 flags
         if grad_grad_offsets is None or not (need_z or need_embeddings):
             return (None, None) + (None,) * n_rest
+        consumer = ctx.next_functions[1] if need_embeddings else None
+        shared = _shared_gradient(consumer)
+        if shared is not None:
+            grad_z, _, _ = backend.query_backward_backward(
+                grad_grad_embeddings,
+                grad_grad_offsets,
+                *ctx.saved_tensors,
+                ctx.grid_dim,
+                ctx.interpolation,
+                need_z=need_z,
+                need_embeddings=True,
+                accumulate_into=shared,
+            )
+            return (grad_z, None) + (None,) * n_rest
         if need_z and need_embeddings:
             grad_z, grad_embeddings, _ = backend.query_backward_backward(
                 grad_grad_embeddings,
@@ -175,4 +251,5 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
                 need_z=need_z,
                 need_embeddings=need_embeddings,
             )
+        _share_gradient(consumer, grad_embeddings)
         return (grad_z, grad_embeddings) + (None,) * n_rest

@@ -1629,16 +1629,17 @@ int ash_query_forward(const ash_query_args* a, void* output, void* stream) {
                                : dispatch_forward<float>(d, output, s);
 }
 
-int ash_query_backward_forward(const ash_query_args* a, const void* z,
-                               void* grad_embeddings, void* grad_offsets,
-                               void* stream) {
+namespace {
+
+int backward_forward(const ash_query_args* a, const void* z, void* grad_embeddings,
+                     void* grad_offsets, void* stream, bool clear) {
     QDev d;
     if (check_args(a, d)) return 1;
     if (grad_embeddings == nullptr && grad_offsets == nullptr) {
         ASH_FAIL("at least one of grad_embeddings / grad_offsets is required");
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (grad_embeddings != nullptr &&
+    if (clear && grad_embeddings != nullptr &&
         zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
         return 1;
     }
@@ -1651,17 +1652,16 @@ int ash_query_backward_forward(const ash_query_args* a, const void* z,
                                              grad_offsets, s);
 }
 
-int ash_query_backward_backward(const ash_query_args* a,
-                                const void* grad_grad_offsets, const void* z,
-                                void* grad_z, void* grad_embeddings,
-                                void* stream) {
+int backward_backward(const ash_query_args* a, const void* grad_grad_offsets,
+                      const void* z, void* grad_z, void* grad_embeddings,
+                      void* stream, bool clear) {
     QDev d;
     if (check_args(a, d)) return 1;
     if (grad_embeddings == nullptr && grad_z == nullptr) {
         ASH_FAIL("at least one of grad_z / grad_embeddings is required");
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (grad_embeddings != nullptr &&
+    if (clear && grad_embeddings != nullptr &&
         zero_fill(grad_embeddings, d.B * d.M * d.E * elem_bytes(a->dtype), s)) {
         return 1;
     }
@@ -1672,6 +1672,36 @@ int ash_query_backward_backward(const ash_query_args* a,
                                               grad_embeddings, s)
                    : dispatch_bwd_bwd<float>(d, grad_grad_offsets, z, grad_z,
                                              grad_embeddings, s);
+}
+
+}  // namespace
+
+int ash_query_backward_forward(const ash_query_args* a, const void* z,
+                               void* grad_embeddings, void* grad_offsets,
+                               void* stream) {
+    return backward_forward(a, z, grad_embeddings, grad_offsets, stream, true);
+}
+
+int ash_query_backward_forward_accumulate(const ash_query_args* a, const void* z,
+                                          void* grad_embeddings, void* grad_offsets,
+                                          void* stream) {
+    if (grad_embeddings == nullptr) ASH_FAIL("accumulate: null grad_embeddings");
+    return backward_forward(a, z, grad_embeddings, grad_offsets, stream, false);
+}
+
+int ash_query_backward_backward(const ash_query_args* a,
+                                const void* grad_grad_offsets, const void* z,
+                                void* grad_z, void* grad_embeddings,
+                                void* stream) {
+    return backward_backward(a, grad_grad_offsets, z, grad_z, grad_embeddings, stream, true);
+}
+
+int ash_query_backward_backward_accumulate(const ash_query_args* a,
+                                           const void* grad_grad_offsets, const void* z,
+                                           void* grad_z, void* grad_embeddings,
+                                           void* stream) {
+    if (grad_embeddings == nullptr) ASH_FAIL("accumulate: null grad_embeddings");
+    return backward_backward(a, grad_grad_offsets, z, grad_z, grad_embeddings, stream, false);
 }
 
 int ash_convolution_forward(const void* inputs, const void* weights,
