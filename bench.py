@@ -138,7 +138,8 @@ def measure_ceilings(torch, ash, dev, table_bytes, n):
     buf = torch.empty(table_bytes // 128 * 128, dtype=torch.uint8, device=dev).fill_(255)
     sink = torch.empty(n, dtype=torch.int32, device=dev)
     out = {}
-    for mode, name in ((0, "random_line_reads"), (1, "random_line_updates")):
+    for mode, name in ((0, "random_line_reads"), (1, "random_line_updates"),
+                       (2, "random_half_line_reads")):
         timer = EventTimer(torch)
         for it in range(6):
             call = lambda: lib.ash_diag_random_lines(

@@ -455,7 +455,9 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
  * that keep the accesses alive.  The caller times the call.
  *   mode 0: every line is read in full by 8 lanes x 16 bytes (a table probe);
  *   mode 1: per line one 64-bit read, one 64-bit compare-and-swap and one
- *           32-bit store (the accesses of an insert); modifies `buf`. */
+ *           32-bit store (the accesses of an insert); modifies `buf`;
+ *   mode 2: `n` pseudo-random aligned 64-byte halves of lines, each read by 4
+ *           lanes x 16 bytes (what a table of 64-byte buckets would fetch). */
 int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes, int64_t n,
                           uint32_t* sink, uint64_t seed, void* stream);
 

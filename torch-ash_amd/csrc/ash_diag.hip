@@ -44,6 +44,31 @@ __global__ __launch_bounds__(kBlock) void probe_line_reads(
     if (t < n) sink[t] = s;
 }
 
+// Every group of 4 lanes reads 4 pseudo-random aligned 64-byte halves of
+// lines, 16 bytes per lane: what a probe of a table with 64-byte buckets would
+// fetch (n counts the halves).
+__global__ __launch_bounds__(kBlock) void probe_half_line_reads(
+        const uint4* __restrict__ buf, uint32_t nlines, int64_t n,
+        uint32_t* __restrict__ sink, uint64_t seed) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int j = lane & 3;
+    const int gbase = lane & ~3;
+    const uint64_t h = mix64(static_cast<uint64_t>(t) + seed);
+    const uint32_t half = 2u * __umulhi(static_cast<uint32_t>(h >> 32), nlines) +
+                          (static_cast<uint32_t>(h) & 1u);
+    uint4 v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t hr = __shfl(half, gbase | r);
+        v[r] = buf[static_cast<size_t>(hr) * 4 + j];
+    }
+    uint32_t s = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s += v[r].x ^ v[r].y ^ v[r].z ^ v[r].w;
+    if (t < n) sink[t] = s;
+}
+
 // One thread per line: read one 64-bit word, compare-and-swap it, store one
 // dword elsewhere in the line -- the three accesses an insert makes.
 __global__ __launch_bounds__(kBlock) void probe_line_updates(
@@ -88,6 +113,9 @@ extern "C" int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes,
     } else if (mode == 1) {
         probe_line_updates<<<g, kBlock, 0, s>>>(
                 static_cast<unsigned long long*>(buf), nlines, n, sink, seed);
+    } else if (mode == 2) {
+        probe_half_line_reads<<<g, kBlock, 0, s>>>(static_cast<const uint4*>(buf),
+                                                   nlines, n, sink, seed);
     } else {
         ASH_FAIL("unknown probe mode");
     }
