@@ -19,16 +19,16 @@ _N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
 # and the second-order backward, and each would zero-fill a dense gradient of the
 # whole parameter and leave the sum of the two to autograd (two fills and an add
 # over the parameter: about a third of such a step).  Instead, the first node of
-# a pass that produces the gradient for a consumer remembers it here, and a
-# later node of the same pass adds its contribution to that tensor in place and
-# returns no gradient of its own.
-#   consumer (graph node, input number) -> (graph task id, weak reference)
+# a pass that produces the gradient for a consumer (graph node, input number)
+# leaves a note with that consumer -- the graph task and a weak reference to the
+# tensor, in the node's own metadata dictionary, so that the note lives and dies
+# with the node -- and a later node of the same pass adds its contribution to
+# that tensor in place and returns no gradient of its own.
 # Only passes without create_graph share (an in-place change would be invisible
 # to a graph recorded over the first gradient); the tensor is only referenced
 # weakly, so autograd can still adopt it as .grad without a copy, and a tensor
 # that autograd has already replaced by a sum is gone and not written to.
-_shared_gradients = {}
-_SHARED_MAX = 8
+_NOTE = "ash_shared_gradient"
 
 
 def _pass_id() -> int:
@@ -40,25 +40,36 @@ def _pass_id() -> int:
         return -1
 
 
-def _shared_gradient(consumer):
-    """The gradient another node of the running pass already produced for
-    `consumer`, or None."""
+def _notes(consumer):
+    """(graph task, dictionary of the consumer node, key) or None."""
     task = _pass_id()
     if task < 0 or consumer is None or consumer[0] is None:
         return None
-    entry = _shared_gradients.get(consumer)
+    try:
+        return task, consumer[0].metadata, (_NOTE, consumer[1])
+    except Exception:  # a node without metadata
+        return None
+
+
+def _shared_gradient(consumer):
+    """The gradient another node of the running pass already produced for
+    `consumer`, or None."""
+    notes = _notes(consumer)
+    if notes is None:
+        return None
+    task, where, key = notes
+    entry = where.get(key)
     if entry is None or entry[0] != task:
         return None
     return entry[1]()
 
 
 def _share_gradient(consumer, gradient) -> None:
-    task = _pass_id()
-    if task < 0 or gradient is None or consumer is None or consumer[0] is None:
+    notes = _notes(consumer)
+    if notes is None or gradient is None:
         return
-    if len(_shared_gradients) >= _SHARED_MAX:
-        _shared_gradients.clear()
-    _shared_gradients[consumer] = (task, weakref.ref(gradient))
+    task, where, key = notes
+    where[key] = (task, weakref.ref(gradient))
 
 
 def _grad_requested(ctx, index: int) -> bool:
