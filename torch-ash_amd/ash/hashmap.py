@@ -1,7 +1,9 @@
-"""HashMap and HashSet: an ASHEngine plus (for the map) value tensors it owns.
+"""HashSet and HashMap: an ASHEngine, plus (for the map) the value tensors it
+addresses.
 
-Same constructor arguments, method names, return orders and buffer names as
-the reference wrappers (ash/hashmap.py:7-178).
+Constructor arguments, method names, return orders and buffer names are those
+of the reference wrappers (ash/hashmap.py:7-178); how values are declared and
+handed over is kept in one place, `_ValueLayout`.
 """
 from typing import Dict, List, Tuple, Union
 
@@ -13,124 +15,55 @@ ValueSpec = Union[int, List[int], Dict[str, int]]
 Values = Union[torch.Tensor, List[torch.Tensor], Dict[str, torch.Tensor]]
 
 
-def _value_names(value_dims: ValueSpec) -> Dict[str, int]:
-    """Buffer name -> row width for the three ways of declaring values
-    (ash/hashmap.py:23-36): a single width is called "default", a list
-    "default_<i>", a dict keeps its own names."""
-    if isinstance(value_dims, int):
-        return {"default": value_dims}
-    if isinstance(value_dims, list):
-        return {f"default_{i}": d for i, d in enumerate(value_dims)}
-    if isinstance(value_dims, dict):
-        return dict(value_dims)
-    raise ValueError("value_dims must be int, list or dict")
+class _ValueLayout:
+    """The three ways of declaring a map's values (ash/hashmap.py:23-36) and
+    the matching shapes in which values are passed in and handed back: one
+    width -> one tensor, stored as "default"; a list of widths -> a list of
+    tensors, stored as "default_<i>"; a dict -> a dict under its own names."""
 
+    def __init__(self, value_dims: ValueSpec):
+        if not isinstance(value_dims, (int, list, dict)):
+            raise ValueError("value_dims must be int, list or dict")
+        self.kind = next(k for k in (int, list, dict) if isinstance(value_dims, k))
+        if self.kind is int:
+            self.widths = {"default": value_dims}
+        elif self.kind is list:
+            self.widths = {f"default_{i}": width for i, width in enumerate(value_dims)}
+        else:
+            self.widths = dict(value_dims)
 
-class HashMap(ASHModule):
-    """Hash map whose values live in float tensors registered as buffers under
-    their value names, one row per index."""
+    @property
+    def names(self) -> Tuple[str, ...]:
+        return tuple(self.widths)
 
-    def __init__(
-        self,
-        key_dim: int,
-        value_dims: ValueSpec,
-        capacity: int,
-        device: Union[str, torch.device] = torch.device("cpu"),
-    ):
-        super().__init__()
-        self.engine = ASHEngine(key_dim, capacity, device)
-        self.value_dims = value_dims
-        self.values = {
+    def storage(self, capacity: int, device) -> Dict[str, torch.Tensor]:
+        """Zeroed (capacity, width) tensors, one per value."""
+        return {
             name: torch.zeros(capacity, width, device=device)
-            for name, width in _value_names(value_dims).items()
+            for name, width in self.widths.items()
         }
-        for name, store in self.values.items():
-            self.register_buffer(name, store)
 
-    # -- value plumbing ----------------------------------------------------
-    def _to_named(self, values: Values) -> Dict[str, torch.Tensor]:
+    def named(self, values: Values) -> Dict[str, torch.Tensor]:
+        """Values as passed by the caller -> name -> tensor; the shape has to
+        be the declared one."""
         if isinstance(values, torch.Tensor):
-            assert isinstance(self.value_dims, int)
+            assert self.kind is int
             return {"default": values}
         if isinstance(values, list):
-            assert isinstance(self.value_dims, list)
+            assert self.kind is list
             return {f"default_{i}": v for i, v in enumerate(values)}
         if isinstance(values, dict):
-            assert isinstance(self.value_dims, dict)
+            assert self.kind is dict
             return values
         raise ValueError("values must be Tensor, list, or dict")
 
-    def reinterpret_value_dict(self, values: Dict[str, torch.Tensor]) -> Values:
-        """Back from named values to the shape the map was declared with."""
-        if isinstance(self.value_dims, int):
-            return values["default"]
-        if isinstance(self.value_dims, list):
-            return [values[f"default_{i}"] for i in range(len(self.value_dims))]
-        if isinstance(self.value_dims, dict):
-            return values
-        raise ValueError("values must be Tensor, list, or dict")
-
-    def _gather(self, indices: torch.Tensor) -> Values:
-        return self.reinterpret_value_dict(
-            {name: store[indices] for name, store in self.values.items()}
-        )
-
-    # -- map operations ------------------------------------------------------
-    def insert(self, keys: torch.Tensor, values: Values) -> None:
-        self.engine.insert(keys, self._to_named(values), self.values)
-
-    def find(
-        self, keys: torch.Tensor, return_indices: bool = True, return_values: bool = False
-    ) -> Tuple:
-        """(masks[, indices][, values]) -- the mask comes first
-        (ash/hashmap.py:82-95)."""
-        assert return_indices or return_values, "Must return at least one of indices or values"
-        indices, masks = self.engine.find(keys)
-        out = (masks,)
-        if return_indices:
-            out += (indices,)
-        if return_values:
-            out += (self._gather(indices),)
-        return out
-
-    def erase(self, keys: torch.Tensor) -> None:
-        self.engine.erase(keys)
-
-    def clear(self) -> None:
-        for store in self.values.values():
-            store.zero_()
-        self.engine.clear()
-
-    def size(self) -> int:
-        return self.engine.size()
-
-    def resize(self, new_capacity: int) -> None:
-        """Moves keys and value rows into freshly sized storage and swaps the
-        registered buffers (ash/hashmap.py:108-122)."""
-        grown = {
-            name: torch.zeros(new_capacity, *store.shape[1:], device=self.engine.device)
-            for name, store in self.values.items()
-        }
-        self.engine.resize(new_capacity, self.values, grown)
-        for name in self.values:
-            delattr(self, name)
-        self.values = grown
-        for name, store in grown.items():
-            self.register_buffer(name, store)
-
-    def keys(self) -> torch.Tensor:
-        return self.engine.keys()
-
-    def items(self, return_indices: bool = True, return_values: bool = False) -> Tuple:
-        """(keys[, indices][, values]) of the live entries."""
-        assert return_indices or return_values, "Must return at least one of indices or values"
-        live_keys, live_indices = self.engine.items()
-        out = (live_keys,)
-        if return_indices:
-            out += (live_indices,)
-        if return_values:
-            out += (self._gather(live_indices),)
-        return out
+    def declared(self, named: Dict[str, torch.Tensor]) -> Values:
+        """name -> tensor back to the declared shape."""
+        if self.kind is int:
+            return named["default"]
+        if self.kind is list:
+            return [named[name] for name in self.names]
+        return named
 
 
 class HashSet(ASHModule):
@@ -144,7 +77,9 @@ class HashSet(ASHModule):
         self.engine.insert_keys(keys)
 
     def find(self, keys: torch.Tensor) -> torch.Tensor:
-        return self.engine.find(keys)[1]
+        """Mask of the keys that are stored."""
+        _, masks = self.engine.find(keys)
+        return masks
 
     def erase(self, keys: torch.Tensor) -> None:
         self.engine.erase(keys)
@@ -160,3 +95,88 @@ class HashSet(ASHModule):
 
     def keys(self) -> torch.Tensor:
         return self.engine.keys()
+
+
+class HashMap(ASHModule):
+    """Keys with values.  Every value is a float tensor with one row per index
+    of the engine, registered as a buffer under its name (so it travels with
+    `state_dict`) and also reachable through `self.values`."""
+
+    def __init__(
+        self,
+        key_dim: int,
+        value_dims: ValueSpec,
+        capacity: int,
+        device: Union[str, torch.device] = torch.device("cpu"),
+    ):
+        super().__init__()
+        self._layout = _ValueLayout(value_dims)
+        self.value_dims = value_dims
+        self.engine = ASHEngine(key_dim, capacity, device)
+        self.values: Dict[str, torch.Tensor] = {}
+        self._adopt(self._layout.storage(capacity, device))
+
+    def _adopt(self, storage: Dict[str, torch.Tensor]) -> None:
+        """Makes `storage` the map's value tensors and buffers."""
+        for name in self.values:
+            delattr(self, name)
+        self.values = storage
+        for name, rows in storage.items():
+            self.register_buffer(name, rows)
+
+    def reinterpret_value_dict(self, values: Dict[str, torch.Tensor]) -> Values:
+        """name -> tensor in the shape the map was declared with."""
+        return self._layout.declared(values)
+
+    def _rows(self, indices: torch.Tensor) -> Values:
+        return self._layout.declared({name: rows[indices] for name, rows in self.values.items()})
+
+    def _answer(self, first, indices, return_indices: bool, return_values: bool) -> Tuple:
+        assert return_indices or return_values, "Must return at least one of indices or values"
+        answer = [first]
+        if return_indices:
+            answer.append(indices)
+        if return_values:
+            answer.append(self._rows(indices))
+        return tuple(answer)
+
+    def insert(self, keys: torch.Tensor, values: Values) -> None:
+        self.engine.insert(keys, self._layout.named(values), self.values)
+
+    def find(
+        self, keys: torch.Tensor, return_indices: bool = True, return_values: bool = False
+    ) -> Tuple:
+        """(masks[, indices][, values]) -- the mask comes first
+        (ash/hashmap.py:82-95)."""
+        indices, masks = self.engine.find(keys)
+        return self._answer(masks, indices, return_indices, return_values)
+
+    def items(self, return_indices: bool = True, return_values: bool = False) -> Tuple:
+        """(keys[, indices][, values]) of the stored entries."""
+        keys, indices = self.engine.items()
+        return self._answer(keys, indices, return_indices, return_values)
+
+    def keys(self) -> torch.Tensor:
+        return self.engine.keys()
+
+    def erase(self, keys: torch.Tensor) -> None:
+        self.engine.erase(keys)
+
+    def clear(self) -> None:
+        """Empties the table and zeroes the values (ash/hashmap.py:100-103)."""
+        for rows in self.values.values():
+            rows.zero_()
+        self.engine.clear()
+
+    def size(self) -> int:
+        return self.engine.size()
+
+    def resize(self, new_capacity: int) -> None:
+        """New storage of `new_capacity` rows per value; the engine moves keys
+        and rows over, then the buffers are swapped (ash/hashmap.py:108-122)."""
+        roomier = {
+            name: torch.zeros(new_capacity, *rows.shape[1:], device=self.engine.device)
+            for name, rows in self.values.items()
+        }
+        self.engine.resize(new_capacity, self.values, roomier)
+        self._adopt(roomier)
