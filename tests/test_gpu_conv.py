@@ -57,6 +57,49 @@ def test_masked_cells_and_unlisted_blocks_stay_zero(gpu_ash, oracle):
     assert bool((none == 0).all())
 
 
+@pytest.mark.parametrize("channels,radius,reorder", [(16, 1, False), (4, 1, False), (3, 2, False),
+                                                     (5, 1, True), (8, 3, False)])
+def test_entries_with_and_without_block_scratch_agree(gpu_ash, oracle, channels, radius, reorder):
+    """ash_convolution_forward clears the whole output and leaves skipped cells
+    alone; ash_convolution_forward_listed clears the rows of unlisted blocks
+    only and writes zeros into skipped cells of listed ones.  Both from an
+    output full of NaNs, half of the blocks listed, a third of the cells masked
+    out, also with the taps in another order (cells then go through the
+    tables): equal to the oracle bit for bit."""
+    import ctypes
+
+    from ash.common import _DTYPE, _stream_of
+
+    grid, _, _ = workloads.build_grid(gpu_ash, 300, channels, 8, 32, device=DEV)
+    g = torch.Generator().manual_seed(870 + channels)
+    inputs = torch.randn(grid.embeddings.shape, generator=g).to(DEV)
+    k = (2 * radius + 1) ** 3
+    weights = torch.randn(k, channels, generator=g).to(DEV)
+    c2g, c2c, g2g, gi, ci = _tables(grid, radius)
+    if reorder:
+        perm = torch.randperm(k, generator=g).to(DEV)
+        c2g, c2c, weights = c2g[:, perm].contiguous(), c2c[:, perm].contiguous(), weights[perm].contiguous()
+    listed = gi.view(-1)[1::2].contiguous()
+    masks = (torch.rand(listed.numel() * 512, generator=g) < 0.67).to(DEV)
+    ref = oracle.convolution_forward(inputs, weights, masks, listed, ci, g2g, c2c, c2g, 8)
+    lib = gpu_ash.grid.backend.lib
+    b, m, e = inputs.shape
+    ci = ci.view(-1).contiguous()
+    common = (inputs.data_ptr(), weights.data_ptr(), masks.data_ptr(), listed.data_ptr(),
+              ci.data_ptr(), g2g.data_ptr(), c2c.data_ptr(), c2g.data_ptr())
+    sizes = (listed.numel(), b, m, e, k, g2g.shape[1], _DTYPE[inputs.dtype])
+    plain = torch.full_like(inputs, float("nan"))
+    assert lib.ash_convolution_forward(*common, plain.data_ptr(), *sizes, _stream_of(DEV)) == 0
+    scratch = torch.full((b,), 7, dtype=torch.uint8, device=DEV)
+    with_scratch = torch.full_like(inputs, float("nan"))
+    assert lib.ash_convolution_forward_listed(*common, with_scratch.data_ptr(), *sizes,
+                                              scratch.data_ptr(), _stream_of(DEV)) == 0
+    assert torch.equal(plain.cpu(), ref)
+    assert torch.equal(with_scratch.cpu(), ref)
+    assert lib.ash_convolution_forward_listed(*common, with_scratch.data_ptr(), *sizes,
+                                              None, _stream_of(DEV)) != 0
+
+
 def test_gaussian_filter_device_equals_oracle_backend(gpu_ash, oracle, monkeypatch):
     """SparseDenseGrid.gaussian_filter_ (ash/grid.py:435-476) end to end: the
     same blocks and the same field, filtered on the device and on the CPU with
@@ -193,9 +236,12 @@ def test_impulse_and_constant_field_on_a_dense_volume(gpu_ash, radius):
 
 @pytest.mark.parametrize("grid_dim,radius,channels", [(4, 1, 3), (4, 2, 2), (16, 1, 2), (6, 2, 4),
                                                       (12, 3, 1)])
-def test_other_block_edges(gpu_ash, oracle, grid_dim, radius, channels):
+def test_other_block_edges(gpu_ash, oracle, grid_dim, radius, channels, monkeypatch):
     """Block edges that are and are not multiples of four (the latter compute
-    one cell per lane), windows reaching two blocks deep into a small block."""
+    one cell per lane), windows reaching two blocks deep into a small block.
+    Outputs start as NaNs and a fifth of the cells is masked out: every cell
+    has to be written, by the clear or by the kernel."""
+    monkeypatch.setattr(torch, "empty_like", lambda t, **kw: torch.full_like(t, float("nan")))
     s = 5
     g = torch.Generator().manual_seed(850 + grid_dim)
     blocks = torch.stack(torch.meshgrid(*[torch.arange(s)] * 3, indexing="ij"), -1).view(-1, 3)
@@ -209,7 +255,7 @@ def test_other_block_edges(gpu_ash, oracle, grid_dim, radius, channels):
     size = 2 * radius + 1
     weights = torch.randn(size**3, channels, generator=g).to(DEV)
     c2g, c2c, g2g, gi, ci = _tables(grid, radius)
-    masks = torch.ones(inputs.shape[:2], dtype=torch.bool)
+    masks = torch.rand(inputs.shape[:2], generator=g) < 0.8
     out = gpu_ash.grid.backend.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g,
                                                    grid_dim)
     ref = oracle.convolution_forward(inputs, weights, masks, gi, ci, g2g, c2c, c2g, grid_dim)

@@ -159,6 +159,10 @@ _SIGNATURES = {
         ctypes.c_int,
         [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR],
     ),
+    "ash_convolution_forward_listed": (
+        ctypes.c_int,
+        [_PTR] * 9 + [_I64] * 6 + [ctypes.c_int32, _PTR, _PTR],
+    ),
     "ash_marching_cubes_workspace_ints": (ctypes.c_int64, [_I64, _I64]),
     "ash_marching_cubes_classify": (
         ctypes.c_int,
@@ -388,13 +392,16 @@ class _Backend:
         if masks.numel() < gi.numel() * m:
             raise RuntimeError("masks must cover every listed cell")
         outputs = torch.empty_like(inputs)
+        # one scratch byte per block: the library then clears only the rows of
+        # the blocks that are not listed
+        listed = torch.empty(b, dtype=torch.uint8, device=dev)
         with torch.cuda.device(dev):
             self.check(
-                self.lib.ash_convolution_forward(
+                self.lib.ash_convolution_forward_listed(
                     inputs.data_ptr(), weights.data_ptr(), masks.data_ptr(), gi.data_ptr(),
                     ci.data_ptr(), lut_g.data_ptr(), lut_c2c.data_ptr(), lut_c2g.data_ptr(),
                     outputs.data_ptr(), gi.numel(), b, m, e, k, lut_g.shape[1],
-                    _DTYPE[inputs.dtype], _stream_of(dev),
+                    _DTYPE[inputs.dtype], listed.data_ptr(), _stream_of(dev),
                 )
             )
         return outputs

@@ -543,6 +543,7 @@ struct ConvDev {
     const int64_t* lut_c2g;   // [M, K]
     void* out;
     int64_t n_grids, B, M, E, K, GN;
+    int owns;   // the kernel writes every cell of the listed blocks (zeros where it has no result)
 };
 
 // One lane per cell with all channels of the row in registers (EC >= E, a
@@ -855,9 +856,20 @@ __global__ __launch_bounds__(kConvThreads, (EC >= 16 && NY >= 8) ? 2 : 4) void c
     __syncthreads();
     const bool by_table = s_bad != 0;
 
+    // a.owns: nobody cleared the rows of the listed blocks, so cells without a
+    // result get their zeros here.  The paths that visit cells through
+    // cell_indices clear the whole block first, in the pass of the first
+    // channels; the y-blocked path writes a zero where it skips a cell.
+    auto clear_block = [&](int64_t g) {
+        if (!a.owns || e0 != 0) return;
+        T* rows = out + g * a.M * a.E;
+        for (int64_t i = tid; i < a.M * a.E; i += kConvThreads) rows[i] = T(0);
+        __syncthreads();
+    };
     for (int64_t blk = blockIdx.x; by_table && blk < a.n_grids; blk += gridDim.x) {
         const int64_t g = a.grid_indices[blk];
         if (g < 0 || g >= a.B) continue;  // the same for the whole workgroup
+        clear_block(g);
         {
             const int64_t* nb_g = a.lut_g + g * a.GN;
             for (int c_i = tid; c_i < M; c_i += kConvThreads) {
@@ -1078,10 +1090,12 @@ __global__ __launch_bounds__(kConvThreads, (EC >= 16 && NY >= 8) ? 2 : 4) void c
                             const int c = i / kQ;
                             const int q4 = i - c * kQ;
                             const int c_i = s_inv[c];
-                            if (c_i == 0xFFFF || !mask_b[c_i]) continue;
+                            const bool keep = c_i != 0xFFFF && mask_b[c_i];
+                            if (!keep && !a.owns) continue;
                             const T* sp = stage + c * (EC + 1) + 4 * q4;
                             reinterpret_cast<float4*>(out_g + static_cast<uint32_t>(c) * E)[q4] =
-                                    make_float4(sp[0], sp[1], sp[2], sp[3]);
+                                    keep ? make_float4(sp[0], sp[1], sp[2], sp[3])
+                                         : make_float4(0.f, 0.f, 0.f, 0.f);
                         }
                     }
                 } else {
@@ -1089,8 +1103,9 @@ __global__ __launch_bounds__(kConvThreads, (EC >= 16 && NY >= 8) ? 2 : 4) void c
                         const int c = i / ec;
                         const int q = i - c * ec;
                         const int c_i = s_inv[c];
-                        if (c_i == 0xFFFF || !mask_b[c_i]) continue;
-                        out_g[static_cast<uint32_t>(c) * E + q] = stage[c * (EC + 1) + q];
+                        const bool keep = c_i != 0xFFFF && mask_b[c_i];
+                        if (!keep && !a.owns) continue;
+                        out_g[static_cast<uint32_t>(c) * E + q] = keep ? stage[c * (EC + 1) + q] : T(0);
                     }
                 }
             } else {
@@ -1109,13 +1124,15 @@ __global__ __launch_bounds__(kConvThreads, (EC >= 16 && NY >= 8) ? 2 : 4) void c
                     for (int j = 0; j < kNy; ++j) {
                         const int c = x + G * (y0 + j) + G * G * z;
                         const int c_i = s_inv[c];
-                        if (c_i == 0xFFFF || !a.masks[blk * a.M + c_i]) continue;
-                        out[(g * a.M + c) * E + e0 + q] = acc[j];
+                        const bool keep = c_i != 0xFFFF && a.masks[blk * a.M + c_i];
+                        if (!keep && !a.owns) continue;
+                        out[(g * a.M + c) * E + e0 + q] = keep ? acc[j] : T(0);
                     }
                 }
             }
             continue;
         }
+        clear_block(g);
         for (int c_i = tid; c_i < M; c_i += kConvThreads) {
             if (!a.masks[blk * a.M + c_i]) continue;
             const int64_t c64 = a.cell_indices[c_i];
@@ -1186,8 +1203,9 @@ inline int cube_edge(int64_t m) {
 
 // Takes the tile kernel when the sizes describe a cube window over cubic
 // blocks with 27 neighbour blocks and the tile fits; returns -1 when not.
+// `probe`: only say whether the tile kernel would take these sizes.
 template <typename T>
-int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
+int launch_convolution_tile(const ConvDev& a, hipStream_t s, bool probe = false) {
     const int G = cube_edge(a.M);
     const int W = cube_edge(a.K);
     if (G == 0 || W < 3 || W % 2 == 0 || a.GN != 27 || a.n_grids < 64) return -1;
@@ -1226,6 +1244,7 @@ int launch_convolution_tile(const ConvDev& a, hipStream_t s) {
     int ec_max = kMaxEc;
     while (ec_max > 1 && cell_bytes * ec_max > budget) ec_max /= 2;
     if (cell_bytes * ec_max > budget) return -1;
+    if (probe) return 0;
     const uintptr_t align = reinterpret_cast<uintptr_t>(a.in);
     for (int e0 = 0; e0 < a.E;) {
         int width = ec_max;                  // channels of the template instance
@@ -1358,6 +1377,29 @@ __global__ __launch_bounds__(kBlock) void zero1_kernel(
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
          i < n; i += stride) {
         p[i] = 0;
+    }
+}
+
+// listed[b] = 1 for every block of the listing.
+__global__ __launch_bounds__(kBlock) void mark_listed_kernel(
+        const int64_t* __restrict__ grid_indices, int64_t n, int64_t B,
+        uint8_t* __restrict__ listed) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t g = grid_indices[i];
+    if (g >= 0 && g < B) listed[g] = 1;
+}
+
+// Zeroes the rows of the blocks that are not listed: `units` 16-byte pieces
+// per block, one workgroup per block at a time.
+__global__ __launch_bounds__(kBlock) void zero_unlisted_kernel(
+        uint4* __restrict__ out, const uint8_t* __restrict__ listed, int64_t B,
+        int64_t units) {
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    for (int64_t b = blockIdx.x; b < B; b += gridDim.x) {
+        if (listed[b]) continue;  // the same for the whole workgroup
+        uint4* rows = out + b * units;
+        for (int64_t u = threadIdx.x; u < units; u += kBlock) rows[u] = zero;
     }
 }
 
@@ -1704,16 +1746,18 @@ int ash_query_backward_backward_accumulate(const ash_query_args* a,
     return backward_backward(a, grad_grad_offsets, z, grad_z, grad_embeddings, stream, false);
 }
 
-int ash_convolution_forward(const void* inputs, const void* weights,
-                            const uint8_t* masks, const int64_t* grid_indices,
-                            const int64_t* cell_indices,
-                            const int64_t* lut_grid_nb2grid_idx,
-                            const int64_t* lut_cell_nb2cell_idx,
-                            const int64_t* lut_cell_nb2grid_nb, void* outputs,
-                            int64_t num_grids, int64_t num_embeddings,
-                            int64_t cells_per_grid, int64_t embedding_dim,
-                            int64_t num_cell_nbs, int64_t num_grid_nbs,
-                            int32_t dtype, void* stream) {
+namespace {
+
+int convolution_forward(const void* inputs, const void* weights,
+                        const uint8_t* masks, const int64_t* grid_indices,
+                        const int64_t* cell_indices,
+                        const int64_t* lut_grid_nb2grid_idx,
+                        const int64_t* lut_cell_nb2cell_idx,
+                        const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                        int64_t num_grids, int64_t num_embeddings,
+                        int64_t cells_per_grid, int64_t embedding_dim,
+                        int64_t num_cell_nbs, int64_t num_grid_nbs,
+                        int32_t dtype, uint8_t* listed, void* stream) {
     if (dtype != ASH_F32 && dtype != ASH_F64) ASH_FAIL("unknown dtype");
     if (num_grids < 0 || num_embeddings < 1 || cells_per_grid < 1 ||
         embedding_dim < 1 || num_cell_nbs < 1 || num_grid_nbs < 1) {
@@ -1730,11 +1774,6 @@ int ash_convolution_forward(const void* inputs, const void* weights,
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t scalar = dtype == ASH_F32 ? 4 : 8;
-    // rows of blocks that are not listed stay zero (at::zeros_like, grid.cu:1010)
-    if (zero_fill(outputs, num_embeddings * cells_per_grid * embedding_dim * scalar, s)) {
-        return 1;
-    }
-    if (num_grids == 0) return 0;
     ConvDev a;
     a.in = inputs;
     a.w = weights;
@@ -1751,6 +1790,29 @@ int ash_convolution_forward(const void* inputs, const void* weights,
     a.E = embedding_dim;
     a.K = num_cell_nbs;
     a.GN = num_grid_nbs;
+    a.owns = 0;
+    // Rows of blocks that are not listed stay zero (at::zeros_like,
+    // grid.cu:1010).  With a scratch byte per block and the tile kernel, which
+    // writes every cell of the blocks it is given, only those rows are cleared.
+    const int64_t block_bytes = cells_per_grid * embedding_dim * scalar;
+    const bool tile = num_grids > 0 && embedding_dim <= 16 && num_cell_nbs >= kTileMinTaps &&
+                      (dtype == ASH_F32 ? launch_convolution_tile<float>(a, s, true)
+                                        : launch_convolution_tile<double>(a, s, true)) == 0;
+    if (listed != nullptr && tile && block_bytes % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(outputs) % 16 == 0) {
+        if (zero_fill(listed, num_embeddings, s)) return 1;
+        mark_listed_kernel<<<static_cast<unsigned>((num_grids + kBlock - 1) / kBlock), kBlock, 0,
+                             s>>>(grid_indices, num_grids, num_embeddings, listed);
+        ASH_LAUNCH_CHECK();
+        const int64_t g = num_embeddings < 256 * 32 ? num_embeddings : 256 * 32;
+        zero_unlisted_kernel<<<static_cast<unsigned>(g), kBlock, 0, s>>>(
+                static_cast<uint4*>(outputs), listed, num_embeddings, block_bytes / 16);
+        ASH_LAUNCH_CHECK();
+        a.owns = 1;
+    } else if (zero_fill(outputs, num_embeddings * block_bytes, s)) {
+        return 1;
+    }
+    if (num_grids == 0) return 0;
     if (embedding_dim <= 16) {
         return dtype == ASH_F32 ? launch_convolution_cells<float>(a, s)
                                 : launch_convolution_cells<double>(a, s);
@@ -1765,6 +1827,41 @@ int ash_convolution_forward(const void* inputs, const void* weights,
     }
     ASH_LAUNCH_CHECK();
     return 0;
+}
+
+}  // namespace
+
+int ash_convolution_forward(const void* inputs, const void* weights,
+                            const uint8_t* masks, const int64_t* grid_indices,
+                            const int64_t* cell_indices,
+                            const int64_t* lut_grid_nb2grid_idx,
+                            const int64_t* lut_cell_nb2cell_idx,
+                            const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                            int64_t num_grids, int64_t num_embeddings,
+                            int64_t cells_per_grid, int64_t embedding_dim,
+                            int64_t num_cell_nbs, int64_t num_grid_nbs,
+                            int32_t dtype, void* stream) {
+    return convolution_forward(inputs, weights, masks, grid_indices, cell_indices,
+                               lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb,
+                               outputs, num_grids, num_embeddings, cells_per_grid, embedding_dim,
+                               num_cell_nbs, num_grid_nbs, dtype, nullptr, stream);
+}
+
+int ash_convolution_forward_listed(const void* inputs, const void* weights,
+                                   const uint8_t* masks, const int64_t* grid_indices,
+                                   const int64_t* cell_indices,
+                                   const int64_t* lut_grid_nb2grid_idx,
+                                   const int64_t* lut_cell_nb2cell_idx,
+                                   const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                                   int64_t num_grids, int64_t num_embeddings,
+                                   int64_t cells_per_grid, int64_t embedding_dim,
+                                   int64_t num_cell_nbs, int64_t num_grid_nbs,
+                                   int32_t dtype, uint8_t* listed, void* stream) {
+    if (listed == nullptr) ASH_FAIL("convolution_forward_listed: null scratch");
+    return convolution_forward(inputs, weights, masks, grid_indices, cell_indices,
+                               lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb,
+                               outputs, num_grids, num_embeddings, cells_per_grid, embedding_dim,
+                               num_cell_nbs, num_grid_nbs, dtype, listed, stream);
 }
 
 }  // extern "C"
