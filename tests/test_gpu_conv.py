@@ -100,6 +100,37 @@ def test_entries_with_and_without_block_scratch_agree(gpu_ash, oracle, channels,
                                               None, _stream_of(DEV)) != 0
 
 
+def test_window_tables_follow_the_table(gpu_ash, oracle):
+    """grid.convolution keeps its tables between calls: the per-cell pair per
+    radius, the per-block one while the table holds the same keys.  After more
+    blocks are dropped or activated the result has to follow."""
+    grid, _, _ = workloads.build_grid(gpu_ash, 200, 2, 8, 32, device=DEV)
+    g = torch.Generator().manual_seed(880)
+    weights = torch.randn(3, 3, 3, 2, generator=g).to(DEV)
+
+    def check():
+        inputs = torch.randn(grid.embeddings.shape, generator=g).to(DEV)
+        out = grid.convolution(inputs, weights)
+        c2g, c2c, g2g, gi, ci = _tables(grid, 1)
+        masks = torch.ones(inputs.shape[:2], dtype=torch.bool)
+        ref = oracle.convolution_forward(inputs, weights.view(27, 2), masks, gi, ci, g2g, c2c, c2g, 8)
+        assert torch.equal(out.cpu(), ref)
+        return out
+
+    check()
+    first_tables = grid._window_tables(1)
+    check()
+    assert all(a is b for a, b in zip(first_tables, grid._window_tables(1)))
+    keys, _ = grid.engine.items()
+    grid.engine.erase(keys[:40].contiguous())
+    assert grid.engine.size() == len(keys) - 40
+    check()
+    grid.engine.insert_keys((keys[:25] + torch.tensor([[1, 0, 0]], device=DEV, dtype=keys.dtype)).clamp(0, 31))
+    check()
+    assert grid._window_tables(1)[2] is not first_tables[2]
+    assert grid._window_tables(1)[0] is first_tables[0]
+
+
 def test_gaussian_filter_device_equals_oracle_backend(gpu_ash, oracle, monkeypatch):
     """SparseDenseGrid.gaussian_filter_ (ash/grid.py:435-476) end to end: the
     same blocks and the same field, filtered on the device and on the CPU with

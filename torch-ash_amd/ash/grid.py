@@ -433,11 +433,7 @@ class SparseDenseGrid(ASHModule):
         assert weights.shape[3] == inputs.shape[-1]
         assert weights.device == inputs.device
 
-        lut_cell_nb2grid_nb, lut_cell_nb2cell_idx = self.construct_cell_neighbor_lut(
-            radius, bidirectional=True
-        )
-        grid_radius = (radius + self.grid_dim - 1) // self.grid_dim
-        _, lut_grid_nb2grid_idx = self.construct_grid_neighbor_lut(grid_radius, bidirectional=True)
+        lut_cell_nb2grid_nb, lut_cell_nb2cell_idx, lut_grid_nb2grid_idx = self._window_tables(radius)
         _, grid_indices = self._blocks_in_spatial_order()
         cell_indices = self.cell_indices
         num_cell_nbs = lut_cell_nb2grid_nb.shape[1]
@@ -452,6 +448,28 @@ class SparseDenseGrid(ASHModule):
             lut_cell_nb2grid_nb,
             self.grid_dim,
         )
+
+    def _window_tables(self, radius: int):
+        """The three tables of a (2 radius + 1)^3 window: the per-cell pair
+        depends on the block size alone and is built once per radius, the
+        per-block one is kept while the table holds the same keys (as the
+        Z-order listing)."""
+        cell_tables = getattr(self, "_window_cell_tables", None)
+        if cell_tables is None:
+            cell_tables = self._window_cell_tables = {}
+        if radius not in cell_tables:
+            cell_tables[radius] = self.construct_cell_neighbor_lut(radius, bidirectional=True)
+        lut_cell_nb2grid_nb, lut_cell_nb2cell_idx = cell_tables[radius]
+        grid_radius = (radius + self.grid_dim - 1) // self.grid_dim
+        table = self.engine.backend
+        stamp = (id(table), getattr(table, "version", None), grid_radius)
+        cached = getattr(self, "_window_block_table", None)
+        if stamp[1] is not None and cached is not None and cached[0] == stamp:
+            lut_grid_nb2grid_idx = cached[1]
+        else:
+            _, lut_grid_nb2grid_idx = self.construct_grid_neighbor_lut(grid_radius, bidirectional=True)
+            self._window_block_table = (stamp, lut_grid_nb2grid_idx)
+        return lut_cell_nb2grid_nb, lut_cell_nb2cell_idx, lut_grid_nb2grid_idx
 
     @torch.no_grad()
     def isosurface_points(
