@@ -148,6 +148,56 @@ def test_block_sizes_match_oracle(gpu_ash, oracle, grid_dim):
     assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))
 
 
+@pytest.mark.parametrize("grid_dim", [8, 20])
+def test_cells_numbered_in_another_order(gpu_ash, oracle, grid_dim):
+    """The kernels work the corners of a cell out when the per-cell tables are
+    the usual ones (cell = x + G y + G^2 z) and follow the tables otherwise:
+    with the cells renumbered by a random permutation, consistently in the
+    field, the weights and the three per-cell tables, mesh and points still
+    equal the oracle's, which only ever follows the tables."""
+    s = 4 if grid_dim == 8 else 3
+    g = torch.Generator().manual_seed(890 + grid_dim)
+    blocks = torch.stack(torch.meshgrid(*[torch.arange(s)] * 3, indexing="ij"), -1).view(-1, 3)
+    blocks = blocks[torch.rand(len(blocks), generator=g) < 0.9]
+    grid = gpu_ash.BoundedSparseDenseGrid(
+        3, len(blocks) + 5, 1, grid_dim=grid_dim, sparse_grid_dim=s, bbox_min=torch.zeros(3),
+        bbox_max=torch.ones(3), device=DEV)
+    grid.engine.insert_keys(blocks.int().to(DEV))
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    _, idx = grid.engine.items()
+    shape = grid.embeddings.shape[:2]
+    m = shape[1]
+    sdf = (torch.rand(shape, generator=g) - 0.45).to(DEV)
+    weights = (torch.rand(shape, generator=g) * 10).to(DEV)
+    perm = torch.randperm(m, generator=g).to(DEV)            # old cell c becomes cell perm[c]
+    sdf_p, weights_p = torch.empty_like(sdf), torch.empty_like(weights)
+    sdf_p[:, perm], weights_p[:, perm] = sdf, weights
+    coords_p = torch.empty_like(grid.cell_coords)
+    coords_p[perm] = grid.cell_coords
+    c2c_p = torch.empty_like(grid.lut_cell_nb2cell_idx)
+    c2c_p[perm] = perm[grid.lut_cell_nb2cell_idx]
+    c2g_p = torch.empty_like(grid.lut_cell_nb2grid_nb)
+    c2g_p[perm] = grid.lut_cell_nb2grid_nb
+    backend = gpu_ash.grid.backend
+    usual = (idx, grid.grid_coords, grid.lut_grid_nb2grid_idx, grid.cell_coords,
+             grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, grid_dim, 0.02, 0.4)
+    renumbered = (idx, grid.grid_coords, grid.lut_grid_nb2grid_idx, coords_p, c2c_p, c2g_p,
+                  grid_dim, 0.02, 0.4)
+    tri, pts = backend.marching_cubes(sdf_p, weights_p, *renumbered)
+    tri_ref, pts_ref = oracle.marching_cubes(sdf_p, weights_p, *renumbered)
+    assert len(tri_ref) > 300 and tri.shape == tri_ref.shape
+    assert np.array_equal(_sorted_rows(pts), _sorted_rows(pts_ref))
+    assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_ref, pts_ref))
+    tri_u, pts_u = backend.marching_cubes(sdf, weights, *usual)
+    assert np.array_equal(_triangle_set(tri, pts), _triangle_set(tri_u, pts_u))
+    points = backend.isosurface_extraction(sdf_p, weights_p, *renumbered)
+    points_ref = oracle.isosurface_extraction(sdf_p, weights_p, *renumbered)
+    assert len(points_ref) > 200
+    assert np.array_equal(_sorted_rows(points), _sorted_rows(points_ref))
+    assert np.array_equal(_sorted_rows(points),
+                          _sorted_rows(backend.isosurface_extraction(sdf, weights, *usual)))
+
+
 def test_spatial_listing_follows_the_table(gpu_ash):
     """The Z-order listing of the blocks is kept while the table is unchanged
     and rebuilt after every call that can change its keys."""

@@ -45,7 +45,7 @@ constexpr int64_t kMaxVertices = int64_t{1} << 29;  // ids live in 29 bits
 
 // Layout of the int32 workspace: totals, then per chunk of kChunk cells the
 // number (after mc_scan_kernel: the running sum) of vertices and of triangles.
-enum McWorkspace { kMcTriangles32 = 0, kMcVertices32 = 1, kMcHeader = 4 };
+enum McWorkspace { kMcTriangles32 = 0, kMcVertices32 = 1, kMcStandard = 3, kMcHeader = 4 };
 
 struct McDev {
     const void* sdfs;
@@ -144,6 +144,65 @@ __device__ __forceinline__ bool corner_cell(const McDev& a, int64_t g, int64_t c
     if (gi < 0 || gi >= a.B) return false;
     ci = a.lut_c2c[c * 8 + nb];
     return ci >= 0 && ci < a.M;
+}
+
+// The Python layer numbers cells x + G y + G^2 z and builds the two per-cell
+// tables from that; layout_check_kernel compares the tables it is given with
+// this layout and leaves the verdict in the workspace header (kMcStandard).
+// The output kernels then work corners out instead of asking three tables in
+// a row for each of them; any other tables are followed as before.
+struct CellAt {
+    int x, y, z;
+};
+
+__device__ __forceinline__ CellAt cell_at(int G, int c) {
+    CellAt p;
+    p.x = c % G;
+    const int r = c / G;
+    p.y = r % G;
+    p.z = r / G;
+    return p;
+}
+
+__device__ __forceinline__ bool corner_cell_standard(const McDev& a, int64_t g, const CellAt& p,
+                                                     int nb, int64_t& gi, int64_t& ci) {
+    const int G = a.g;
+    const int tx = p.x + (nb & 1), ty = p.y + ((nb >> 1) & 1), tz = p.z + (nb >> 2);
+    const int bx = tx >= G, by = ty >= G, bz = tz >= G;
+    const int gn = bx | (by << 1) | (bz << 2);
+    ci = (tx - bx * G) + G * ((ty - by * G) + G * (tz - bz * G));
+    gi = gn == 0 ? g : a.lut_g[g * 8 + gn];
+    return gi >= 0 && gi < a.B;
+}
+
+constexpr int kCheckThreads = 1024;
+
+__global__ __launch_bounds__(kCheckThreads) void layout_check_kernel(McDev a) {
+    __shared__ int s_bad;
+    if (threadIdx.x == 0) s_bad = 0;
+    __syncthreads();
+    const int G = a.g;
+    const int M = static_cast<int>(a.M);
+    int bad = static_cast<int64_t>(G) * G * G != a.M;
+    // no early way out of the loop: its loads are then all in flight together
+#pragma unroll 4
+    for (int t = threadIdx.x; t < (bad ? 0 : M * 8); t += kCheckThreads) {
+        const int c = t >> 3;
+        const int nb = t & 7;
+        const CellAt p = cell_at(G, c);
+        const int tx = p.x + (nb & 1), ty = p.y + ((nb >> 1) & 1), tz = p.z + (nb >> 2);
+        const int bx = tx >= G, by = ty >= G, bz = tz >= G;
+        const int64_t gn = bx | (by << 1) | (bz << 2);
+        const int64_t ci = (tx - bx * G) + G * ((ty - by * G) + G * (tz - bz * G));
+        bad |= a.lut_c2g[t] != gn || a.lut_c2c[t] != ci;
+        if (nb == 0) {
+            bad |= a.cell_coords[c * 3] != p.x || a.cell_coords[c * 3 + 1] != p.y ||
+                   a.cell_coords[c * 3 + 2] != p.z;
+        }
+    }
+    if (bad) s_bad = 1;
+    __syncthreads();
+    if (threadIdx.x == 0) a.counters[kMcStandard] = s_bad ? 0 : 1;
 }
 
 __device__ __forceinline__ int edge_low_corner(int e) {
@@ -569,21 +628,31 @@ __global__ __launch_bounds__(kScanThreads) void mc_scan_kernel(int32_t* ws, int6
 // g, linear between the two ends of an edge, to positions[out...]
 // (ash/src/grid.cu:510-527 and :748-771).
 template <typename T>
-__device__ __forceinline__ void write_edge_points(const McDev& a, int64_t g, int64_t c,
-                                                  int64_t own, int f, int64_t out) {
+__device__ __forceinline__ void write_edge_points(const McDev& a, bool standard, int64_t g,
+                                                  int64_t c, int64_t own, int f, int64_t out) {
     const T* sdfs = static_cast<const T*>(a.sdfs);
     const T self = sdfs[own] - static_cast<T>(a.iso);
+    CellAt at = {0, 0, 0};
+    if (standard) {
+        at = cell_at(a.g, static_cast<int>(c));
+    } else {
+        at.x = a.cell_coords[c * 3];
+        at.y = a.cell_coords[c * 3 + 1];
+        at.z = a.cell_coords[c * 3 + 2];
+    }
+    const int cell[3] = {at.x, at.y, at.z};
     float base[3];
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
-        base[d] = static_cast<float>(a.grid_coords[g * 3 + d] * a.g + a.cell_coords[c * 3 + d]);
+        base[d] = static_cast<float>(a.grid_coords[g * 3 + d] * a.g + cell[d]);
     }
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
         if (!(f & (1 << d))) continue;
         int64_t gi, ci;
         float ratio = 0.f;
-        if (corner_cell(a, g, c, 1 << d, gi, ci)) {
+        if (standard ? corner_cell_standard(a, g, at, 1 << d, gi, ci)
+                     : corner_cell(a, g, c, 1 << d, gi, ci)) {
             const T other = sdfs[gi * a.M + ci] - static_cast<T>(a.iso);
             ratio = static_cast<float>(self / (self - other));
         }
@@ -606,6 +675,7 @@ __global__ __launch_bounds__(kBlock) void edge_points_kernel(McDev a) {
     __shared__ uint16_t s_cell[kChunk];   // cell of the chunk | flags << 12
     __shared__ uint16_t s_id[kChunk];     // its first point, from the chunk's first
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
+    const bool standard = a.counters[kMcStandard] != 0;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint64_t flags = 0;   // 3 bits per own cell
         int part[kPerThread / VEC] = {};   // per group: listed cells | points << 16
@@ -656,7 +726,7 @@ __global__ __launch_bounds__(kBlock) void edge_points_kernel(McDev a) {
                 a.slots[own] = static_cast<uint32_t>(f) | (static_cast<uint32_t>(out) << 3);
             }
             if (out + __popc(f) > a.n_vertices) continue;  // never with the counts of classify
-            write_edge_points<T>(a, g, c, own, f, out);
+            write_edge_points<T>(a, standard, g, c, own, f, out);
         }
     }
 }
@@ -671,6 +741,7 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
     __shared__ McTables tables;
     load_tables(tables);
     const int64_t chunks = (a.n_grids * a.M + kChunk - 1) / kChunk;
+    const bool standard = a.counters[kMcStandard] != 0;
     for (int64_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         uint32_t codes[kPerThread / 4] = {};   // one byte per own cell
         for_own_groups<VEC>(a, ch, [&](int j, uint32_t, int64_t at) {
@@ -714,10 +785,14 @@ __global__ __launch_bounds__(kBlock) void mc_triangles_kernel(McDev a) {
                 if (edge_crossed(code, e)) need |= 1 << edge_low_corner(e);
             }
             int64_t at[8];
+            const CellAt where = cell_at(a.g, static_cast<int>(c));
 #pragma unroll
             for (int nb = 0; nb < 8; ++nb) {
                 int64_t gi, ci;
-                at[nb] = ((need >> nb) & 1) && corner_cell(a, g, c, nb, gi, ci) ? gi * a.M + ci : -1;
+                const bool found = ((need >> nb) & 1) &&
+                                   (standard ? corner_cell_standard(a, g, where, nb, gi, ci)
+                                             : corner_cell(a, g, c, nb, gi, ci));
+                at[nb] = found ? gi * a.M + ci : -1;
             }
             int32_t vid[12];
 #pragma unroll
@@ -983,6 +1058,8 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     }
     ASH_LAUNCH_CHECK();
     if (num_grids == 0) return 0;
+    layout_check_kernel<<<1, kCheckThreads, 0, s>>>(a);   // after the clear of the header
+    ASH_LAUNCH_CHECK();
     const bool tiled = grid_dim <= kMaxTileG &&
                        static_cast<int64_t>(grid_dim) * grid_dim * grid_dim == cells_per_grid;
     if (tiled) {
@@ -1097,6 +1174,8 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
     const int64_t cells = num_grids * cells_per_grid;
     const int64_t chunks = (cells + kChunk - 1) / kChunk;
     if (num_grids > 0) {
+        layout_check_kernel<<<1, kCheckThreads, 0, s>>>(a);
+        ASH_LAUNCH_CHECK();
         const size_t cell_bytes = dtype == ASH_F32 ? 4 : 8;
         const size_t lds = (cell_bytes + 3) * tile_cells(grid_dim < 64 ? grid_dim : 64) +
                            2 * static_cast<size_t>(cells_per_grid);
