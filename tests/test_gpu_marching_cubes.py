@@ -229,3 +229,8 @@ def test_spatial_listing_follows_the_table(gpu_ash):
     grid.engine.erase(blocks[:100])
     shrunk = grid._blocks_in_spatial_order()
     assert len(shrunk[1]) == 17 ** 3 - 98 and same_set(shrunk)
+    # a resized engine is a new table (possibly at the old one's address) that
+    # hands the same keys other indices
+    grid.engine.resize(grid.engine.capacity + 64)
+    resized = grid._blocks_in_spatial_order()
+    assert len(resized[1]) == 17 ** 3 - 98 and same_set(resized)

@@ -10,6 +10,7 @@ There is no CPU or PyTorch fallback: if the library is missing, or a tensor is
 not on a HIP device, the calls raise.
 """
 import ctypes
+import itertools
 import os
 import warnings
 from typing import Dict, Optional, Tuple
@@ -196,6 +197,12 @@ _SIGNATURES = {
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 _INTERPOLATION = {"linear": 0, "smooth_step": 1}
+
+# Stamps of the tables' contents: a table takes a new one whenever its keys may
+# have changed, and no two tables ever share one (a table made by `resize` may
+# sit at the address of the one it replaces), so that what callers derive from
+# the keys can be kept under the stamp alone.
+_VERSIONS = itertools.count(1)
 
 # Largest number of staged sample slots (rays x stride, 8 bytes each) for which
 # ray_sample keeps the samples of its allocation pass; beyond it the march is
@@ -826,7 +833,7 @@ class _HashMap:
         self._maybe_tombstones = False
         # counts the calls that may have changed the stored keys; lets callers
         # keep results derived from the key set (orderings, tables) while it stands
-        self.version = 0
+        self.version = next(_VERSIONS)
         handle = _PTR()
         with torch.cuda.device(self._device):
             self._check(
@@ -893,7 +900,7 @@ class _HashMap:
         the kernel; attach the region once and let the caller re-issue."""
         st = self.status()
         self._status_after_insert = st
-        self.version += 1
+        self.version = next(_VERSIONS)
         if st["dropped"] > 0 or st["tombstones"] > 0:
             self._maybe_tombstones = True
         if st["exotic_pending"] == 0:
@@ -1130,7 +1137,7 @@ class _HashMap:
         keys = self._keys(keys)
         self._maybe_tombstones = True
         self._status_after_insert = None
-        self.version += 1
+        self.version = next(_VERSIONS)
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_erase(
@@ -1143,7 +1150,7 @@ class _HashMap:
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
         self._maybe_tombstones = False
         self._status_after_insert = None
-        self.version += 1
+        self.version = next(_VERSIONS)
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
         n = self.size()
