@@ -374,15 +374,15 @@ int ash_convolution_forward(const void* inputs, const void* weights,
  * not take run exactly as in the plain call.  No counterpart in the reference
  * (at::zeros_like, ash/src/grid.cu:1010). */
 int ash_convolution_forward_listed(const void* inputs, const void* weights,
-                            const uint8_t* masks, const int64_t* grid_indices,
-                            const int64_t* cell_indices,
-                            const int64_t* lut_grid_nb2grid_idx,
-                            const int64_t* lut_cell_nb2cell_idx,
-                            const int64_t* lut_cell_nb2grid_nb, void* outputs,
-                            int64_t num_grids, int64_t num_embeddings,
-                            int64_t cells_per_grid, int64_t embedding_dim,
-                            int64_t num_cell_nbs, int64_t num_grid_nbs,
-                            int32_t dtype, uint8_t* listed, void* stream);
+                                   const uint8_t* masks, const int64_t* grid_indices,
+                                   const int64_t* cell_indices,
+                                   const int64_t* lut_grid_nb2grid_idx,
+                                   const int64_t* lut_cell_nb2cell_idx,
+                                   const int64_t* lut_cell_nb2grid_nb, void* outputs,
+                                   int64_t num_grids, int64_t num_embeddings,
+                                   int64_t cells_per_grid, int64_t embedding_dim,
+                                   int64_t num_cell_nbs, int64_t num_grid_nbs,
+                                   int32_t dtype, uint8_t* listed, void* stream);
 
 /* Replace the two launches of `isosurface_extraction` (ash/src/grid.cu:453-602,
  * pybind.cpp:30; the reference counts, allocates and runs the same kernel again
