@@ -157,3 +157,90 @@ def test_bulk_equals_per_key_kernel(gpu_ash, monkeypatch):
     (ia, ma), (ib, mb) = a.find(probe), b.find(probe)
     assert torch.equal(ma, mb)
     assert_is_bijection_into(a.items()[1], capacity)
+
+
+@pytest.mark.parametrize("policy", ["always", "never"])
+def test_clear_leaves_the_fill_to_the_next_call(gpu_ash, monkeypatch, policy):
+    """clear() resets counters and heap at once and leaves the fill of the
+    bucket array to the next call on the table; a streaming insert rewrites
+    every bucket instead.  Whatever comes first after a clear -- find, items,
+    erase, size, a per-key or a streaming insert (also one that reaches only a
+    few partitions) -- sees an empty table, and nothing of the old keys comes
+    back later."""
+    monkeypatch.setattr(gpu_ash.common, "BULK_INSERT", policy)
+    rng = np.random.default_rng(61)
+    old = torch.unique(_random_keys(rng, 60_000, 3, 300), dim=0).to(DEV)
+    new = torch.unique(_random_keys(rng, 50_000, 3, 300), dim=0).to(DEV)
+    few = new[:3000].contiguous()
+
+    def fresh():
+        hm = gpu_ash.HashMap(3, 2, 2_000_000, DEV)
+        hm.insert(old, torch.ones(len(old), 2, device=DEV))
+        assert hm.size() == len(old)
+        hm.clear()
+        return hm
+
+    hm = fresh()
+    assert hm.size() == 0
+    masks, _ = hm.find(old)
+    assert not bool(masks.any())
+    hm = fresh()
+    keys, idx = hm.items()
+    assert len(keys) == 0 and len(idx) == 0
+    hm = fresh()
+    hm.erase(old[:100])
+    assert hm.size() == 0
+    for batch in (new, few):
+        hm = fresh()
+        values = torch.arange(len(batch), device=DEV, dtype=torch.float32).view(-1, 1).repeat(1, 2)
+        hm.insert(batch, values)
+        assert hm.size() == len(batch)
+        masks, idx, got = hm.find(batch, return_values=True)
+        assert bool(masks.all()) and torch.equal(got, values)
+        assert_is_bijection_into(idx.cpu(), 2_000_000)
+        keys, _ = hm.items()
+        assert torch.equal(sort_rows(keys)[0], sort_rows(batch)[0])
+    # a streaming insert that leaves many partitions of a large table without a
+    # record: those are written as empty ones, or old keys would reappear
+    import ctypes
+    big = gpu_ash.HashMap(3, 2, 20_000_000, DEV)
+    spread = torch.unique(_random_keys(rng, 400_000, 3, 2000), dim=0).to(DEV)
+    big.insert(spread, torch.ones(len(spread), 2, device=DEV))
+    big.clear()
+    sparse_batch = torch.unique(_random_keys(rng, 20_000, 3, 2000), dim=0).to(DEV)
+    if policy == "always":
+        rows = (ctypes.c_int64 * 1)(8)
+        assert big.engine.backend._bulk_workspace(len(sparse_batch), 1, rows) is not None
+    big.insert(sparse_batch, torch.zeros(len(sparse_batch), 2, device=DEV))
+    keys, _ = big.items()
+    assert torch.equal(sort_rows(keys)[0], sort_rows(sparse_batch)[0])
+    masks, _ = big.find(spread)
+    assert int(masks.sum()) <= len(sparse_batch)   # only keys that are in both sets
+    del big
+    # twice in a row, and a clear right after a clear
+    hm = fresh()
+    hm.clear()
+    hm.insert(few, torch.zeros(len(few), 2, device=DEV))
+    hm.clear()
+    hm.insert(new, torch.zeros(len(new), 2, device=DEV))
+    keys, _ = hm.items()
+    assert torch.equal(sort_rows(keys)[0], sort_rows(new)[0])
+
+
+def test_pending_fill_is_refused_under_capture(gpu_ash):
+    """A look-up recorded into a HIP graph right after a clear would record the
+    pending fill with it and empty the table at every replay: the call fails
+    instead, and works once the fill has run outside the capture."""
+    engine = gpu_ash.ASHEngine(3, 5000, DEV)
+    keys = torch.randint(-50, 50, (3000, 3), dtype=torch.int32, device=DEV)
+    engine.insert_keys(keys)
+    engine.clear()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with pytest.raises(RuntimeError, match="cleared"):
+            with torch.cuda.graph(graph, stream=side):
+                engine.find(keys)
+    torch.cuda.synchronize()
+    _, masks = engine.find(keys)
+    assert not bool(masks.any())

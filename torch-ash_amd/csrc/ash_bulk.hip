@@ -405,8 +405,11 @@ __device__ __forceinline__ int staged(int lb, int q) {
 }
 
 // Pass 3: one workgroup per partition builds its 512 buckets in LDS.
+// `stale`: the bucket array holds leftovers of a table that has been cleared
+// since (the clear left the fill to its successor): every partition is then
+// written, those without records as empty ones.
 __global__ __launch_bounds__(kBuildThreads) void build_kernel(
-        MapDev m, BulkPlan pl, ValueArgs va) {
+        MapDev m, BulkPlan pl, ValueArgs va, int stale) {
     __shared__ uint4 tab[kPartBuckets * kGroup];
     // winners per (record slot k, wavefront), then their exclusive prefix
     __shared__ int s_wcnt[kBuildRecs * (kBuildThreads / 64)];
@@ -417,13 +420,21 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
     const uint32_t p = blockIdx.x;
     int cnt = pl.cursor_part[p];
     if (cnt > static_cast<int>(pl.cap_part)) cnt = static_cast<int>(pl.cap_part);
-    if (cnt == 0) return;
     const uint32_t b0 = p << kPartShift;
+    if (b0 >= m.nb) return;
     const int nbk = static_cast<int>(m.nb - b0 < static_cast<uint32_t>(kPartBuckets)
                                              ? m.nb - b0
                                              : static_cast<uint32_t>(kPartBuckets));
     uint4* __restrict__ gl =
             reinterpret_cast<uint4*>(m.buckets) + static_cast<size_t>(b0) * kGroup;
+    if (cnt == 0) {
+        if (stale) {
+            for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
+                gl[t] = make_uint4(~0u, ~0u, ~0u, ~0u);
+            }
+        }
+        return;
+    }
     const bool was_empty = pl.hdr[kHdrWasEmpty] != 0;
     const int64_t bbase = static_cast<int64_t>(p) * pl.cap_part;
     // The first round's records are requested before the table range is
@@ -699,8 +710,12 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     split_records_kernel<<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl,
                                                                       user);
     ASH_LAUNCH_CHECK();
-    build_kernel<<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, from_b);
+    // A cleared table whose fill is still pending is empty by its counters, so
+    // the build starts every partition from scratch and writes all of them.
+    build_kernel<<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, from_b,
+                                                    map->table_stale ? 1 : 0);
     ASH_LAUNCH_CHECK();
+    map->table_stale = false;
     if (insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys,
                         user, s)) {
         return 1;

@@ -93,4 +93,8 @@ struct ash_map {
     ash::MapDev d;
     int64_t table_bytes;
     bool general_attached;
+    // clear() has reset the counters and the heap but left the bucket array as
+    // it was: the next call that reads the table fills it first, a streaming
+    // insert that rewrites every bucket does not need to
+    bool table_stale;
 };

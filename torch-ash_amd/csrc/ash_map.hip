@@ -1273,11 +1273,22 @@ int check_map(const ash_map* map) {
     return 0;
 }
 
-int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size) {
+int fill_buckets(ash_map* map, hipStream_t s) {
     const int64_t n16 = static_cast<int64_t>(map->d.nb) * kGroup;
     fill16_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
             reinterpret_cast<uint4*>(map->d.buckets), n16, 0xFFFFFFFFu);
     ASH_LAUNCH_CHECK();
+    map->table_stale = false;
+    return 0;
+}
+
+// `lazy`: leave the bucket array to the next call that needs it (settle_table).
+int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool lazy = false) {
+    if (lazy) {
+        map->table_stale = true;
+    } else if (fill_buckets(map, s)) {
+        return 1;
+    }
     if (map->general_attached) {
         const int64_t g16 = static_cast<int64_t>(map->d.gslots) / 4;
         fill16_kernel<<<capped_grid(g16), kBlock, 0, s>>>(
@@ -1352,6 +1363,18 @@ int launch_selected(ash_map* map, bool codes, const int32_t* keys,
 
 }  // namespace
 
+// Every entry that reads or updates buckets calls this first.  The fill must
+// not end up in a captured graph: replays would empty the table again.
+int settle_table(ash_map* map, hipStream_t s) {
+    if (!map->table_stale) return 0;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) == hipSuccess &&
+        capturing != hipStreamCaptureStatusNone) {
+        ASH_FAIL("the table was cleared and not used since: run one call outside the capture first");
+    }
+    return fill_buckets(map, s);
+}
+
 int check_batch(const ash_map* map, const void* keys, int64_t n) {
     if (check_map(map)) return 1;
     if (n < 0) ASH_FAIL("negative key count");
@@ -1413,6 +1436,7 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->device = device;
     map->table_bytes = table_bytes;
     map->general_attached = false;
+    map->table_stale = false;
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
@@ -1470,6 +1494,7 @@ int ash_map_find(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
     const unsigned g = grid_for(n);
     switch (map->key_dim) {
         case 1:
@@ -1502,6 +1527,7 @@ int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
     }
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
+    if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
     grid_query_kernel<<<grid_for(n), kBlock, 0,
                         static_cast<hipStream_t>(stream)>>>(
             map->d, x, n, static_cast<float>(grid_dim), grid_dim, grid_indices,
@@ -1526,6 +1552,7 @@ int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
     const int lo = bidirectional ? -dilation : 0;
     const int width = dilation - lo + 1;
     const float g = static_cast<float>(grid_dim);
@@ -1564,6 +1591,7 @@ int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
     }
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
+    if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
     // every step must advance t (else the march never ends), and their number
     // must stay finite
     const float half_block = static_cast<float>(grid2cell_multiplier * 0.5);
@@ -1604,6 +1632,7 @@ int ash_ray_sample(ash_map_t* map, const float* ray_origins,
     }
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
+    if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
     launch_ray_sample(map, ray_origins, ray_directions, ray_nears, ray_fars, n,
                       static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
                       prefix, ray_indices, t_nears, t_fars, nullptr, 0,
@@ -1632,6 +1661,7 @@ int ash_ray_sample_staged(ash_map_t* map, const float* ray_origins,
     if (reinterpret_cast<uintptr_t>(stage) % 8 != 0) ASH_FAIL("ray_sample_staged: stage must be 8-byte aligned");
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
+    if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
     launch_ray_sample(map, ray_origins, ray_directions, ray_nears, ray_fars, n,
                       static_cast<float>(max_samples_per_ray), grid2cell_multiplier, counts,
                       nullptr, nullptr, nullptr, nullptr, reinterpret_cast<float2*>(stage),
@@ -1663,6 +1693,7 @@ int ash_map_insert_keys(ash_map_t* map, const int32_t* keys, int64_t n,
     if (n == 0) return 0;
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
+    if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
     ValueArgs va = {};
     return launch_insert<kInsertKeys>(map, keys, n, va, nullptr, nullptr,
                                       static_cast<hipStream_t>(stream));
@@ -1726,6 +1757,7 @@ int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
     ValueArgs va = {};
     if (!ash_map_insert_needs_scratch(n_values, row_bytes)) {
         va.n = n_values;
@@ -1758,6 +1790,7 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
     const unsigned g = grid_for(n, kEraseBlock);
     switch (map->key_dim) {
         case 1:
@@ -1781,7 +1814,7 @@ int ash_map_clear(ash_map_t* map, void* stream) {
     if (check_map(map)) return 1;
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    return clear_table(map, static_cast<hipStream_t>(stream), true, 0);
+    return clear_table(map, static_cast<hipStream_t>(stream), true, 0, true);
 }
 
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
@@ -1821,6 +1854,7 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrCursor, 0);
     ASH_LAUNCH_CHECK();
     const int64_t units = static_cast<int64_t>(map->d.nb) * kGroup;
@@ -1894,10 +1928,7 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t n16 = static_cast<int64_t>(map->d.nb) * kGroup;
-    fill16_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
-            reinterpret_cast<uint4*>(map->d.buckets), n16, 0xFFFFFFFFu);
-    ASH_LAUNCH_CHECK();
+    if (fill_buckets(map, s)) return 1;
     if (map->general_attached) {
         const int64_t g16 = static_cast<int64_t>(map->d.gslots) / 4;
         fill16_kernel<<<capped_grid(g16), kBlock, 0, s>>>(

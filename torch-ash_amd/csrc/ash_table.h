@@ -123,5 +123,7 @@ int insert_selected(ash_map* map, bool codes, const void* keys,
                     const ValueArgs& va, hipStream_t s);
 
 int check_batch(const ash_map* map, const void* keys, int64_t n);
+// Fills the bucket array if a clear() left that to the next user of the table.
+int settle_table(ash_map* map, hipStream_t s);
 
 }  // namespace ash
