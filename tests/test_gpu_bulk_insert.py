@@ -2,6 +2,8 @@
 on for every batch that it accepts, it must leave the same map as the oracle and
 as the per-key kernel -- same key set, masks, sizes, heap protocol, and each
 stored key carrying the value rows of ONE of its source rows."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -202,7 +204,6 @@ def test_clear_leaves_the_fill_to_the_next_call(gpu_ash, monkeypatch, policy):
         assert torch.equal(sort_rows(keys)[0], sort_rows(batch)[0])
     # a streaming insert that leaves many partitions of a large table without a
     # record: those are written as empty ones, or old keys would reappear
-    import ctypes
     big = gpu_ash.HashMap(3, 2, 20_000_000, DEV)
     spread = torch.unique(_random_keys(rng, 400_000, 3, 2000), dim=0).to(DEV)
     big.insert(spread, torch.ones(len(spread), 2, device=DEV))
