@@ -511,3 +511,41 @@ def test_config5_fusion_reduced_against_oracle(gpu_ash, oracle, monkeypatch):
     assert float((~same).float().mean()) < 5e-4
     assert torch.allclose(cells_gpu[..., 0][same], cells_cpu[..., 0][same], rtol=1e-3, atol=2e-4)
     assert float(cells_gpu[..., 1].sum()) > 1e5
+
+
+@pytest.mark.parametrize("policy", ["auto", "always"])
+def test_table_larger_than_4_gib(gpu_ash, monkeypatch, policy):
+    """A bucket array of 6.4 GB (capacity 300 M): every byte offset into the
+    table needs more than 32 bits.  Keys spread over the whole array are
+    inserted (per key, and through the streaming path where it applies), found,
+    listed and erased."""
+    monkeypatch.setattr(gpu_ash.common, "BULK_INSERT", policy)
+    capacity = 300_000_000
+    hm = gpu_ash.HashMap(3, 1, capacity, DEV)
+    table_bytes = hm.engine.backend._table.numel()
+    assert table_bytes > 5 * 2**30
+    g = torch.Generator().manual_seed(97)
+    keys = torch.unique(torch.randint(-100_000, 100_000, (6_000_000, 3), generator=g,
+                                      dtype=torch.int32), dim=0).to(DEV)
+    n = len(keys)
+    values = torch.arange(n, device=DEV, dtype=torch.float32).view(-1, 1)
+    hm.insert(keys, values)
+    assert hm.size() == n
+    masks, indices, got = hm.find(keys, return_values=True)
+    assert bool(masks.all()) and torch.equal(got, values)
+    assert int(indices.min()) == 0 and int(indices.max()) == n - 1
+    assert len(torch.unique(indices)) == n
+    shifted = keys + torch.tensor([[250_000, 0, 0]], dtype=torch.int32, device=DEV)
+    masks_absent, _ = hm.find(shifted)
+    assert not bool(masks_absent.any())
+    listed, listed_idx = hm.items()
+    assert len(listed) == n
+    assert torch.equal(sort_rows(listed, listed_idx)[0], sort_rows(keys, indices)[0])
+    hm.erase(keys[: n // 2].contiguous())
+    assert hm.size() == n - n // 2
+    masks_after, _ = hm.find(keys)
+    assert not bool(masks_after[: n // 2].any()) and bool(masks_after[n // 2:].all())
+    hm.clear()
+    assert hm.size() == 0 and not bool(hm.find(keys[:1000].contiguous())[0].any())
+    del hm
+    torch.cuda.empty_cache()
