@@ -243,6 +243,13 @@ int ash_map_clear(ash_map_t* map, void* stream);
  *   out[4] duplicate (key,index) pairs seen by ash_map_load */
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
 
+/* ash_map_status through eight int32 of page-locked host memory of the
+ * caller's (`staging`, e.g. a pinned tensor kept with the map): the counters
+ * are copied there directly instead of through the runtime's staging of
+ * pageable memory, which halves the latency of the read-back that ends every
+ * insert.  No counterpart in the reference. */
+int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream);
+
 /* Replaces `HashMap::size` (ash/src/hashmap_gpu.cuh:157); synchronises. */
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream);
 

@@ -135,6 +135,7 @@ _SIGNATURES = {
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
     "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_map_status_staged": (ctypes.c_int, [_PTR, _PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_items": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_map_load": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR, _PTR]),
@@ -922,8 +923,16 @@ class _HashMap:
 
     def status(self) -> Dict[str, int]:
         out = (_I64 * 5)()
+        staging = getattr(self, "_status_staging", None)
+        if staging is None:
+            # page-locked landing place of the counters, kept with the map
+            staging = self._status_staging = torch.zeros(8, dtype=torch.int32, pin_memory=True)
         with torch.cuda.device(self._device):
-            self._check(self._lib.ash_map_status(self._handle, out, self._stream()))
+            self._check(
+                self._lib.ash_map_status_staged(
+                    self._handle, staging.data_ptr(), out, self._stream()
+                )
+            )
         return {
             "size": out[0],
             "dropped": out[1],

@@ -1817,15 +1817,20 @@ int ash_map_clear(ash_map_t* map, void* stream) {
     return clear_table(map, static_cast<hipStream_t>(stream), true, 0, true);
 }
 
-int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
+namespace {
+
+// `staging`: eight int32 of page-locked host memory of the caller's, or NULL.
+// A copy into pageable memory goes through the runtime's own staging and
+// takes about twice as long (25 against 13 us on an idle device).
+int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream) {
     if (check_map(map)) return 1;
     if (out == nullptr) ASH_FAIL("null status output");
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    int32_t host[8] = {0};
-    ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(host), hipMemcpyDeviceToHost,
-                           s));
+    int32_t pageable[8] = {0};
+    int32_t* host = staging != nullptr ? staging : pageable;
+    ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(pageable), hipMemcpyDeviceToHost, s));
     ASH_HIP(hipStreamSynchronize(s));
     out[0] = host[kCtrSize];
     out[1] = host[kCtrDropped];
@@ -1833,6 +1838,17 @@ int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
     out[3] = host[kCtrExotic];
     out[4] = host[kCtrLoadDup];
     return 0;
+}
+
+}  // namespace
+
+int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
+    return read_status(map, nullptr, out, stream);
+}
+
+int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream) {
+    if (staging == nullptr) ASH_FAIL("null staging buffer");
+    return read_status(map, staging, out, stream);
 }
 
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream) {
