@@ -244,7 +244,7 @@ int ash_map_clear(ash_map_t* map, void* stream);
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
 
 /* ash_map_status through eight int32 of page-locked host memory of the
- * caller's (`staging`, e.g. a pinned tensor kept with the map): the counters
+ * caller's (`staging`, e.g. one pinned tensor per host thread): the counters
  * are copied there directly instead of through the runtime's staging of
  * pageable memory, which halves the latency of the read-back that ends every
  * insert.  No counterpart in the reference. */

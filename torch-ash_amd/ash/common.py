@@ -12,6 +12,7 @@ not on a HIP device, the calls raise.
 import ctypes
 import itertools
 import os
+import threading
 import warnings
 from typing import Dict, Optional, Tuple
 
@@ -769,6 +770,20 @@ class _Backend:
         return grad_z, grad_embeddings, grad_offsets
 
 
+_STAGING: Dict[int, torch.Tensor] = {}
+
+
+def _status_staging() -> torch.Tensor:
+    """Page-locked landing place for the counters of a status read-back: one
+    per host thread for all maps (a read-back is complete when it returns, and
+    short-lived scratch sets would otherwise each allocate their own)."""
+    key = threading.get_ident()
+    staging = _STAGING.get(key)
+    if staging is None:
+        staging = _STAGING[key] = torch.zeros(8, dtype=torch.int32, pin_memory=True)
+    return staging
+
+
 def _accumulator(t: torch.Tensor, embeddings: torch.Tensor) -> torch.Tensor:
     """Checks that `t` can take a gradient of `embeddings` in place."""
     if (
@@ -923,10 +938,7 @@ class _HashMap:
 
     def status(self) -> Dict[str, int]:
         out = (_I64 * 5)()
-        staging = getattr(self, "_status_staging", None)
-        if staging is None:
-            # page-locked landing place of the counters, kept with the map
-            staging = self._status_staging = torch.zeros(8, dtype=torch.int32, pin_memory=True)
+        staging = _status_staging()
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_status_staged(
