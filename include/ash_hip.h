@@ -113,6 +113,18 @@ int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
                       int bound_lo, int bound_hi, uint8_t* touched,
                       int32_t* coords, int32_t* heads_scratch, void* stream);
 
+/* After ash_grid_activate: the rows whose flag is set in `touched`, in
+ * ascending order, to out_indices int64[capacity] and their block coordinates
+ * to out_coords int32[capacity, 3]; the flags are cleared and the count is left
+ * in the table's counters (out[5] of ash_map_status_staged), so that the
+ * read-back that follows an activation anyway also sizes the result -- instead
+ * of a `nonzero` over the flags with a read-back of its own.  One workgroup;
+ * tables of up to ASH_COLLECT_MAX_BLOCKS rows.  No counterpart in the
+ * reference. */
+#define ASH_COLLECT_MAX_BLOCKS (1 << 20)
+int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* block_coords,
+                             int64_t* out_indices, int32_t* out_coords, void* stream);
+
 /* Stands for `project_points_to_rgbd` plus the fusion arithmetic of
  * `fuse_frame` in the reference's TSDF demo (demo/rgbd_fusion.py:76-110,
  * 216-254), which are torch expressions around
@@ -247,8 +259,9 @@ int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
  * caller's (`staging`, e.g. one pinned tensor per host thread): the counters
  * are copied there directly instead of through the runtime's staging of
  * pageable memory, which halves the latency of the read-back that ends every
- * insert.  No counterpart in the reference. */
-int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream);
+ * insert.  out[5] is the number of rows the latest ash_grid_collect_touched
+ * listed.  No counterpart in the reference. */
+int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[6], void* stream);
 
 /* Replaces `HashMap::size` (ash/src/hashmap_gpu.cuh:157); synchronises. */
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream);

@@ -199,3 +199,29 @@ def test_fused_fusion_against_oracle_harness(gpu_ash, oracle, monkeypatch):
     assert float((~same).float().mean()) < 5e-4
     assert torch.allclose(cells_gpu[..., 0][same], cells_cpu[..., 0][same], rtol=1e-3, atol=2e-4)
     assert float(cells_gpu[..., 1].sum()) > 1e5
+
+
+@pytest.mark.parametrize("capacity", [5, 1000, 80_000, 131_073, 200_000, 1_048_576])
+def test_touched_rows_are_listed_in_order(gpu_ash, capacity):
+    """ash_grid_collect_touched against torch.nonzero: ascending rows, their
+    coordinates, flags cleared, count in the sixth status value -- for runs of
+    flags per thread that fit the registers, that do not, and that end inside
+    the last word."""
+    engine = gpu_ash.ASHEngine(3, capacity, DEV)
+    backend = engine.backend
+    g = torch.Generator().manual_seed(capacity)
+    for density in (0.0, 0.05, 1.0):
+        flags = (torch.rand(capacity, generator=g) < density).to(torch.uint8).to(DEV)
+        flags = flags * torch.randint(1, 255, (capacity,), generator=g, dtype=torch.uint8).to(DEV)
+        coords = torch.randint(-1000, 1000, (capacity, 3), generator=g, dtype=torch.int32).to(DEV)
+        expected = flags.nonzero().view(-1)
+        rows = torch.full((capacity,), -1, dtype=torch.int64, device=DEV)
+        out_coords = torch.zeros((capacity, 3), dtype=torch.int32, device=DEV)
+        rc = backend._lib.ash_grid_collect_touched(
+            backend._handle, flags.data_ptr(), coords.data_ptr(), rows.data_ptr(),
+            out_coords.data_ptr(), backend._stream())
+        assert rc == 0, backend._lib.ash_last_error().decode()
+        n = backend.status()["touched"]
+        assert n == len(expected)
+        assert torch.equal(rows[:n], expected) and torch.equal(out_coords[:n], coords[expected])
+        assert bool((rows[n:] == -1).all()) and int(flags.sum()) == 0

@@ -137,6 +137,7 @@ _SIGNATURES = {
     "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
     "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_status_staged": (ctypes.c_int, [_PTR, _PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_grid_collect_touched": (ctypes.c_int, [_PTR] * 6),
     "ash_map_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_items": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_map_load": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR, _PTR]),
@@ -212,6 +213,9 @@ _VERSIONS = itertools.count(1)
 RAY_STAGE_LIMIT = 1 << 30
 # Staged slots per ray beyond max_samples_per_ray.
 RAY_STAGE_EXTRA = 2
+# Largest table whose touched rows ash_grid_collect_touched lists (the header's
+# ASH_COLLECT_MAX_BLOCKS).
+COLLECT_MAX_BLOCKS = 1 << 20
 
 # Which inserts take the streaming (partition + build in LDS) path of the
 # library instead of the per-key kernel: "auto" = when the library says the
@@ -937,7 +941,7 @@ class _HashMap:
         return self._device
 
     def status(self) -> Dict[str, int]:
-        out = (_I64 * 5)()
+        out = (_I64 * 6)()
         staging = _status_staging()
         with torch.cuda.device(self._device):
             self._check(
@@ -951,6 +955,7 @@ class _HashMap:
             "tombstones": out[2],
             "exotic_pending": out[3],
             "load_duplicates": out[4],
+            "touched": out[5],
         }
 
     def status_after_insert(self) -> Dict[str, int]:
@@ -1034,6 +1039,13 @@ class _HashMap:
             )
         self._make_room(cells.shape[0])
         heads = torch.empty(64 + 3 * cells.shape[0], dtype=torch.int32, device=self._device)
+        # the touched rows are listed on the device and their count travels with
+        # the read-back that ends the activation (tables beyond the listing
+        # kernel's one workgroup take torch's nonzero and a second read-back)
+        listing = self.capacity <= COLLECT_MAX_BLOCKS
+        if listing:
+            rows = torch.empty(self.capacity, dtype=torch.int64, device=self._device)
+            coords = torch.empty((self.capacity, 3), dtype=torch.int32, device=self._device)
         for _ in range(2):
             with torch.cuda.device(self._device):
                 self._check(
@@ -1044,8 +1056,18 @@ class _HashMap:
                         heads.data_ptr(), self._stream(),
                     )
                 )
+                if listing:
+                    self._check(
+                        self._lib.ash_grid_collect_touched(
+                            self._handle, self._touched.data_ptr(), self._block_coords.data_ptr(),
+                            rows.data_ptr(), coords.data_ptr(), self._stream(),
+                        )
+                    )
             if not self._attach_general_if_needed():
                 break
+        if listing:
+            n = self._status_after_insert["touched"]
+            return coords[:n], rows[:n]
         grid_indices = self._touched.nonzero().view(-1)
         grid_coords = self._block_coords[grid_indices]
         self._touched[grid_indices] = 0

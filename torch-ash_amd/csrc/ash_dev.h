@@ -52,6 +52,7 @@ enum Counter {
     kCtrExotic = 3,    // unpackable keys seen while no general region exists
     kCtrLoadDup = 4,   // duplicate pairs met by load
     kCtrCursor = 5,    // output cursor of items()
+    kCtrTouched = 6,   // blocks listed by the latest ash_grid_collect_touched
     kNumCounters = 64
 };
 constexpr int64_t kHeaderBytes = 256;

@@ -1232,6 +1232,85 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(
     }
 }
 
+// The rows whose flag an activation has set, in ascending order, with their
+// block coordinates; the flags are cleared on the way and the count goes to
+// the table's counters, where the read-back that follows every activation
+// finds it.  One workgroup: every thread takes a run of `span` flags (a
+// multiple of four, read as words), an exclusive scan over the workgroup
+// gives each run its place in the output.
+constexpr int kCollectThreads = 1024;
+constexpr int64_t kCollectMaxBlocks = int64_t{1} << 20;   // ASH_COLLECT_MAX_BLOCKS of the header
+
+__global__ __launch_bounds__(kCollectThreads) void collect_touched_kernel(
+        uint8_t* __restrict__ touched, const int32_t* __restrict__ block_coords,
+        int64_t capacity, int span, int64_t* __restrict__ out_idx,
+        int32_t* __restrict__ out_coords, int32_t* __restrict__ ctr) {
+    __shared__ int s_wave[kCollectThreads / 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t first = static_cast<int64_t>(threadIdx.x) * span;
+    int cnt = 0;
+    for (int o = 0; o < span; o += 4) {
+        const int64_t at = first + o;
+        if (at >= capacity) break;
+        uint32_t w = at + 4 <= capacity ? *reinterpret_cast<const uint32_t*>(touched + at) : 0u;
+        if (at + 4 > capacity) {
+            for (int b = 0; at + b < capacity; ++b) w |= static_cast<uint32_t>(touched[at + b]) << (8 * b);
+        }
+        cnt += (w & 0xFFu ? 1 : 0) + (w & 0xFF00u ? 1 : 0) + (w & 0xFF0000u ? 1 : 0) +
+               (w & 0xFF000000u ? 1 : 0);
+    }
+    int incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    int pos = incl - cnt;
+    int total = 0;
+    for (int q = 0; q < kCollectThreads / 64; ++q) {
+        if (q < wave) pos += s_wave[q];
+        total += s_wave[q];
+    }
+    if (threadIdx.x == 0) ctr[kCtrTouched] = total;
+    if (cnt == 0) return;
+    auto list = [&](int64_t at) {
+        out_idx[pos] = at;
+        out_coords[pos * 3 + 0] = block_coords[at * 3 + 0];
+        out_coords[pos * 3 + 1] = block_coords[at * 3 + 1];
+        out_coords[pos * 3 + 2] = block_coords[at * 3 + 2];
+        ++pos;
+    };
+    constexpr int kWords = 32;   // runs of up to 128 flags are held in registers
+    if (span <= 4 * kWords && first + span <= capacity) {
+        uint32_t w[kWords];
+#pragma unroll
+        for (int i = 0; i < kWords; ++i) {
+            w[i] = 4 * i < span ? *reinterpret_cast<const uint32_t*>(touched + first + 4 * i) : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < kWords; ++i) {
+            if (w[i] == 0u) continue;
+            *reinterpret_cast<uint32_t*>(touched + first + 4 * i) = 0u;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                if ((w[i] >> (8 * b)) & 0xFFu) list(first + 4 * i + b);
+            }
+        }
+        return;
+    }
+    for (int o = 0; o < span; ++o) {
+        const int64_t at = first + o;
+        if (at >= capacity) break;
+        if (touched[at]) {
+            touched[at] = 0;
+            list(at);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- host
 inline unsigned grid_for(int64_t n, int per_block = kBlock) {
     return static_cast<unsigned>((n + per_block - 1) / per_block);
@@ -1822,7 +1901,7 @@ namespace {
 // `staging`: eight int32 of page-locked host memory of the caller's, or NULL.
 // A copy into pageable memory goes through the runtime's own staging and
 // takes about twice as long (25 against 13 us on an idle device).
-int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream) {
+int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], int64_t* touched, void* stream) {
     if (check_map(map)) return 1;
     if (out == nullptr) ASH_FAIL("null status output");
     DeviceGuard guard;
@@ -1837,18 +1916,39 @@ int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream) 
     out[2] = host[kCtrTombs];
     out[3] = host[kCtrExotic];
     out[4] = host[kCtrLoadDup];
+    if (touched != nullptr) *touched = host[kCtrTouched];
     return 0;
 }
 
 }  // namespace
 
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
-    return read_status(map, nullptr, out, stream);
+    return read_status(map, nullptr, out, nullptr, stream);
 }
 
-int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[5], void* stream) {
+int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[6], void* stream) {
     if (staging == nullptr) ASH_FAIL("null staging buffer");
-    return read_status(map, staging, out, stream);
+    if (out == nullptr) ASH_FAIL("null status output");
+    return read_status(map, staging, out, out + 5, stream);
+}
+
+int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* block_coords,
+                             int64_t* out_indices, int32_t* out_coords, void* stream) {
+    if (check_map(map)) return 1;
+    if (touched == nullptr || block_coords == nullptr || out_indices == nullptr ||
+        out_coords == nullptr) {
+        ASH_FAIL("null pointer in grid_collect_touched");
+    }
+    if (map->capacity > kCollectMaxBlocks) ASH_FAIL("grid_collect_touched: too many blocks for one workgroup");
+    if (reinterpret_cast<uintptr_t>(touched) % 4 != 0) ASH_FAIL("grid_collect_touched: flags must be 4-byte aligned");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    int span = static_cast<int>((map->capacity + kCollectThreads - 1) / kCollectThreads);
+    span = (span + 3) / 4 * 4;
+    collect_touched_kernel<<<1, kCollectThreads, 0, static_cast<hipStream_t>(stream)>>>(
+            touched, block_coords, map->capacity, span, out_indices, out_coords, map->d.ctr);
+    ASH_LAUNCH_CHECK();
+    return 0;
 }
 
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream) {
