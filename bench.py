@@ -507,6 +507,9 @@ def bench_fusion(torch, ash, workloads, args, dev, frames=20):
     integration kernels and once in the reference's formulation (candidate
     expansion + scratch set, torch expressions around
     embeddings[grid_indices, cell_indices])."""
+    # same allocator state whatever ran before: the reference formulation
+    # allocates tens of MB per frame and is sensitive to what is cached
+    torch.cuda.empty_cache()
     scene = workloads.FusionScene()
     intrinsic = scene.intrinsic.to(dev)
     data = []
