@@ -239,7 +239,10 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n, void* stream);
 
 /* Replaces `HashMap::clear` (ash/src/hashmap_gpu.cuh:354-358,
  * ash/src/hashmap_impl.h:26-33).  Counters, heap and the second region are
- * reset on `stream` at once; the fill of the bucket array runs with the next
+ * reset on `stream` at once (the heap array is rewritten to 0..capacity-1 only
+ * when ash_map_erase or ash_map_load has written to it since it was last in
+ * that state: inserts only read it, and nothing but this library may write to
+ * it while the map lives); the fill of the bucket array runs with the next
  * call that reads or updates the table, on that call's stream, and not at all
  * when that call is an ash_map_insert_bulk, which rewrites every bucket.  A
  * call whose stream is being captured refuses to run that pending fill (the

@@ -549,3 +549,36 @@ def test_table_larger_than_4_gib(gpu_ash, monkeypatch, policy):
     assert hm.size() == 0 and not bool(hm.find(keys[:1000].contiguous())[0].any())
     del hm
     torch.cuda.empty_cache()
+
+
+def test_heap_starts_over_after_clear(gpu_ash):
+    """clear() gives the indices back in their first order: the heap array is
+    rewritten when an erase or a load has written to it and left alone when
+    nothing has; either way the next n distinct keys get the indices 0..n-1."""
+    engine = gpu_ash.ASHEngine(3, 6000, DEV)
+    g = torch.Generator().manual_seed(99)
+    keys = torch.unique(torch.randint(-40, 40, (5000, 3), generator=g, dtype=torch.int32), dim=0).to(DEV)
+    n = len(keys)
+
+    def fresh_indices():
+        engine.insert_keys(keys)
+        indices, masks = engine.find(keys)
+        assert bool(masks.all())
+        return torch.sort(indices)[0]
+
+    assert torch.equal(fresh_indices(), torch.arange(n, device=DEV))
+    engine.clear()                                   # nothing wrote to the heap
+    assert torch.equal(fresh_indices(), torch.arange(n, device=DEV))
+    engine.erase(keys[::3].contiguous())             # freed indices go back in another order
+    engine.insert_keys(keys[::3].contiguous())
+    engine.clear()
+    assert torch.equal(fresh_indices(), torch.arange(n, device=DEV))
+    state = {k: v.clone() for k, v in engine.state_dict().items()}
+    engine.erase(keys[: n // 2].contiguous())
+    engine.load_state_dict(state)                    # the heap comes from the caller
+    engine.clear()
+    half = keys[: n // 2].contiguous()
+    engine.insert_keys(half)
+    indices, masks = engine.find(half)
+    assert bool(masks.all())
+    assert torch.equal(torch.sort(indices)[0], torch.arange(len(half), device=DEV))

@@ -98,4 +98,7 @@ struct ash_map {
     // it was: the next call that reads the table fills it first, a streaming
     // insert that rewrites every bucket does not need to
     bool table_stale;
+    // the heap array may differ from 0, 1, 2, ... (an erase or a load has
+    // written to it since it was last reset): clear() rewrites it only then
+    bool heap_dirty;
 };

@@ -1374,10 +1374,14 @@ int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool
                 reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
         ASH_LAUNCH_CHECK();
     }
-    int64_t span = map->capacity > kNumCounters ? map->capacity : kNumCounters;
+    // Inserts only read the heap; while nothing has written to it since the
+    // last reset it still is 0, 1, 2, ... and only the counters are reset.
+    const bool rewrite = write_heap && map->heap_dirty;
+    int64_t span = rewrite && map->capacity > kNumCounters ? map->capacity : kNumCounters;
     reset_heap_kernel<<<grid_for(span), kBlock, 0, s>>>(
-            map->d.heap, map->capacity, map->d.ctr, size, write_heap);
+            map->d.heap, map->capacity, map->d.ctr, size, rewrite);
     ASH_LAUNCH_CHECK();
+    if (rewrite) map->heap_dirty = false;
     return 0;
 }
 
@@ -1516,6 +1520,7 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->table_bytes = table_bytes;
     map->general_attached = false;
     map->table_stale = false;
+    map->heap_dirty = true;   // the caller's buffer holds anything
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
@@ -1870,6 +1875,7 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
+    map->heap_dirty = true;   // freed indices go back onto the heap
     const unsigned g = grid_for(n, kEraseBlock);
     switch (map->key_dim) {
         case 1:
@@ -2068,6 +2074,7 @@ int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (clear_table(map, s, false, static_cast<int32_t>(n))) return 1;
+    map->heap_dirty = true;   // the heap is the caller's from here on
     if (heap_src != nullptr && heap_src != map->d.heap) {
         ASH_HIP(hipMemcpyAsync(map->d.heap, heap_src,
                                static_cast<size_t>(map->capacity) * 4,
