@@ -573,8 +573,9 @@ def test_heap_starts_over_after_clear(gpu_ash):
     engine.insert_keys(keys[::3].contiguous())
     engine.clear()
     assert torch.equal(fresh_indices(), torch.arange(n, device=DEV))
+    engine.erase(keys[::2].contiguous())             # the saved heap is out of order
     state = {k: v.clone() for k, v in engine.state_dict().items()}
-    engine.erase(keys[: n // 2].contiguous())
+    engine.clear()                                   # in order again, and marked so
     engine.load_state_dict(state)                    # the heap comes from the caller
     engine.clear()
     half = keys[: n // 2].contiguous()
