@@ -113,6 +113,25 @@ int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
                       int bound_lo, int bound_hi, uint8_t* touched,
                       int32_t* coords, int32_t* heads_scratch, void* stream);
 
+/* ash_grid_activate for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops that must not reach hipMalloc, harnesses
+ * that forbid it): same arguments, same result, but the list of run heads lives
+ * in a device array inside the library instead of `heads_scratch`, and the call
+ * allocates nothing on the host or the device.  No counterpart in the
+ * reference.
+ *   - at most ASH_ACTIVATE_STATIC_MAX_POSITIONS positions per call (a 1024 x
+ *     1024 depth image); more is an error, nothing is launched;
+ *   - the array (64 + 3 * ASH_ACTIVATE_STATIC_MAX_POSITIONS int32, 12.6 MB) is
+ *     held by every device that loads the library until the process ends;
+ *   - all calls on one device share it, on whatever map or stream: two calls
+ *     whose work overlaps in time on one device race.  Issue them on one
+ *     stream, or order the streams with events. */
+#define ASH_ACTIVATE_STATIC_MAX_POSITIONS (1 << 20)
+int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
+                             int grid_dim, int dilation, int bidirectional,
+                             int bound_lo, int bound_hi, uint8_t* touched,
+                             int32_t* coords, void* stream);
+
 /* After ash_grid_activate: the rows whose flag is set in `touched`, in
  * ascending order, to out_indices int64[capacity] and their block coordinates
  * to out_coords int32[capacity, 3]; the flags are cleared and the count is left

@@ -76,6 +76,11 @@ _SIGNATURES = {
         [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
          _PTR, _PTR, _PTR, _PTR],
     ),
+    "ash_grid_activate_static": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         _PTR, _PTR, _PTR],
+    ),
     "ash_grid_integrate_depth": (
         ctypes.c_int,
         [_PTR, _I64, ctypes.c_int, ctypes.c_int, _PTR, _PTR, _I64, ctypes.c_float,

@@ -24,9 +24,16 @@
 
 #include "../../include/ash_hip.h"
 
-#ifndef ASH_HEAP_BLOCK
-#define ASH_HEAP_BLOCK 256
-#endif
+#include <mutex>
+
+// Scratch of ash_grid_activate_static, the entry point that allocates nothing:
+// the list of run heads that ash_grid_activate keeps in a caller-provided
+// temporary (one counter line + three int32 per position).  Every device that
+// loads the library holds its own copy until the process ends.  In host code
+// this name is only a handle for hipGetSymbolAddress; kernels are given the
+// address that call returned for the current device.
+constexpr int64_t kActivateStaticMax = ASH_ACTIVATE_STATIC_MAX_POSITIONS;
+static __device__ __align__(256) int32_t scratch[64 + 3 * kActivateStaticMax];
 
 namespace ash {
 
@@ -40,7 +47,7 @@ constexpr int kBlock = 256;
 // workgroup).  Larger groups mean fewer updates of that single address but
 // make every wavefront wait for the slowest probe of the group; measured on
 // 16 M keys: 256 -> 1.28 ms, 512 -> 1.46 ms, 1024 -> 1.42 ms.
-constexpr int kHeapBlock = ASH_HEAP_BLOCK;
+constexpr int kHeapBlock = 256;
 constexpr uint32_t kSpinLimit = 1u << 22;
 
 __device__ __forceinline__ uint32_t spread8(uint32_t x) {
@@ -990,10 +997,7 @@ __global__ __launch_bounds__(kBlock) void ray_compact_kernel(
 // each), so larger groups pay off here: measured on 16 M stored keys,
 // 256 threads with a tombstone update per wavefront 3.0 ms, 1024 threads with
 // one update of each counter per workgroup 0.85 ms.
-#ifndef ASH_ERASE_BLOCK
-#define ASH_ERASE_BLOCK 1024
-#endif
-constexpr int kEraseBlock = ASH_ERASE_BLOCK;
+constexpr int kEraseBlock = 1024;
 
 template <int DIM>
 __global__ __launch_bounds__(kEraseBlock) void erase_kernel(
@@ -1620,41 +1624,106 @@ int ash_grid_query(ash_map_t* map, const float* x, int64_t n, int grid_dim,
     return 0;
 }
 
-int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
-                      int grid_dim, int dilation, int bidirectional,
-                      int bound_lo, int bound_hi, uint8_t* touched,
-                      int32_t* coords, int32_t* heads_scratch, void* stream) {
+namespace {
+
+// Argument checks shared by the two activation entry points; `heads` is
+// checked by the caller.
+int check_activate(ash_map_t* map, const float* cells, int64_t n, int grid_dim,
+                   int dilation, int bound_lo, int bound_hi, const uint8_t* touched,
+                   const int32_t* coords) {
     if (check_batch(map, cells, n)) return 1;
     if (map->key_dim != 3) ASH_FAIL("block activation needs a map with 3-d keys");
     if (grid_dim < 1 || grid_dim > 1024) ASH_FAIL("grid_dim must be in 1..1024");
     if (dilation < 0 || dilation > 8) ASH_FAIL("dilation must be in 0..8");
     if (bound_lo > bound_hi) ASH_FAIL("empty block bounds");
-    if (n == 0) return 0;
-    if (touched == nullptr || coords == nullptr || heads_scratch == nullptr) {
+    if (n > 0 && (touched == nullptr || coords == nullptr)) {
         ASH_FAIL("null output or scratch pointer");
     }
-    DeviceGuard guard;
-    ASH_HIP(guard.enter(map->device));
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    return 0;
+}
+
+// The launches of an activation; the map's device is current, `heads` points
+// to 64 + 3 n int32 of device memory.
+int launch_activate(ash_map_t* map, const float* cells, int64_t n, int grid_dim,
+                    int dilation, int bidirectional, int bound_lo, int bound_hi,
+                    uint8_t* touched, int32_t* coords, int32_t* heads, hipStream_t s) {
     if (settle_table(map, s)) return 1;
     const int lo = bidirectional ? -dilation : 0;
     const int width = dilation - lo + 1;
     const float g = static_cast<float>(grid_dim);
-    set_counter_kernel<<<1, 64, 0, s>>>(heads_scratch, 0, 0);
+    set_counter_kernel<<<1, 64, 0, s>>>(heads, 0, 0);
     ASH_LAUNCH_CHECK();
     activate_heads_kernel<<<grid_for(n, kHeadsBlock), kHeadsBlock, 0, s>>>(
-            cells, n, g, bound_lo, bound_hi, heads_scratch);
+            cells, n, g, bound_lo, bound_hi, heads);
     ASH_LAUNCH_CHECK();
     int64_t blocks = (n * width * width * width + kHeapBlock - 1) / kHeapBlock;
     if (blocks > 2048) blocks = 2048;
     const unsigned gb = static_cast<unsigned>(blocks);
     activate_kernel<false><<<gb, kHeapBlock, 0, s>>>(
-            map->d, heads_scratch, lo, width, bound_lo, bound_hi, touched, coords);
+            map->d, heads, lo, width, bound_lo, bound_hi, touched, coords);
     ASH_LAUNCH_CHECK();
     activate_kernel<true><<<gb, kHeapBlock, 0, s>>>(
-            map->d, heads_scratch, lo, width, bound_lo, bound_hi, touched, coords);
+            map->d, heads, lo, width, bound_lo, bound_hi, touched, coords);
     ASH_LAUNCH_CHECK();
     return 0;
+}
+
+// Address of `scratch` on each device, asked for once per device with that
+// device current (every device holds its own copy at its own address).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+int32_t* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_on_current_device(int device, int32_t** out) {
+    if (device < 0 || device >= kMaxDevices) ASH_FAIL("device number out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        void* p = nullptr;
+        ASH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) ASH_FAIL("hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[device] = static_cast<int32_t*>(p);
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
+
+}  // namespace
+
+int ash_grid_activate(ash_map_t* map, const float* cells, int64_t n,
+                      int grid_dim, int dilation, int bidirectional,
+                      int bound_lo, int bound_hi, uint8_t* touched,
+                      int32_t* coords, int32_t* heads_scratch, void* stream) {
+    if (check_activate(map, cells, n, grid_dim, dilation, bound_lo, bound_hi, touched, coords)) {
+        return 1;
+    }
+    if (n == 0) return 0;
+    if (heads_scratch == nullptr) ASH_FAIL("null output or scratch pointer");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    return launch_activate(map, cells, n, grid_dim, dilation, bidirectional, bound_lo, bound_hi,
+                           touched, coords, heads_scratch, static_cast<hipStream_t>(stream));
+}
+
+int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
+                             int grid_dim, int dilation, int bidirectional,
+                             int bound_lo, int bound_hi, uint8_t* touched,
+                             int32_t* coords, void* stream) {
+    if (check_activate(map, cells, n, grid_dim, dilation, bound_lo, bound_hi, touched, coords)) {
+        return 1;
+    }
+    if (n > kActivateStaticMax) {
+        ASH_FAIL("ash_grid_activate_static takes at most " +
+                 std::to_string(kActivateStaticMax) +
+                 " positions per call (ASH_ACTIVATE_STATIC_MAX_POSITIONS); use "
+                 "ash_grid_activate with a scratch buffer of the caller's for more");
+    }
+    if (n == 0) return 0;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    int32_t* heads = nullptr;
+    if (scratch_on_current_device(map->device, &heads)) return 1;
+    return launch_activate(map, cells, n, grid_dim, dilation, bidirectional, bound_lo, bound_hi,
+                           touched, coords, heads, static_cast<hipStream_t>(stream));
 }
 
 int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
