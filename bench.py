@@ -4,7 +4,7 @@
 
 Headline (`value`): configuration 2 of the baseline -- HashMap with values
 {color: fp32[3], depth: fp32[1]}, 16 M distinct voxel keys into capacity 24 M,
-16 M queries (70 % hits), full items() enumeration.  One step is
+16 M queries (70 % hits), full items(return_indices=True, return_values=True) enumeration.  One step is
 clear + insert + find + items through the public Python API (including its
 host read-backs), inputs resident in HBM; `value` counts the 32 M keys that
 were inserted or looked up per step.
@@ -37,6 +37,38 @@ for sub in ("torch-ash_amd", "oracle", ""):
         sys.path.insert(0, path)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X, published
+
+PROBES_SRC = os.path.join(ROOT, "bench_probes.hip")
+PROBES_LIB = os.path.join(ROOT, "bench_probes.so")
+
+
+def build_probes(force: bool = False) -> str:
+    """Compiles bench_probes.hip (the random-line probes behind `ceilings`) for
+    gfx950 into bench_probes.so beside this file.  The probes belong to the
+    benchmark, not to libash_hip.so."""
+    import shutil
+    import subprocess
+
+    if not force and os.path.exists(PROBES_LIB) and \
+            os.path.getmtime(PROBES_LIB) >= os.path.getmtime(PROBES_SRC):
+        return PROBES_LIB
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    tmp = PROBES_LIB + ".tmp"
+    subprocess.check_call([
+        hipcc, "-O3", "-std=c++17", "-fPIC", "-shared", "--offload-arch=gfx950",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", PROBES_SRC, "-o", tmp])
+    os.replace(tmp, PROBES_LIB)
+    return PROBES_LIB
+
+
+def load_probes():
+    lib = ctypes.CDLL(build_probes())
+    lib.bench_probe_last_error.restype = ctypes.c_char_p
+    lib.bench_probe_random_lines.restype = ctypes.c_int
+    lib.bench_probe_random_lines.argtypes = [
+        ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
+        ctypes.c_uint64, ctypes.c_void_p]
+    return lib
 
 # Algorithmic bytes per unit of work.  A stored slot counts as 16 B (12 B key +
 # 4 B index) whatever the physical layout; E = embedding width; fp32.
@@ -86,7 +118,8 @@ def parse_args():
     ap.add_argument("--no-trilinear", action="store_true", help="skip the trilinear kernel figures")
     ap.add_argument("--no-fusion", action="store_true", help="skip the configuration 5 figure")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--cpu-keys", type=int, default=4_000_000, help="CPU baseline sample size")
+    ap.add_argument("--cpu-keys", type=int, default=0,
+                    help="CPU baseline size (0 = the configuration itself: --keys into --capacity)")
     ap.add_argument("--calibrate", action="store_true",
                     help="run a 1 GiB device copy first (reference point for HBM counters)")
     return ap.parse_args()
@@ -129,11 +162,11 @@ def roofline_entry(name, alg_bytes, ms, traffic=None):
 
 def measure_ceilings(torch, ash, dev, table_bytes, n):
     """What this device's memory system delivers for the two access patterns
-    that bound the table kernels, measured with the library's probes on a
+    that bound the table kernels, measured with the probes of bench_probes.hip on a
     buffer of the table's size: random 128-byte line reads (a probe) and random
     line read + compare-and-swap + dword store (an insert); plus a plain
     device-to-device copy for the streaming rate."""
-    lib = ash.core.backend.lib
+    lib = load_probes()
     stream = torch.cuda.current_stream(dev).cuda_stream
     buf = torch.empty(table_bytes // 128 * 128, dtype=torch.uint8, device=dev).fill_(255)
     sink = torch.empty(n, dtype=torch.int32, device=dev)
@@ -142,10 +175,10 @@ def measure_ceilings(torch, ash, dev, table_bytes, n):
                        (2, "random_half_line_reads")):
         timer = EventTimer(torch)
         for it in range(6):
-            call = lambda: lib.ash_diag_random_lines(
+            call = lambda: lib.bench_probe_random_lines(
                 mode, buf.data_ptr(), buf.numel(), n, sink.data_ptr(), 7919 * it, stream)
             if it == 0:
-                assert call() == 0, lib.ash_last_error().decode()
+                assert call() == 0, lib.bench_probe_last_error().decode()
             else:
                 timer(call)
         ms = timer.mean_ms()
@@ -176,7 +209,7 @@ def bench_hash(torch, ash, workloads, args, dev):
         hm.clear()
         hm.insert(w["keys"], values)
         masks, indices = hm.find(w["query_keys"])
-        keys_out, idx_out = hm.items()
+        keys_out, idx_out, values_out = hm.items(return_indices=True, return_values=True)
         return masks, keys_out
 
     for _ in range(args.warmup):
@@ -486,15 +519,23 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         loss = (feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
         loss.backward()
 
-    for _ in range(2):
-        train_step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        train_step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / reps * 1e3
-    out["cfg4_module_train_step"] = {"ms": round(ms, 3), "Mqueries_per_s": round(n4 / ms / 1e3, 1)}
+    # as shipped every backward node fills a dense gradient of its own (the
+    # reference's behaviour); ash.grid_query.SHARE_DENSE_GRADIENT lets the nodes
+    # of one pass share one
+    step_ms = {}
+    for label, share in (("", False), ("_shared_gradient", True)):
+        ash.grid_query.SHARE_DENSE_GRADIENT = share
+        for _ in range(2):
+            train_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            train_step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / reps * 1e3
+        out["cfg4_module_train_step" + label] = {
+            "ms": round(ms, 3), "Mqueries_per_s": round(n4 / ms / 1e3, 1)}
+    ash.grid_query.SHARE_DENSE_GRADIENT = False
     if not args.no_cpu:
         # The CPU baseline runs after every section that is timed with the wall
         # clock: its OpenMP workers keep spinning for a while after a parallel
@@ -503,7 +544,7 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     return out
 
 
-def bench_fusion(torch, ash, workloads, args, dev, frames=20):
+def bench_fusion(torch, ash, workloads, args, dev, frames=100):
     """Configuration 5 (secondary figure): depth frames of the synthetic scene
     fused into an unbounded grid, once with the library's fused activation and
     integration kernels and once in the reference's formulation (candidate
@@ -546,13 +587,15 @@ def bench_fusion(torch, ash, workloads, args, dev, frames=20):
 
 
 def cpu_baseline(torch, workloads, args):
-    """The oracle (OpenMP) on a bounded sample of configuration 2: same
-    generator, `--cpu-keys` distinct keys, capacity 1.5x, insert + find + items."""
+    """The oracle (OpenMP) on configuration 2 itself (same generator, the same
+    keys, capacity, queries and value rows as the device run; `--cpu-keys`
+    picks a smaller sample with capacity 1.5x): insert + find + items with the
+    value rows gathered, as in the device step."""
     import ash_oracle
 
     oracle = ash_oracle.OracleBackend()
-    n = args.cpu_keys
-    cap = n * 3 // 2
+    n = args.cpu_keys or args.keys
+    cap = n * 3 // 2 if args.cpu_keys else args.capacity
     w = workloads.hashmap_sphere_voxels(num_keys=n, device="cpu")
     heap = torch.arange(cap, dtype=torch.int32)
     omap = oracle.HashMap(3, cap, heap)
@@ -566,7 +609,8 @@ def cpu_baseline(torch, workloads, args):
         t1 = time.perf_counter()
         omap.find(w["query_keys"])
         t2 = time.perf_counter()
-        omap.items()
+        _, idx = omap.items()
+        gathered = {name: rows[idx] for name, rows in stores.items()}
         t3 = time.perf_counter()
         if best is None or t3 - t0 < best[0]:
             best = (t3 - t0, t1 - t0, t2 - t1, t3 - t2)
@@ -576,11 +620,12 @@ def cpu_baseline(torch, workloads, args):
         "unit": "Mkeys/s",
         "cores": oracle.num_threads(),
         "kind": "port",
-        "sample": f"configuration 2 generator at {n} keys, capacity {cap}: insert+find+items, best of 2",
+        "sample": f"configuration 2 at {n} keys, capacity {cap}: insert + find + items with "
+                  "values, best of 2",
         "insert_Mkeys_per_s": round(n / t_ins / 1e6, 2),
         "find_Mkeys_per_s": round(n / t_find / 1e6, 2),
     }
-    del omap, stores, values, w
+    del omap, stores, values, w, gathered
 
     # configuration 1 at full size (HashSet, 1 M inserts with 50 % duplicates
     # into capacity 2 M, 1 M finds), all threads and one thread

@@ -1,13 +1,23 @@
-// Memory-system probes of libash_hip.so.  The hash kernels are bound by how
-// many random 128-byte lines per second the device can read or update, not by
-// streaming bandwidth; these kernels measure those ceilings on the device at
-// hand so that a benchmark can price the table kernels against them.
-#include "ash_dev.h"
+// Memory-system probes of bench.py (built into bench_probes.so by
+// bench.py's build_probes(); not part of libash_hip.so or its C ABI).  The hash
+// kernels are bound by how many random 128-byte lines per second the device
+// can read or update, not by streaming bandwidth; these kernels measure those
+// ceilings on the device at hand so that the benchmark can price the table
+// kernels against them.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-#include "../../include/ash_hip.h"
+#include <string>
 
-namespace ash {
 namespace {
+
+std::string g_error;
+
+#define PROBE_FAIL(msg)   \
+    do {                  \
+        g_error = (msg);  \
+        return 1;         \
+    } while (0)
 
 constexpr int kBlock = 256;
 
@@ -87,22 +97,30 @@ __global__ __launch_bounds__(kBlock) void probe_line_updates(
 }
 
 }  // namespace
-}  // namespace ash
 
-using namespace ash;
+extern "C" const char* bench_probe_last_error(void) { return g_error.c_str(); }
 
-extern "C" int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes,
+// `buf` is a 128-byte aligned device buffer of `buf_bytes` bytes treated as
+// 128-byte lines; `n` (a multiple of 256) pseudo-random lines are touched and
+// `sink` (uint32[n]) receives values that keep the accesses alive.  The caller
+// times the call.
+//   mode 0: every line is read in full by 8 lanes x 16 bytes (a table probe);
+//   mode 1: per line one 64-bit read, one 64-bit compare-and-swap and one
+//           32-bit store (the accesses of an insert); modifies `buf`;
+//   mode 2: `n` pseudo-random aligned 64-byte halves of lines, each read by 4
+//           lanes x 16 bytes (what a table of 64-byte buckets would fetch).
+extern "C" int bench_probe_random_lines(int mode, void* buf, int64_t buf_bytes,
                                      int64_t n, uint32_t* sink, uint64_t seed,
                                      void* stream) {
-    if (buf == nullptr || sink == nullptr) ASH_FAIL("null buffer");
+    if (buf == nullptr || sink == nullptr) PROBE_FAIL("null buffer");
     if (buf_bytes < 128 || buf_bytes / 128 > 0xFFFFFFFFll) {
-        ASH_FAIL("buffer must hold between 1 and 2^32-1 lines of 128 bytes");
+        PROBE_FAIL("buffer must hold between 1 and 2^32-1 lines of 128 bytes");
     }
     if (n <= 0 || n % kBlock != 0 || n > (int64_t{1} << 31)) {
-        ASH_FAIL("n must be a positive multiple of 256 below 2^31");
+        PROBE_FAIL("n must be a positive multiple of 256 below 2^31");
     }
     if (reinterpret_cast<uintptr_t>(buf) % 128 != 0) {
-        ASH_FAIL("buffer must be 128-byte aligned");
+        PROBE_FAIL("buffer must be 128-byte aligned");
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t nlines = static_cast<uint32_t>(buf_bytes / 128);
@@ -117,8 +135,9 @@ extern "C" int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes,
         probe_half_line_reads<<<g, kBlock, 0, s>>>(static_cast<const uint4*>(buf),
                                                    nlines, n, sink, seed);
     } else {
-        ASH_FAIL("unknown probe mode");
+        PROBE_FAIL("unknown probe mode");
     }
-    ASH_LAUNCH_CHECK();
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) PROBE_FAIL(hipGetErrorString(e));
     return 0;
 }

@@ -21,7 +21,12 @@
  *   - launches are asynchronous on `stream`; only `ash_map_status` /
  *     `ash_map_size` (which return host values) synchronise that stream;
  *   - a map handle is not thread-safe; operations on one handle must be issued
- *     in order on one stream (as the reference issues them on the null stream).
+ *     in order on one stream (as the reference issues them on the null stream);
+ *   - calls on a map run on the map's device (ash_map_create's `device`); the
+ *     calls that take tensors but no map (queries, convolution, surface
+ *     extraction, depth integration) run on the device that holds their first
+ *     tensor argument.  Either way the caller's current device is restored on
+ *     return, and `stream` must belong to the device the call runs on.
  */
 #ifndef ASH_HIP_H_
 #define ASH_HIP_H_
@@ -157,7 +162,7 @@ int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* bl
  * int64[n_blocks] rows of it, grid_coords int32[n_blocks,3]; intrinsic 3x3 and
  * extrinsic 4x4 row-major fp32 ON THE DEVICE; origin: host float[3] or NULL;
  * depth fp32[height,width] (0 = no reading), color fp32[height,width,3] or
- * NULL.  Runs on the current device. */
+ * NULL. */
 int ash_grid_integrate_depth(float* embeddings, int64_t num_embeddings,
                              int grid_dim, int embedding_dim,
                              const int64_t* grid_indices,
@@ -511,21 +516,6 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
                                uint32_t* edge_slots, int32_t* workspace, int64_t n_vertices,
                                int64_t n_triangles, float* positions, int32_t* triangles,
                                void* stream);
-
-/* -------------------------------------------------------------- diagnostics */
-
-/* Measures the device's random-access ceilings that bound the table kernels
- * (no counterpart in the reference).  `buf` is a 128-byte aligned device
- * buffer of `buf_bytes` bytes treated as 128-byte lines; `n` (a multiple of
- * 256) pseudo-random lines are touched and `sink` (uint32[n]) receives values
- * that keep the accesses alive.  The caller times the call.
- *   mode 0: every line is read in full by 8 lanes x 16 bytes (a table probe);
- *   mode 1: per line one 64-bit read, one 64-bit compare-and-swap and one
- *           32-bit store (the accesses of an insert); modifies `buf`;
- *   mode 2: `n` pseudo-random aligned 64-byte halves of lines, each read by 4
- *           lanes x 16 bytes (what a table of 64-byte buckets would fetch). */
-int ash_diag_random_lines(int mode, void* buf, int64_t buf_bytes, int64_t n,
-                          uint32_t* sink, uint64_t seed, void* stream);
 
 #ifdef __cplusplus
 }

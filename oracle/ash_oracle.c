@@ -579,6 +579,85 @@ int64_t ash_oracle_map_load(ash_oracle_map* m, const int32_t* keys,
 DEFINE_QUERY(float, f32)
 DEFINE_QUERY(double, f64)
 
+/* Magnitudes behind the three query functions, for error bounds in the tests:
+ * for every output element the sum of the ABSOLUTE values of the terms that
+ * the kernels above add up to form it, in double.  A sum of n fp32 terms
+ * evaluated in any order differs from the exact sum by at most about
+ * n * 2^-24 * (sum of |terms|), so these are what a tolerance for sums that two
+ * implementations accumulate in different orders has to scale with.  Same
+ * addressing, early-outs and weights as the kernels (ash/src/grid.cu:68-132,
+ * :177-255, :309-387); not a restatement of anything in the reference.
+ *   sum_forward[i,k]      = sum_c w_c |emb_c[k]|
+ *   sum_bf_emb[row,k]     = sum_i w_c |z[i,k]|              (row = corner c of query i)
+ *   sum_bf_off[i,d]       = sum_c |dw_c/do_d| sum_k |emb_c[k] z[i,k]|
+ *   sum_bb_z[i,k]         = sum_c (sum_d |dw_c/do_d u[i,d]|) |emb_c[k]|
+ *   sum_bb_emb[row,k]     = sum_i (sum_d |dw_c/do_d u[i,d]|) |z[i,k]|
+ * Any output may be NULL; z / u may be NULL when no output needs them. */
+void ash_oracle_query_term_sums(
+        const double* u, const double* z, const double* embeddings,
+        const float* offsets, const int64_t* grid_indices,
+        const int64_t* cell_indices, const uint8_t* masks,
+        const int64_t* lut_grid_nb2grid_idx, const int64_t* lut_cell_nb2cell_idx,
+        const int64_t* lut_cell_nb2grid_nb, double* sum_forward, double* sum_bf_emb,
+        double* sum_bf_off, double* sum_bb_z, double* sum_bb_emb, int64_t len,
+        int64_t num_embeddings, int64_t cells_per_grid, int64_t embedding_dims,
+        int kind) {
+    const size_t dense = (size_t)(num_embeddings * cells_per_grid * embedding_dims);
+    if (sum_forward) memset(sum_forward, 0, (size_t)(len * embedding_dims) * sizeof(double));
+    if (sum_bf_emb) memset(sum_bf_emb, 0, dense * sizeof(double));
+    if (sum_bf_off) memset(sum_bf_off, 0, (size_t)(len * 3) * sizeof(double));
+    if (sum_bb_z) memset(sum_bb_z, 0, (size_t)(len * embedding_dims) * sizeof(double));
+    if (sum_bb_emb) memset(sum_bb_emb, 0, dense * sizeof(double));
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < len; ++i) {
+        if (!masks[i]) continue;
+        const float* offset = offsets + i * 3;
+        const int64_t* nb_g2g = lut_grid_nb2grid_idx + grid_indices[i] * 8;
+        const int64_t* nb_c2c = lut_cell_nb2cell_idx + cell_indices[i] * 8;
+        const int64_t* nb_c2g = lut_cell_nb2grid_nb + cell_indices[i] * 8;
+        int complete = 1;
+        for (int c = 0; c < 8; ++c) {
+            if (nb_g2g[nb_c2g[c]] == -1) complete = 0;
+        }
+        if (!complete) continue;
+        for (int c = 0; c < 8; ++c) {
+            double w = 1.0, wg[3] = {1, 1, 1};
+            for (int d = 0; d < 3; ++d) {
+                double x = ((c >> d) & 1) ? (double)offset[d] : (double)(1 - offset[d]);
+                double f = interp_f64(x, kind);
+                double df = fabs(diff_interp_f64(x, kind));
+                w *= f;
+                for (int e = 0; e < 3; ++e) wg[e] *= (e == d) ? df : f;
+            }
+            w = fabs(w);
+            double du = 0;
+            if (u) {
+                for (int d = 0; d < 3; ++d) du += fabs(wg[d] * u[i * 3 + d]);
+            }
+            const int64_t base = (nb_g2g[nb_c2g[c]] * cells_per_grid + nb_c2c[c]) * embedding_dims;
+            double dot = 0;
+            for (int64_t k = 0; k < embedding_dims; ++k) {
+                const double e_k = fabs(embeddings[base + k]);
+                const double z_k = z ? fabs(z[i * embedding_dims + k]) : 0.0;
+                if (sum_forward) sum_forward[i * embedding_dims + k] += w * e_k;
+                if (sum_bf_emb) {
+#pragma omp atomic
+                    sum_bf_emb[base + k] += w * z_k;
+                }
+                dot += e_k * z_k;
+                if (sum_bb_z) sum_bb_z[i * embedding_dims + k] += du * e_k;
+                if (sum_bb_emb) {
+#pragma omp atomic
+                    sum_bb_emb[base + k] += du * z_k;
+                }
+            }
+            if (sum_bf_off) {
+                for (int d = 0; d < 3; ++d) sum_bf_off[i * 3 + d] += wg[d] * dot;
+            }
+        }
+    }
+}
+
 /* ------------------------------------------------------- iso-surface points
  * ash/src/grid.cu:453-531, cells in launch order.  Returns the number of
  * points; positions (may be NULL) receives them in that order. */

@@ -77,6 +77,7 @@ def load(build_if_missing: bool = True) -> ctypes.CDLL:
         getattr(lib, f"ash_oracle_query_backward_backward_{sfx}").argtypes = (
             [_PTR] * 12 + [_I64, _I64, _I64, _I64, ctypes.c_int]
         )
+    lib.ash_oracle_query_term_sums.argtypes = [_PTR] * 15 + [_I64] * 4 + [ctypes.c_int]
     return lib
 
 
@@ -312,6 +313,41 @@ class OracleBackend:
             grad_emb if need_embeddings else None,
             torch.zeros((n, 3), dtype=emb.dtype),
         )
+
+
+    def query_term_sums(
+        self, grad_grad_offsets, z, embeddings, offsets, grid_indices, cell_indices, masks,
+        lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb, grid_dim, interpolation,
+        dense: bool = True,
+    ) -> Dict[str, torch.Tensor]:
+        """Per output element of the three query functions, the sum of the
+        absolute values of the terms that form it (float64): what a bound on
+        the rounding of sums accumulated in another order scales with.  Keys:
+        forward, bf_embeddings, bf_offsets, bb_z, bb_embeddings (the two dense
+        ones only with `dense`)."""
+        held = self._tables(
+            embeddings, offsets, grid_indices, cell_indices, masks,
+            lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb,
+        )
+        held[0] = held[0].double()
+        emb = held[0]
+        n = held[2].shape[0]
+        b, m, e = emb.shape
+        z = _cpu(z, torch.float64)
+        u = _cpu(grad_grad_offsets, torch.float64)
+        out = {
+            "forward": torch.empty((n, e), dtype=torch.float64),
+            "bf_embeddings": torch.empty_like(emb) if dense else None,
+            "bf_offsets": torch.empty((n, 3), dtype=torch.float64),
+            "bb_z": torch.empty((n, e), dtype=torch.float64),
+            "bb_embeddings": torch.empty_like(emb) if dense else None,
+        }
+        self.lib.ash_oracle_query_term_sums(
+            u.data_ptr(), z.data_ptr(), *[t.data_ptr() for t in held],
+            *[(t.data_ptr() if t is not None else None) for t in out.values()],
+            n, b, m, e, _INTERP[interpolation],
+        )
+        return {k: v for k, v in out.items() if v is not None}
 
 
 class _OracleHashMap:

@@ -37,6 +37,60 @@ def torch_query(
     return y * ok.unsqueeze(-1).to(dtype)
 
 
+def torch_term_sums(embeddings, offsets, grid_indices, cell_indices, masks, lut_g, lut_c2c,
+                    lut_c2g, interpolation, z, u):
+    """Sum of |terms| behind every output element of the three query functions
+    (float64, vectorised): an independent statement of what the oracle's
+    query_term_sums computes."""
+    emb = embeddings.double()
+    n = grid_indices.shape[0]
+    nbn = lut_c2g[cell_indices]
+    g = torch.gather(lut_g[grid_indices], 1, nbn)
+    cell = lut_c2c[cell_indices]
+    ok = (masks & (g >= 0).all(dim=1)).double()
+    corner = torch.arange(8)
+    bits = torch.stack([(corner >> d) & 1 for d in range(3)], dim=1).to(torch.bool)
+    x = torch.where(bits.unsqueeze(0), offsets.unsqueeze(1), (1.0 - offsets).unsqueeze(1)).double()
+    f = basis(x, interpolation)                                           # (N, 8, 3)
+    df = (6 * x * (1 - x)).abs() if interpolation == "smooth_step" else torch.ones_like(x)
+    w = f.prod(dim=2).abs() * ok.unsqueeze(1)                             # (N, 8)
+    wg = torch.stack([df[..., d] * f[..., [e for e in range(3) if e != d]].prod(dim=2)
+                      for d in range(3)], dim=2).abs() * ok.view(-1, 1, 1)  # (N, 8, 3)
+    rows = emb[g.clamp(min=0), cell].abs()                                # (N, 8, E)
+    za, ua = z.double().abs(), u.double().abs()
+    du = (wg * ua.unsqueeze(1)).sum(dim=2)                                # (N, 8)
+    flat = (g.clamp(min=0) * emb.shape[1] + cell).view(-1)
+    dense = lambda t: torch.zeros(emb.shape[0] * emb.shape[1], emb.shape[2], dtype=torch.float64
+                                  ).index_add_(0, flat, t.reshape(n * 8, -1)).view(emb.shape)
+    return {
+        "forward": (w.unsqueeze(-1) * rows).sum(dim=1),
+        "bf_embeddings": dense(w.unsqueeze(-1) * za.unsqueeze(1)),
+        "bf_offsets": (wg * (rows * za.unsqueeze(1)).sum(dim=2, keepdim=True)).sum(dim=1),
+        "bb_z": (du.unsqueeze(-1) * rows).sum(dim=1),
+        "bb_embeddings": dense(du.unsqueeze(-1) * za.unsqueeze(1)),
+    }
+
+
+# Bound on the difference between two evaluations of a sum of fp terms in
+# different orders: K_ROUND * eps * sum|terms| on top of the stated tolerance.
+# Each side rounds every term (a product of up to five factors: ~5 eps) and
+# every partial sum (a tree or a chain of additions: ~log2(n)..n eps, sqrt(n)
+# eps typically); 16 eps covers both sides for the sums met here (up to a few
+# thousand terms per element) and is what the tests state.
+K_ROUND = 16.0
+
+
+def assert_close_sums(got, ref, term_sums, rtol, atol, eps, what=""):
+    """|got - ref| <= rtol |ref| + atol + K_ROUND eps sum|terms|, elementwise."""
+    got, ref = got.detach().cpu().double(), ref.detach().cpu().double()
+    bound = rtol * ref.abs() + atol + K_ROUND * eps * term_sums
+    excess = (got - ref).abs() - bound
+    worst = int(excess.argmax())
+    assert float(excess.view(-1)[worst]) <= 0, (
+        f"{what}: |diff| {float((got - ref).abs().view(-1)[worst]):.3e} exceeds the bound "
+        f"{float(bound.view(-1)[worst]):.3e} (sum|terms| {float(term_sums.reshape(-1)[worst]):.3e})")
+
+
 class DictMap:
     """Sequential dictionary model of the map with the reference's heap
     protocol (ash/src/hashmap_gpu.cuh:211-232,316-336)."""

@@ -163,22 +163,28 @@ def test_integrate_depth_equals_torch_expressions(gpu_ash, with_color, bounded):
         assert int((~close_rgb & same).sum()) < 2e-3 * n_cells
 
 
-def test_fused_fusion_against_oracle_harness(gpu_ash, oracle, monkeypatch):
-    """Configuration 5 at reduced size: the fused step on the device against the
-    reference's formulation run on the CPU with the oracle as backend."""
+@pytest.mark.parametrize("width,height,poses,capacity",
+                         [(160, 120, (0, 10, 20), 20_000), (640, 480, (0, 33, 66), 80_000)])
+def test_fused_fusion_against_oracle_harness(gpu_ash, oracle, monkeypatch, width, height, poses,
+                                             capacity):
+    """Configuration 5, at reduced size and at its full frame size (640 x 480
+    depth frames, 307 200 positions and 8.3 M candidate keys per frame,
+    capacity 80 000 as in the reference's demo): the fused step on the device
+    against the reference's formulation run on the CPU with the oracle as
+    backend."""
     import ash.core
     import ash.grid
     import ash.grid_query
 
-    scene = workloads.FusionScene(width=160, height=120)
+    scene = workloads.FusionScene(width=width, height=height)
     frames = []
-    for f in (0, 10, 20):
+    for f in poses:
         ext = scene.pose(f)
         depth = scene.depth(ext)
         frames.append((scene.unproject(depth, ext), depth, ext))
 
     def run(device, fused):
-        grid = gpu_ash.UnBoundedSparseDenseGrid(3, 20000, 2, 8, cell_size=0.015, device=device)
+        grid = gpu_ash.UnBoundedSparseDenseGrid(3, capacity, 2, 8, cell_size=0.015, device=device)
         touched = [
             workloads.fuse_frame(grid, p.to(device), d.to(device), scene.intrinsic.to(device),
                                  e.to(device), trunc=0.04, fused=fused)
@@ -195,9 +201,17 @@ def test_fused_fusion_against_oracle_harness(gpu_ash, oracle, monkeypatch):
         touched_cpu, keys_cpu, cells_cpu = run(torch.device("cpu"), False)
     assert touched_gpu == touched_cpu and len(keys_gpu) > 5000
     assert torch.equal(keys_gpu, keys_cpu)
+    # A cell whose projection falls on a pixel boundary (x.5) may read the
+    # neighbouring pixel on the other side (fused multiply-adds against torch's
+    # matrix products): its weight flips when one of the two pixels has no
+    # valid reading, its distance changes when both have.  Their fraction is
+    # bounded; every other cell agrees to fp32 rounding.
     same = cells_gpu[..., 1] == cells_cpu[..., 1]
-    assert float((~same).float().mean()) < 5e-4
-    assert torch.allclose(cells_gpu[..., 0][same], cells_cpu[..., 0][same], rtol=1e-3, atol=2e-4)
+    flipped = float((~same).float().mean())
+    assert flipped < 5e-4, flipped
+    close = torch.isclose(cells_gpu[..., 0], cells_cpu[..., 0], rtol=1e-3, atol=2e-4)
+    other_pixel = float((same & ~close).float().mean())
+    assert other_pixel < 5e-4, other_pixel
     assert float(cells_gpu[..., 1].sum()) > 1e5
 
 

@@ -105,6 +105,27 @@ def test_engine_state_dict_round_trip(gpu_ash, dim, num, tmp_path):
         assert_is_bijection_into(engine.items()[1], capacity)
 
 
+def test_state_with_duplicate_keys_is_refused(gpu_ash):
+    """A saved state whose active keys repeat a key (the reference prints
+    "should never reach here", ash/src/hashmap_gpu.cuh:420-422, and goes on
+    with a heap counter that exceeds the stored entries) is refused and leaves
+    the map empty and usable."""
+    capacity = 5000
+    engine = gpu_ash.ASHEngine(3, capacity, DEV)
+    keys = _tiled_keys(3, 3000, seed=77)
+    engine.insert_keys(keys)
+    state = {k: v.clone() for k, v in engine.state_dict().items()}
+    state["_keys"][10] = state["_keys"][20]
+    other = gpu_ash.ASHEngine(3, capacity, DEV)
+    with pytest.raises(RuntimeError, match="duplicate keys"):
+        other.load_state_dict(state)
+    assert other.size() == 0 and other.items()[0].shape[0] == 0
+    other.insert_keys(keys[:100])
+    idx, mask = other.find(keys[:200])
+    assert int(mask.sum()) == 100 and other.size() == 100
+    assert torch.equal(torch.sort(idx[:100])[0].cpu(), torch.arange(100))
+
+
 @pytest.mark.parametrize(
     "dim,num,old,new", [(1, 50000, 100000, 50000), (1, 100000, 100000, 200000),
                         (3, 50000, 100000, 50000), (3, 100000, 100000, 200000)]

@@ -245,7 +245,13 @@ def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
     the first node's gradient instead of producing a dense tensor of its own,
     and the result is what separate passes give -- also with another user of
     the embeddings in the loss, on a second pass into an existing .grad, and
-    not at all while a graph of the backward is being recorded."""
+    not at all while a graph of the backward is being recorded.  That is with
+    ash.grid_query.SHARE_DENSE_GRADIENT switched on; as shipped (off) every
+    node produces its own dense gradient, as in the reference, which is also
+    right when a hook keeps a node's gradients while a third contribution
+    arrives (the case the switch cannot see and is off for)."""
+    import ash.grid_query as gq
+
     torch.manual_seed(7)
     g_dim = 2
     grid = cpu_ash.SparseDenseGrid(3, 8, 3, g_dim, device=CPU)
@@ -280,13 +286,34 @@ def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
             total += grid.embeddings.grad
         return total
 
+    assert gq.SHARE_DENSE_GRADIENT is False          # as shipped
+    expected = separate()
+    grid.embeddings.grad = None
+    value, eikonal = losses(x.clone().requires_grad_(True))
+    (value + eikonal).backward()
+    assert shared_calls == [] and gq.LAST_GRADIENT_PATH == "own"
+    assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
+    # a hook that keeps the gradients of the query node + a third contribution
+    kept = []
+    grid.embeddings.grad = None
+    xq = x.clone().requires_grad_(True)
+    feats, _ = grid(xq, "smooth_step")
+    feats.grad_fn.register_hook(lambda grad_inputs, grad_outputs: kept.append(grad_inputs))
+    (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+    ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
+     + 0.5 * (grid.embeddings ** 2).sum()).backward()
+    assert shared_calls == [] and len(kept) >= 1
+    assert torch.allclose(grid.embeddings.grad, expected + grid.embeddings.detach(),
+                          rtol=1e-5, atol=1e-6)
+
+    monkeypatch.setattr(gq, "SHARE_DENSE_GRADIENT", True)
     expected = separate()
     assert shared_calls == []          # one producer per pass: nothing to share
 
     grid.embeddings.grad = None
     value, eikonal = losses(x.clone().requires_grad_(True))
     (value + eikonal).backward()
-    assert len(shared_calls) == 1
+    assert len(shared_calls) == 1 and gq.LAST_GRADIENT_PATH == "shared"
     assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
 
     # a second pass adds to the existing .grad
@@ -322,6 +349,19 @@ def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
     (a.sum() + 2 * b.sum()).backward()
     assert len(shared_calls) == before
     assert torch.allclose(alias.grad, 2 * grid.embeddings.grad)
+
+    # a consumer that is not the accumulation node of a leaf is never shared with
+    scaled = grid.embeddings * 1.0
+    gi, ci, off, masks = grid.query(x)
+    xq = x.clone().requires_grad_(True)
+    gi, ci, off, masks = grid.query(xq)
+    feats = cpu_ash.SparseDenseGridQuery.apply(scaled, off, gi, ci, masks, *tables, "smooth_step")
+    (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+    grid.embeddings.grad = None
+    before = len(shared_calls)
+    ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()).backward()
+    assert len(shared_calls) == before and gq.LAST_GRADIENT_PATH == "own"
+    assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
 
 
 # ---------------------------------------------- engine / set / map / embedding

@@ -15,7 +15,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import torch_query
+from helpers import torch_query, torch_term_sums
 
 
 def _dense_grid(ash, grid_dim, embedding_dim, bound, dtype=torch.float32, seed=0):
@@ -194,3 +194,23 @@ def test_finite_differences_of_forward(cpu_ash, oracle):
             ym = oracle.query_forward(*minus, 4, interpolation)
             fd = ((yp - ym) * z).sum(dim=1) / (plus[1][:, d] - minus[1][:, d]).double()
             assert torch.allclose(go[:, d], fd, rtol=1e-3, atol=1e-4)
+
+
+@pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
+def test_term_sums_equal_an_independent_formula(cpu_ash, oracle, interpolation):
+    """The magnitudes that the GPU tests scale their rounding bound with
+    (sum of |terms| per output element) against a vectorised torch statement,
+    with masked-out queries and missing neighbour blocks in the batch."""
+    grid = _dense_grid(cpu_ash, 4, 3, 1, seed=9)
+    x = _queries(4, 1, 1500, seed=10) + 2.5          # some queries leave the populated blocks
+    ops = _operands(grid, x)
+    g = torch.Generator().manual_seed(11)
+    z = torch.rand(1500, 3, generator=g) - 0.5
+    u = torch.rand(1500, 3, generator=g) - 0.5
+    got = oracle.query_term_sums(u, z, *ops, 4, interpolation)
+    ref = torch_term_sums(*ops, interpolation, z, u)
+    assert set(got) == set(ref)
+    for name in ref:
+        assert torch.allclose(got[name], ref[name], rtol=1e-12, atol=1e-14), name
+        assert float(ref[name].sum()) > 1.0
+    assert 0.2 < float(ops[4].float().mean()) < 0.99

@@ -149,10 +149,6 @@ _SIGNATURES = {
     "ash_map_should_rebuild": (ctypes.c_int, [_PTR, _I64, _I64, _I64]),
     "ash_map_rebuild": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_scatter_rows": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _I64, _PTR]),
-    "ash_diag_random_lines": (
-        ctypes.c_int,
-        [ctypes.c_int, _PTR, _I64, _I64, _PTR, ctypes.c_uint64, _PTR],
-    ),
     "ash_isosurface_workspace_ints": (ctypes.c_int64, [_I64, _I64]),
     "ash_isosurface_classify": (
         ctypes.c_int,
@@ -1238,7 +1234,14 @@ class _HashMap:
                 break
         dup = self.status()["load_duplicates"]
         if dup:
-            warnings.warn(f"load_states met {dup} duplicate keys; they were stored once")
+            # The reference prints "Error loading, should never reach here!"
+            # (ash/src/hashmap_gpu.cuh:420-422) and goes on with a heap counter
+            # that no longer matches the stored entries.  Here such a state is
+            # refused: the map is left empty.
+            self.clear()
+            raise RuntimeError(
+                f"load_states: active_keys holds {dup} duplicate keys; nothing was loaded"
+            )
 
 
 class _MissingBackend:

@@ -3,6 +3,7 @@ backward.  Two chained Functions with the same operands and return
 conventions as the reference (ash/grid_query.py:10-283); each one is a single
 call into the HIP library.
 """
+import os
 import weakref
 from typing import Literal
 
@@ -16,23 +17,41 @@ _N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
 
 # One backward pass can reach the same embeddings through several nodes: a
 # training step with a value loss and a gradient-norm loss runs both the first-
-# and the second-order backward, and each would zero-fill a dense gradient of the
-# whole parameter and leave the sum of the two to autograd (two fills and an add
-# over the parameter: about a third of such a step).  Instead, the first node of
-# a pass that produces the gradient for a consumer (graph node, input number)
-# leaves a note with that consumer -- the graph task and a weak reference to the
-# tensor, in the node's own metadata dictionary, so that the note lives and dies
-# with the node -- and a later node of the same pass adds its contribution to
-# that tensor in place and returns no gradient of its own.
-# Only passes without create_graph share (an in-place change would be invisible
-# to a graph recorded over the first gradient); the tensor is only referenced
-# weakly, so autograd can still adopt it as .grad without a copy, and a tensor
-# that autograd has already replaced by a sum is gone and not written to.
+# and the second-order backward, and each zero-fills a dense gradient of the
+# whole parameter and leaves the sum of the two to autograd (two fills and an
+# add over the parameter: about a third of such a step), as in the reference.
+#
+# SHARE_DENSE_GRADIENT (off unless the caller switches it on, here or with
+# ASH_SHARE_DENSE_GRADIENT=1) saves the second fill and the add: the first node
+# of a pass that produces the gradient for a leaf parameter leaves a note with
+# the parameter's accumulation node -- the graph task, the stream and a weak
+# reference to the tensor, in the node's own metadata dictionary, so that the
+# note lives and dies with the node -- and a later node of the same pass adds its
+# contribution to that tensor in place and returns no gradient of its own.
+#
+# Why it is a switch: the in-place addition is only right while the tensor the
+# first node returned still is what the autograd engine holds for the
+# parameter.  The engine replaces it by a new tensor when a further gradient
+# for the same parameter arrives (a weight-decay term, say) while something
+# else still refers to the first one -- a hook on this function's grad_fn that
+# keeps its grad_inputs is enough -- and this code cannot see that; the later
+# contribution would then be lost.  Without such references the engine adds
+# in place (or autograd drops the tensor and the weak reference dies, and the
+# node falls back to a gradient of its own).  So: switch it on for training
+# loops that keep no references to intermediate gradients.
+#
+# Shared only: with the switch on, without create_graph (an in-place change
+# would be invisible to a graph recorded over the first gradient), towards the
+# accumulation node of a leaf, by nodes that run on the same stream.
 _NOTE = "ash_shared_gradient"
+SHARE_DENSE_GRADIENT = os.environ.get("ASH_SHARE_DENSE_GRADIENT", "0") not in ("", "0")
+# which way the embedding gradient of the latest backward node went: "own"
+# (a dense tensor of its own), "shared" (added to another node's), "skipped"
+LAST_GRADIENT_PATH = None
 
 
 def _pass_id() -> int:
-    if torch.is_grad_enabled():
+    if not SHARE_DENSE_GRADIENT or torch.is_grad_enabled():
         return -1
     try:
         return torch._C._current_graph_task_id()
@@ -45,10 +64,19 @@ def _notes(consumer):
     task = _pass_id()
     if task < 0 or consumer is None or consumer[0] is None:
         return None
+    node = consumer[0]
+    # only the accumulation node of a leaf: what it receives is added to .grad
+    # and goes nowhere else
+    if type(node).__name__ != "AccumulateGrad":
+        return None
     try:
-        return task, consumer[0].metadata, (_NOTE, consumer[1])
+        return task, node.metadata, (_NOTE, consumer[1])
     except Exception:  # a node without metadata
         return None
+
+
+def _stream_id(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream if t.is_cuda else 0
 
 
 def _shared_gradient(consumer):
@@ -61,7 +89,10 @@ def _shared_gradient(consumer):
     entry = where.get(key)
     if entry is None or entry[0] != task:
         return None
-    return entry[1]()
+    gradient = entry[2]()
+    if gradient is None or entry[1] != _stream_id(gradient):
+        return None
+    return gradient
 
 
 def _share_gradient(consumer, gradient) -> None:
@@ -69,7 +100,12 @@ def _share_gradient(consumer, gradient) -> None:
     if notes is None or gradient is None:
         return
     task, where, key = notes
-    where[key] = (task, weakref.ref(gradient))
+    where[key] = (task, _stream_id(gradient), weakref.ref(gradient))
+
+
+def _record_path(path: str) -> None:
+    global LAST_GRADIENT_PATH
+    LAST_GRADIENT_PATH = path
 
 
 def _grad_requested(ctx, index: int) -> bool:
@@ -138,6 +174,7 @@ class SparseDenseGridQuery(torch.autograd.Function):
         # autograd.grad(y, x, create_graph=True).
         consumer = ctx.next_functions[0] if need_embeddings else None
         shared = _shared_gradient(consumer)
+        _record_path("shared" if shared is not None else "own" if need_embeddings else "skipped")
         if shared is not None:
             # no graph is being recorded: the library is called directly
             _, grad_offsets = backend.query_backward_forward(
@@ -232,6 +269,7 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
             return (None, None) + (None,) * n_rest
         consumer = ctx.next_functions[1] if need_embeddings else None
         shared = _shared_gradient(consumer)
+        _record_path("shared" if shared is not None else "own" if need_embeddings else "skipped")
         if shared is not None:
             grad_z, _, _ = backend.query_backward_backward(
                 grad_grad_embeddings,

@@ -16,8 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "ash", "lib")
 OUT = os.path.join(OUT_DIR, "libash_hip.so")
-SOURCES = ["ash_map.hip", "ash_bulk.hip", "ash_query.hip", "ash_fusion.hip", "ash_mesh.hip",
-           "ash_diag.hip"]
+SOURCES = ["ash_map.hip", "ash_bulk.hip", "ash_query.hip", "ash_fusion.hip", "ash_mesh.hip"]
 HEADERS = [
     os.path.join(CSRC, "ash_dev.h"),
     os.path.join(CSRC, "ash_table.h"),

@@ -13,7 +13,7 @@
 // fp32 (no fused multiply-add), i.e. exactly like the elementwise torch
 // expressions; the projection uses fused multiply-adds where torch calls a
 // matrix product, whose rounding is not specified either.
-#include "ash_dev.h"
+#include "ash_table.h"
 
 #include "../../include/ash_hip.h"
 
@@ -150,6 +150,8 @@ extern "C" int ash_grid_integrate_depth(
     for (int d = 0; d < 3; ++d) a.origin[d] = origin ? origin[d] : 0.f;
     a.trunc = trunc;
     a.depth_max = depth_max;
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(embeddings));
     const int64_t threads = n_blocks * a.m;
     if (threads > (int64_t{1} << 40)) ASH_FAIL("too many cells in one call");
     const int64_t blocks = (threads + kBlock - 1) / kBlock;

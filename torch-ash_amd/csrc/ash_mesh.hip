@@ -28,7 +28,7 @@
 // A cell takes part when it and the seven cells at its other corners exist
 // and weigh at least the threshold; its case has bit c set when corner c is
 // below the iso value.
-#include "ash_dev.h"
+#include "ash_table.h"
 #include "ash_mc_table.h"
 
 #include "../../include/ash_hip.h"
@@ -1046,6 +1046,8 @@ int ash_marching_cubes_classify(const void* sdfs, const void* weights,
     if (num_grids > 0 && weights == nullptr) ASH_FAIL("null pointer in marching_cubes");
     a.weights = weights;
     a.weight_thr = weight_thr;
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(sdfs));
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cells = num_grids * cells_per_grid;
     const unsigned by_cell = chunk_grid((cells + kBlock - 1) / kBlock);
@@ -1120,6 +1122,8 @@ int ash_marching_cubes_extract(const void* sdfs, const int64_t* grid_indices,
     a.triangles = triangles;
     a.n_vertices = n_vertices;
     a.n_triangles = n_triangles;
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(sdfs));
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cells = num_grids * cells_per_grid;
     const unsigned by_chunk = chunk_grid((cells + kChunk - 1) / kChunk);
@@ -1170,6 +1174,8 @@ int ash_isosurface_classify(const void* sdfs, const void* weights, const int64_t
     if (num_grids > 0 && weights == nullptr) ASH_FAIL("null pointer in isosurface_classify");
     a.weights = weights;
     a.weight_thr = weight_thr;
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(sdfs));
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int64_t cells = num_grids * cells_per_grid;
     const int64_t chunks = (cells + kChunk - 1) / kChunk;
@@ -1235,6 +1241,8 @@ int ash_isosurface_points(const void* sdfs, const int64_t* grid_indices,
     a.grid_coords = grid_coords_table;
     a.positions = positions;
     a.n_vertices = n_points;
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(sdfs));
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned by_chunk = chunk_grid((num_grids * cells_per_grid + kChunk - 1) / kChunk);
     const bool vec = a.M % 4 == 0 && reinterpret_cast<uintptr_t>(flags) % 4 == 0;

@@ -112,6 +112,23 @@ struct DeviceGuard {
     }
 };
 
+// The entry points that take tensors but no map (queries, convolution, surface
+// extraction, depth integration) run on the device that holds their first
+// tensor: the runtime is asked where the pointer lives and that device is made
+// current for the call.  A pointer the runtime does not know leaves the
+// current device as it is.
+struct PointerGuard : DeviceGuard {
+    hipError_t enter_for(const void* p) {
+        if (p == nullptr) return hipSuccess;
+        hipPointerAttribute_t attr;
+        if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+            (void)hipGetLastError();
+            return hipSuccess;
+        }
+        if (attr.type != hipMemoryTypeDevice) return hipSuccess;
+        return enter(attr.device);
+    }
+};
 
 // Inserts the keys selected by `sel[0 .. *nsel)` (both on the device) with the
 // per-key atomic kernel.  `codes` false: `keys` are int32[.., key_dim] rows and
