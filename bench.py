@@ -85,15 +85,14 @@ MEASURED_TRAFFIC_BYTES = {
     "insert_values": 2_563_000_000 + 1_819_000_000,
     "insert_keys": 2_303_000_000 + 1_564_000_000,
     "find": 2_230_000_000 + 146_000_000,
-    "items": 512_000_000 + 324_000_000,
-    # sums over split_keys_kernel, split_records_kernel and build_kernel
-    "insert_values_bulk": 1_285_000_000 + 1_592_000_000,
-    "insert_keys_bulk": 515_000_000 + 786_000_000,
 }
 
 
-def items_bytes(slots: int, n: int) -> int:
-    return 16 * slots + 20 * n
+def items_bytes(scanned: int, n: int) -> int:
+    """items(): the key log is scanned (8 B per index, `scanned` indices: the
+    size while the heap is in its initial order, else the capacity), 12 B key +
+    8 B index written per live entry."""
+    return 8 * scanned + 20 * n
 
 
 def fwd_bytes(e: int) -> int:
@@ -287,13 +286,27 @@ def bench_hash(torch, ash, workloads, args, dev):
         run(t_erase, lambda: check(lib.ash_map_erase(handle, keys.data_ptr(), n, stream)))
     assert int(mask_out.sum()) == hits
     assert backend.status()["size"] == 0   # a fresh read: the launches above went past the shim
-    slots = (backend._table.numel() - 256) // 128 * 10
+    c_count = (ctypes.c_int64 * k)(args.capacity, args.capacity)
+    gathered = [torch.empty((n, 3), device=dev), torch.empty((n, 1), device=dev)]
+    c_out = (ctypes.c_void_p * k)(gathered[0].data_ptr(), gathered[1].data_ptr())
+    t_gather = EventTimer(torch)
+    for it in range(args.warmup + args.steps):
+        fn = lambda: check(lib.ash_gather_rows(k, c_dst, c_out, c_rows, c_count,
+                                               items_idx.data_ptr(), n, stream))
+        if it >= args.warmup:
+            t_gather(fn)
+        else:
+            fn()
     kernels = {
         "insert_values": roofline_entry(
             "insert_kernel<3,fused>", (INSERT_KEY_BYTES + VALUE_ROW_BYTES) * n, t_insert.mean_ms()),
         "insert_keys": roofline_entry("insert_kernel<3,keys>", INSERT_KEY_BYTES * n, t_insert_keys.mean_ms()),
         "find": roofline_entry("find_kernel<3>", FIND_BYTES * n, t_find.mean_ms()),
-        "items": roofline_entry("items_kernel<3>", items_bytes(slots, n), t_items.mean_ms()),
+        # the heap is in its initial order when items() runs here: n indices scanned
+        "items": roofline_entry("items_kernel<3>", items_bytes(n, n), t_items.mean_ms()),
+        # value rows of the enumerated entries: index in, 16 B read and written
+        "items_values": roofline_entry("gather_rows_kernel (color + depth by items() index)",
+                                       (8 + VALUE_ROW_BYTES) * n, t_gather.mean_ms()),
         # the heap array is rewritten only after an erase or a load wrote to it;
         # none did before the clear timed here
         "clear": roofline_entry("reset counters + deferred fill16 (+ a one-key find)",

@@ -326,6 +326,17 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
 int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
                      int64_t n, int64_t row_bytes, void* stream);
 
+/* The gather behind `HashMap.find(return_values=True)` /
+ * `HashMap.items(return_values=True)` (ash/hashmap.py:87-95,138-146: the
+ * reference indexes every value tensor with the returned indices, one torch
+ * launch per tensor): dst[v][i] = src[v][indices[i]] for up to four tensors in
+ * one launch.  Rows of tensor v are row_bytes[v] bytes (a multiple of 4), the
+ * source has src_rows[v] rows; an index outside the source gives a zero row.
+ * dst[v] holds n rows.  Runs on the device that holds `indices`. */
+int ash_gather_rows(int n_values, const void* const* src, void* const* dst,
+                    const int64_t* row_bytes, const int64_t* src_rows,
+                    const int64_t* indices, int64_t n, void* stream);
+
 /* -------------------------------------------------------- trilinear queries */
 
 enum { ASH_INTERP_LINEAR = 0, ASH_INTERP_SMOOTH_STEP = 1 };

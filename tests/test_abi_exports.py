@@ -44,11 +44,12 @@ def _error(lib):
 def test_workspace_sizes(lib):
     table, general = ctypes.c_int64(0), ctypes.c_int64(0)
     assert lib.ash_map_workspace_bytes(3, 24_000_000, ctypes.byref(table), ctypes.byref(general)) == 0
-    # 256-byte header + one 128-byte bucket per 6 entries of capacity
-    assert table.value == 256 + 4_000_000 * 128
+    # 256-byte header + one 128-byte bucket per 6 entries of capacity + the key
+    # log (8 bytes per entry, in 16-byte units, 256-byte aligned)
+    assert table.value == 256 + 4_000_000 * 128 + 24_000_000 * 8
     assert general.value == 2**26 * 20  # next power of two >= 2 * capacity, 20 B per slot
     assert lib.ash_map_workspace_bytes(1, 1, ctypes.byref(table), ctypes.byref(general)) == 0
-    assert table.value == 256 + 2 * 128
+    assert table.value == 256 + 2 * 128 + 16
     for dim in (0, 5):
         assert lib.ash_map_workspace_bytes(dim, 10, ctypes.byref(table), ctypes.byref(general)) != 0
         assert "key_dim" in _error(lib)

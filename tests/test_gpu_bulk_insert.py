@@ -245,3 +245,152 @@ def test_pending_fill_is_refused_under_capture(gpu_ash):
     torch.cuda.synchronize()
     _, masks = engine.find(keys)
     assert not bool(masks.any())
+
+
+def _assert_indices_and_free_list_partition(hm, size, capacity):
+    both = torch.cat([hm.engine.items()[1], hm.engine._heap[size:].long()])
+    assert torch.equal(torch.sort(both)[0].cpu(), torch.arange(capacity))
+
+
+def _check_value_map(hm, keys, values, capacity, untouched):
+    """Every distinct key of `keys` is stored once; its rows come from ONE
+    source row that holds this key; the indices in use and the free list
+    heap[size ..] together are every index once (ash/src/hashmap_gpu.cuh:226-231:
+    a new key takes heap[counter++], inserts never write to the heap); rows of
+    free indices still hold `untouched`."""
+    uniq = torch.unique(keys, dim=0)
+    n = keys.shape[0]
+    size = hm.size()
+    idx, masks = hm.engine.find(uniq)
+    assert bool(masks.all())
+    assert_is_bijection_into(idx, capacity)
+    heap = hm.engine._heap
+    _assert_indices_and_free_list_partition(hm, size, capacity)
+    color, depth = hm.color[idx], hm.depth[idx]
+    src = depth[:, 0].long()
+    assert bool((src >= 0).all()) and bool((src < n).all())
+    assert torch.equal(color, values["color"][src]) and torch.equal(keys[src], uniq)
+    free = heap[size:].long()
+    assert bool((hm.color[free] == untouched).all()) and bool((hm.depth[free] == untouched).all())
+    return uniq
+
+
+@pytest.mark.parametrize("duplicates", [0.0, 0.001, 0.5])
+def test_bulk_values_keep_the_heap_protocol(bulk_ash, oracle, duplicates):
+    """The streaming insert with value rows promises row i the heap position
+    counter + i and repairs the promise where keys lose: no duplicates (the
+    promise holds), a few (a handful of moves), half of the batch (most winners
+    of the upper half move).  Checked each time: key set against the oracle,
+    one source row per key, indices = heap[0 .. size), free rows untouched."""
+    dim, capacity = 3, 300_000
+    rng = np.random.default_rng(960 + int(duplicates * 1000))
+    n = 200_000
+    distinct = torch.unique(_random_keys(rng, 3 * n, dim, 60), dim=0)
+    distinct = distinct[torch.from_numpy(rng.permutation(len(distinct)))][:n]
+    n_dup = int(n * duplicates)
+    keys = distinct.clone()
+    if n_dup:
+        keys[rng.permutation(n)[:n_dup]] = distinct[rng.integers(0, n, size=n_dup)]
+    keys = keys.to(DEV)
+    row = torch.arange(n, device=DEV, dtype=torch.float32)
+    values = {"color": torch.stack([row, row + 0.5, 2 * row], dim=1), "depth": row.view(-1, 1).clone()}
+    hm = bulk_ash.HashMap(dim, {"color": 3, "depth": 1}, capacity, DEV)
+    hm.color.fill_(-7.0)
+    hm.depth.fill_(-7.0)
+    hm.insert(keys, values)
+    uniq = _check_value_map(hm, keys, values, capacity, -7.0)
+    assert hm.size() == len(uniq)
+    # a fresh heap: the indices are 0 .. size-1
+    assert torch.equal(torch.sort(hm.engine.items()[1])[0].cpu(), torch.arange(len(uniq)))
+    omap = _oracle_map(oracle, dim, capacity)
+    omap.insert_keys(keys.cpu())
+    _assert_same_map(hm.engine, omap, _random_keys(rng, 50_000, dim, 62).to(DEV))
+
+
+def test_bulk_values_into_a_populated_map_with_a_shuffled_heap(bulk_ash, oracle):
+    """Second batch with value rows into a map that holds keys (half of the
+    batch is already stored), after erases have put indices back on the heap in
+    another order (the heap is read instead of assumed to be 0, 1, 2, ...), and
+    a third batch that asks for more than the heap still has."""
+    dim, capacity = 3, 260_000
+    rng = np.random.default_rng(970)
+    pool = torch.unique(_random_keys(rng, 900_000, dim, 70), dim=0)
+    pool = pool[torch.from_numpy(rng.permutation(len(pool)))].to(DEV)
+    first, second_new, third_new = pool[:120_000], pool[120_000:200_000], pool[200_000:420_000]
+
+    def rows_for(keys, offset):
+        row = torch.arange(len(keys), device=DEV, dtype=torch.float32) + offset
+        return {"color": torch.stack([row, row + 0.5, 2 * row], dim=1), "depth": row.view(-1, 1).clone()}
+
+    hm = bulk_ash.HashMap(dim, {"color": 3, "depth": 1}, capacity, DEV)
+    omap = _oracle_map(oracle, dim, capacity)
+    hm.insert(first, rows_for(first, 0))
+    omap.insert_keys(first.cpu())
+    gone = first[torch.from_numpy(rng.permutation(len(first))[:50_000]).to(DEV)]
+    hm.erase(gone)
+    omap.erase(gone.cpu())
+    assert hm.size() == 70_000
+    hm.color[hm.engine._heap[70_000:].long()] = -7.0
+    hm.depth[hm.engine._heap[70_000:].long()] = -7.0
+    second = torch.cat([second_new, first[:80_000]])
+    second = second[torch.from_numpy(rng.permutation(len(second))).to(DEV)]
+    before = {k: v.clone() for k, v in hm.values.items()}
+    old_idx, old_mask = hm.engine.find(second)
+    hm.insert(second, rows_for(second, 1_000_000))
+    omap.insert_keys(second.cpu())
+    _assert_same_map(hm.engine, omap, pool[:450_000:3].contiguous())
+    size = hm.size()
+    heap = hm.engine._heap
+    _assert_indices_and_free_list_partition(hm, size, capacity)
+    # keys that were stored keep their index and their rows
+    new_idx, new_mask = hm.engine.find(second)
+    assert bool(new_mask.all()) and torch.equal(new_idx[old_mask], old_idx[old_mask])
+    kept = old_idx[old_mask]
+    assert torch.equal(hm.color[kept], before["color"][kept])
+    # new keys carry the rows of their source row
+    fresh = ~old_mask
+    src = (hm.depth[new_idx[fresh], 0] - 1_000_000).long()
+    assert torch.equal(second[src], second[fresh])
+    free = heap[size:].long()
+    assert bool((hm.color[free] == -7.0).all()) and bool((hm.depth[free] == -7.0).all())
+    # third batch: more new keys than the heap has left
+    with pytest.warns(UserWarning, match="exceeds the hash map capacity"):
+        hm.insert(third_new, rows_for(third_new, 2_000_000))
+    assert hm.size() == capacity
+    idx3, mask3 = hm.engine.find(third_new)
+    assert int(mask3.sum()) == capacity - size
+    src3 = (hm.depth[idx3[mask3], 0] - 2_000_000).long()
+    assert torch.equal(third_new[src3], third_new[mask3])
+    assert_is_bijection_into(hm.engine.items()[1], capacity)
+
+
+def test_streaming_insert_refuses_a_pending_fill_under_capture(gpu_ash):
+    """ash_map_insert_bulk after a clear decides on the host that the build
+    pass rewrites every bucket; recorded into a graph that decision would be
+    replayed against whatever the table holds then, so the call fails while
+    the stream is being captured and works outside."""
+    lib = gpu_ash.common.load_library()
+    engine = gpu_ash.ASHEngine(3, 50_000, DEV)
+    backend = engine.backend
+    keys = torch.unique(torch.randint(-40, 40, (30_000, 3), dtype=torch.int32), dim=0).to(DEV)
+    engine.insert_keys(keys)
+    engine.clear()
+    nbytes, worth = ctypes.c_int64(0), ctypes.c_int(0)
+    assert lib.ash_map_bulk_workspace_bytes(backend._handle, len(keys), 0, None,
+                                            ctypes.byref(nbytes), ctypes.byref(worth)) == 0
+    assert nbytes.value > 0
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=DEV)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.ash_map_insert_bulk(backend._handle, keys.data_ptr(), len(keys), 0, None, None,
+                                         None, ws.data_ptr(), ws.numel(), side.cuda_stream)
+    assert rc != 0 and "cleared" in lib.ash_last_error().decode()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(DEV).cuda_stream
+    rc = lib.ash_map_insert_bulk(backend._handle, keys.data_ptr(), len(keys), 0, None, None, None,
+                                 ws.data_ptr(), ws.numel(), stream)
+    assert rc == 0, lib.ash_last_error().decode()
+    assert backend.status()["size"] == len(keys)
+    assert bool(engine.find(keys)[1].all())

@@ -105,6 +105,48 @@ def test_engine_state_dict_round_trip(gpu_ash, dim, num, tmp_path):
         assert_is_bijection_into(engine.items()[1], capacity)
 
 
+def test_gather_rows_equals_torch_indexing(gpu_ash):
+    """ash_gather_rows behind HashMap.find / items (return_values=True) against
+    the reference's formulation, values[name][indices] (ash/hashmap.py:87-95):
+    one to five tensors (more than one launch), row widths 1..5 and 20 words,
+    float and int rows, sorted and random indices, and the tables torch keeps
+    (rows of 2 bytes)."""
+    backend = gpu_ash.core.backend
+    g = torch.Generator().manual_seed(5)
+    rows = 50_000
+    tables = {
+        "a": torch.rand(rows, 3, generator=g),
+        "b": torch.rand(rows, 1, generator=g),
+        "c": torch.randint(-9, 9, (rows, 5), generator=g, dtype=torch.int32),
+        "d": torch.rand(rows, 4, generator=g, dtype=torch.float64),
+        "e": torch.rand(rows, 20, generator=g),
+        "f": torch.rand(rows, 1, generator=g).to(torch.float16),
+    }
+    tables = {k: v.to(DEV) for k, v in tables.items()}
+    for n in (0, 1, 70_001):
+        for order in ("random", "sorted"):
+            idx = torch.randint(0, rows, (n,), generator=g)
+            idx = (torch.sort(idx)[0] if order == "sorted" else idx).to(DEV)
+            for names in (("a",), ("a", "b"), tuple("abcdef")):
+                got = backend.gather_rows({k: tables[k] for k in names}, idx)
+                assert tuple(got) == names
+                for k in names:
+                    assert got[k].dtype == tables[k].dtype
+                    assert torch.equal(got[k], tables[k][idx]), (k, n, order)
+    # through the map: values of found keys and of items()
+    hm = gpu_ash.HashMap(3, {"color": 3, "depth": 1}, 40_000, DEV)
+    keys = torch.unique(torch.randint(-30, 30, (30_000, 3), generator=g, dtype=torch.int32), dim=0).to(DEV)
+    values = {"color": torch.rand(len(keys), 3, device=DEV), "depth": torch.rand(len(keys), 1, device=DEV)}
+    hm.insert(keys, values)
+    masks, idx, found = hm.find(keys, return_values=True)
+    assert bool(masks.all())
+    assert torch.equal(found["color"], values["color"]) and torch.equal(found["depth"], values["depth"])
+    k2, i2, v2 = hm.items(return_indices=True, return_values=True)
+    assert torch.equal(v2["color"], hm.color[i2]) and torch.equal(v2["depth"], hm.depth[i2])
+    order = sort_rows(k2, i2)
+    assert torch.equal(order[0], sort_rows(keys)[0])
+
+
 def test_state_with_duplicate_keys_is_refused(gpu_ash):
     """A saved state whose active keys repeat a key (the reference prints
     "should never reach here", ash/src/hashmap_gpu.cuh:420-422, and goes on

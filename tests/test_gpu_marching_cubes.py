@@ -207,7 +207,9 @@ def test_spatial_listing_follows_the_table(gpu_ash):
         3, 17 ** 3 + 10, 1, grid_dim=2, sparse_grid_dim=20, bbox_min=torch.zeros(3),
         bbox_max=torch.ones(3), device=DEV)
     r = torch.arange(17, dtype=torch.int32)
-    blocks = torch.stack(torch.meshgrid(r, r, r, indexing="ij"), -1).view(-1, 3).to(DEV)
+    blocks = torch.stack(torch.meshgrid(r, r, r, indexing="ij"), -1).view(-1, 3)
+    # inserted in a random order: items() lists by index, i.e. roughly as inserted
+    blocks = blocks[torch.randperm(len(blocks), generator=torch.Generator().manual_seed(3))].to(DEV)
     grid.engine.insert_keys(blocks)
 
     def same_set(listing):
@@ -217,7 +219,7 @@ def test_spatial_listing_follows_the_table(gpu_ash):
 
     first = grid._blocks_in_spatial_order()
     assert same_set(first) and len(first[1]) == 17 ** 3
-    # neighbours in the listing are neighbours in space far more often than in table order
+    # neighbours in the listing are neighbours in space far more often than in items() order
     step = (first[0][1:] - first[0][:-1]).abs().sum(dim=1).float().mean()
     table_step = (grid.engine.items()[0][1:] - grid.engine.items()[0][:-1]).abs().sum(dim=1).float().mean()
     assert float(step) < 0.3 * float(table_step)

@@ -149,6 +149,11 @@ _SIGNATURES = {
     "ash_map_should_rebuild": (ctypes.c_int, [_PTR, _I64, _I64, _I64]),
     "ash_map_rebuild": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
     "ash_scatter_rows": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _I64, _PTR]),
+    "ash_gather_rows": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.POINTER(_PTR), ctypes.POINTER(_PTR), ctypes.POINTER(_I64),
+         ctypes.POINTER(_I64), _PTR, _I64, _PTR],
+    ),
     "ash_isosurface_workspace_ints": (ctypes.c_int64, [_I64, _I64]),
     "ash_isosurface_classify": (
         ctypes.c_int,
@@ -569,6 +574,42 @@ class _Backend:
                     _stream_of(dev),
                 )
             )
+
+    # -- value rows by index (ash/hashmap.py:87-95,138-146) -------------------
+    def gather_rows(self, tables: Dict[str, torch.Tensor], indices: torch.Tensor) -> Dict[str, torch.Tensor]:
+        """{name: table[indices]} for value tables on a HIP device, four tables
+        per launch.  Tables the kernel does not take (rows that are not a
+        multiple of 4 bytes, non-contiguous storage) are indexed by torch."""
+        out: Dict[str, torch.Tensor] = {}
+        batch = []
+        indices = indices.reshape(-1)
+        n = indices.shape[0]
+        for name, table in tables.items():
+            row_bytes = (table.numel() // max(table.shape[0], 1)) * table.element_size()
+            fits = (table.is_cuda and table.is_contiguous() and table.shape[0] > 0
+                    and row_bytes % 4 == 0 and row_bytes > 0 and indices.device == table.device
+                    and indices.dtype == torch.int64 and not table.requires_grad)
+            if not fits:
+                out[name] = table[indices]
+                continue
+            out[name] = torch.empty((n,) + tuple(table.shape[1:]), dtype=table.dtype,
+                                    device=table.device)
+            batch.append((table, out[name], row_bytes))
+        indices = indices.contiguous()
+        for first in range(0, len(batch), 4):
+            part = batch[first:first + 4]
+            if n == 0:
+                break
+            k = len(part)
+            c_src = (_PTR * k)(*[t.data_ptr() for t, _, _ in part])
+            c_dst = (_PTR * k)(*[d.data_ptr() for _, d, _ in part])
+            c_rows = (_I64 * k)(*[rb for _, _, rb in part])
+            c_count = (_I64 * k)(*[t.shape[0] for t, _, _ in part])
+            dev = part[0][0].device
+            with torch.cuda.device(dev):
+                self.check(self.lib.ash_gather_rows(k, c_src, c_dst, c_rows, c_count,
+                                                    indices.data_ptr(), n, _stream_of(dev)))
+        return {name: out[name] for name in tables}
 
     # -- trilinear queries (ash/src/pybind.cpp:25-29) ---------------------
     def _query_args(

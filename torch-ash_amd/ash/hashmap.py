@@ -9,6 +9,7 @@ from typing import Dict, List, Tuple, Union
 
 import torch
 
+from . import core
 from .core import ASHEngine, ASHModule
 
 ValueSpec = Union[int, List[int], Dict[str, int]]
@@ -129,6 +130,12 @@ class HashMap(ASHModule):
         return self._layout.declared(values)
 
     def _rows(self, indices: torch.Tensor) -> Values:
+        """The value rows at `indices` (ash/hashmap.py:87-95,138-146 index every
+        tensor with torch); the native backend gathers all tensors in one
+        launch."""
+        gather = getattr(core.backend, "gather_rows", None)
+        if gather is not None:
+            return self._layout.declared(gather(self.values, indices))
         return self._layout.declared({name: rows[indices] for name, rows in self.values.items()})
 
     def _answer(self, first, indices, return_indices: bool, return_values: bool) -> Tuple:

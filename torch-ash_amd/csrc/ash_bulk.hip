@@ -2,24 +2,42 @@
 // slots with one global compare-and-swap per key.
 //
 // The per-key kernel (ash_map.hip) is bound by the rate at which the device
-// executes atomics on random lines (about 2e10 per second, whatever cache the
-// line sits in).  When a batch is of the order of the table itself it is
-// cheaper to stream: the batch is split by bucket range in two coalesced
-// passes (coarse bins, then partitions of 512 buckets inside each bin), and one
-// workgroup per partition then owns 64 KB of the table exclusively: it loads
-// that range into LDS (or starts from an empty one), inserts its records with
-// LDS compare-and-swap, takes all indices of the partition from the heap with a
-// single update of the heap counter, copies the value rows of the new keys and
-// writes the range back with full-line stores.
+// executes atomics on random lines.  When a batch is of the order of the table
+// itself it is cheaper to stream: the batch is split by bucket range in two
+// coalesced passes (coarse bins, then partitions of 512 buckets inside each
+// bin), and one workgroup per partition then owns 64 KB of the table
+// exclusively: it loads that range into LDS (or starts from an empty one),
+// inserts its records with LDS compare-and-swap and writes the range back with
+// full-line stores.
 //
-// Records travel as a plane of 64-bit key codes plus one plane per value
-// tensor, so every pass reads and writes contiguous runs.  Bins and partitions
-// have a fixed capacity (expected count + ten standard deviations); what does
-// not fit -- duplicates piled on one key, unpackable keys, a probe sequence
-// that leaves its partition, an exhausted heap -- is put on a spill list and
+// Two ways of handing out indices, both with the reference's heap protocol
+// (ash/src/hashmap_gpu.cuh:211-232: a new key takes heap[counter++]):
+//
+//  * keys only: records are bare 64-bit key codes; the build pass ranks the
+//    winners of a partition and takes their indices with one update of the
+//    heap counter.
+//
+//  * keys with value rows ("provisional" indices): moving the rows through the
+//    two split passes would triple their traffic, so they never travel.  Row i
+//    of the batch is promised heap position base + i (base = the counter on
+//    entry) and records are (code, i) pairs of 12 bytes.  If every key turns
+//    out to be new the promise holds and the value rows are copied in input
+//    order, source and destination both contiguous.  Keys that lose (already
+//    stored, repeated inside the batch, or handed to the per-key kernel) leave
+//    holes among the promised positions; with U winners the positions
+//    base .. base + U - 1 must be the ones in use, so every winner at or beyond
+//    base + U ("high" winner) is moved into a hole below it -- there are
+//    exactly as many of one as of the other.  A flag byte per row tells losers
+//    from winners; the value copy skips losers, and when rows lost two small
+//    kernels list the holes and re-point the high winners' slots and copy
+//    their rows.  Rows of keys that are not inserted are never written.
+//
+// Bins and partitions have a fixed capacity (expected count + ten standard
+// deviations); what does not fit -- duplicates piled on one key, unpackable
+// keys, rows beyond the capacity of the heap -- is put on a spill list and
 // handled afterwards by the per-key kernel, so the result is the same map for
-// any input.  The heap protocol is the reference's
-// (ash/src/hashmap_gpu.cuh:211-232): a new key takes heap[counter++].
+// any input.  (A probe sequence stays inside its partition by the table's own
+// rule, ash_table.h: next_bucket.)
 #include "ash_table.h"
 
 #include "../../include/ash_hip.h"
@@ -29,21 +47,25 @@
 namespace ash {
 namespace {
 
-constexpr int kPartShift = 9;
-constexpr int kPartBuckets = 1 << kPartShift;   // buckets per build workgroup
-// Chunk geometry measured on 16 M keys with two value planes (ms per insert):
-// 1024x4 1.03, 1024x2 1.06, 512x4 1.13, 512x8 1.17, 256x8 1.29.
+// A build workgroup owns one probe range of the table: kPartBuckets buckets
+// (ash_dev.h), the range a probe sequence never leaves.
+// Chunk geometry measured on 16 M keys (ms per insert): 1024x4 1.03,
+// 1024x2 1.06, 512x4 1.13, 512x8 1.17, 256x8 1.29.
 constexpr int kSplitThreads = 1024;
 constexpr int kSplitKeys = 4;                   // records per thread
-constexpr int kStageDwords = 4;                 // widest row slice staged in LDS
 constexpr int kSplitChunk = kSplitThreads * kSplitKeys;
 constexpr int kMaxBins = 256;
 constexpr int kBuildThreads = 512;
 constexpr int kBuildRecs = 4;                   // records per thread and round
+constexpr int kCopyThreads = 256;
 constexpr int64_t kMinKeys = 1 << 12;
 
 // Header words at the start of the workspace.
-enum { kHdrSpillKeys = 0, kHdrSpillA = 1, kHdrSpillB = 2, kHdrWasEmpty = 3,
+enum { kHdrSpillKeys = 0, kHdrSpillA = 1, kHdrWasEmpty = 3,
+       kHdrBase = 4,      // heap counter on entry
+       kHdrLosers = 5,    // rows that did not win a slot in the build pass
+       kHdrHoles = 6,     // listed holes
+       kHdrTaken = 7,     // holes handed to high winners
        kHdrWords = 64 };
 
 struct BulkPlan {
@@ -59,11 +81,14 @@ struct BulkPlan {
     int32_t* cursor_part;  // bins << fine_shift
     uint64_t* codes_a;     // bins * cap_bin
     uint64_t* codes_b;     // parts * cap_part
-    uint32_t* plane_a[kMaxFusedValues];
-    uint32_t* plane_b[kMaxFusedValues];
-    int32_t* spill_keys;   // n input row numbers
-    int32_t* spill_a;      // n positions in the coarse planes
-    int32_t* spill_b;      // n positions in the partition planes
+    // keys only
+    int32_t* spill_keys;   // n input row numbers (also the one list of the provisional scheme)
+    int32_t* spill_a;      // n positions in the coarse plane
+    // provisional scheme
+    int32_t* rows_a;       // bins * cap_bin input row numbers
+    int32_t* rows_b;       // parts * cap_part
+    uint8_t* flags;        // n: 1 = row i did not win a slot
+    int32_t* holes;        // n / 2 + 64 row numbers
 };
 
 inline int64_t align256(int64_t x) { return (x + 255) & ~int64_t{255}; }
@@ -119,17 +144,18 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
     pl.cursor_part = reinterpret_cast<int32_t*>(take((bins << fine_shift) * 4));
     pl.codes_a = reinterpret_cast<uint64_t*>(take(na * 8));
     pl.codes_b = reinterpret_cast<uint64_t*>(take(nbp * 8));
-    for (int v = 0; v < kMaxFusedValues; ++v) {
-        pl.plane_a[v] = nullptr;
-        pl.plane_b[v] = nullptr;
-        if (v < n_values) {
-            pl.plane_a[v] = reinterpret_cast<uint32_t*>(take(na * row_bytes[v]));
-            pl.plane_b[v] = reinterpret_cast<uint32_t*>(take(nbp * row_bytes[v]));
-        }
-    }
     pl.spill_keys = reinterpret_cast<int32_t*>(take(n * 4));
-    pl.spill_a = reinterpret_cast<int32_t*>(take(n * 4));
-    pl.spill_b = reinterpret_cast<int32_t*>(take(n * 4));
+    pl.spill_a = nullptr;
+    pl.rows_a = pl.rows_b = pl.holes = nullptr;
+    pl.flags = nullptr;
+    if (n_values == 0) {
+        pl.spill_a = reinterpret_cast<int32_t*>(take(n * 4));
+    } else {
+        pl.rows_a = reinterpret_cast<int32_t*>(take(na * 4));
+        pl.rows_b = reinterpret_cast<int32_t*>(take(nbp * 4));
+        pl.flags = reinterpret_cast<uint8_t*>(take(n));
+        pl.holes = reinterpret_cast<int32_t*>(take((n / 2 + 64) * 4));
+    }
     return off;
 }
 
@@ -139,36 +165,40 @@ __global__ void bulk_init_kernel(MapDev m, BulkPlan pl, int ncursors) {
     // cursor_bin and cursor_part are zeroed separately: they are not adjacent
     if (t < static_cast<int>(pl.bins)) pl.cursor_bin[t] = 0;
     if (t < ncursors) pl.cursor_part[t] = 0;
-    if (t == 0) {
-        pl.hdr[kHdrSpillKeys] = 0;
-        pl.hdr[kHdrSpillA] = 0;
-        pl.hdr[kHdrSpillB] = 0;
-        pl.hdr[kHdrWasEmpty] =
-                (m.ctr[kCtrSize] == 0 && m.ctr[kCtrTombs] == 0) ? 1 : 0;
+    if (t < kHdrWords) {
+        int32_t v = 0;
+        if (t == kHdrWasEmpty) v = (m.ctr[kCtrSize] == 0 && m.ctr[kCtrTombs] == 0) ? 1 : 0;
+        if (t == kHdrBase) v = m.ctr[kCtrSize];
+        pl.hdr[t] = v;
     }
 }
 
-__device__ __forceinline__ void copy_row(const uint32_t* __restrict__ s,
-                                         uint32_t* __restrict__ d, int rd) {
-    for (int q = 0; q < rd; ++q) d[q] = s[q];
+// Rows of the batch that can be promised a heap position.
+__device__ __forceinline__ int64_t rows_that_fit(const MapDev& m, const BulkPlan& pl) {
+    const int64_t room = static_cast<int64_t>(m.capacity) - pl.hdr[kHdrBase];
+    return room < 0 ? 0 : (room < pl.n ? room : pl.n);
 }
 
 // LDS of the two split passes.  Every record of the workgroup's chunk gets a
 // bin and its arrival rank inside that bin (LDS counter); reserve_runs turns
 // the counts into start[b] (first sorted position of bin b inside the chunk)
 // and base[b] (position of the chunk's run inside the bin's global buffer,
-// reserved with one atomic per bin).  The chunk is then moved plane by plane:
-// each thread drops its records at their sorted positions in `stage`, and the
-// workgroup writes the stage out front to back, so that global reads and
-// writes both have consecutive lanes on consecutive records.
+// reserved with one atomic per bin).  Each thread then drops its records at
+// their sorted positions in `stage`, and the workgroup writes the stage out
+// front to back, so that global reads and writes both have consecutive lanes
+// on consecutive records.
 struct SplitShared {
     int cnt[kMaxBins];
     int start[kMaxBins];
     int base[kMaxBins];
     int wave_total[kMaxBins / 64];
-    uint16_t perm[kSplitChunk];    // sorted position -> record of the chunk
+    int losers;
+    int nspill;        // rows of this chunk that pass 1 leaves to the per-key kernel
+    int spill_first;   // their place in the spill list
+    // sorted position -> input row (provisional scheme) or record of the chunk
+    int32_t aux[kSplitChunk];
     uint8_t bin_of[kSplitChunk];   // sorted position -> bin
-    uint32_t stage[kSplitChunk * kStageDwords];
+    uint64_t stage[kSplitChunk];   // sorted position -> code
 };
 
 __device__ __forceinline__ int reserve_runs(SplitShared& sh, int32_t* cursors,
@@ -200,120 +230,82 @@ __device__ __forceinline__ int reserve_runs(SplitShared& sh, int32_t* cursors,
     return total;
 }
 
-// Moves the ranked records of a chunk to their runs.  code/bin/rank describe
-// the calling thread's kSplitKeys records (record k of the thread is record
-// k * kSplitThreads + tid of the chunk, bin < 0 = not taking part); the value
-// rows of record r are row `row0 + r` of src[v].  Destination of a record with
-// bin b and position pos inside the bin: dst_first(b) + pos, valid while
-// pos < cap; the others are reported through `spill` with their record number.
-template <typename DstFirst, typename Spill>
+// Moves the ranked records of a chunk to their runs.  code/aux/bin/rank
+// describe the calling thread's kSplitKeys records (bin < 0 = not taking
+// part); aux is what travels with the code: the input row in the provisional
+// scheme (written to aux_dst), the record's number inside the chunk otherwise
+// (only used to name a record that does not fit).  Destination of a record
+// with bin b and position pos inside the bin: dst_first(b) + pos, valid while
+// pos < cap; the others are reported through `spill` with their aux value.
+template <bool PROV, typename DstFirst, typename Spill>
 __device__ __forceinline__ void move_chunk(
         SplitShared& sh, int total, const uint64_t (&code)[kSplitKeys],
-        const int (&bin)[kSplitKeys], const int (&rank)[kSplitKeys],
-        int64_t row0, const uint32_t* const (&src)[kMaxFusedValues],
-        uint32_t* const (&dst)[kMaxFusedValues],
-        const int32_t (&row_dwords)[kMaxFusedValues], int n_values,
-        uint64_t* __restrict__ codes_dst, uint32_t cap, DstFirst dst_first,
-        Spill spill) {
+        const int32_t (&aux)[kSplitKeys], const int (&bin)[kSplitKeys],
+        const int (&rank)[kSplitKeys], uint64_t* __restrict__ codes_dst,
+        int32_t* __restrict__ aux_dst, uint32_t cap, DstFirst dst_first, Spill spill) {
     const int tid = threadIdx.x;
-    uint32_t regs[kSplitKeys][kStageDwords];
-    auto load_slice = [&](int v, int q0) {
-        const int rd = row_dwords[v];
-        const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
-#pragma unroll
-        for (int k = 0; k < kSplitKeys; ++k) {
-            if (bin[k] >= 0) {
-                const uint32_t* s =
-                        src[v] + (row0 + k * kSplitThreads + tid) * rd + q0;
-#pragma unroll
-                for (int q = 0; q < kStageDwords; ++q) {
-                    if (q < w) regs[k][q] = s[q];
-                }
-            }
-        }
-    };
-    int v = 0, q0 = 0;
-    bool have = n_values > 0;
-    if (have) load_slice(0, 0);
-    int sp[kSplitKeys];
 #pragma unroll
     for (int k = 0; k < kSplitKeys; ++k) {
-        sp[k] = -1;
         if (bin[k] >= 0) {
-            sp[k] = sh.start[bin[k]] + rank[k];
-            sh.perm[sp[k]] = static_cast<uint16_t>(k * kSplitThreads + tid);
-            sh.bin_of[sp[k]] = static_cast<uint8_t>(bin[k]);
-            reinterpret_cast<uint64_t*>(sh.stage)[sp[k]] = code[k];
+            const int sp = sh.start[bin[k]] + rank[k];
+            sh.aux[sp] = aux[k];
+            sh.bin_of[sp] = static_cast<uint8_t>(bin[k]);
+            sh.stage[sp] = code[k];
         }
     }
     __syncthreads();
-    int64_t d[kSplitKeys];
 #pragma unroll
     for (int j = 0; j < kSplitKeys; ++j) {
         const int s = j * kSplitThreads + tid;
-        d[j] = -1;
         if (s < total) {
             const int b = sh.bin_of[s];
             const uint32_t pos =
                     static_cast<uint32_t>(sh.base[b] + (s - sh.start[b]));
             if (pos < cap) {
-                d[j] = dst_first(b) + pos;
-                codes_dst[d[j]] = reinterpret_cast<const uint64_t*>(sh.stage)[s];
+                const int64_t d = dst_first(b) + pos;
+                codes_dst[d] = sh.stage[s];
+                if constexpr (PROV) aux_dst[d] = sh.aux[s];
             } else {
-                spill(static_cast<int>(sh.perm[s]));
+                spill(sh.aux[s]);
             }
         }
-    }
-    // Value rows, one slice of up to kStageDwords words at a time.  The rows of
-    // the next slice are requested while the current one is written out.
-    while (have) {
-        const int rd = row_dwords[v];
-        const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < kSplitKeys; ++k) {
-            if (sp[k] >= 0) {
-#pragma unroll
-                for (int q = 0; q < kStageDwords; ++q) {
-                    if (q < w) sh.stage[sp[k] * w + q] = regs[k][q];
-                }
-            }
-        }
-        int nv = v, nq0 = q0 + kStageDwords;
-        if (nq0 >= rd) {
-            ++nv;
-            nq0 = 0;
-        }
-        const bool nhave = nv < n_values;
-        if (nhave) load_slice(nv, nq0);
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < kSplitKeys; ++j) {
-            if (d[j] >= 0) {
-                const int s = j * kSplitThreads + tid;
-                uint32_t* o = dst[v] + d[j] * rd + q0;
-                for (int q = 0; q < w; ++q) o[q] = sh.stage[s * w + q];
-            }
-        }
-        v = nv;
-        q0 = nq0;
-        have = nhave;
     }
 }
 
+// A row of the provisional scheme that will not be placed by the build pass:
+// flagged, counted, and (unless it is a plain duplicate) left to the per-key
+// kernel.
+__device__ __forceinline__ void give_up_row(const BulkPlan& pl, int32_t row, int* losers,
+                                            bool to_per_key_kernel) {
+    pl.flags[row] = 1;
+    atomicAdd(losers, 1);
+    if (to_per_key_kernel) pl.spill_keys[atomicAdd(pl.hdr + kHdrSpillKeys, 1)] = row;
+}
+
 // Pass 1: input rows -> coarse bins, 4096 keys per workgroup.
-template <int DIM>
+// `identity` (provisional scheme): the heap is 0, 1, 2, ..., so row i's promised
+// index is base + i and the key log can be written here, in input order; with a
+// heap in another order the build pass writes it.
+template <int DIM, bool PROV>
 __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
-        MapDev m, BulkPlan pl, const int32_t* __restrict__ keys, ValueArgs va) {
+        MapDev m, BulkPlan pl, const int32_t* __restrict__ keys, int identity) {
     __shared__ SplitShared sh;
     const int tid = threadIdx.x;
     if (tid < kMaxBins) sh.cnt[tid] = 0;
+    if (tid == 0) {
+        sh.losers = 0;
+        sh.nspill = 0;
+    }
     __syncthreads();
     const int64_t base = static_cast<int64_t>(blockIdx.x) * kSplitChunk;
     const int bin_shift = kPartShift + static_cast<int>(pl.fine_shift);
+    const int64_t fit = PROV ? rows_that_fit(m, pl) : pl.n;
+    const int64_t heap_base = PROV ? pl.hdr[kHdrBase] : 0;
     uint64_t code[kSplitKeys];
+    int32_t aux[kSplitKeys];
     int bin[kSplitKeys];
     int rank[kSplitKeys];
+    int spill_rank[kSplitKeys];
 #pragma unroll
     for (int k = 0; k < kSplitKeys; ++k) {
         const int64_t i = base + k * kSplitThreads + tid;
@@ -323,31 +315,57 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
         const bool fits = pack_key<DIM>(key, code[k]);
         bin[k] = -1;
         rank[k] = 0;
-        if (active && fits) {
+        spill_rank[k] = -1;
+        aux[k] = PROV ? static_cast<int32_t>(i) : k * kSplitThreads + tid;
+        if (active && fits && i < fit) {
             bin[k] = static_cast<int>(bucket_of(code[k], m.nb) >> bin_shift);
             rank[k] = atomicAdd(&sh.cnt[bin[k]], 1);
+            if constexpr (PROV) {
+                pl.flags[i] = 0;
+                if (identity) m.klog[heap_base + i] = code[k];
+            }
         } else if (active) {
-            // unpackable: left to the per-key kernel
-            pl.spill_keys[atomicAdd(pl.hdr + kHdrSpillKeys, 1)] =
-                    static_cast<int32_t>(i);
+            // unpackable, or beyond what the heap can still give: left to the
+            // per-key kernel (listed below, one update of the list's counter
+            // per workgroup: a batch far beyond the capacity lands here)
+            spill_rank[k] = atomicAdd(&sh.nspill, 1);
+            if constexpr (PROV) pl.flags[i] = 1;
         }
     }
     __syncthreads();
+    if (tid == 0 && sh.nspill) {
+        sh.spill_first = atomicAdd(pl.hdr + kHdrSpillKeys, sh.nspill);
+        if constexpr (PROV) sh.losers = sh.nspill;
+    }
     const int total = reserve_runs(sh, pl.cursor_bin, static_cast<int>(pl.bins));
-    move_chunk(
-            sh, total, code, bin, rank, base, va.src, pl.plane_a, va.row_dwords,
-            va.n, pl.codes_a, pl.cap_bin,
+#pragma unroll
+    for (int k = 0; k < kSplitKeys; ++k) {
+        if (spill_rank[k] >= 0) {
+            pl.spill_keys[sh.spill_first + spill_rank[k]] =
+                    static_cast<int32_t>(base + k * kSplitThreads + tid);
+        }
+    }
+    move_chunk<PROV>(
+            sh, total, code, aux, bin, rank, pl.codes_a, pl.rows_a, pl.cap_bin,
             [&](int b) { return static_cast<int64_t>(b) * pl.cap_bin; },
-            [&](int rec) {
-                pl.spill_keys[atomicAdd(pl.hdr + kHdrSpillKeys, 1)] =
-                        static_cast<int32_t>(base + rec);
+            [&](int32_t a) {
+                if constexpr (PROV) {
+                    give_up_row(pl, a, &sh.losers, true);
+                } else {
+                    pl.spill_keys[atomicAdd(pl.hdr + kHdrSpillKeys, 1)] =
+                            static_cast<int32_t>(base + a);
+                }
             });
+    if constexpr (PROV) {
+        __syncthreads();
+        if (tid == 0 && sh.losers) atomicAdd(pl.hdr + kHdrLosers, sh.losers);
+    }
 }
 
 // Pass 2: coarse bin -> partitions.  Workgroup (bin, chunk) takes 4096 records
 // of its bin.
-__global__ __launch_bounds__(kSplitThreads) void split_records_kernel(
-        MapDev m, BulkPlan pl, ValueArgs va) {
+template <bool PROV>
+__global__ __launch_bounds__(kSplitThreads) void split_records_kernel(MapDev m, BulkPlan pl) {
     __shared__ SplitShared sh;
     const int tid = threadIdx.x;
     const uint32_t c = blockIdx.x / pl.chunks;
@@ -357,10 +375,12 @@ __global__ __launch_bounds__(kSplitThreads) void split_records_kernel(
     const int start = static_cast<int>(chunk) * kSplitChunk;
     if (start >= cnt) return;
     if (tid < kMaxBins) sh.cnt[tid] = 0;
+    if (tid == 0) sh.losers = 0;
     __syncthreads();
     const int64_t abase = static_cast<int64_t>(c) * pl.cap_bin + start;
     const uint32_t fmask = (1u << pl.fine_shift) - 1u;
     uint64_t code[kSplitKeys];
+    int32_t aux[kSplitKeys];
     int bin[kSplitKeys];
     int rank[kSplitKeys];
 #pragma unroll
@@ -369,8 +389,10 @@ __global__ __launch_bounds__(kSplitThreads) void split_records_kernel(
         bin[k] = -1;
         rank[k] = 0;
         code[k] = 0;
+        aux[k] = j;
         if (start + j < cnt) {
             code[k] = pl.codes_a[abase + j];
+            if constexpr (PROV) aux[k] = pl.rows_a[abase + j];
             bin[k] = static_cast<int>((bucket_of(code[k], m.nb) >> kPartShift) & fmask);
             rank[k] = atomicAdd(&sh.cnt[bin[k]], 1);
         }
@@ -379,21 +401,25 @@ __global__ __launch_bounds__(kSplitThreads) void split_records_kernel(
     const int total = reserve_runs(
             sh, pl.cursor_part + (static_cast<size_t>(c) << pl.fine_shift),
             static_cast<int>(fmask) + 1);
-    const uint32_t* src[kMaxFusedValues];
-#pragma unroll
-    for (int v = 0; v < kMaxFusedValues; ++v) src[v] = pl.plane_a[v];
-    move_chunk(
-            sh, total, code, bin, rank, abase, src, pl.plane_b, va.row_dwords,
-            va.n, pl.codes_b, pl.cap_part,
+    move_chunk<PROV>(
+            sh, total, code, aux, bin, rank, pl.codes_b, pl.rows_b, pl.cap_part,
             [&](int b) {
                 return static_cast<int64_t>((c << pl.fine_shift) +
                                             static_cast<uint32_t>(b)) *
                        pl.cap_part;
             },
-            [&](int rec) {
-                pl.spill_a[atomicAdd(pl.hdr + kHdrSpillA, 1)] =
-                        static_cast<int32_t>(abase + rec);
+            [&](int32_t a) {
+                if constexpr (PROV) {
+                    give_up_row(pl, a, &sh.losers, true);
+                } else {
+                    pl.spill_a[atomicAdd(pl.hdr + kHdrSpillA, 1)] =
+                            static_cast<int32_t>(abase + a);
+                }
             });
+    if constexpr (PROV) {
+        __syncthreads();
+        if (tid == 0 && sh.losers) atomicAdd(pl.hdr + kHdrLosers, sh.losers);
+    }
 }
 
 // Where the q-th 16 bytes of local bucket lb sit in the LDS copy of the table
@@ -404,16 +430,62 @@ __device__ __forceinline__ int staged(int lb, int q) {
     return lb * kGroup + ((q + lb) & (kGroup - 1));
 }
 
+enum { kPlaced = 0, kKnown = 1, kFull = 2 };
+
+// Inserts `code` into the LDS copy of the partition, starting at local bucket
+// lb and going round inside the partition (next_bucket's rule).  kPlaced: the
+// calling thread owns slot `where` (local bucket * 16 + slot) now; kKnown: the
+// code was there already (or another thread of this round placed it); kFull:
+// every bucket of the partition has been visited.
+__device__ __forceinline__ int place_code(uint4* tab, uint64_t code, int lb, int nbk,
+                                          int& where) {
+    unsigned long long* tab64 = reinterpret_cast<unsigned long long*>(tab);
+    for (int visited = 0; visited < nbk; ++visited) {
+        uint64_t c[kSlots];
+#pragma unroll
+        for (int q = 0; q < kSlots / 2; ++q) {
+            const uint4 w = tab[staged(lb, q)];
+            c[2 * q] = static_cast<uint64_t>(w.x) | (static_cast<uint64_t>(w.y) << 32);
+            c[2 * q + 1] = static_cast<uint64_t>(w.z) | (static_cast<uint64_t>(w.w) << 32);
+        }
+        bool known = false;
+        uint32_t em = 0;
+#pragma unroll
+        for (int s = 0; s < kSlots; ++s) {
+            known |= c[s] == code;
+            em |= (c[s] == kEmpty ? 1u : 0u) << s;
+        }
+        if (known) return kKnown;
+        while (em) {
+            const int s = __builtin_ctz(em);
+            const unsigned long long old =
+                    atomicCAS(tab64 + staged(lb, s >> 1) * 2 + (s & 1), kEmpty, code);
+            if (old == kEmpty) {
+                where = lb * kBucketQwords + s;
+                return kPlaced;
+            }
+            if (old == code) return kKnown;
+            em &= em - 1;
+        }
+        if (++lb == nbk) lb = 0;
+    }
+    return kFull;
+}
+
 // Pass 3: one workgroup per partition builds its 512 buckets in LDS.
 // `stale`: the bucket array holds leftovers of a table that has been cleared
 // since (the clear left the fill to its successor): every partition is then
-// written, those without records as empty ones.
+// written, those without records as empty ones.  `identity`: the heap is
+// 0, 1, 2, ... (nothing has written to it since it was last reset), so
+// position p holds index p and need not be read.
+template <bool PROV>
 __global__ __launch_bounds__(kBuildThreads) void build_kernel(
-        MapDev m, BulkPlan pl, ValueArgs va, int stale) {
+        MapDev m, BulkPlan pl, int stale, int identity) {
     __shared__ uint4 tab[kPartBuckets * kGroup];
     // winners per (record slot k, wavefront), then their exclusive prefix
     __shared__ int s_wcnt[kBuildRecs * (kBuildThreads / 64)];
     __shared__ int s_base;
+    __shared__ int s_losers;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -436,14 +508,18 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
         return;
     }
     const bool was_empty = pl.hdr[kHdrWasEmpty] != 0;
+    const int32_t heap_base = pl.hdr[kHdrBase];
     const int64_t bbase = static_cast<int64_t>(p) * pl.cap_part;
+    if (tid == 0) s_losers = 0;
     // The first round's records are requested before the table range is
     // staged, so that both latencies overlap.
     uint64_t codes[kBuildRecs];
+    int32_t rows[kBuildRecs];
 #pragma unroll
     for (int k = 0; k < kBuildRecs; ++k) {
         const int r = k * kBuildThreads + tid;
         codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
+        if constexpr (PROV) rows[k] = r < cnt ? pl.rows_b[bbase + r] : 0;
     }
     for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
         tab[staged(t >> 3, t & 7)] =
@@ -453,15 +529,20 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
 
     unsigned long long* tab64 = reinterpret_cast<unsigned long long*>(tab);
     int32_t* tab32 = reinterpret_cast<int32_t*>(tab);
+    auto store_index = [&](int where, int32_t idx) {
+        const int wlb = where >> 4;
+        const int ws = where & 15;
+        tab32[staged(wlb, (kValDword0 + ws) >> 2) * 4 + (ws & 3)] = idx;
+    };
 
     for (int rb = 0; rb < cnt; rb += kBuildThreads * kBuildRecs) {
         int wslot[kBuildRecs];
-        int wrank[kBuildRecs];
         if (rb > 0) {
 #pragma unroll
             for (int k = 0; k < kBuildRecs; ++k) {
                 const int r = rb + k * kBuildThreads + tid;
                 codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
+                if constexpr (PROV) rows[k] = r < cnt ? pl.rows_b[bbase + r] : 0;
             }
         }
 #pragma unroll
@@ -469,136 +550,71 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
             const int r = rb + k * kBuildThreads + tid;
             wslot[k] = -1;
             if (r >= cnt) continue;
-            const uint64_t code = codes[k];
-
-            int lb = static_cast<int>(bucket_of(code, m.nb) - b0);
-            for (;;) {
-                uint64_t c[kSlots];
-#pragma unroll
-                for (int q = 0; q < kSlots / 2; ++q) {
-                    const uint4 w = tab[staged(lb, q)];
-                    c[2 * q] = static_cast<uint64_t>(w.x) |
-                               (static_cast<uint64_t>(w.y) << 32);
-                    c[2 * q + 1] = static_cast<uint64_t>(w.z) |
-                                   (static_cast<uint64_t>(w.w) << 32);
-                }
-                bool done = false;
-                uint32_t em = 0;
-#pragma unroll
-                for (int s = 0; s < kSlots; ++s) {
-                    done |= c[s] == code;
-                    em |= (c[s] == kEmpty ? 1u : 0u) << s;
-                }
-                while (!done && em) {
-                    const int s = __builtin_ctz(em);
-                    const unsigned long long old =
-                            atomicCAS(tab64 + staged(lb, s >> 1) * 2 + (s & 1),
-                                      kEmpty, code);
-                    if (old == kEmpty) {
-                        wslot[k] = lb * kBucketQwords + s;
-                        done = true;
-                    } else if (old == code) {
-                        done = true;
+            const int lb = static_cast<int>(bucket_of(codes[k], m.nb) - b0);
+            const int how = place_code(tab, codes[k], lb, nbk, wslot[k]);
+            if (how == kFull) atomicAdd(m.ctr + kCtrDropped, 1);   // refused
+            if constexpr (PROV) {
+                if (how == kPlaced) {
+                    // the promised position; re-pointed later if it turns out
+                    // to lie beyond the last position in use
+                    const int32_t pos = heap_base + rows[k];
+                    if (identity) {
+                        store_index(wslot[k], pos);   // the log was written by pass 1
+                    } else {
+                        const int32_t idx = m.heap[pos];
+                        store_index(wslot[k], idx);
+                        m.klog[idx] = codes[k];
                     }
-                    em &= em - 1;
-                }
-                if (done) break;
-                if (++lb == nbk) {
-                    // The probe sequence leaves this partition.
-                    pl.spill_b[atomicAdd(pl.hdr + kHdrSpillB, 1)] =
-                            static_cast<int32_t>(bbase + r);
-                    break;
+                } else {
+                    give_up_row(pl, rows[k], &s_losers, false);
                 }
             }
         }
-        // Winners are ranked in record order, so that consecutive lanes take
-        // consecutive heap entries and their value rows land side by side.
-#pragma unroll
-        for (int k = 0; k < kBuildRecs; ++k) {
-            const uint64_t wm = __ballot(wslot[k] >= 0);
-            wrank[k] = __popcll(wm & ((1ull << lane) - 1ull));
-            if (lane == 0) s_wcnt[k * (kBuildThreads / 64) + wave] = __popcll(wm);
-        }
-        // The first slice of the winners' value rows does not depend on the
-        // indices: it is requested now and travels while the heap counter and
-        // the heap entries are fetched.
-        uint32_t rows[kBuildRecs][kStageDwords];
-        auto load_rows = [&](int v, int q0) {
-            const int rd = va.row_dwords[v];
-            const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
+        if constexpr (!PROV) {
+            // Winners are ranked in record order, so that consecutive lanes
+            // take consecutive heap entries.
+            int wrank[kBuildRecs];
 #pragma unroll
             for (int k = 0; k < kBuildRecs; ++k) {
-                if (wslot[k] >= 0) {
-                    const uint32_t* s = pl.plane_b[v] +
-                            (bbase + rb + k * kBuildThreads + tid) * rd + q0;
-#pragma unroll
-                    for (int q = 0; q < kStageDwords; ++q) {
-                        if (q < w) rows[k][q] = s[q];
+                const uint64_t wm = __ballot(wslot[k] >= 0);
+                wrank[k] = __popcll(wm & ((1ull << lane) - 1ull));
+                if (lane == 0) s_wcnt[k * (kBuildThreads / 64) + wave] = __popcll(wm);
+            }
+            __syncthreads();
+            if (tid == 0) {
+                int tot = 0;
+                for (int q = 0; q < kBuildRecs * (kBuildThreads / 64); ++q) {
+                    const int c = s_wcnt[q];
+                    s_wcnt[q] = tot;
+                    tot += c;
+                }
+                int base = 0;
+                if (tot > 0) {
+                    base = atomicAdd(m.ctr + kCtrSize, tot);
+                    if (base + tot > m.capacity) {
+                        const int lo = base > m.capacity ? base : m.capacity;
+                        const int excess = base + tot - lo;
+                        atomicSub(m.ctr + kCtrSize, excess);
+                        atomicAdd(m.ctr + kCtrDropped, excess);
                     }
                 }
+                s_base = base;
             }
-        };
-        if (va.n > 0) load_rows(0, 0);
-        __syncthreads();
-        if (tid == 0) {
-            int tot = 0;
-            for (int q = 0; q < kBuildRecs * (kBuildThreads / 64); ++q) {
-                const int c = s_wcnt[q];
-                s_wcnt[q] = tot;
-                tot += c;
-            }
-            int base = 0;
-            if (tot > 0) {
-                base = atomicAdd(m.ctr + kCtrSize, tot);
-                if (base + tot > m.capacity) {
-                    const int lo = base > m.capacity ? base : m.capacity;
-                    const int excess = base + tot - lo;
-                    atomicSub(m.ctr + kCtrSize, excess);
-                    atomicAdd(m.ctr + kCtrDropped, excess);
-                }
-            }
-            s_base = base;
-        }
-        __syncthreads();
-        int32_t idx[kBuildRecs];
+            __syncthreads();
 #pragma unroll
-        for (int k = 0; k < kBuildRecs; ++k) {
-            idx[k] = -1;
-            if (wslot[k] < 0) continue;
-            const int top = s_base + s_wcnt[k * (kBuildThreads / 64) + wave] + wrank[k];
-            if (top < m.capacity) {
-                idx[k] = m.heap[top];
-            } else {
-                // Heap exhausted: give the slot up again.
-                const int wlb = wslot[k] >> 4;
-                const int ws = wslot[k] & 15;
-                tab64[staged(wlb, ws >> 1) * 2 + (ws & 1)] = kTomb;
-                atomicAdd(m.ctr + kCtrTombs, 1);
-                wslot[k] = -1;
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < kBuildRecs; ++k) {
-            if (idx[k] >= 0) {
-                const int wlb = wslot[k] >> 4;
-                const int ws = wslot[k] & 15;
-                tab32[staged(wlb, (kValDword0 + ws) >> 2) * 4 + (ws & 3)] = idx[k];
-            }
-        }
-        for (int v = 0; v < va.n; ++v) {
-            const int rd = va.row_dwords[v];
-            for (int q0 = 0; q0 < rd; q0 += kStageDwords) {
-                const int w = rd - q0 < kStageDwords ? rd - q0 : kStageDwords;
-                if (v > 0 || q0 > 0) load_rows(v, q0);
-#pragma unroll
-                for (int k = 0; k < kBuildRecs; ++k) {
-                    if (idx[k] >= 0) {
-                        uint32_t* o = va.dst[v] + static_cast<int64_t>(idx[k]) * rd + q0;
-#pragma unroll
-                        for (int q = 0; q < kStageDwords; ++q) {
-                            if (q < w) o[q] = rows[k][q];
-                        }
-                    }
+            for (int k = 0; k < kBuildRecs; ++k) {
+                if (wslot[k] < 0) continue;
+                const int top = s_base + s_wcnt[k * (kBuildThreads / 64) + wave] + wrank[k];
+                if (top < m.capacity) {
+                    const int32_t idx = identity ? top : m.heap[top];
+                    store_index(wslot[k], idx);
+                    m.klog[idx] = codes[k];
+                } else {
+                    // Heap exhausted: give the slot up again.
+                    const int wlb = wslot[k] >> 4;
+                    const int ws = wslot[k] & 15;
+                    tab64[staged(wlb, ws >> 1) * 2 + (ws & 1)] = kTomb;
+                    atomicAdd(m.ctr + kCtrTombs, 1);
                 }
             }
         }
@@ -606,6 +622,245 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
     }
     for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
         gl[t] = tab[staged(t >> 3, t & 7)];
+    }
+    if constexpr (PROV) {
+        if (tid == 0 && s_losers) atomicAdd(pl.hdr + kHdrLosers, s_losers);
+    }
+}
+
+// Provisional scheme, after the build pass: U = n - losers rows won a slot and
+// the heap positions base .. base + U - 1 are the ones in use.  Thread t moves
+// 32-bit word t of a value plane: row i = t / RD goes to the row of its
+// promised position when i is a winner below U; with the heap in its initial
+// order that is one contiguous copy.  RD = row width in words, 0 = read it from
+// `rd` (widths 1..4 are compiled in so that the division is by a constant).
+template <int RD>
+__device__ __forceinline__ void copy_plane(const MapDev& m, const BulkPlan& pl,
+                                           const uint32_t* __restrict__ src,
+                                           uint32_t* __restrict__ dst, int rd_runtime,
+                                           int64_t winners, int32_t heap_base, int identity) {
+    const uint32_t rd = RD > 0 ? static_cast<uint32_t>(RD) : static_cast<uint32_t>(rd_runtime);
+    const int64_t words = winners * rd;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kCopyThreads;
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * kCopyThreads + threadIdx.x;
+    const bool narrow = words <= 0xFFFFFFFFll;   // the common case: 32-bit divisions
+    auto row_of = [&](int64_t w) {
+        return narrow ? static_cast<int64_t>(static_cast<uint32_t>(w) / rd) : w / rd;
+    };
+    auto move_word = [&](int64_t w) {
+        const int64_t row = row_of(w);
+        if (pl.flags[row] != 0) return;
+        const uint32_t q = static_cast<uint32_t>(w - row * rd);
+        const int64_t pos = heap_base + row;
+        const int64_t idx = identity ? pos : m.heap[pos];
+        dst[idx * rd + q] = src[w];
+    };
+    uint32_t* __restrict__ to = dst + static_cast<int64_t>(heap_base) * rd;
+    const bool wide = identity && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(to) % 16 == 0;
+    if (!wide) {
+        for (int64_t w = tid; w < words; w += stride) move_word(w);
+        return;
+    }
+    // With the heap in its initial order the rows go to one contiguous range
+    // that starts at `to`: 16 bytes per thread wherever none of the (up to four)
+    // rows under them lost; the flags are not even read when no row lost.
+    const bool clean = pl.hdr[kHdrLosers] == 0;
+    const int64_t quads = words / 4;
+    for (int64_t t = tid; t < quads; t += stride) {
+        bool all = clean;
+        if (!clean) {
+            const int64_t lo = row_of(4 * t), hi = row_of(4 * t + 3);
+            all = true;
+            for (int64_t r = lo; r <= hi; ++r) all = all && pl.flags[r] == 0;
+        }
+        if (all) {
+            reinterpret_cast<uint4*>(to)[t] = reinterpret_cast<const uint4*>(src)[t];
+        } else {
+            for (int q = 0; q < 4; ++q) move_word(4 * t + q);
+        }
+    }
+    if (tid < words - 4 * quads) move_word(4 * quads + tid);
+}
+
+__global__ __launch_bounds__(kCopyThreads) void copy_rows_kernel(
+        MapDev m, BulkPlan pl, ValueArgs va, int identity) {
+    const int32_t heap_base = pl.hdr[kHdrBase];
+    const int64_t winners = pl.n - pl.hdr[kHdrLosers];
+    for (int v = 0; v < va.n; ++v) {
+        const int rd = va.row_dwords[v];
+        switch (rd) {
+            case 1:
+                copy_plane<1>(m, pl, va.src[v], va.dst[v], rd, winners, heap_base, identity);
+                break;
+            case 2:
+                copy_plane<2>(m, pl, va.src[v], va.dst[v], rd, winners, heap_base, identity);
+                break;
+            case 3:
+                copy_plane<3>(m, pl, va.src[v], va.dst[v], rd, winners, heap_base, identity);
+                break;
+            case 4:
+                copy_plane<4>(m, pl, va.src[v], va.dst[v], rd, winners, heap_base, identity);
+                break;
+            default:
+                copy_plane<0>(m, pl, va.src[v], va.dst[v], rd, winners, heap_base, identity);
+                break;
+        }
+    }
+}
+
+// Positions of `mine` set lanes of the workgroup in a list that grows through
+// the counter `cursor`: one update of the counter per workgroup (updates of a
+// single address serialise across the device).  Every thread calls this; the
+// return value is the caller's position (meaningful when `mine`).
+constexpr int kListThreads = 1024;
+
+__device__ __forceinline__ int reserve_in_list(bool mine, int32_t* cursor, int* s_wave,
+                                               int* s_first) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const uint64_t mm = __ballot(mine);
+    if (lane == 0) s_wave[wave] = __popcll(mm);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int tot = 0;
+        for (int q = 0; q < kListThreads / 64; ++q) {
+            const int c = s_wave[q];
+            s_wave[q] = tot;
+            tot += c;
+        }
+        *s_first = tot ? atomicAdd(cursor, tot) : 0;
+    }
+    __syncthreads();
+    const int at = *s_first + s_wave[wave] + __popcll(mm & ((1ull << lane) - 1ull));
+    __syncthreads();   // s_wave / s_first are reused by the next call
+    return at;
+}
+
+// Provisional scheme, only when rows lost: the losers below row U are the
+// holes that the winners at or beyond U move into.  Sixteen flags per thread;
+// a workgroup that meets no loser (the usual case: a handful of rows lost among
+// millions) goes on without touching the list.
+__global__ __launch_bounds__(kListThreads) void list_holes_kernel(BulkPlan pl) {
+    __shared__ int s_wave[kListThreads / 64];
+    __shared__ int s_first;
+    const int32_t losers = pl.hdr[kHdrLosers];
+    if (losers == 0) return;
+    const int64_t winners = pl.n - losers;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    for (int64_t first = static_cast<int64_t>(blockIdx.x) * kListThreads * 16; first < winners;
+         first += static_cast<int64_t>(gridDim.x) * kListThreads * 16) {
+        const int64_t i0 = first + static_cast<int64_t>(threadIdx.x) * 16;
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (i0 + 16 <= winners) {
+            // flags start 256-byte aligned and i0 is a multiple of 16
+            const uint4 q = *reinterpret_cast<const uint4*>(pl.flags + i0);
+            w[0] = q.x;
+            w[1] = q.y;
+            w[2] = q.z;
+            w[3] = q.w;
+        } else {
+            for (int b = 0; b < 16 && i0 + b < winners; ++b) {
+                w[b >> 2] |= static_cast<uint32_t>(pl.flags[i0 + b] != 0) << (8 * (b & 3));
+            }
+        }
+        int cnt = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            cnt += (w[q] & 0xFFu ? 1 : 0) + (w[q] & 0xFF00u ? 1 : 0) +
+                   (w[q] & 0xFF0000u ? 1 : 0) + (w[q] & 0xFF000000u ? 1 : 0);
+        }
+        if (!__syncthreads_or(cnt)) continue;
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int tot = 0;
+            for (int q = 0; q < kListThreads / 64; ++q) {
+                const int c = s_wave[q];
+                s_wave[q] = tot;
+                tot += c;
+            }
+            s_first = atomicAdd(pl.hdr + kHdrHoles, tot);
+        }
+        __syncthreads();
+        int at = s_first + s_wave[wave] + incl - cnt;
+        for (int b = 0; b < 16 && cnt > 0; ++b) {
+            if ((w[b >> 2] >> (8 * (b & 3))) & 0xFFu) {
+                pl.holes[at++] = static_cast<int32_t>(i0 + b);
+            }
+        }
+        __syncthreads();   // s_wave / s_first are reused by the next round
+    }
+}
+
+// The slot that holds `code` (which is stored), by one lane on its own.
+__device__ __forceinline__ int32_t* locate_index(const MapDev& m, uint64_t code) {
+    uint32_t b = bucket_of(code, m.nb);
+    for (uint32_t steps = 0; steps < kPartBuckets; ++steps) {
+        const uint64_t* line = m.buckets + static_cast<size_t>(b) * kBucketQwords;
+        for (int s = 0; s < kSlots; ++s) {
+            if (line[s] == code) {
+                return reinterpret_cast<int32_t*>(m.buckets) +
+                       static_cast<size_t>(b) * kBucketDwords + kValDword0 + s;
+            }
+        }
+        b = next_bucket(b, m.nb);
+    }
+    return nullptr;
+}
+
+// Provisional scheme, last step: sets the heap counter, and if rows lost,
+// moves every winner at or beyond row U into a hole below U: its slot gets the
+// index of the hole's position and its value rows are copied there.
+template <int DIM>
+__global__ __launch_bounds__(kListThreads) void settle_rows_kernel(
+        MapDev m, BulkPlan pl, const int32_t* __restrict__ keys, ValueArgs va,
+        int identity) {
+    __shared__ int s_wave[kListThreads / 64];
+    __shared__ int s_first;
+    const int32_t heap_base = pl.hdr[kHdrBase];
+    const int32_t losers = pl.hdr[kHdrLosers];
+    const int64_t winners = pl.n - losers;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        m.ctr[kCtrSize] = heap_base + static_cast<int32_t>(winners);
+    }
+    if (losers == 0) return;
+    const int64_t fit = rows_that_fit(m, pl);
+    for (int64_t first = winners + static_cast<int64_t>(blockIdx.x) * kListThreads; first < fit;
+         first += static_cast<int64_t>(gridDim.x) * kListThreads) {
+        const int64_t i = first + threadIdx.x;
+        const bool high = i < fit && pl.flags[i] == 0;
+        const int at = reserve_in_list(high, pl.hdr + kHdrTaken, s_wave, &s_first);
+        // positions from base + U on are free again: those of the rows that lost
+        // (pass 1 has written their log entry when the heap is in its initial
+        // order) and those that the high winners leave
+        if (i < fit && (identity || high)) {
+            const int64_t old_pos = heap_base + i;
+            m.klog[identity ? old_pos : static_cast<int64_t>(m.heap[old_pos])] = kEmpty;
+        }
+        if (!high) continue;
+        const int64_t pos = heap_base + pl.holes[at];
+        const int32_t idx = identity ? static_cast<int32_t>(pos) : m.heap[pos];
+        int32_t key[DIM];
+        load_key<DIM>(keys, i, true, key);
+        uint64_t code;
+        pack_key<DIM>(key, code);
+        int32_t* slot = locate_index(m, code);
+        if (slot != nullptr) *slot = idx;
+        m.klog[idx] = code;
+        for (int v = 0; v < va.n; ++v) {
+            const int rd = va.row_dwords[v];
+            const uint32_t* s = va.src[v] + i * rd;
+            uint32_t* d = va.dst[v] + static_cast<int64_t>(idx) * rd;
+            for (int q = 0; q < rd; ++q) d[q] = s[q];
+        }
     }
 }
 
@@ -620,6 +875,52 @@ int check_values(int n_values, const void* const* src, void* const* dst,
         if (src[v] == nullptr || dst[v] == nullptr) ASH_FAIL("null value tensor");
         if (row_bytes[v] <= 0) ASH_FAIL("value rows must not be empty");
     }
+    return 0;
+}
+
+template <bool PROV>
+int launch_split_keys(ash_map* map, const BulkPlan& pl, const int32_t* keys, int identity,
+                      hipStream_t s) {
+    const unsigned g = static_cast<unsigned>((pl.n + kSplitChunk - 1) / kSplitChunk);
+    switch (map->key_dim) {
+        case 1:
+            split_keys_kernel<1, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            break;
+        case 2:
+            split_keys_kernel<2, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            break;
+        case 3:
+            split_keys_kernel<3, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            break;
+        default:
+            split_keys_kernel<4, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_settle_rows(ash_map* map, const BulkPlan& pl, const int32_t* keys,
+                       const ValueArgs& va, int identity, hipStream_t s) {
+    // both leave at once when no row lost: grids that cost little to launch
+    constexpr unsigned g = 128;
+    list_holes_kernel<<<g, kListThreads, 0, s>>>(pl);
+    ASH_LAUNCH_CHECK();
+    switch (map->key_dim) {
+        case 1:
+            settle_rows_kernel<1><<<g, kListThreads, 0, s>>>(map->d, pl, keys, va, identity);
+            break;
+        case 2:
+            settle_rows_kernel<2><<<g, kListThreads, 0, s>>>(map->d, pl, keys, va, identity);
+            break;
+        case 3:
+            settle_rows_kernel<3><<<g, kListThreads, 0, s>>>(map->d, pl, keys, va, identity);
+            break;
+        default:
+            settle_rows_kernel<4><<<g, kListThreads, 0, s>>>(map->d, pl, keys, va, identity);
+            break;
+    }
+    ASH_LAUNCH_CHECK();
     return 0;
 }
 
@@ -642,8 +943,7 @@ int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
         // The build pass streams the whole table once, the per-key kernel costs
         // about as much per key as streaming three buckets.  Measured on
         // MI355X (16 M-slot table): keys only, the streaming path wins from
-        // about one key per bucket; with value rows, which travel through both
-        // split passes, from about 1.5.
+        // about one key per bucket; with value rows from about 1.5.
         // A table below 2^19 buckets has too few partitions to fill the device
         // in the build pass (a batch that large for it is mostly duplicates,
         // which the per-key kernel handles without atomics).
@@ -674,58 +974,58 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (map->table_stale) {
+        // A cleared table whose fill is still pending is rewritten whole by the
+        // build pass.  Captured into a graph that decision would be replayed
+        // against whatever the table holds then.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &capturing) == hipSuccess &&
+            capturing != hipStreamCaptureStatusNone) {
+            ASH_FAIL("the table was cleared and not used since: run one call outside the capture first");
+        }
+    }
 
     ValueArgs user = {};
-    ValueArgs from_a = {};
-    ValueArgs from_b = {};
-    user.n = from_a.n = from_b.n = n_values;
+    user.n = n_values;
     for (int v = 0; v < n_values; ++v) {
-        const int32_t rd = static_cast<int32_t>(row_bytes[v] / 4);
         user.src[v] = static_cast<const uint32_t*>(src[v]);
-        from_a.src[v] = pl.plane_a[v];
-        from_b.src[v] = pl.plane_b[v];
-        user.dst[v] = from_a.dst[v] = from_b.dst[v] = static_cast<uint32_t*>(dst[v]);
-        user.row_dwords[v] = from_a.row_dwords[v] = from_b.row_dwords[v] = rd;
+        user.dst[v] = static_cast<uint32_t*>(dst[v]);
+        user.row_dwords[v] = static_cast<int32_t>(row_bytes[v] / 4);
     }
+    const ValueArgs none = {};
+    const int stale = map->table_stale ? 1 : 0;
+    const int identity = map->heap_dirty ? 0 : 1;
 
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);
-    bulk_init_kernel<<<(ncursors + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
+    const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
+    bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
-    const unsigned g1 = static_cast<unsigned>((n + kSplitChunk - 1) / kSplitChunk);
-    switch (map->key_dim) {
-        case 1:
-            split_keys_kernel<1><<<g1, kSplitThreads, 0, s>>>(map->d, pl, keys, user);
-            break;
-        case 2:
-            split_keys_kernel<2><<<g1, kSplitThreads, 0, s>>>(map->d, pl, keys, user);
-            break;
-        case 3:
-            split_keys_kernel<3><<<g1, kSplitThreads, 0, s>>>(map->d, pl, keys, user);
-            break;
-        default:
-            split_keys_kernel<4><<<g1, kSplitThreads, 0, s>>>(map->d, pl, keys, user);
-            break;
+    if (n_values == 0) {
+        if (launch_split_keys<false>(map, pl, keys, identity, s)) return 1;
+        split_records_kernel<false><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
+        ASH_LAUNCH_CHECK();
+        build_kernel<false><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
+        ASH_LAUNCH_CHECK();
+        map->table_stale = false;
+        if (insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys, none, s)) {
+            return 1;
+        }
+        return insert_selected(map, true, pl.codes_a, pl.spill_a, pl.hdr + kHdrSpillA, none, s);
     }
+    if (launch_split_keys<true>(map, pl, keys, identity, s)) return 1;
+    split_records_kernel<true><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
-    split_records_kernel<<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl,
-                                                                      user);
-    ASH_LAUNCH_CHECK();
-    // A cleared table whose fill is still pending is empty by its counters, so
-    // the build starts every partition from scratch and writes all of them.
-    build_kernel<<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, from_b,
-                                                    map->table_stale ? 1 : 0);
+    build_kernel<true><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
     ASH_LAUNCH_CHECK();
     map->table_stale = false;
-    if (insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys,
-                        user, s)) {
-        return 1;
-    }
-    if (insert_selected(map, true, pl.codes_a, pl.spill_a, pl.hdr + kHdrSpillA,
-                        from_a, s)) {
-        return 1;
-    }
-    return insert_selected(map, true, pl.codes_b, pl.spill_b,
-                           pl.hdr + kHdrSpillB, from_b, s);
+    int64_t words = 0;
+    for (int v = 0; v < n_values; ++v) words = words > n * user.row_dwords[v] ? words : n * user.row_dwords[v];
+    int64_t blocks = (words + kCopyThreads - 1) / kCopyThreads;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    copy_rows_kernel<<<static_cast<unsigned>(blocks), kCopyThreads, 0, s>>>(map->d, pl, user, identity);
+    ASH_LAUNCH_CHECK();
+    if (launch_settle_rows(map, pl, keys, user, identity, s)) return 1;
+    return insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys, user, s);
 }
 
 }  // extern "C"

@@ -44,6 +44,17 @@ constexpr int kTargetFill = 6;                  // entries per bucket at capacit
 constexpr uint64_t kEmpty = ~0ull;
 constexpr uint64_t kTomb = ~0ull - 1ull;
 
+// A probe sequence never leaves the aligned range of 512 buckets (64 KB) that
+// the key's hash names: from the range's last bucket it goes on at its first.
+// The streaming insert builds one such range per workgroup in LDS, and a range
+// is what a key's neighbours in the table share in the caches.  At the table's
+// load (six entries per ten-slot bucket at capacity) a range that is full is
+// out of reach (its 5120 slots against a mean of 3072 entries with a standard
+// deviation of 55); a key that finds its range full is refused and counted
+// like a key that finds the heap exhausted.
+constexpr int kPartShift = 9;
+constexpr uint32_t kPartBuckets = 1u << kPartShift;
+
 // Device counters kept in the first 256 bytes of the table workspace.
 enum Counter {
     kCtrSize = 0,      // heap counter == number of live entries
@@ -65,6 +76,12 @@ constexpr int32_t kGenNoIndex = -4;  // key visible, index not yet assigned
 
 struct MapDev {
     uint64_t* buckets;   // nb * 16 qwords
+    // key log: klog[index] = packed code of the key stored under `index`,
+    // kTomb when that key lives in the general region, kEmpty when the index
+    // is free.  items() enumerates from here (8 bytes per index instead of the
+    // whole bucket array) and therefore in index order, which is the order of
+    // the callers' value rows.
+    uint64_t* klog;      // capacity qwords
     int32_t* ctr;        // kNumCounters int32
     int32_t* heap;       // capacity int32 (caller-owned)
     int32_t* gstate;     // general region state/index words (or nullptr)
@@ -77,6 +94,17 @@ struct MapDev {
 inline int64_t num_buckets(int64_t capacity) {
     int64_t nb = (capacity + kTargetFill - 1) / kTargetFill;
     return nb < 2 ? 2 : nb;
+}
+
+// Byte offset of the key log inside the table workspace.
+inline int64_t klog_offset(int64_t capacity) {
+    const int64_t end = kHeaderBytes + num_buckets(capacity) * kBucketDwords * 4;
+    return (end + 255) & ~int64_t{255};
+}
+
+inline int64_t table_workspace_bytes(int64_t capacity) {
+    // whole 16-byte units: the log is cleared and read two entries at a time
+    return klog_offset(capacity) + ((capacity + 1) / 2) * 16;
 }
 
 inline int64_t general_slots(int64_t capacity) {

@@ -284,7 +284,7 @@ __device__ __forceinline__ bool find_key(const MapDev& m, const int32_t (&k)[DIM
                 pend = false;
             } else {
                 b = next_bucket(b, m.nb);
-                if (++steps >= m.nb) pend = false;
+                if (++steps >= kPartBuckets) pend = false;
             }
         }
     }
@@ -344,7 +344,7 @@ __device__ __forceinline__ bool find_key_shared(const MapDev& m, const int32_t (
                 pend = false;
             } else {
                 b = next_bucket(b, m.nb);
-                if (++steps >= m.nb) pend = false;
+                if (++steps >= kPartBuckets) pend = false;
             }
         }
     }
@@ -395,7 +395,7 @@ __device__ __forceinline__ bool find_key_alone(const MapDev& m, const int32_t (&
             pend = false;
         } else {
             b = next_bucket(b, m.nb);
-            if (++steps >= m.nb) pend = false;
+            if (++steps >= kPartBuckets) pend = false;
         }
     }
     if (active && !fits) {
@@ -540,7 +540,7 @@ __device__ __forceinline__ void insert_key(
                 }
                 if (pend) {
                     b = next_bucket(b, m.nb);
-                    if (++steps >= m.nb) {
+                    if (++steps >= kPartBuckets) {
                         pend = false;
                         refused = true;
                     }
@@ -613,9 +613,11 @@ __device__ __forceinline__ void insert_key(
     if (idx >= 0) {
         if (won) {
             *value_ptr(m, wb, ws) = idx;
+            if (idx < m.capacity) m.klog[idx] = code;   // (a loaded index may be anything)
         } else {
             __hip_atomic_store(m.gstate + gp, idx, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
+            if (idx < m.capacity) m.klog[idx] = kTomb;   // "stored in the general region"
         }
         if constexpr (MODE == kInsertFused) {
 #pragma unroll
@@ -1037,7 +1039,7 @@ __global__ __launch_bounds__(kEraseBlock) void erase_kernel(
                 pend = false;
             } else {
                 b = next_bucket(b, m.nb);
-                if (++steps >= m.nb) pend = false;
+                if (++steps >= kPartBuckets) pend = false;
             }
         }
     }
@@ -1080,92 +1082,85 @@ __global__ __launch_bounds__(kEraseBlock) void erase_kernel(
         for (int q = 0; q < wave; ++q) below += s_cnt[q];
         const int pos = s_base - 1 - below;
         if (pos >= 0 && pos < m.capacity) m.heap[pos] = idx;
+        m.klog[idx] = kEmpty;
     }
 }
 
-// items(): thread t reads the 16-byte unit t of the bucket array (two code
-// slots, or index words for the last lanes of a line), four units per thread.
-// Output positions come from one global cursor; atomics on that single address
-// serialise (about 7 ns each across the XCDs), so the workgroup is made as
-// large as possible (1024 threads, one atomic per 4096 units): with 256-thread
-// groups the cursor alone cost more than reading the whole table.
+// items(): the live entries are read from the key log (8 bytes per index,
+// against 21 bytes per index of bucket array).  A workgroup takes 8192
+// consecutive indices, each of its wavefronts 512 of them in eight rounds of
+// 64, so that reads are contiguous and -- positions being ranks in index order
+// -- so are the writes of every round; the entries of a workgroup come out
+// sorted by index, workgroups in the order in which they reserve their output
+// range.  `limit` indices are scanned: the capacity, or -- when nothing has
+// written to the heap since it was last 0, 1, 2, ... (`identity`) and the
+// indices in use therefore are 0 .. size-1 -- only the size.
+// Output ranges come from one global cursor; atomics on that single address
+// serialise (about 7 ns each across the XCDs), hence the large workgroups.
 constexpr int kItemsBlock = 1024;
-constexpr int kItemsUnroll = 4;
+constexpr int kItemsRounds = 8;
+constexpr int kItemsSpan = kItemsBlock * kItemsRounds;   // indices per workgroup
 
 template <int DIM>
 __global__ __launch_bounds__(kItemsBlock) void items_kernel(
         MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out,
-        int64_t n_expected) {
-    constexpr int kUnroll = kItemsUnroll;
+        int64_t n_expected, int identity) {
     constexpr int kWaves = kItemsBlock / 64;
+    __shared__ int s_cnt[kWaves * kItemsRounds];
+    __shared__ int s_base;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int j = lane & (kGroup - 1);
-    const bool v0 = (2 * j) < kSlots;
-    const bool v1 = (2 * j + 1) < kSlots;
-    const uint64_t units = static_cast<uint64_t>(m.nb) * kGroup;
-    const uint64_t t0 =
-            static_cast<uint64_t>(blockIdx.x) * (kItemsBlock * kUnroll) +
-            threadIdx.x;
-    uint64_t qa[kUnroll], qb[kUnroll];
-    int32_t va[kUnroll], vb[kUnroll];
-    bool l0[kUnroll], l1[kUnroll];
-    int cnt = 0;
-    // The index of slot s is dword 20+s of the line: for the code lane j (slots
-    // 2j, 2j+1) that is lane 5 + j/2 of the same group, components x,y (j even)
-    // or z,w (j odd).
-    const int vsrc = (lane & ~(kGroup - 1)) + 5 + (j >> 1);
+    const int64_t limit = identity ? static_cast<int64_t>(m.ctr[kCtrSize])
+                                   : static_cast<int64_t>(m.capacity);
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * kItemsSpan;
+    if (first >= limit) return;
+    const int64_t mine = first + wave * (64 * kItemsRounds) + lane;
+    uint64_t code[kItemsRounds];
+    int rank[kItemsRounds];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-        const uint64_t t = t0 + static_cast<uint64_t>(u) * kItemsBlock;
-        uint4 q = make_uint4(~0u, ~0u, ~0u, ~0u);
-        if (t < units) q = reinterpret_cast<const uint4*>(m.buckets)[t];
-        const int sx = __shfl(static_cast<int>(q.x), vsrc);
-        const int sy = __shfl(static_cast<int>(q.y), vsrc);
-        const int sz = __shfl(static_cast<int>(q.z), vsrc);
-        const int sw = __shfl(static_cast<int>(q.w), vsrc);
-        va[u] = (j & 1) ? sz : sx;
-        vb[u] = (j & 1) ? sw : sy;
-        qa[u] = static_cast<uint64_t>(q.x) | (static_cast<uint64_t>(q.y) << 32);
-        qb[u] = static_cast<uint64_t>(q.z) | (static_cast<uint64_t>(q.w) << 32);
-        l0[u] = v0 && qa[u] < kTomb;
-        l1[u] = v1 && qb[u] < kTomb;
-        cnt += (l0[u] ? 1 : 0) + (l1[u] ? 1 : 0);
+    for (int r = 0; r < kItemsRounds; ++r) {
+        const int64_t i = mine + r * 64;
+        code[r] = i < limit ? m.klog[i] : kEmpty;
+        const uint64_t live = __ballot(code[r] < kTomb);
+        rank[r] = __popcll(live & ((1ull << lane) - 1ull));
+        if (lane == 0) s_cnt[wave * kItemsRounds + r] = __popcll(live);
     }
-    // exclusive scan of cnt over the block
-    int incl = cnt;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d);
-        if (lane >= d) incl += up;
-    }
-    __shared__ int s_cnt[kWaves];
-    __shared__ int s_base;
-    if (lane == 63) s_cnt[wave] = incl;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int tot = 0;
+    // exclusive scan of the 128 counts by the first two wavefronts
+    const bool scanner = threadIdx.x < kWaves * kItemsRounds;
+    int c = 0, incl = 0;
+    if (scanner) {
+        c = s_cnt[threadIdx.x];
+        incl = c;
 #pragma unroll
-        for (int q = 0; q < kWaves; ++q) tot += s_cnt[q];
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+    }
+    __syncthreads();
+    if (scanner) {
+        s_cnt[threadIdx.x] = incl - c;
+        if (threadIdx.x == 63) s_base = incl;   // total of the first 64 counts
+    }
+    __syncthreads();
+    if (scanner && threadIdx.x >= 64) s_cnt[threadIdx.x] += s_base;
+    __syncthreads();
+    if (threadIdx.x == kWaves * kItemsRounds - 1) {
+        const int tot = s_cnt[threadIdx.x] + c;
         s_base = tot > 0 ? atomicAdd(m.ctr + kCtrCursor, tot) : 0;
     }
     __syncthreads();
-    int64_t pos = s_base + (incl - cnt);
-    for (int q = 0; q < wave; ++q) pos += s_cnt[q];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int r = 0; r < kItemsRounds; ++r) {
+        if (code[r] < kTomb) {
+            const int64_t pos = static_cast<int64_t>(s_base) + s_cnt[wave * kItemsRounds + r] + rank[r];
+            if (pos < n_expected) {
+                int32_t k[DIM];
+                unpack_key<DIM>(code[r], k);
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const bool live = h == 0 ? l0[u] : l1[u];
-            if (live) {
-                if (pos < n_expected) {
-                    int32_t k[DIM];
-                    unpack_key<DIM>(h == 0 ? qa[u] : qb[u], k);
-#pragma unroll
-                    for (int d = 0; d < DIM; ++d) keys_out[pos * DIM + d] = k[d];
-                    idx_out[pos] = h == 0 ? va[u] : vb[u];
-                }
-                ++pos;
+                for (int d = 0; d < DIM; ++d) keys_out[pos * DIM + d] = k[d];
+                idx_out[pos] = mine + r * 64;
             }
         }
     }
@@ -1209,6 +1204,27 @@ __global__ __launch_bounds__(kBlock) void fill16_kernel(uint4* __restrict__ p,
     }
 }
 
+// klog[0 .. limit) := free, limit = the capacity or (prefix_only) the size
+// counter rounded up to whole 16-byte units.  The log's allocation is a
+// multiple of 16 bytes plus slack (256-byte aligned workspace regions), so the
+// last unit of an odd capacity is written whole.
+__global__ __launch_bounds__(kBlock) void empty_log_kernel(
+        uint4* __restrict__ log16, int64_t capacity, const int32_t* __restrict__ ctr,
+        int prefix_only) {
+    int64_t entries = capacity;
+    if (prefix_only) {
+        const int64_t used = ctr[kCtrSize];
+        entries = used < capacity ? used : capacity;
+    }
+    const int64_t n16 = (entries + 1) / 2;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    const uint4 v = make_uint4(~0u, ~0u, ~0u, ~0u);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n16;
+         i += stride) {
+        log16[i] = v;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void reset_heap_kernel(
         int32_t* __restrict__ heap, int64_t capacity, int32_t* __restrict__ ctr,
         int32_t size_value, bool write_heap) {
@@ -1233,6 +1249,61 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(
         const int64_t u = t - row * units_per_row;
         const int32_t a = assigned[row];
         if (a >= 0) dst[static_cast<int64_t>(a) * units_per_row + u] = src[t];
+    }
+}
+
+// Row gather for up to kMaxFusedValues tensors at once: word t of output plane
+// v is word t % rd of row indices[t / rd] of source plane v.  One launch reads
+// the indices once per word of a row (the repeats hit the first-level cache);
+// with indices in ascending runs, as items() returns them, source reads are
+// contiguous.  RD = row width in words, 0 = read it from the arguments.
+struct GatherArgs {
+    int n;
+    const uint32_t* src[kMaxFusedValues];
+    uint32_t* dst[kMaxFusedValues];
+    int32_t row_dwords[kMaxFusedValues];
+    int64_t src_rows[kMaxFusedValues];
+};
+
+template <int RD>
+__device__ __forceinline__ void gather_plane(const uint32_t* __restrict__ src,
+                                             uint32_t* __restrict__ dst, int rd_runtime,
+                                             const int64_t* __restrict__ indices, int64_t n,
+                                             int64_t src_rows) {
+    const uint32_t rd = RD > 0 ? static_cast<uint32_t>(RD) : static_cast<uint32_t>(rd_runtime);
+    const int64_t words = n * rd;
+    const bool narrow = words <= 0xFFFFFFFFll;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; t < words;
+         t += stride) {
+        const int64_t row = narrow ? static_cast<int64_t>(static_cast<uint32_t>(t) / rd) : t / rd;
+        const uint32_t q = static_cast<uint32_t>(t - row * rd);
+        const int64_t from = indices[row];
+        // an index outside the source reads as zero instead of faulting
+        dst[t] = (from >= 0 && from < src_rows) ? src[from * rd + q] : 0u;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(
+        GatherArgs a, const int64_t* __restrict__ indices, int64_t n) {
+    for (int v = 0; v < a.n; ++v) {
+        switch (a.row_dwords[v]) {
+            case 1:
+                gather_plane<1>(a.src[v], a.dst[v], 1, indices, n, a.src_rows[v]);
+                break;
+            case 2:
+                gather_plane<2>(a.src[v], a.dst[v], 2, indices, n, a.src_rows[v]);
+                break;
+            case 3:
+                gather_plane<3>(a.src[v], a.dst[v], 3, indices, n, a.src_rows[v]);
+                break;
+            case 4:
+                gather_plane<4>(a.src[v], a.dst[v], 4, indices, n, a.src_rows[v]);
+                break;
+            default:
+                gather_plane<0>(a.src[v], a.dst[v], a.row_dwords[v], indices, n, a.src_rows[v]);
+                break;
+        }
     }
 }
 
@@ -1378,6 +1449,17 @@ int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool
                 reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
         ASH_LAUNCH_CHECK();
     }
+    // The key log: every index is free again.  While nothing has written to the
+    // heap since its last reset the indices in use are 0 .. size-1, and only
+    // that part of the log (the size is read on the device, before the counters
+    // are reset below) needs clearing.
+    {
+        const int64_t n16 = (map->capacity + 1) / 2;
+        empty_log_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
+                reinterpret_cast<uint4*>(map->d.klog), map->capacity, map->d.ctr,
+                map->heap_dirty ? 0 : 1);
+        ASH_LAUNCH_CHECK();
+    }
     // Inserts only read the heap; while nothing has written to it since the
     // last reset it still is 0, 1, 2, ... and only the counters are reset.
     const bool rewrite = write_heap && map->heap_dirty;
@@ -1420,7 +1502,9 @@ template <int MODE>
 int launch_selected(ash_map* map, bool codes, const int32_t* keys,
                     const int32_t* sel, const int32_t* nsel,
                     const ValueArgs& va, hipStream_t s) {
-    constexpr unsigned g = 512;
+    // the selection is empty or short as a rule: a grid that costs little to
+    // launch, whose workgroups stride over a long one
+    constexpr unsigned g = 128;
     if (codes) {
         insert_selected_kernel<1, MODE, true>
                 <<<g, kHeapBlock, 0, s>>>(map->d, keys, sel, nsel, va);
@@ -1496,9 +1580,7 @@ int ash_map_workspace_bytes(int key_dim, int64_t capacity, int64_t* table_bytes,
     if (capacity < 1 || capacity > 0x7FFFFFF0ll) {
         ASH_FAIL("capacity must be in 1..2^31-16");
     }
-    if (table_bytes) {
-        *table_bytes = kHeaderBytes + num_buckets(capacity) * kBucketDwords * 4;
-    }
+    if (table_bytes) *table_bytes = table_workspace_bytes(capacity);
     if (general_bytes) *general_bytes = general_slots(capacity) * 20;
     return 0;
 }
@@ -1528,6 +1610,8 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
+    map->d.klog = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
+                                              klog_offset(capacity));
     map->d.heap = heap;
     map->d.gstate = nullptr;
     map->d.gkeys = nullptr;
@@ -1893,6 +1977,42 @@ int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
     return 0;
 }
 
+int ash_gather_rows(int n_values, const void* const* src, void* const* dst,
+                    const int64_t* row_bytes, const int64_t* src_rows,
+                    const int64_t* indices, int64_t n, void* stream) {
+    if (n_values < 1 || n_values > kMaxFusedValues) {
+        ASH_FAIL("gather_rows takes 1.." + std::to_string(kMaxFusedValues) + " tensors per call");
+    }
+    if (n < 0) ASH_FAIL("negative row count");
+    if (src == nullptr || dst == nullptr || row_bytes == nullptr || src_rows == nullptr) {
+        ASH_FAIL("null value tables");
+    }
+    if (n == 0) return 0;
+    if (indices == nullptr) ASH_FAIL("null indices pointer");
+    GatherArgs a = {};
+    a.n = n_values;
+    int64_t most = 0;
+    for (int v = 0; v < n_values; ++v) {
+        if (src[v] == nullptr || dst[v] == nullptr) ASH_FAIL("null value tensor");
+        if (row_bytes[v] <= 0 || row_bytes[v] % 4 != 0) {
+            ASH_FAIL("gather_rows: rows must be a positive multiple of 4 bytes");
+        }
+        if (src_rows[v] < 0) ASH_FAIL("negative source row count");
+        a.src[v] = static_cast<const uint32_t*>(src[v]);
+        a.dst[v] = static_cast<uint32_t*>(dst[v]);
+        a.row_dwords[v] = static_cast<int32_t>(row_bytes[v] / 4);
+        a.src_rows[v] = src_rows[v];
+        const int64_t words = n * a.row_dwords[v];
+        most = words > most ? words : most;
+    }
+    PointerGuard guard;
+    ASH_HIP(guard.enter_for(indices));
+    gather_rows_kernel<<<capped_grid(most), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+            a, indices, n);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
 int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
                    const void* const* src, void* const* dst,
                    const int64_t* row_bytes, int32_t* assigned, void* stream) {
@@ -2048,24 +2168,24 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     if (settle_table(map, s)) return 1;
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrCursor, 0);
     ASH_LAUNCH_CHECK();
-    const int64_t units = static_cast<int64_t>(map->d.nb) * kGroup;
-    const unsigned g = grid_for(units, kItemsBlock * kItemsUnroll);
+    const unsigned g = grid_for(map->capacity, kItemsSpan);
+    const int identity = map->heap_dirty ? 0 : 1;
     switch (map->key_dim) {
         case 1:
             items_kernel<1><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
-                                                 n_expected);
+                                                 n_expected, identity);
             break;
         case 2:
             items_kernel<2><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
-                                                 n_expected);
+                                                 n_expected, identity);
             break;
         case 3:
             items_kernel<3><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
-                                                 n_expected);
+                                                 n_expected, identity);
             break;
         default:
             items_kernel<4><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
-                                                 n_expected);
+                                                 n_expected, identity);
             break;
     }
     ASH_LAUNCH_CHECK();

@@ -73,8 +73,12 @@ __device__ __forceinline__ uint32_t bucket_of(uint64_t code, uint32_t nb) {
     return __umulhi(static_cast<uint32_t>(mix64(code) >> 32), nb);
 }
 
+// The bucket after b in b's probe sequence: the next one of b's aligned range
+// of kPartBuckets buckets, wrapping inside that range (the table's last range
+// may be shorter).  A sequence visits at most kPartBuckets buckets.
 __device__ __forceinline__ uint32_t next_bucket(uint32_t b, uint32_t nb) {
-    return (b + 1 == nb) ? 0u : b + 1;
+    const uint32_t n = b + 1;
+    return ((n & (kPartBuckets - 1)) == 0 || n == nb) ? (b & ~(kPartBuckets - 1)) : n;
 }
 
 template <int DIM>
