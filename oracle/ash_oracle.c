@@ -31,13 +31,12 @@
  *     iso-surface point extraction (grid.cu:453-531) and marching cubes
  *     (grid.cu:606-946), each described at its function below.
  *
- * Marching cubes: the 256-row case table of the reference (mc_macros.h) is not
- * restated here; the functions take a table as an argument, and the tests pass
- * the one that the library's generator derives from the cube.  That table is
- * pinned against the reference case by case in the outline, the facing and the
- * number of triangles of every patch, and by the geometry of the meshes it
- * gives; how a polygon of more than three corners is cut into triangles is the
- * generator's choice, so the triangle list is "parity unpinned" beyond that.
+ * Marching cubes: the functions take the 256-row case table as an argument.
+ * The Python face passes the reference's triangles (ash/src/mc_macros.h:32-288
+ * in the reversed order of ash/src/grid.cu:818-841), re-expressed in the corner
+ * and edge numbering used here and kept as a fixture under tests/golden/ by the
+ * script that reads the reference's header as text.  The library's own table
+ * comes from its generator and is compared with that fixture case by case.
  *
  * Where the reference has undefined behaviour (inserting more distinct keys
  * than `capacity` reads past the heap, ash/src/hashmap_gpu.cuh:226-227) the

@@ -85,17 +85,23 @@ _MC_TABLE = None
 
 
 def _mc_table():
-    """The 256 x 16 case table of the library's generator script."""
+    """The 256 x 16 marching-cubes case table (rows of edge triples, -1 padded)
+    with the reference's triangles: read from the fixture that
+    tests/golden/make_mc_case_fixture.py derives from ash/src/mc_macros.h, not
+    from the library's generator, so that the library's table is checked against
+    an input it did not produce."""
     global _MC_TABLE
     if _MC_TABLE is None:
-        import importlib.util
+        import json
 
-        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), os.pardir,
-                            "torch-ash_amd", "csrc", "gen_mc_table.py")
-        spec = importlib.util.spec_from_file_location("gen_mc_table", path)
-        mod = importlib.util.module_from_spec(spec)
-        spec.loader.exec_module(mod)
-        _MC_TABLE = mod.build_table()
+        path = os.path.join(HERE, os.pardir, "tests", "golden", "mc_case_boundaries.json")
+        with open(path) as f:
+            cases = json.load(f)
+        table = []
+        for case in range(256):
+            flat = [e for tri in cases[str(case)]["set"] for e in tri]
+            table.append(flat + [-1] * (16 - len(flat)))
+        _MC_TABLE = table
     return _MC_TABLE
 
 
@@ -149,8 +155,7 @@ class OracleBackend:
                        lut_grid_nb2grid_idx, cell_coords_table, lut_cell_nb2cell_idx,
                        lut_cell_nb2grid_nb, grid_dim, iso_value, weight_thr):
         """(triangles int32 (T, 3), vertices float32 (V, 3)), cells in launch
-        order.  The case table comes from the library's generator, whose
-        output the tests pin on their own."""
+        order, with the reference's case table (see _mc_table)."""
         x = _cpu(sdfs)
         b, m = x.shape[0], x.shape[1]
         x = x.reshape(b, m).contiguous()

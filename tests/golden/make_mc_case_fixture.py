@@ -1,6 +1,12 @@
 """Writes mc_case_boundaries.json: for each of the 256 marching-cubes cases the
-outline of the surface patch the reference emits, as a set of directed segments
-between cube edges, plus its triangle count.
+triangles the reference emits ("set": oriented edge triples, each starting at
+its lowest edge, sorted), their number, and the outline of the patch they form,
+as a set of directed segments between cube edges.
+
+With --cuts it also prints the CUTS dictionary of
+torch-ash_amd/csrc/gen_mc_table.py: for every polygon of more than three
+corners of that generator's loops, the number of the cut (in the generator's
+enumeration) whose triangles are the reference's.
 
 The outline is what the reference's case table (ash/src/mc_macros.h:32-288)
 fixes about a cell's surface independently of how each polygon is cut into
@@ -16,9 +22,11 @@ case bit c set when corner c is below the iso value, edge 4*axis + j.  The
 reference header is read as text and must be present at /root/reference; the
 JSON this script writes is what the tests load.
 """
+import importlib.util
 import json
 import os
 import re
+import sys
 
 REF = "/root/reference/ash/src/mc_macros.h"
 OUT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mc_case_boundaries.json")
@@ -55,18 +63,52 @@ def main():
                 mine |= 1 << corner[k]
         row = tri[16 * ref_case : 16 * ref_case + 16]
         sides = []
-        count = 0
+        triangles = []
         for t in range(0, 15, 3):
             if row[t] < 0:
                 break
-            count += 1
             a, b, c = (edge[row[t + 2]], edge[row[t + 1]], edge[row[t]])
             sides += [(a, b), (b, c), (c, a)]
+            triangles.append(_from_lowest([a, b, c]))
         outline = sorted(s for s in sides if (s[1], s[0]) not in sides)
-        cases[str(mine)] = {"triangles": count, "outline": outline}
+        cases[str(mine)] = {"triangles": len(triangles), "outline": outline,
+                            "set": sorted(triangles)}
     with open(OUT, "w") as f:
         json.dump(cases, f, separators=(",", ":"), sort_keys=True)
     print(f"wrote {OUT}")
+    if "--cuts" in sys.argv:
+        print_cuts(cases)
+
+
+def _from_lowest(t):
+    i = t.index(min(t))
+    return t[i:] + t[:i]
+
+
+def print_cuts(cases):
+    """The CUTS dictionary of the library's generator: per case, which cut of
+    each polygon of more than three corners gives the reference's triangles."""
+    here = os.path.dirname(os.path.abspath(__file__))
+    path = os.path.join(here, os.pardir, os.pardir, "torch-ash_amd", "csrc", "gen_mc_table.py")
+    spec = importlib.util.spec_from_file_location("gen_mc_table", path)
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    cuts = {}
+    for case in range(256):
+        want = {tuple(t) for t in cases[str(case)]["set"]}
+        picked = []
+        for loop in gen.case_loops(case):
+            loop = gen.from_lowest_edge(loop)
+            if len(loop) <= 3:
+                continue
+            mine = {t for t in want if set(t) <= set(loop)}
+            which = [n for n, cut in enumerate(gen.triangulations(loop))
+                     if {tuple(_from_lowest(list(t))) for t in cut} == mine]
+            assert len(which) == 1, f"case {case}: no cut of {loop} gives {sorted(mine)}"
+            picked.append(which[0])
+        if picked:
+            cuts[case] = tuple(picked)
+    print("CUTS =", cuts)
 
 
 if __name__ == "__main__":

@@ -2,14 +2,14 @@
 (restating ash/src/grid.cu:606-946 behind SparseDenseGrid.marching_cubes,
 ash/grid.py:680-711).
 
-The case table is derived by torch-ash_amd/csrc/gen_mc_table.py.  It is pinned
-(a) against the reference: for every case, the outline of the emitted patch --
-which crossed edges are joined across the faces of the cube, and the side the
-patch faces -- and the number of triangles equal those of the reference's
-table (tests/golden/mc_case_boundaries.json, written by
-tests/golden/make_mc_case_fixture.py); what is left open is only how a polygon
-with more than three corners is cut into triangles, which the reference fixes
-by hand and this library by a fan; (b) by geometry: meshes of closed surfaces
+The library's case table is written by torch-ash_amd/csrc/gen_mc_table.py.  It
+is pinned (a) against the reference: for every case the set of oriented
+triangles, and with it the outline of the emitted patch and the number of
+triangles, equal those of the reference's table
+(tests/golden/mc_case_boundaries.json, written by
+tests/golden/make_mc_case_fixture.py from ash/src/mc_macros.h:32-288 and the
+reversed order of ash/src/grid.cu:818-841); the oracle takes its table from
+that fixture, the library from the generator; (b) by geometry: meshes of closed surfaces
 are closed, oriented, have the Euler characteristic of the surface and
 enclose its volume, and a random field gives a mesh whose only open edges lie
 on the border of the volume -- a wrong entry in any of the 256 rows tears it.
@@ -54,6 +54,34 @@ def test_table_outlines_equal_the_reference_for_all_cases():
         ref = golden[str(case)]
         assert len(tris) == ref["triangles"], case
         assert _outline(tris) == [tuple(s) for s in ref["outline"]], case
+
+
+def test_table_triangles_equal_the_reference_for_all_cases():
+    """Every row of the library's table holds the reference's triangles: same
+    oriented triples (up to where a triple starts), for all 256 cases; and the
+    oracle's table, read from the fixture, is that set as well."""
+    import ash_oracle
+
+    gen = _gen()
+    with open(os.path.join(ROOT, "tests", "golden", "mc_case_boundaries.json")) as f:
+        golden = json.load(f)
+
+    def as_set(row):
+        tris = [row[i:i + 3] for i in range(0, 15, 3) if row[i] >= 0]
+        return sorted(tuple(gen.from_lowest_edge(list(t))) for t in tris)
+
+    table, oracle_table = gen.build_table(), ash_oracle._mc_table()
+    polygons = 0
+    for case in range(256):
+        want = [tuple(t) for t in golden[str(case)]["set"]]
+        assert as_set(table[case]) == want, case
+        assert as_set(oracle_table[case]) == want, case
+        polygons += sum(len(loop) > 3 for loop in gen.case_loops(case))
+    assert polygons > 200     # the cuts were a choice in most cases
+    # the generator's enumeration really offers a choice: another cut differs
+    loop = gen.from_lowest_edge(gen.case_loops(3)[0])
+    assert len(loop) == 4 and len(gen.triangulations(loop)) == 2
+    assert sorted(gen.triangulations(loop)[0]) != sorted(gen.triangulations(loop)[1])
 
 
 def test_table_rows_use_exactly_the_crossed_edges():

@@ -1,7 +1,8 @@
 """Builds the marching-cubes case table that ash_mc_table.h holds.
 
-The table is derived here from the geometry of the cube, not taken from a
-published listing.  Conventions:
+The outline of every case's patch is derived here from the geometry of the
+cube; how its polygons are cut into triangles follows the reference's table
+(see below).  Conventions:
 
 * corner c of a cell sits at offset (c & 1, (c >> 1) & 1, (c >> 2) & 1), which
   is also entry c of the 8-entry neighbour tables of a sparse-dense grid;
@@ -16,10 +17,19 @@ Per case: on each face of the cube the inside corners form runs along the
 face's corner cycle, and one segment joins the two crossed edges that bound a
 run.  A face with two diagonal inside corners therefore isolates each of them
 -- the same decision on both cells that share the face, so surfaces close
-across cells.  The segments chain into closed loops, each loop is oriented so
-that its normal points from the inside corners to the outside ones, and is cut
-into a fan of triangles whose diagonals all run through the interior of the
-cube.
+across cells.  The segments chain into closed loops and each loop is oriented
+so that its normal points from the inside corners to the outside ones: that
+fixes the outline of a case's patch, and it is the outline of the reference's
+table (ash/src/mc_macros.h:32-288) for all 256 cases.
+
+What the geometry leaves open is how a loop of more than three corners is cut
+into triangles.  So that a cell gives the very triangles the reference gives,
+the cut of every such loop is the reference's: `triangulations` enumerates the
+cuts of a polygon in a fixed order and CUTS names, per case and loop, the
+number of the one whose triangles are those of the reference's row.  CUTS is
+written by tests/golden/make_mc_case_fixture.py (which reads the reference's
+header as text) and pinned by tests/test_oracle_marching_cubes.py against the
+fixture that script also writes.
 
 Run as a script to rewrite ash_mc_table.h beside this file.
 """
@@ -135,33 +145,68 @@ def case_loops(case: int) -> List[List[int]]:
     return [_oriented(loop, case) for loop in _loops(case_segments(case))]
 
 
-def _share_a_face(e1: int, e2: int) -> bool:
-    def faces(e):
-        low, _ = edge_corners(e)
-        return {(a, (low >> a) & 1) for a in range(3) if a != e // 4}
+def triangulations(polygon: List[int]) -> List[List[Tuple[int, int, int]]]:
+    """Every way of cutting the polygon into triangles, in a fixed order: the
+    triangle over the side (first, last) takes each other corner k in turn,
+    with every cut of the part before k and of the part after it."""
+    n = len(polygon)
+    if n < 3:
+        return [[]]
+    if n == 3:
+        return [[tuple(polygon)]]
+    cuts = []
+    for k in range(1, n - 1):
+        for before in triangulations(polygon[: k + 1]):
+            for after in triangulations(polygon[k:]):
+                cuts.append(before + [(polygon[0], polygon[k], polygon[n - 1])] + after)
+    return cuts
 
-    return bool(faces(e1) & faces(e2))
+
+def from_lowest_edge(loop: List[int]) -> List[int]:
+    """The loop's corners in the same cyclic order, starting at its lowest edge."""
+    i = loop.index(min(loop))
+    return loop[i:] + loop[:i]
 
 
-def _fan(loop: List[int]) -> List[int]:
-    """The loop rotated so that the fan from its first corner has as few
-    diagonals inside a face of the cube as possible (none, for every loop that
-    occurs): such a diagonal could coincide with one of the neighbouring cell
-    and give an edge shared by four triangles."""
-    def flat_diagonals(start):
-        r = loop[start:] + loop[:start]
-        return sum(_share_a_face(r[0], r[i]) for i in range(2, len(r) - 1))
-
-    best = min(range(len(loop)), key=lambda s: (flat_diagonals(s), s))
-    return loop[best:] + loop[:best]
+# case -> for each of its loops with more than three corners (in the order of
+# case_loops, each taken from its lowest edge), the number of the cut in
+# triangulations() whose triangles the reference's table holds
+CUTS: Dict[int, Tuple[int, ...]] = {
+    3: (0,), 5: (1,), 7: (1,), 10: (0,), 11: (2,), 12: (1,), 13: (2,), 14: (1,), 15: (1,),
+    17: (0,), 19: (2,), 21: (0,), 23: (10,), 25: (0,), 26: (0,), 27: (11,), 28: (1,), 29: (2,),
+    30: (3,), 31: (3,), 34: (1,), 35: (1,), 37: (1,), 38: (1,), 39: (11,), 42: (0,), 43: (10,),
+    44: (1,), 45: (0,), 46: (11,), 47: (0,), 48: (1,), 49: (1,), 50: (2,), 51: (1,), 52: (1,),
+    53: (2,), 54: (0,), 55: (0,), 56: (1,), 57: (3,), 58: (2,), 59: (3,), 60: (1, 0), 61: (41,),
+    62: (41,), 63: (0,), 67: (0,), 68: (1,), 69: (4,), 70: (1,), 71: (2,), 74: (0,), 75: (0,),
+    76: (1,), 77: (3,), 78: (11,), 79: (0,), 80: (0,), 81: (3,), 82: (0,), 83: (2,), 84: (4,),
+    85: (0,), 86: (2,), 87: (2,), 88: (0,), 89: (4,), 90: (0, 1), 91: (13,), 92: (2,), 93: (4,),
+    94: (0,), 95: (1,), 98: (1,), 99: (3,), 100: (1,), 101: (2,), 102: (1, 0), 103: (20,),
+    106: (1,), 107: (10,), 108: (3,), 109: (10,), 110: (20,), 111: (6,), 112: (2,), 113: (12,),
+    114: (11,), 115: (3,), 116: (11,), 117: (2,), 118: (13,), 119: (0,), 120: (0,), 121: (8,),
+    122: (23,), 123: (4,), 124: (41,), 125: (13,), 131: (0,), 133: (1,), 135: (3,), 136: (0,),
+    137: (0,), 138: (3,), 139: (11,), 140: (2,), 141: (11,), 142: (8,), 143: (3,), 145: (0,),
+    147: (0,), 149: (1,), 151: (10,), 152: (0,), 153: (0, 1), 154: (4,), 155: (23,), 156: (0,),
+    157: (23,), 158: (8,), 159: (4,), 160: (1,), 161: (1,), 162: (4,), 163: (2,), 164: (1,),
+    165: (0, 1), 166: (2,), 167: (0,), 168: (3,), 169: (4,), 170: (0,), 171: (4,), 172: (2,),
+    173: (13,), 174: (2,), 175: (0,), 176: (1,), 177: (11,), 178: (1,), 179: (0,), 180: (3,),
+    181: (20,), 182: (1,), 183: (0,), 184: (2,), 185: (0,), 186: (4,), 187: (1,), 188: (41,),
+    190: (13,), 192: (0,), 193: (0,), 194: (0,), 195: (0, 1), 196: (2,), 197: (2,), 198: (0,),
+    199: (41,), 200: (1,), 201: (3,), 202: (2,), 203: (41,), 204: (1,), 205: (3,), 206: (0,),
+    207: (1,), 208: (1,), 209: (11,), 210: (3,), 211: (41,), 212: (5,), 213: (1,), 214: (1,),
+    215: (13,), 216: (11,), 217: (18,), 218: (18,), 220: (0,), 221: (1,), 222: (6,), 224: (2,),
+    225: (0,), 226: (2,), 227: (41,), 228: (11,), 229: (28,), 230: (28,), 232: (5,), 233: (1,),
+    234: (1,), 235: (7,), 236: (3,), 237: (4,), 238: (0,), 240: (1,), 241: (0,), 242: (3,),
+    243: (1,), 244: (3,), 245: (0,), 246: (4,), 248: (0,), 249: (0,), 250: (1,), 252: (0,),
+}
 
 
 def case_triangles(case: int) -> List[Tuple[int, int, int]]:
     tris = []
+    cuts = iter(CUTS.get(case, ()))
     for loop in case_loops(case):
-        loop = _fan(loop)
-        for i in range(1, len(loop) - 1):
-            tris.append((loop[0], loop[i], loop[i + 1]))
+        loop = from_lowest_edge(loop)
+        which = next(cuts) if len(loop) > 3 else 0
+        tris.extend(triangulations(loop)[which])
     return tris
 
 
