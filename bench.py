@@ -576,7 +576,11 @@ def bench_fusion(torch, ash, workloads, args, dev, frames=100):
     points = sum(d[0].shape[0] for d in data) / frames
     out = {"frames": frames, "points_per_frame": round(points),
            "candidate_keys_per_frame": round(points * 27)}
-    for name, fused in (("reference_formulation", False), ("fused", True)):
+    # "fused": the library's activation + integration kernels with the number of
+    # touched blocks read back per frame (what spatial_init_ returns needs it);
+    # "fused_no_readback": the same kernels with that number left on the device
+    for name, fused, count in (("reference_formulation", False, True), ("fused", True, True),
+                               ("fused_no_readback", True, False)):
         for rep in range(2):  # the first pass warms allocations up
             grid = ash.UnBoundedSparseDenseGrid(3, 80000, 2, 8, cell_size=0.015, device=dev)
             torch.cuda.synchronize()
@@ -584,7 +588,7 @@ def bench_fusion(torch, ash, workloads, args, dev, frames=100):
             touched = 0
             for pts, depth, ext in data:
                 touched += workloads.fuse_frame(grid, pts, depth, intrinsic, ext, trunc=0.04,
-                                                fused=fused)
+                                                fused=fused, count_blocks=count) or 0
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
         out[name] = {

@@ -173,6 +173,23 @@ int ash_grid_integrate_depth(float* embeddings, int64_t num_embeddings,
                              int width, float trunc, float depth_max,
                              void* stream);
 
+/* ash_grid_integrate_depth over the listing that the latest
+ * ash_grid_collect_touched on `map` left (out_indices / out_coords of that
+ * call, both of `capacity` rows), whose length is read on the device from the
+ * table's counters: no host value depends on the activation, so a frame of a
+ * fusion loop (activate, list, integrate) needs no read-back at all.  A fixed
+ * grid strides over the listed blocks' cells.  Same arithmetic and arguments
+ * otherwise.  No counterpart in the reference, whose loop sizes tensors by the
+ * number of touched blocks (demo/rgbd_fusion.py:216-254). */
+int ash_grid_integrate_depth_touched(ash_map_t* map, float* embeddings,
+                                     int64_t num_embeddings, int grid_dim,
+                                     int embedding_dim, const int64_t* grid_indices,
+                                     const int32_t* grid_coords, float cell_size,
+                                     const float* origin, const float* intrinsic,
+                                     const float* extrinsic, const float* depth,
+                                     const float* color, int height, int width,
+                                     float trunc, float depth_max, void* stream);
+
 /* Replaces `ray_find_near_far` (ash/src/sampler.cu:7-121, pybind.cpp:35): per
  * ray, march from t_min in steps of half a block while inside the box
  * [bbox_min, bbox_max] and report the range [near, far] that contains active

@@ -215,6 +215,45 @@ def test_fused_fusion_against_oracle_harness(gpu_ash, oracle, monkeypatch, width
     assert float(cells_gpu[..., 1].sum()) > 1e5
 
 
+def test_frames_without_read_back_equal_counted_frames(gpu_ash):
+    """ash.fusion.fuse_frame(count_blocks=False): activation, listing and
+    integration are queued with the number of touched blocks left on the device
+    (ash_grid_integrate_depth_touched).  Same blocks and, block by block, the
+    same embedding rows bit for bit as the frames that read the number back;
+    an overfull table shows at the next call that reads the counters."""
+    scene = workloads.FusionScene(width=320, height=240)
+    intrinsic = scene.intrinsic.to(DEV)
+    frames = []
+    for f in (0, 9, 18, 27, 36):
+        ext = scene.pose(f)
+        depth = scene.depth(ext)
+        frames.append((scene.unproject(depth, ext).to(DEV), depth.to(DEV), ext.to(DEV)))
+
+    def run(count_blocks, capacity=30_000):
+        grid = gpu_ash.UnBoundedSparseDenseGrid(3, capacity, 2, 8, cell_size=0.015, device=DEV)
+        with torch.no_grad():
+            grid.embeddings.zero_()
+        touched = [gpu_ash.fusion.fuse_frame(grid, p, d, intrinsic, e, 0.04, 6.0,
+                                             count_blocks=count_blocks) for p, d, e in frames]
+        keys, idx = grid.engine.items()
+        order = sort_rows(keys, idx)
+        return grid, touched, order[0], grid.embeddings.detach()[order[1].to(DEV)].cpu()
+
+    _, touched, keys_a, cells_a = run(True)
+    grid, nothing, keys_b, cells_b = run(False)
+    assert all(t > 100 for t in touched) and nothing == [None] * len(frames)
+    assert torch.equal(keys_a, keys_b) and len(keys_a) > 1000
+    assert torch.equal(cells_a, cells_b)
+    assert float(cells_a[..., 1].sum()) > 1e5
+    # the count of the last listing is still in the counters
+    assert grid.engine.backend.status()["touched"] == touched[-1]
+    # too small a table: the frames run, the table is full, the next insert warns
+    small, _, keys_c, _ = run(False, capacity=1500)
+    assert small.engine.size() == 1500 and len(keys_c) == 1500
+    with pytest.warns(UserWarning, match="exceeds the hash map capacity"):
+        small.engine.insert_keys(torch.tensor([[900, 900, 900]], dtype=torch.int32, device=DEV))
+
+
 @pytest.mark.parametrize("capacity", [5, 1000, 80_000, 131_073, 200_000, 1_048_576])
 def test_touched_rows_are_listed_in_order(gpu_ash, capacity):
     """ash_grid_collect_touched against torch.nonzero: ascending rows, their

@@ -87,6 +87,12 @@ _SIGNATURES = {
          ctypes.POINTER(ctypes.c_float), _PTR, _PTR, _PTR, _PTR, ctypes.c_int, ctypes.c_int,
          ctypes.c_float, ctypes.c_float, _PTR],
     ),
+    "ash_grid_integrate_depth_touched": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, _PTR, _PTR, ctypes.c_float,
+         ctypes.POINTER(ctypes.c_float), _PTR, _PTR, _PTR, _PTR, ctypes.c_int, ctypes.c_int,
+         ctypes.c_float, ctypes.c_float, _PTR],
+    ),
     "ash_ray_find_near_far": (
         ctypes.c_int,
         [_PTR, _PTR, _PTR, _PTR, _PTR, _I64, ctypes.c_float, ctypes.c_float, ctypes.c_float,
@@ -222,6 +228,11 @@ RAY_STAGE_EXTRA = 2
 # Largest table whose touched rows ash_grid_collect_touched lists (the header's
 # ASH_COLLECT_MAX_BLOCKS).
 COLLECT_MAX_BLOCKS = 1 << 20
+# Most positions per call of ash_grid_activate_static (the header's
+# ASH_ACTIVATE_STATIC_MAX_POSITIONS).
+ACTIVATE_STATIC_MAX = 1 << 20
+# Deferred activations between two looks at the table's counters.
+DEFERRED_UPKEEP_EVERY = 64
 
 # Which inserts take the streaming (partition + build in LDS) path of the
 # library instead of the per-key kernel: "auto" = when the library says the
@@ -537,8 +548,11 @@ class _Backend:
         color: Optional[torch.Tensor],
         trunc: float,
         depth_max: float,
+        counted_by=None,
     ) -> None:
-        """In-place TSDF update of the cells of the listed blocks."""
+        """In-place TSDF update of the cells of the listed blocks.  With
+        `counted_by` (a map whose latest deferred activation made the listing)
+        the number of listed blocks is read on the device."""
         _require_hip(embeddings, "embeddings")
         dev = embeddings.device
         if embeddings.dtype != torch.float32 or not embeddings.is_contiguous():
@@ -549,6 +563,8 @@ class _Backend:
         grid_coords = grid_coords.reshape(-1, 3).to(dev, torch.int32).contiguous()
         if grid_coords.shape[0] != grid_indices.shape[0]:
             raise RuntimeError("one coordinate row per block index is needed")
+        if counted_by is not None and grid_indices.shape[0] != counted_by.capacity:
+            raise RuntimeError("a listing counted on the device has one row per block of the map")
         intrinsic = intrinsic.to(dev, torch.float32).contiguous()
         extrinsic = extrinsic.to(dev, torch.float32).contiguous()
         if intrinsic.shape != (3, 3) or extrinsic.shape != (4, 4):
@@ -563,17 +579,26 @@ class _Backend:
         c_origin = None
         if origin is not None:
             c_origin = (ctypes.c_float * 3)(*[float(v) for v in origin.reshape(-1).tolist()])
+        tail = (float(cell_size), c_origin, intrinsic.data_ptr(), extrinsic.data_ptr(),
+                depth.data_ptr(), color.data_ptr() if color is not None else None,
+                depth.shape[0], depth.shape[1], float(trunc), float(depth_max), _stream_of(dev))
         with torch.cuda.device(dev):
-            self.check(
-                self.lib.ash_grid_integrate_depth(
-                    embeddings.data_ptr(), embeddings.shape[0], int(grid_dim), embeddings.shape[2],
-                    grid_indices.data_ptr(), grid_coords.data_ptr(), grid_indices.shape[0],
-                    float(cell_size), c_origin, intrinsic.data_ptr(), extrinsic.data_ptr(),
-                    depth.data_ptr(), color.data_ptr() if color is not None else None,
-                    depth.shape[0], depth.shape[1], float(trunc), float(depth_max),
-                    _stream_of(dev),
+            if counted_by is not None:
+                self.check(
+                    self.lib.ash_grid_integrate_depth_touched(
+                        counted_by._handle, embeddings.data_ptr(), embeddings.shape[0],
+                        int(grid_dim), embeddings.shape[2], grid_indices.data_ptr(),
+                        grid_coords.data_ptr(), *tail,
+                    )
                 )
-            )
+            else:
+                self.check(
+                    self.lib.ash_grid_integrate_depth(
+                        embeddings.data_ptr(), embeddings.shape[0], int(grid_dim),
+                        embeddings.shape[2], grid_indices.data_ptr(), grid_coords.data_ptr(),
+                        grid_indices.shape[0], *tail,
+                    )
+                )
 
     # -- value rows by index (ash/hashmap.py:87-95,138-146) -------------------
     def gather_rows(self, tables: Dict[str, torch.Tensor], indices: torch.Tensor) -> Dict[str, torch.Tensor]:
@@ -1114,6 +1139,83 @@ class _HashMap:
         grid_coords = self._block_coords[grid_indices]
         self._touched[grid_indices] = 0
         return grid_coords, grid_indices
+
+    def activate_blocks_deferred(
+        self,
+        cells: torch.Tensor,
+        grid_dim: int,
+        dilation: int,
+        bidirectional: bool,
+        bound_lo: int,
+        bound_hi: int,
+    ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """activate_blocks without its read-back: the blocks are inserted and
+        the touched ones listed on the device, and (grid_coords int32[capacity,3],
+        grid_indices int64[capacity]) are returned whole -- how many of their
+        rows the listing filled stays in the table's counters, where
+        ash_grid_integrate_depth_touched reads it.  Nothing here waits for the
+        device; keys refused for lack of capacity show in the counters at the
+        next call that reads them (`status`, `size` after it, any insert).
+        Both tensors are reused by the next deferred activation of this map."""
+        if self.key_dim != 3:
+            raise RuntimeError("block activation needs 3-d keys")
+        if cells.dim() != 2 or cells.shape[1] != 3 or cells.dtype != torch.float32:
+            raise RuntimeError("positions must be float32 (N, 3)")
+        if cells.device != self._device:
+            raise RuntimeError(f"positions are on {cells.device}, the map on {self._device}")
+        if self.capacity > COLLECT_MAX_BLOCKS:
+            raise RuntimeError("deferred activation lists at most 2^20 blocks")
+        cells = cells.contiguous()
+        n = cells.shape[0]
+        if getattr(self, "_touched", None) is None:
+            self._touched = torch.zeros(self.capacity, dtype=torch.uint8, device=self._device)
+            self._block_coords = torch.zeros(
+                (self.capacity, 3), dtype=torch.int32, device=self._device
+            )
+        if getattr(self, "_listing", None) is None:
+            self._listing = (
+                torch.empty((self.capacity, 3), dtype=torch.int32, device=self._device),
+                torch.empty(self.capacity, dtype=torch.int64, device=self._device),
+            )
+        if self._general is None:
+            # a key beyond the packed range would otherwise wait for a read-back
+            # that this path does not make
+            self._general = torch.empty(self._general_bytes, dtype=torch.uint8, device=self._device)
+            with torch.cuda.device(self._device):
+                self._check(
+                    self._lib.ash_map_attach_general(
+                        self._handle, self._general.data_ptr(), self._general_bytes, self._stream()
+                    )
+                )
+        self._make_room(n)
+        coords, rows = self._listing
+        head = (self._handle, cells.data_ptr(), n, int(grid_dim), int(dilation),
+                int(bool(bidirectional)), int(bound_lo), int(bound_hi),
+                self._touched.data_ptr(), self._block_coords.data_ptr())
+        with torch.cuda.device(self._device):
+            if n <= ACTIVATE_STATIC_MAX:
+                # run heads in the library's own device array: no allocation
+                self._check(self._lib.ash_grid_activate_static(*head, self._stream()))
+            else:
+                heads = torch.empty(64 + 3 * n, dtype=torch.int32, device=self._device)
+                self._check(self._lib.ash_grid_activate(*head, heads.data_ptr(), self._stream()))
+            self._check(
+                self._lib.ash_grid_collect_touched(
+                    self._handle, self._touched.data_ptr(), self._block_coords.data_ptr(),
+                    rows.data_ptr(), coords.data_ptr(), self._stream(),
+                )
+            )
+        self._status_after_insert = None
+        self.version = next(_VERSIONS)
+        # Keys refused for lack of capacity leave tombstones behind and are
+        # only visible in the counters: every DEFERRED_UPKEEP_EVERY-th call the
+        # next insert looks at them (one read-back) and re-places the entries if
+        # tombstones have piled up.
+        self._deferred_calls = getattr(self, "_deferred_calls", 0) + 1
+        if self._deferred_calls >= DEFERRED_UPKEEP_EVERY:
+            self._deferred_calls = 0
+            self._maybe_tombstones = True
+        return coords, rows
 
     def _bulk_workspace(self, n: int, k: int, c_rows) -> Optional[torch.Tensor]:
         """Workspace for the streaming insert path, or None when this batch goes

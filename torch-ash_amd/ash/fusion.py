@@ -13,7 +13,7 @@ from typing import Optional
 
 import torch
 
-from .common import _get_c_extension
+from .common import COLLECT_MAX_BLOCKS, _get_c_extension
 from .grid import SparseDenseGrid
 
 backend = _get_c_extension()
@@ -30,11 +30,14 @@ def integrate_depth(
     trunc: float,
     depth_max: float,
     color: Optional[torch.Tensor] = None,
+    counted_by=None,
 ) -> None:
     """Projects every cell of the listed blocks into `depth` (H, W; metres, 0 =
     no reading) with the pinhole `intrinsic` (3, 3) and the world-to-camera
     `extrinsic` (4, 4) and folds the truncated signed distance (and `color`
-    (H, W, 3), if given) into the grid's embedding rows."""
+    (H, W, 3), if given) into the grid's embedding rows.  `counted_by`: the
+    table whose deferred activation made the listing (its length is then read
+    on the device)."""
     scale, origin = grid._cell_to_world_affine()
     backend.integrate_depth(
         grid.embeddings.data,
@@ -49,6 +52,7 @@ def integrate_depth(
         color,
         trunc,
         depth_max,
+        counted_by=counted_by,
     )
 
 
@@ -63,10 +67,29 @@ def fuse_frame(
     depth_max: float,
     color: Optional[torch.Tensor] = None,
     dilation: int = 1,
-) -> int:
+    count_blocks: bool = True,
+) -> Optional[int]:
     """One fusion step: activate the blocks around the unprojected `points`
     (world coordinates) with a two-sided dilation, then integrate the frame
-    into them.  Returns the number of touched blocks."""
+    into them.  Returns the number of touched blocks -- or, with
+    `count_blocks=False`, nothing: the frame then runs without a single
+    read-back from the device (the reference's loop needs the number to size
+    its tensors, demo/rgbd_fusion.py:216-254; the kernels here read it where it
+    is), the host only queues launches, and the reference's capacity warning
+    comes with the next call that reads the table's counters."""
+    if not count_blocks and points.shape[0] > 0 and grid.engine.capacity <= COLLECT_MAX_BLOCKS:
+        cells = grid.transform_world_to_cell(points)
+        if cells.dtype == torch.float32:
+            lo, hi = grid._block_bounds()
+            table = grid.engine.backend
+            grid_coords, grid_indices = table.activate_blocks_deferred(
+                cells, grid.grid_dim, dilation, True, lo, hi
+            )
+            integrate_depth(
+                grid, grid_coords, grid_indices, depth, intrinsic, extrinsic, trunc, depth_max,
+                color, counted_by=table,
+            )
+            return None
     grid_coords, _, grid_indices, _ = grid.spatial_init_(
         points, dilation=dilation, bidirectional=True
     )

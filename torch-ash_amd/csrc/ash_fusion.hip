@@ -39,9 +39,8 @@ struct IntegrateArgs {
     float trunc, depth_max;
 };
 
-__global__ __launch_bounds__(kBlock) void integrate_depth_kernel(IntegrateArgs a) {
-    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (t >= a.n * a.m) return;
+// The update of cell t of the listing (block t / m, cell t % m).
+__device__ __forceinline__ void integrate_cell(const IntegrateArgs& a, int64_t t) {
     const int64_t blk = t / a.m;
     const int cell = static_cast<int>(t - blk * a.m);
     const int64_t row = a.grid_idx[blk];
@@ -106,19 +105,38 @@ __global__ __launch_bounds__(kBlock) void integrate_depth_kernel(IntegrateArgs a
     e[a.e - 1] = w_new;
 }
 
+__global__ __launch_bounds__(kBlock) void integrate_depth_kernel(IntegrateArgs a) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t < a.n * a.m) integrate_cell(a, t);
+}
+
+// The same over a listing whose length is on the device (`count`, at most
+// a.n): a fixed grid strides over count * m cells, so no host value depends on
+// the activation that made the listing.
+__global__ __launch_bounds__(kBlock) void integrate_depth_counted_kernel(
+        IntegrateArgs a, const int32_t* __restrict__ count) {
+    int64_t blocks = *count;
+    if (blocks > a.n) blocks = a.n;
+    const int64_t cells = blocks * a.m;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; t < cells;
+         t += static_cast<int64_t>(gridDim.x) * kBlock) {
+        integrate_cell(a, t);
+    }
+}
+
 }  // namespace
 }  // namespace ash
 
 using namespace ash;
 
-extern "C" int ash_grid_integrate_depth(
-        float* embeddings, int64_t num_embeddings, int grid_dim, int embedding_dim,
-        const int64_t* grid_indices, const int32_t* grid_coords, int64_t n_blocks,
-        float cell_size, const float* origin, const float* intrinsic,
-        const float* extrinsic, const float* depth, const float* color, int height,
-        int width, float trunc, float depth_max, void* stream) {
-    if (n_blocks < 0) ASH_FAIL("negative block count");
-    if (n_blocks == 0) return 0;
+namespace {
+
+int fill_integrate_args(IntegrateArgs& a, float* embeddings, int64_t num_embeddings,
+                        int grid_dim, int embedding_dim, const int64_t* grid_indices,
+                        const int32_t* grid_coords, int64_t n_blocks, float cell_size,
+                        const float* origin, const float* intrinsic, const float* extrinsic,
+                        const float* depth, const float* color, int height, int width,
+                        float trunc, float depth_max) {
     if (embeddings == nullptr || grid_indices == nullptr || grid_coords == nullptr ||
         intrinsic == nullptr || extrinsic == nullptr || depth == nullptr) {
         ASH_FAIL("null pointer in depth integration");
@@ -130,7 +148,6 @@ extern "C" int ash_grid_integrate_depth(
     }
     if (height < 1 || width < 1) ASH_FAIL("empty depth image");
     if (num_embeddings < 1) ASH_FAIL("empty embedding table");
-    IntegrateArgs a;
     a.emb = embeddings;
     a.grid_idx = grid_indices;
     a.grid_xyz = grid_coords;
@@ -150,10 +167,54 @@ extern "C" int ash_grid_integrate_depth(
     for (int d = 0; d < 3; ++d) a.origin[d] = origin ? origin[d] : 0.f;
     a.trunc = trunc;
     a.depth_max = depth_max;
+    if (n_blocks * a.m > (int64_t{1} << 40)) ASH_FAIL("too many cells in one call");
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int ash_grid_integrate_depth_touched(
+        ash_map_t* map, float* embeddings, int64_t num_embeddings, int grid_dim,
+        int embedding_dim, const int64_t* grid_indices, const int32_t* grid_coords,
+        float cell_size, const float* origin, const float* intrinsic, const float* extrinsic,
+        const float* depth, const float* color, int height, int width, float trunc,
+        float depth_max, void* stream) {
+    if (map == nullptr) ASH_FAIL("null map handle");
+    IntegrateArgs a;
+    if (fill_integrate_args(a, embeddings, num_embeddings, grid_dim, embedding_dim, grid_indices,
+                            grid_coords, map->capacity, cell_size, origin, intrinsic, extrinsic,
+                            depth, color, height, width, trunc, depth_max)) {
+        return 1;
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    // enough workgroups to fill the device; they stride over the listing
+    int64_t blocks = (map->capacity * a.m + kBlock - 1) / kBlock;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    integrate_depth_counted_kernel<<<static_cast<unsigned>(blocks), kBlock, 0,
+                                     static_cast<hipStream_t>(stream)>>>(
+            a, map->d.ctr + kCtrTouched);
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ash_grid_integrate_depth(
+        float* embeddings, int64_t num_embeddings, int grid_dim, int embedding_dim,
+        const int64_t* grid_indices, const int32_t* grid_coords, int64_t n_blocks,
+        float cell_size, const float* origin, const float* intrinsic,
+        const float* extrinsic, const float* depth, const float* color, int height,
+        int width, float trunc, float depth_max, void* stream) {
+    if (n_blocks < 0) ASH_FAIL("negative block count");
+    if (n_blocks == 0) return 0;
+    IntegrateArgs a;
+    if (fill_integrate_args(a, embeddings, num_embeddings, grid_dim, embedding_dim, grid_indices,
+                            grid_coords, n_blocks, cell_size, origin, intrinsic, extrinsic, depth,
+                            color, height, width, trunc, depth_max)) {
+        return 1;
+    }
     PointerGuard guard;
     ASH_HIP(guard.enter_for(embeddings));
     const int64_t threads = n_blocks * a.m;
-    if (threads > (int64_t{1} << 40)) ASH_FAIL("too many cells in one call");
     const int64_t blocks = (threads + kBlock - 1) / kBlock;
     if (blocks > 0x7FFFFFFFll) ASH_FAIL("too many cells in one call");
     integrate_depth_kernel<<<static_cast<unsigned>(blocks), kBlock, 0,

@@ -337,18 +337,21 @@ class FusionScene:
 
 
 def fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc: float, depth_max: float = 6.0,
-               fused: bool = False):
+               fused: bool = False, count_blocks: bool = True):
     """One fusion step on `grid` (embedding channels: tsdf, weight), following
     the reference demo (demo/rgbd_fusion.py:200-254 and :76-110): activate the
     blocks around `points` with a one-block two-sided dilation, project every
     cell of the touched blocks into the depth image, and update the running
     weighted mean.  All tensors must live on the grid's device.  Returns the
     number of touched blocks.  `fused` takes the library's integration kernel
-    instead of the torch expressions below (the reference's statement)."""
+    instead of the torch expressions below (the reference's statement), and
+    with `count_blocks=False` runs the frame without a read-back (returns
+    None)."""
     if fused:
         import ash.fusion
 
-        return ash.fusion.fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc, depth_max)
+        return ash.fusion.fuse_frame(grid, points, depth, intrinsic, extrinsic, trunc, depth_max,
+                                     count_blocks=count_blocks)
     import ash.grid
 
     switch, ash.grid.FUSED_ACTIVATION = ash.grid.FUSED_ACTIVATION, False
