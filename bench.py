@@ -77,15 +77,45 @@ INSERT_KEY_BYTES = 12 + 16 + 16 + 4          # key in, probe, slot write, heap p
 VALUE_ROW_BYTES = 2 * (12 + 4)               # color + depth, read and written
 
 
-# HBM bytes per launch (read + written) at the default sizes, from two
-# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
-# counters read for a plain 1 GiB copy: FETCH_SIZE x 1024 / 0.50,
-# WRITE_SIZE x 1024 / 1.00.  Only attached when the run uses those sizes.
-MEASURED_TRAFFIC_BYTES = {
-    "insert_values": 2_563_000_000 + 1_819_000_000,
-    "insert_keys": 2_303_000_000 + 1_564_000_000,
-    "find": 2_230_000_000 + 146_000_000,
+# Counters per launch at the default sizes, from rocprofv3 --pmc runs of this
+# file (one counter set per run; the summaries are in profiles/).  Only attached
+# when the run uses those sizes.
+#   traffic: bytes that cross the far side of the L2s (read + written), i.e.
+#     HBM plus what the Infinity Cache answers: FETCH_SIZE x 1024 / 0.50 +
+#     WRITE_SIZE x 1024 / 1.00, the factors being what the same counters read
+#     for kernels that move a known number of bytes;
+#   l2_hit_rate: TCC_HIT / (TCC_HIT + TCC_MISS);
+#   atomic_requests: TCC_ATOMIC (all of them are forwarded to the memory side:
+#     TCC_EA0_ATOMIC reads the same).
+MEASURED_COUNTERS = {
+    "insert_values": (2_564_000_000 + 1_947_000_000, 0.343, 16_404_000),
+    "insert_keys": (2_304_000_000 + 1_691_000_000, 0.243, 16_465_000),
+    "find": (2_230_000_000 + 146_000_000, 0.064, 0),
+    "erase": (2_234_000_000 + 1_217_000_000, 0.447, 16_031_000),
+    "items": (128_000_000 + 320_000_000, 0.417, 1_954),
+    "items_values": (528_000_000 + 256_000_000, 0.247, 0),
+    # sums over the split, build and row-copy kernels
+    "insert_values_bulk": (834_000_000 + 1_330_000_000, 0.390, 47_000),
+    "insert_keys_bulk": (449_000_000 + 914_000_000, 0.411, 59_000),
+    "cfg3_forward_linear": (3_519_000_000 + 282_000_000, 0.171, 0),
+    "cfg3_forward_smooth_step": (3_519_000_000 + 282_000_000, 0.171, 0),
+    "cfg4_forward": (369_000_000 + 67_000_000, 0.258, 0),
+    # kernel only: the zero fill of the dense gradient adds 1.64 GB written
+    "cfg4_backward": (431_000_000 + 311_000_000 + 1_638_400_000, 0.078, 7_589_000),
+    "cfg4_double_backward": (478_000_000 + 328_000_000 + 1_638_400_000, 0.087, 7_589_000),
+    "cfg4_grid_query": (71_000_000 + 122_000_000, 0.399, 0),
 }
+
+
+def attach_counters(kernels):
+    for name, (traffic, hit_rate, atomics) in MEASURED_COUNTERS.items():
+        entry = kernels.get(name)
+        if not isinstance(entry, dict) or "ms" not in entry:
+            continue
+        entry["traffic"] = traffic
+        entry["l2_hit_rate"] = hit_rate
+        entry["atomic_requests"] = atomics
+        entry["atomic_requests_per_s"] = round(atomics / (entry["ms"] * 1e-3)) if entry["ms"] else 0
 
 
 def items_bytes(scanned: int, n: int) -> int:
@@ -328,10 +358,6 @@ def bench_hash(torch, ash, workloads, args, dev):
     for name in ("insert_values", "insert_keys", "find", "erase"):
         kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
-    if n == 16_000_000 and args.capacity == 24_000_000:
-        for name, traffic in MEASURED_TRAFFIC_BYTES.items():
-            if name in kernels:
-                kernels[name]["traffic"] = traffic
     del hm, w, workspace
     torch.cuda.empty_cache()
     return ms_per_step, hits, kernels
@@ -733,6 +759,8 @@ def main():
     kernels["cfg1_hashset"] = bench_config1(torch, ash, workloads, dev)
     if not args.no_fusion:
         kernels["cfg5_fusion"] = bench_fusion(torch, ash, workloads, args, dev)
+    if args.keys == 16_000_000 and args.capacity == 24_000_000:
+        attach_counters(kernels)
     dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
     table_bytes = (args.capacity + 5) // 6 * 128
