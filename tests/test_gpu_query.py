@@ -133,6 +133,29 @@ def test_repeated_cells_merge_path(gpu_ash, oracle):
         _compare_all(gpu_ash, oracle, grid, x, interpolation, seed=13)
 
 
+def test_ordered_and_unordered_stretches_in_one_batch(gpu_ash, oracle):
+    """The four-channel backward kernels gather gradient lines in a per-wavefront
+    table, send rows past it when it is full and leave it aside for a few tiles
+    when most rows went past it.  The batch makes every workgroup walk through
+    all of that (a workgroup takes every n-th tile of its eighth of the batch,
+    so each eighth holds the whole pattern): rays (few lines per tile), one
+    query repeated over several tiles (a single line, runs that span rows of
+    lanes), scattered queries (more lines per tile than the table holds: rows
+    spill, then the table rests), rays again (the table comes back)."""
+    grid = _make_grid(gpu_ash, 8, 4, 1, seed=21)
+    g = torch.Generator().manual_seed(22)
+    parts = []
+    for _ in range(8):
+        starts = torch.rand(1600, 1, 3, generator=g) * 20 - 6
+        steps = torch.arange(128).view(1, -1, 1) * torch.rand(1600, 1, 3, generator=g) * 0.04
+        rays = (starts + steps).view(-1, 3)
+        same = (torch.rand(1, 3, generator=g) * 6 + 1).repeat(12800, 1)
+        scattered = torch.rand(102400, 3, generator=g) * 20 - 6
+        parts += [rays[:102400], same, scattered, rays[102400:]]
+    x = torch.cat(parts).to(DEV)
+    _compare_all(gpu_ash, oracle, grid, x, "smooth_step", seed=23)
+
+
 def test_empty_batch_and_bad_arguments(gpu_ash):
     grid = _make_grid(gpu_ash, 2, 3, 1, seed=5)
     backend = gpu_ash.grid_query.backend

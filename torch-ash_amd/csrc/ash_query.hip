@@ -122,6 +122,7 @@ __device__ __forceinline__ void corner_weight_grad(const AxisTerms<T>& t, int c,
 // ------------------------------------------------------------ LDS layout
 // [ tile: row[8][256] uint32, off[3][256] float ]  (only when LPQ > 1)
 // [ per-cell tables: c2c[M*8] uint16, c2g[M*8] uint8 ]  (only when lds_lut)
+// [ one LineTable per wavefront ]  (E = 4 backward kernels that produce grad_embeddings)
 struct Tile {
     uint32_t row[8][kBlock];
     float off[3][kBlock];
@@ -168,6 +169,13 @@ __device__ __forceinline__ CellLut stage_cell_lut(const QDev& a,
         lut.c2g = s_c2g;
     }
     return lut;
+}
+
+// Where the line tables of the float4 backward kernels start in dynamic LDS.
+__host__ __device__ inline size_t table_offset(const QDev& a, int lpq, bool lds_lut) {
+    size_t bytes = lpq > 1 ? sizeof(Tile) : 0;
+    if (lds_lut) bytes += static_cast<size_t>(a.M) * 8 * 3;
+    return (bytes + 15) & ~static_cast<size_t>(15);
 }
 
 // Tile walk: workgroup w serves XCD (w mod 8); each XCD owns a contiguous
@@ -237,7 +245,6 @@ __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
 template <int LPQ, bool LDS>
 struct TileStage {
     static constexpr int kPasses = LPQ;
-    static constexpr int kQpp = kBlock / LPQ;  // queries per pass
 
     static __device__ __forceinline__ void fill(const QDev& a,
                                                 const CellLut& lut,
@@ -260,7 +267,9 @@ struct TileStage {
                                                     uint32_t (&row)[8],
                                                     float (&o)[3]) {
         if constexpr (LPQ > 1) {
-            const int qi = p * kQpp + threadIdx.x / LPQ;
+            // a wavefront serves the 64 consecutive queries it resolved itself,
+            // 64 / LPQ of them per pass
+            const int qi = (threadIdx.x & ~63) + p * (64 / LPQ) + (threadIdx.x & 63) / LPQ;
 #pragma unroll
             for (int c = 0; c < 8; ++c) row[c] = s->row[c][qi];
 #pragma unroll
@@ -516,6 +525,480 @@ query_backward_backward_kernel(
             if (want_z && q < a.N && chv) {
                 grad_z[q * a.E + ch] = on ? gz : T(0);
             }
+        }
+    }
+}
+
+// ================================================== float4 backward kernels
+// fp32 embeddings of four channels (a signed distance and a colour, say): one
+// lane holds a whole query, as in the forward kernel, so that a wavefront
+// serves 64 queries per tile: four times the loads in flight and a quarter of
+// the per-query arithmetic of the one-lane-per-channel kernels above.
+//
+// Gradient rows.  The memory side executes atomics at a fixed rate of
+// requests, and one request is what one instruction of a wavefront sends to
+// one 64-byte line, whether it carries one float or sixteen (measured: 18 G
+// requests/s for 4-byte and for 64-byte groups alike).  The eight corners of a
+// query and the queries that follow it along a ray meet the same few lines
+// over and over -- the x neighbour is the next row, a corner of this sample is
+// another corner of the next -- but in different instructions.  So every
+// wavefront first adds its contributions into a small table of lines in LDS
+// (open addressing on the line number, sixteen floats per entry) and sends the
+// table out once per tile, one line per sixteen lanes: a third of the requests
+// on ray-ordered samples.  Before that, runs of consecutive queries with the
+// same row are summed in registers (lane exchange inside a row of 16 lanes is
+// a modifier of an ordinary vector instruction, across rows it would be a trip
+// through the LDS pipeline, so a run is cut at the row of lanes; the table
+// joins the pieces).  A row whose line finds no place within kLineProbes steps
+// goes to memory directly, and a wavefront half of whose rows had to do that
+// (unordered queries share no lines) leaves the table aside for the next
+// kLineRest tiles.
+template <int CTRL>
+__device__ __forceinline__ int dpp_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL, typename T>
+__device__ __forceinline__ T dpp(T v) {
+    static_assert(sizeof(T) == 4, "32-bit values");
+    return __builtin_bit_cast(T, dpp_int<CTRL>(__builtin_bit_cast(int, v)));
+}
+constexpr int kRowShl = 0x100;  // lane i takes lane i + n of its row of 16 (0 beyond it)
+constexpr int kRowShr = 0x110;  // lane i takes lane i - n
+
+// One step of the segmented sum: adds what lies `D` lanes below, unless a run
+// starts in between.
+template <int D>
+__device__ __forceinline__ void run_step(float (&v)[4], int& f, int g) {
+    const int fu = dpp_int<kRowShr + D>(f);
+    const bool take = g >= D && !f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float vu = dpp<kRowShr + D>(v[k]);
+        if (take) v[k] += vu;
+    }
+    if (take) f |= fu;
+}
+
+// Sums `v` over runs of consecutive lanes (of one row of 16) with equal `id`;
+// returns whether this lane ends its run and holds the total.  Every lane of
+// the wavefront must take part.
+__device__ __forceinline__ bool merge_runs(uint32_t id, float (&v)[4], int lane) {
+    const int g = lane & 15;
+    const uint32_t prev = dpp<kRowShr + 1>(id);
+    const uint32_t next = dpp<kRowShl + 1>(id);
+    int f = (g == 0 || prev != id) ? 1 : 0;
+    const bool tail = g == 15 || next != id;
+    run_step<1>(v, f, g);
+    run_step<2>(v, f, g);
+    run_step<4>(v, f, g);
+    run_step<8>(v, f, g);
+    return tail;
+}
+
+constexpr int kLineSlots = 128;   // lines per wavefront's table
+constexpr int kLineProbes = 4;
+constexpr int kLineRest = 7;
+constexpr uint32_t kLineFree = 0xFFFFFFFFu;
+// float k of slot h sits at k * kLinePitch + h: the sixteen floats of a line
+// and the same float of neighbouring slots fall into different banks
+constexpr int kLinePitch = kLineSlots + 1;
+
+struct LineTable {
+    float val[16 * kLinePitch];
+    uint32_t key[kLineSlots];
+    // rows on their way to memory without the table; the flush keeps its list
+    // of used slots in the same place
+    union {
+        struct {
+            uint32_t row[64];
+            float v[64 * 4];
+        } out;
+        uint32_t used[kLineSlots];
+    };
+};
+
+// Orders the LDS traffic of one wavefront (whose LDS instructions execute in
+// program order, each for all its lanes) for the compiler.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// at[k * kLinePitch] += v[k], k = 0..3, in LDS.  The LDS executes a
+// floating-point add atomic one lane after the other (about three cycles a
+// lane, measured) and a 32-bit compare-and-swap at full rate: the add is a read
+// and a compare-and-swap of the sum, repeated by the lanes that met another
+// lane's update in between.  The four floats go side by side, two round trips
+// for all of them.
+__device__ __forceinline__ void lds_add4(float* at, const float (&v)[4]) {
+    unsigned int* w = reinterpret_cast<unsigned int*>(at);
+    unsigned int seen[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) seen[k] = w[k * kLinePitch];
+    unsigned int todo = 0xFu;
+    while (todo != 0u) {
+        unsigned int got[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            got[k] = seen[k];
+            if (todo & (1u << k)) {
+                const unsigned int sum = __float_as_uint(__uint_as_float(seen[k]) + v[k]);
+                got[k] = atomicCAS(w + k * kLinePitch, seen[k], sum);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (got[k] == seen[k]) todo &= ~(1u << k);
+            seen[k] = got[k];
+        }
+    }
+}
+
+struct LineAcc {
+    LineTable* tab;
+    int rest;      // tiles left during which the table is left aside
+    int wanted;    // rows handed in since the last flush (whole wavefront)
+    int spilled;   // of those, rows that found no place in the table
+
+    __device__ __forceinline__ void start(LineTable* t, int lane) {
+        tab = t;
+        rest = 0;
+        wanted = 0;
+        spilled = 0;
+        if (tab != nullptr) {
+            for (int i = lane; i < 16 * kLinePitch; i += 64) tab->val[i] = 0.f;
+            tab->key[lane] = kLineFree;
+            tab->key[lane + 64] = kLineFree;
+            wave_lds_fence();
+        }
+    }
+
+    // grad[4 * row .. 4 * row + 3] += v for the lanes that `want`; every lane
+    // of the wavefront must take part.
+    __device__ __forceinline__ void add4(float* __restrict__ grad, bool want, uint32_t row,
+                                         const float (&v)[4], int lane) {
+        bool placed = false;
+        if (want && rest == 0) {
+            const uint32_t line = row >> 2;
+            uint32_t h = (line * 0x9E3779B1u) >> 25;
+            for (int p = 0; p < kLineProbes; ++p) {
+                const uint32_t old = atomicCAS(&tab->key[h], kLineFree, line);
+                if (old == kLineFree || old == line) {
+                    lds_add4(tab->val + (row & 3u) * 4 * kLinePitch + h, v);
+                    placed = true;
+                    break;
+                }
+                h = (h + 1) & (kLineSlots - 1);
+            }
+        }
+        // The rest goes to memory now, regrouped so that the four floats of a
+        // row leave from neighbouring lanes of one instruction (one request a
+        // row; one lane sending its four floats would make four).
+        const uint64_t all = __ballot(want);
+        const uint64_t out = __ballot(want && !placed);
+        wanted += __popcll(all);
+        if (out == 0) return;
+        const int n = __popcll(out);
+        spilled += n;
+        wave_lds_fence();
+        if (want && !placed) {
+            const int at = __popcll(out & ((1ull << lane) - 1ull));
+            tab->out.row[at] = row;
+            *reinterpret_cast<float4*>(tab->out.v + at * 4) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        wave_lds_fence();
+        for (int i = 0; i < n; i += 16) {
+            const int e = i + (lane >> 2);
+            if (e < n) {
+                unsafeAtomicAdd(grad + static_cast<uint64_t>(tab->out.row[e]) * 4 + (lane & 3),
+                                tab->out.v[e * 4 + (lane & 3)]);
+            }
+        }
+        wave_lds_fence();
+    }
+
+    // Whole wavefront: sends the table's lines out and empties it.
+    __device__ __forceinline__ void flush(float* __restrict__ grad, int lane) {
+        if (rest > 0) {
+            --rest;
+        } else {
+            wave_lds_fence();
+            const bool lo = tab->key[lane] != kLineFree;
+            const bool hi = tab->key[lane + 64] != kLineFree;
+            const uint64_t mlo = __ballot(lo), mhi = __ballot(hi);
+            const uint64_t below = (1ull << lane) - 1ull;
+            const int nlo = __popcll(mlo);
+            const int n = nlo + __popcll(mhi);
+            if (lo) tab->used[__popcll(mlo & below)] = lane;
+            if (hi) tab->used[nlo + __popcll(mhi & below)] = lane + 64;
+            wave_lds_fence();
+            // four lines per instruction, sixteen lines per turn: the reads of
+            // a turn are issued together
+            for (int i = 0; i < n; i += 16) {
+                uint32_t h[4], line[4];
+                float v[4];
+                float* at[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = i + j * 4 + (lane >> 4);
+                    h[j] = e < n ? tab->used[e] : 0u;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int e = i + j * 4 + (lane >> 4);
+                    at[j] = tab->val + (lane & 15) * kLinePitch + h[j];
+                    line[j] = tab->key[h[j]];
+                    v[j] = e < n ? *at[j] : 0.f;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    // floats nobody contributed to are zero
+                    if (v[j] != 0.f) {
+                        *at[j] = 0.f;
+                        unsafeAtomicAdd(
+                                grad + ((static_cast<uint64_t>(line[j]) << 4) | (lane & 15)), v[j]);
+                    }
+                }
+            }
+            wave_lds_fence();
+            tab->key[lane] = kLineFree;
+            tab->key[lane + 64] = kLineFree;
+            wave_lds_fence();
+            if (spilled * 2 > wanted) rest = kLineRest;
+        }
+        wanted = 0;
+        spilled = 0;
+    }
+};
+
+// The loop over the corners that scatters is not unrolled (one copy of the
+// code, fewer registers), so the corner number is a run-time value there, and
+// what it selects -- a row number, an axis term -- must come out of registers
+// by conditional moves: an indexed access would move the whole array to
+// scratch memory.  To keep the compiler from building that indexed access
+// itself, both operands of every ?: pass through an empty asm statement, which
+// makes them values without an origin in memory (between two loads from one
+// object the compiler would select the address instead).
+template <typename V>
+__device__ __forceinline__ V in_register(V x) {
+    static_assert(sizeof(V) == 4, "one 32-bit register");
+    asm("" : "+v"(x));
+    return x;
+}
+
+struct Rows8 {
+    uint32_t r[8];
+    __device__ __forceinline__ explicit Rows8(const uint32_t (&row)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = row[i];
+    }
+    __device__ __forceinline__ uint32_t at(int c) const {
+        const uint32_t a = (c & 1) ? in_register(r[1]) : in_register(r[0]);
+        const uint32_t b = (c & 1) ? in_register(r[3]) : in_register(r[2]);
+        const uint32_t d = (c & 1) ? in_register(r[5]) : in_register(r[4]);
+        const uint32_t e = (c & 1) ? in_register(r[7]) : in_register(r[6]);
+        const uint32_t ab = (c & 2) ? in_register(b) : in_register(a);
+        const uint32_t de = (c & 2) ? in_register(e) : in_register(d);
+        return (c & 4) ? in_register(de) : in_register(ab);
+    }
+};
+
+// Corner weights for a corner number known at run time.
+struct AxisValues {
+    float w0a, w0b, w1a, w1b, w2a, w2b;
+    float d0a, d0b, d1a, d1b, d2a, d2b;
+    __device__ __forceinline__ explicit AxisValues(const AxisTerms<float>& t)
+        : w0a(t.w[0][0]), w0b(t.w[0][1]),
+          w1a(t.w[1][0]), w1b(t.w[1][1]),
+          w2a(t.w[2][0]), w2b(t.w[2][1]),
+          d0a(t.dw[0][0]), d0b(t.dw[0][1]),
+          d1a(t.dw[1][0]), d1b(t.dw[1][1]),
+          d2a(t.dw[2][0]), d2b(t.dw[2][1]) {}
+    __device__ __forceinline__ float weight(int c) const {
+        float w = 1.0f;
+        w *= (c & 1) ? in_register(w0b) : in_register(w0a);
+        w *= (c & 2) ? in_register(w1b) : in_register(w1a);
+        w *= (c & 4) ? in_register(w2b) : in_register(w2a);
+        return w;
+    }
+    __device__ __forceinline__ void weight_grad(int c, float (&g)[3]) const {
+        const float w0 = (c & 1) ? in_register(w0b) : in_register(w0a);
+        const float w1 = (c & 2) ? in_register(w1b) : in_register(w1a);
+        const float w2 = (c & 4) ? in_register(w2b) : in_register(w2a);
+        const float d0 = (c & 1) ? in_register(d0b) : in_register(d0a);
+        const float d1 = (c & 2) ? in_register(d1b) : in_register(d1a);
+        const float d2 = (c & 4) ? in_register(d2b) : in_register(d2a);
+        g[0] = d0 * w1 * w2;
+        g[1] = w0 * d1 * w2;
+        g[2] = w0 * w1 * d2;
+    }
+};
+
+// grad_emb[row, 0..3] += v for the lanes that are `on`; every lane of the
+// wavefront must take part.
+__device__ __forceinline__ void accumulate_row4(LineAcc& acc, float* __restrict__ grad_emb,
+                                                uint32_t row, bool on, float (&v)[4],
+                                                int lane) {
+    // lanes that are off get a row number no neighbour shares
+    const uint32_t id = on ? row : (kNoRow - static_cast<uint32_t>(lane & 1));
+    if (!on) v[0] = v[1] = v[2] = v[3] = 0.f;
+    const bool tail = merge_runs(id, v, lane);
+    acc.add4(grad_emb, on && tail, row, v, lane);
+}
+
+__device__ __forceinline__ LineTable* line_table(unsigned char* smem, const QDev& a,
+                                                 bool lds_lut, bool wanted) {
+    if (!wanted) return nullptr;
+    return reinterpret_cast<LineTable*>(smem + table_offset(a, 1, lds_lut)) +
+           (threadIdx.x >> 6);
+}
+
+// First-order backward, E = 4 (formulas as in query_backward_forward_kernel).
+template <bool LDS, int OUT>
+__global__ __launch_bounds__(kBlock, kWavesWide) void
+query_backward_forward_vec_kernel(
+        QDev a, const float* __restrict__ z, float* __restrict__ grad_emb,
+        float* __restrict__ grad_off) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CellLut lut = stage_cell_lut<LDS>(a, smem);
+    const int lane = threadIdx.x & 63;
+    const float* __restrict__ emb = static_cast<const float*>(a.emb);
+    constexpr bool want_emb = (OUT & 1) != 0;
+    constexpr bool want_off = (OUT & 2) != 0;
+    LineAcc acc;
+    acc.start(line_table(smem, a, LDS, want_emb), lane);
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        uint32_t row[8];
+        float o[3];
+        const int64_t q = tile * kBlock + threadIdx.x;
+        resolve_rows<LDS>(a, lut, q, row, o);
+        const bool on = row[0] != kNoRow;
+        float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (on) z4 = *reinterpret_cast<const float4*>(z + q * 4);
+        AxisTerms<float> t;
+        axis_terms<float, true>(o, a.smooth, t);
+        // the gathered rows are used up before the scatter starts, which keeps
+        // them out of the registers the scatter needs
+        if constexpr (want_off) {
+            float4 e[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                e[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (on) {
+                    e[c] = *reinterpret_cast<const float4*>(
+                            emb + static_cast<int64_t>(row[c]) * 4);
+                }
+            }
+            float go[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float gw[3];
+                corner_weight_grad<float>(t, c, gw);
+                float dot = e[c].x * z4.x;
+                dot += e[c].y * z4.y;
+                dot += e[c].z * z4.z;
+                dot += e[c].w * z4.w;
+                go[0] += dot * gw[0];
+                go[1] += dot * gw[1];
+                go[2] += dot * gw[2];
+            }
+            if (q < a.N) {
+                grad_off[q * 3 + 0] = on ? go[0] : 0.f;
+                grad_off[q * 3 + 1] = on ? go[1] : 0.f;
+                grad_off[q * 3 + 2] = on ? go[2] : 0.f;
+            }
+        }
+        if constexpr (want_emb) {
+            // one copy of the scatter code, not eight: fewer registers and a
+            // loop that stays in the instruction cache
+            const AxisValues tv(t);
+            const Rows8 rows(row);
+#pragma unroll 1
+            for (int c = 0; c < 8; ++c) {
+                const float w = tv.weight(c);
+                float v[4] = {w * z4.x, w * z4.y, w * z4.z, w * z4.w};
+                accumulate_row4(acc, grad_emb, rows.at(c), on, v, lane);
+            }
+            acc.flush(grad_emb, lane);
+        }
+    }
+}
+
+// Backward of the backward, E = 4 (formulas as in
+// query_backward_backward_kernel).
+template <bool LDS, int OUT>
+__global__ __launch_bounds__(kBlock, kWavesWide) void
+query_backward_backward_vec_kernel(
+        QDev a, const float* __restrict__ gg_off, const float* __restrict__ z,
+        float* __restrict__ grad_z, float* __restrict__ grad_emb) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const CellLut lut = stage_cell_lut<LDS>(a, smem);
+    const int lane = threadIdx.x & 63;
+    const float* __restrict__ emb = static_cast<const float*>(a.emb);
+    constexpr bool want_emb = (OUT & 1) != 0;
+    constexpr bool want_z = (OUT & 2) != 0;
+    LineAcc acc;
+    acc.start(line_table(smem, a, LDS, want_emb), lane);
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        uint32_t row[8];
+        float o[3];
+        const int64_t q = tile * kBlock + threadIdx.x;
+        resolve_rows<LDS>(a, lut, q, row, o);
+        const bool on = row[0] != kNoRow;
+        float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        float gg[3] = {0.f, 0.f, 0.f};
+        if (on) {
+            z4 = *reinterpret_cast<const float4*>(z + q * 4);
+            gg[0] = gg_off[q * 3 + 0];
+            gg[1] = gg_off[q * 3 + 1];
+            gg[2] = gg_off[q * 3 + 2];
+        }
+        AxisTerms<float> t;
+        axis_terms<float, true>(o, a.smooth, t);
+        if constexpr (want_z) {
+            float4 e[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                e[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (on) {
+                    e[c] = *reinterpret_cast<const float4*>(
+                            emb + static_cast<int64_t>(row[c]) * 4);
+                }
+            }
+            float gz[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float gw[3];
+                corner_weight_grad<float>(t, c, gw);
+                const float d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
+                gz[0] += d * e[c].x;
+                gz[1] += d * e[c].y;
+                gz[2] += d * e[c].z;
+                gz[3] += d * e[c].w;
+            }
+            if (q < a.N) {
+                *reinterpret_cast<float4*>(grad_z + q * 4) =
+                        on ? make_float4(gz[0], gz[1], gz[2], gz[3])
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+        if constexpr (want_emb) {
+            const AxisValues tv(t);
+            const Rows8 rows(row);
+#pragma unroll 1
+            for (int c = 0; c < 8; ++c) {
+                float gw[3];
+                tv.weight_grad(c, gw);
+                const float d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
+                float v[4] = {d * z4.x, d * z4.y, d * z4.z, d * z4.w};
+                accumulate_row4(acc, grad_emb, rows.at(c), on, v, lane);
+            }
+            acc.flush(grad_emb, lane);
         }
     }
 }
@@ -1473,9 +1956,9 @@ int pow2_ceil(int v) {
 
 bool lut_in_lds(const QDev& d) { return d.M <= kMaxLdsCells; }
 
-size_t smem_bytes(const QDev& d, int lpq) {
-    size_t bytes = lpq > 1 ? sizeof(Tile) : 0;
-    if (lut_in_lds(d)) bytes += static_cast<size_t>(d.M) * 8 * 3;
+size_t smem_bytes(const QDev& d, int lpq, bool line_tables = false) {
+    size_t bytes = table_offset(d, lpq, lut_in_lds(d));
+    if (line_tables) bytes += (kBlock / 64) * sizeof(LineTable);
     return bytes;
 }
 
@@ -1572,6 +2055,58 @@ bool aligned16(const void* p) {
     return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
 
+int launch_bwd_fwd_vec(const QDev& d, const void* z, void* ge, void* go,
+                       hipStream_t s) {
+    const size_t smem = smem_bytes(d, 1, ge != nullptr);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    const int out = (ge != nullptr ? 1 : 0) | (go != nullptr ? 2 : 0);
+#define ASH_BF(L, O)                                                          \
+    query_backward_forward_vec_kernel<L, O><<<g, kBlock, smem, s>>>(     \
+            d, static_cast<const float*>(z), static_cast<float*>(ge),         \
+            static_cast<float*>(go))
+    if (lut_in_lds(d)) {
+        if (out == 3) ASH_BF(true, 3);
+        else if (out == 1) ASH_BF(true, 1);
+        else ASH_BF(true, 2);
+    } else {
+        if (out == 3) ASH_BF(false, 3);
+        else if (out == 1) ASH_BF(false, 1);
+        else ASH_BF(false, 2);
+    }
+#undef ASH_BF
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_bwd_bwd_vec(const QDev& d, const void* gg, const void* z, void* gz,
+                       void* ge, hipStream_t s) {
+    const size_t smem = smem_bytes(d, 1, ge != nullptr);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    const int out = (ge != nullptr ? 1 : 0) | (gz != nullptr ? 2 : 0);
+#define ASH_BB(L, O)                                                          \
+    query_backward_backward_vec_kernel<L, O><<<g, kBlock, smem, s>>>(    \
+            d, static_cast<const float*>(gg), static_cast<const float*>(z),   \
+            static_cast<float*>(gz), static_cast<float*>(ge))
+    if (lut_in_lds(d)) {
+        if (out == 3) ASH_BB(true, 3);
+        else if (out == 1) ASH_BB(true, 1);
+        else ASH_BB(true, 2);
+    } else {
+        if (out == 3) ASH_BB(false, 3);
+        else if (out == 1) ASH_BB(false, 1);
+        else ASH_BB(false, 2);
+    }
+#undef ASH_BB
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+// fp32 rows of four channels on 16-byte aligned buffers
+bool rows_as_float4(const QDev& d, const void* p0, const void* p1, const void* p2) {
+    return d.E == 4 && aligned16(d.emb) && aligned16(p0) && aligned16(p1) &&
+           aligned16(p2);
+}
+
 template <typename T>
 int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
     if constexpr (sizeof(T) == 4) {
@@ -1603,6 +2138,9 @@ int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
 template <typename T>
 int dispatch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
                      hipStream_t s) {
+    if constexpr (sizeof(T) == 4) {
+        if (rows_as_float4(d, z, ge, nullptr)) return launch_bwd_fwd_vec(d, z, ge, go, s);
+    }
     switch (pow2_ceil(d.E)) {
         case 1:
             return launch_bwd_fwd<T, 1>(d, z, ge, go, s);
@@ -1620,6 +2158,9 @@ int dispatch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
 template <typename T>
 int dispatch_bwd_bwd(const QDev& d, const void* gg, const void* z, void* gz,
                      void* ge, hipStream_t s) {
+    if constexpr (sizeof(T) == 4) {
+        if (rows_as_float4(d, z, ge, gz)) return launch_bwd_bwd_vec(d, gg, z, gz, ge, s);
+    }
     switch (pow2_ceil(d.E)) {
         case 1:
             return launch_bwd_bwd<T, 1>(d, gg, z, gz, ge, s);
