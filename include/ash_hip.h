@@ -142,8 +142,8 @@ int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
  * to out_coords int32[capacity, 3]; the flags are cleared and the count is left
  * in the table's counters (out[5] of ash_map_status_staged), so that the
  * read-back that follows an activation anyway also sizes the result -- instead
- * of a `nonzero` over the flags with a read-back of its own.  One workgroup;
- * tables of up to ASH_COLLECT_MAX_BLOCKS rows.  No counterpart in the
+ * of a `nonzero` over the flags with a read-back of its own.  Tables of up to
+ * ASH_COLLECT_MAX_BLOCKS rows; `touched` 4-byte aligned.  No counterpart in the
  * reference. */
 #define ASH_COLLECT_MAX_BLOCKS (1 << 20)
 int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* block_coords,

@@ -257,15 +257,19 @@ def test_frames_without_read_back_equal_counted_frames(gpu_ash):
 @pytest.mark.parametrize("capacity", [5, 1000, 80_000, 131_073, 200_000, 1_048_576])
 def test_touched_rows_are_listed_in_order(gpu_ash, capacity):
     """ash_grid_collect_touched against torch.nonzero: ascending rows, their
-    coordinates, flags cleared, count in the sixth status value -- for runs of
-    flags per thread that fit the registers, that do not, and that end inside
-    the last word."""
+    coordinates, flags cleared, count in the sixth status value -- for tables of
+    one workgroup's chunk and of many, with one and with two words of flags per
+    thread, that end inside a word, and for flags that start at a 4-byte but not
+    at a 16-byte boundary.  Three calls in a row on one table: the workgroups'
+    ticket counter has to be back at zero after each."""
     engine = gpu_ash.ASHEngine(3, capacity, DEV)
     backend = engine.backend
     g = torch.Generator().manual_seed(capacity)
-    for density in (0.0, 0.05, 1.0):
-        flags = (torch.rand(capacity, generator=g) < density).to(torch.uint8).to(DEV)
-        flags = flags * torch.randint(1, 255, (capacity,), generator=g, dtype=torch.uint8).to(DEV)
+    for density, shift in ((0.0, 0), (0.05, 4), (1.0, 0)):
+        store = torch.zeros(capacity + 16, dtype=torch.uint8, device=DEV)
+        flags = store[shift : shift + capacity]
+        flags.copy_((torch.rand(capacity, generator=g) < density).to(torch.uint8))
+        flags.mul_(torch.randint(1, 255, (capacity,), generator=g, dtype=torch.uint8).to(DEV))
         coords = torch.randint(-1000, 1000, (capacity, 3), generator=g, dtype=torch.int32).to(DEV)
         expected = flags.nonzero().view(-1)
         rows = torch.full((capacity,), -1, dtype=torch.int64, device=DEV)

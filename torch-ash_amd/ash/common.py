@@ -1108,7 +1108,7 @@ class _HashMap:
         heads = torch.empty(64 + 3 * cells.shape[0], dtype=torch.int32, device=self._device)
         # the touched rows are listed on the device and their count travels with
         # the read-back that ends the activation (tables beyond the listing
-        # kernel's one workgroup take torch's nonzero and a second read-back)
+        # kernel's limit take torch's nonzero and a second read-back)
         listing = self.capacity <= COLLECT_MAX_BLOCKS
         if listing:
             rows = torch.empty(self.capacity, dtype=torch.int64, device=self._device)

@@ -64,6 +64,7 @@ enum Counter {
     kCtrLoadDup = 4,   // duplicate pairs met by load
     kCtrCursor = 5,    // output cursor of items()
     kCtrTouched = 6,   // blocks listed by the latest ash_grid_collect_touched
+    kCtrTicket = 7,    // workgroups of a running ash_grid_collect_touched that have read their input
     kNumCounters = 64
 };
 constexpr int64_t kHeaderBytes = 256;

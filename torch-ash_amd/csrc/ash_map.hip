@@ -1309,81 +1309,122 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(
 
 // The rows whose flag an activation has set, in ascending order, with their
 // block coordinates; the flags are cleared on the way and the count goes to
-// the table's counters, where the read-back that follows every activation
-// finds it.  One workgroup: every thread takes a run of `span` flags (a
-// multiple of four, read as words), an exclusive scan over the workgroup
-// gives each run its place in the output.
+// the table's counters, where the read-back that follows an activation finds
+// it (and where ash_grid_integrate_depth_touched reads it on the device).
+//
+// Up to kCollectGroups workgroups, each with a chunk of the flags: a workgroup
+// holds its own chunk in registers (one run of `words` 4-flag words per thread,
+// so that thread order is flag order), counts the flags of all chunks before
+// its own (they sit in L2: every workgroup reads them) and so knows where its
+// rows go without waiting for anybody.  Nobody may clear flags while others
+// still count them: each workgroup draws a ticket when it has read all it
+// needs, and the one that draws the last ticket clears the whole array and
+// puts the ticket counter back to zero.
 constexpr int kCollectThreads = 1024;
+constexpr int kCollectGroups = 128;
+constexpr int kCollectMaxWords = 2;    // per thread: 2^20 flags / 128 groups / 1024 threads / 4
 constexpr int64_t kCollectMaxBlocks = int64_t{1} << 20;   // ASH_COLLECT_MAX_BLOCKS of the header
 
-__global__ __launch_bounds__(kCollectThreads) void collect_touched_kernel(
-        uint8_t* __restrict__ touched, const int32_t* __restrict__ block_coords,
-        int64_t capacity, int span, int64_t* __restrict__ out_idx,
-        int32_t* __restrict__ out_coords, int32_t* __restrict__ ctr) {
-    __shared__ int s_wave[kCollectThreads / 64];
+__device__ __forceinline__ int flags_in(uint32_t w) {
+    return (w & 0xFFu ? 1 : 0) + (w & 0xFF00u ? 1 : 0) + (w & 0xFF0000u ? 1 : 0) +
+           (w & 0xFF000000u ? 1 : 0);
+}
+
+// word `i` of the flags, bytes beyond `capacity` read as zero
+__device__ __forceinline__ uint32_t flag_word(const uint8_t* touched, int64_t i, int64_t capacity) {
+    const int64_t at = i * 4;
+    if (at + 4 <= capacity) return *reinterpret_cast<const uint32_t*>(touched + at);
+    uint32_t w = 0;
+    for (int b = 0; at + b < capacity; ++b) w |= static_cast<uint32_t>(touched[at + b]) << (8 * b);
+    return w;
+}
+
+// Sum of `v` over the workgroup; `mine` = sum over the threads before this one.
+__device__ __forceinline__ int block_sums(int v, int* s_wave, int& mine) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t first = static_cast<int64_t>(threadIdx.x) * span;
-    int cnt = 0;
-    for (int o = 0; o < span; o += 4) {
-        const int64_t at = first + o;
-        if (at >= capacity) break;
-        uint32_t w = at + 4 <= capacity ? *reinterpret_cast<const uint32_t*>(touched + at) : 0u;
-        if (at + 4 > capacity) {
-            for (int b = 0; at + b < capacity; ++b) w |= static_cast<uint32_t>(touched[at + b]) << (8 * b);
-        }
-        cnt += (w & 0xFFu ? 1 : 0) + (w & 0xFF00u ? 1 : 0) + (w & 0xFF0000u ? 1 : 0) +
-               (w & 0xFF000000u ? 1 : 0);
-    }
-    int incl = cnt;
+    int incl = v;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
         const int up = __shfl_up(incl, d);
         if (lane >= d) incl += up;
     }
+    __syncthreads();   // s_wave free again
     if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
-    int pos = incl - cnt;
+    mine = incl - v;
     int total = 0;
     for (int q = 0; q < kCollectThreads / 64; ++q) {
-        if (q < wave) pos += s_wave[q];
+        if (q < wave) mine += s_wave[q];
         total += s_wave[q];
     }
-    if (threadIdx.x == 0) ctr[kCtrTouched] = total;
-    if (cnt == 0) return;
-    auto list = [&](int64_t at) {
-        out_idx[pos] = at;
-        out_coords[pos * 3 + 0] = block_coords[at * 3 + 0];
-        out_coords[pos * 3 + 1] = block_coords[at * 3 + 1];
-        out_coords[pos * 3 + 2] = block_coords[at * 3 + 2];
-        ++pos;
-    };
-    constexpr int kWords = 32;   // runs of up to 128 flags are held in registers
-    if (span <= 4 * kWords && first + span <= capacity) {
-        uint32_t w[kWords];
+    return total;
+}
+
+__global__ __launch_bounds__(kCollectThreads) void collect_touched_kernel(
+        uint8_t* __restrict__ touched, const int32_t* __restrict__ block_coords,
+        int64_t capacity, int words, int64_t* __restrict__ out_idx,
+        int32_t* __restrict__ out_coords, int32_t* __restrict__ ctr) {
+    __shared__ int s_wave[kCollectThreads / 64];
+    __shared__ int s_last;
+    const int64_t chunk_words = static_cast<int64_t>(words) * kCollectThreads;
+    const int64_t first_word = blockIdx.x * chunk_words + static_cast<int64_t>(threadIdx.x) * words;
+    uint32_t w[kCollectMaxWords];
+    int own = 0;
 #pragma unroll
-        for (int i = 0; i < kWords; ++i) {
-            w[i] = 4 * i < span ? *reinterpret_cast<const uint32_t*>(touched + first + 4 * i) : 0u;
+    for (int i = 0; i < kCollectMaxWords; ++i) {
+        w[i] = i < words ? flag_word(touched, first_word + i, capacity) : 0u;
+        own += flags_in(w[i]);
+    }
+    int before = 0;
+    const int64_t words_before = blockIdx.x * chunk_words;   // whole words, inside the array
+    if (reinterpret_cast<uintptr_t>(touched) % 16 == 0) {
+        const uint4* quads = reinterpret_cast<const uint4*>(touched);
+#pragma unroll 8
+        for (int64_t i = threadIdx.x; i < words_before / 4; i += kCollectThreads) {
+            const uint4 v = quads[i];
+            before += flags_in(v.x) + flags_in(v.y) + flags_in(v.z) + flags_in(v.w);
         }
+    } else {
+#pragma unroll 8
+        for (int64_t i = threadIdx.x; i < words_before; i += kCollectThreads) {
+            before += flags_in(reinterpret_cast<const uint32_t*>(touched)[i]);
+        }
+    }
+    int unused;
+    const int base = block_sums(before, s_wave, unused);
+    int pos;
+    const int total = block_sums(own, s_wave, pos);
+    pos += base;
+    if (threadIdx.x == 0) {
+        if (blockIdx.x == gridDim.x - 1) ctr[kCtrTouched] = base + total;
+        __threadfence();
+        s_last = atomicAdd(ctr + kCtrTicket, 1) == static_cast<int>(gridDim.x) - 1;
+    }
 #pragma unroll
-        for (int i = 0; i < kWords; ++i) {
-            if (w[i] == 0u) continue;
-            *reinterpret_cast<uint32_t*>(touched + first + 4 * i) = 0u;
+    for (int i = 0; i < kCollectMaxWords; ++i) {
+        if (w[i] == 0u) continue;
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                if ((w[i] >> (8 * b)) & 0xFFu) list(first + 4 * i + b);
+        for (int b = 0; b < 4; ++b) {
+            if ((w[i] >> (8 * b)) & 0xFFu) {
+                const int64_t at = (first_word + i) * 4 + b;
+                out_idx[pos] = at;
+                out_coords[pos * 3 + 0] = block_coords[at * 3 + 0];
+                out_coords[pos * 3 + 1] = block_coords[at * 3 + 1];
+                out_coords[pos * 3 + 2] = block_coords[at * 3 + 2];
+                ++pos;
             }
         }
-        return;
     }
-    for (int o = 0; o < span; ++o) {
-        const int64_t at = first + o;
-        if (at >= capacity) break;
-        if (touched[at]) {
-            touched[at] = 0;
-            list(at);
-        }
+    __syncthreads();
+    if (!s_last) return;
+    // every workgroup has read what it needs
+    const int64_t whole = capacity / 4;
+    for (int64_t i = threadIdx.x; i < whole; i += kCollectThreads) {
+        reinterpret_cast<uint32_t*>(touched)[i] = 0u;
     }
+    if (threadIdx.x < capacity - whole * 4) touched[whole * 4 + threadIdx.x] = 0;
+    if (threadIdx.x == 0) ctr[kCtrTicket] = 0;
 }
 
 // ---------------------------------------------------------------- host
@@ -2134,14 +2175,18 @@ int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* bl
         out_coords == nullptr) {
         ASH_FAIL("null pointer in grid_collect_touched");
     }
-    if (map->capacity > kCollectMaxBlocks) ASH_FAIL("grid_collect_touched: too many blocks for one workgroup");
+    if (map->capacity > kCollectMaxBlocks) ASH_FAIL("grid_collect_touched: more than ASH_COLLECT_MAX_BLOCKS rows");
     if (reinterpret_cast<uintptr_t>(touched) % 4 != 0) ASH_FAIL("grid_collect_touched: flags must be 4-byte aligned");
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    int span = static_cast<int>((map->capacity + kCollectThreads - 1) / kCollectThreads);
-    span = (span + 3) / 4 * 4;
-    collect_touched_kernel<<<1, kCollectThreads, 0, static_cast<hipStream_t>(stream)>>>(
-            touched, block_coords, map->capacity, span, out_indices, out_coords, map->d.ctr);
+    const int64_t per_group = int64_t{4} * kCollectThreads;   // flags of a one-word-per-thread chunk
+    int64_t groups = (map->capacity + per_group - 1) / per_group;
+    if (groups > kCollectGroups) groups = kCollectGroups;
+    const int words = static_cast<int>((map->capacity + groups * per_group - 1) / (groups * per_group));
+    groups = (map->capacity + words * per_group - 1) / (words * per_group);   // no empty chunks
+    collect_touched_kernel<<<static_cast<unsigned>(groups), kCollectThreads, 0,
+                             static_cast<hipStream_t>(stream)>>>(
+            touched, block_coords, map->capacity, words, out_indices, out_coords, map->d.ctr);
     ASH_LAUNCH_CHECK();
     return 0;
 }
