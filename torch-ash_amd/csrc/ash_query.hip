@@ -550,9 +550,9 @@ query_backward_backward_kernel(
 // a modifier of an ordinary vector instruction, across rows it would be a trip
 // through the LDS pipeline, so a run is cut at the row of lanes; the table
 // joins the pieces).  A row whose line finds no place within kLineProbes steps
-// goes to memory directly, and a wavefront half of whose rows had to do that
-// (unordered queries share no lines) leaves the table aside for the next
-// kLineRest tiles.
+// goes to memory directly, and a wavefront that sent more rows that way than
+// the table has lines (unordered queries share no lines) leaves the table
+// aside for the next kLineRest tiles.
 template <int CTRL>
 __device__ __forceinline__ int dpp_int(int v) {
     return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
@@ -579,19 +579,48 @@ __device__ __forceinline__ void run_step(float (&v)[4], int& f, int g) {
     if (take) f |= fu;
 }
 
-// Sums `v` over runs of consecutive lanes (of one row of 16) with equal `id`;
-// returns whether this lane ends its run and holds the total.  Every lane of
-// the wavefront must take part.
+constexpr int kRowBcast15 = 0x142;  // every lane of a row takes lane 15 of the row before
+
+// Sums `v` over runs of consecutive lanes with equal `id`; returns whether this
+// lane ends its run and holds the total.  Every lane of the wavefront must take
+// part.  The sums run inside the rows of 16 lanes; a run that goes on in the
+// next row hands its part over: lane 15 keeps quiet and the lane that ends the
+// run in the next row adds what lane 15 had.  (A run that fills a whole row
+// and still goes on is not handed over a second time; its parts meet in the
+// table of lines.)
 __device__ __forceinline__ bool merge_runs(uint32_t id, float (&v)[4], int lane) {
     const int g = lane & 15;
     const uint32_t prev = dpp<kRowShr + 1>(id);
     const uint32_t next = dpp<kRowShl + 1>(id);
-    int f = (g == 0 || prev != id) ? 1 : 0;
-    const bool tail = g == 15 || next != id;
+    const bool starts = g > 0 && prev != id;   // a run starts here, inside the row
+    int f = (g == 0 || starts) ? 1 : 0;
+    bool tail = g == 15 || next != id;
     run_step<1>(v, f, g);
     run_step<2>(v, f, g);
     run_step<4>(v, f, g);
     run_step<8>(v, f, g);
+    // in the first run of its row: no run starts between the row's first lane and here
+    const uint64_t started = __ballot(starts);
+    const uint64_t upto = (2ull << lane) - 1ull;
+    const uint64_t row_lanes = 0xFFFFull << (lane & 48);
+    const bool first_run = (started & upto & row_lanes) == 0;
+    // lane 15 offers its sum unless its run began with the row
+    const int offers = (g == 15 && !first_run) ? 1 : 0;
+    const int offered = dpp_int<kRowBcast15>(offers);
+    const uint32_t offered_id = dpp<kRowBcast15>(id);
+    float part[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) part[k] = dpp<kRowBcast15>(v[k]);
+    if (lane >= 16 && tail && first_run && offered != 0 && offered_id == id) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] += part[k];
+    }
+    // ... and keeps quiet when the next row takes the offer
+    const uint32_t id16 = __builtin_amdgcn_readlane(id, 16);
+    const uint32_t id32 = __builtin_amdgcn_readlane(id, 32);
+    const uint32_t id48 = __builtin_amdgcn_readlane(id, 48);
+    const uint32_t over = lane < 16 ? id16 : lane < 32 ? id32 : id48;
+    if (offers != 0 && lane < 48 && over == id) tail = false;
     return tail;
 }
 
@@ -628,29 +657,29 @@ __device__ __forceinline__ void wave_lds_fence() {
 // at[k * kLinePitch] += v[k], k = 0..3, in LDS.  The LDS executes a
 // floating-point add atomic one lane after the other (about three cycles a
 // lane, measured) and a 32-bit compare-and-swap at full rate: the add is a read
-// and a compare-and-swap of the sum, repeated by the lanes that met another
-// lane's update in between.  The four floats go side by side, two round trips
-// for all of them.
+// and a compare-and-swap of the sum.  The four floats go side by side, two
+// round trips for all of them; lanes that met another lane's update in between
+// (seldom: runs of equal rows have been summed before) repeat float by float.
 __device__ __forceinline__ void lds_add4(float* at, const float (&v)[4]) {
     unsigned int* w = reinterpret_cast<unsigned int*>(at);
-    unsigned int seen[4];
+    unsigned int seen[4], got[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) seen[k] = w[k * kLinePitch];
-    unsigned int todo = 0xFu;
-    while (todo != 0u) {
-        unsigned int got[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            got[k] = seen[k];
-            if (todo & (1u << k)) {
-                const unsigned int sum = __float_as_uint(__uint_as_float(seen[k]) + v[k]);
-                got[k] = atomicCAS(w + k * kLinePitch, seen[k], sum);
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            if (got[k] == seen[k]) todo &= ~(1u << k);
-            seen[k] = got[k];
+    for (int k = 0; k < 4; ++k) {
+        got[k] = atomicCAS(w + k * kLinePitch, seen[k],
+                           __float_as_uint(__uint_as_float(seen[k]) + v[k]));
+    }
+    if (got[0] == seen[0] && got[1] == seen[1] && got[2] == seen[2] && got[3] == seen[3]) return;
+#pragma unroll 1
+    for (int k = 0; k < 4; ++k) {
+        // (selects, not an indexed access: the arrays stay in registers)
+        unsigned int g = k == 0 ? got[0] : k == 1 ? got[1] : k == 2 ? got[2] : got[3];
+        unsigned int s = k == 0 ? seen[0] : k == 1 ? seen[1] : k == 2 ? seen[2] : seen[3];
+        const float add = k == 0 ? v[0] : k == 1 ? v[1] : k == 2 ? v[2] : v[3];
+        while (g != s) {
+            s = g;
+            g = atomicCAS(w + k * kLinePitch, s, __float_as_uint(__uint_as_float(s) + add));
         }
     }
 }
@@ -658,13 +687,11 @@ __device__ __forceinline__ void lds_add4(float* at, const float (&v)[4]) {
 struct LineAcc {
     LineTable* tab;
     int rest;      // tiles left during which the table is left aside
-    int wanted;    // rows handed in since the last flush (whole wavefront)
-    int spilled;   // of those, rows that found no place in the table
+    int spilled;   // rows that found no place in the table since the last flush (whole wavefront)
 
     __device__ __forceinline__ void start(LineTable* t, int lane) {
         tab = t;
         rest = 0;
-        wanted = 0;
         spilled = 0;
         if (tab != nullptr) {
             for (int i = lane; i < 16 * kLinePitch; i += 64) tab->val[i] = 0.f;
@@ -682,22 +709,21 @@ struct LineAcc {
         if (want && rest == 0) {
             const uint32_t line = row >> 2;
             uint32_t h = (line * 0x9E3779B1u) >> 25;
+#pragma unroll 1
             for (int p = 0; p < kLineProbes; ++p) {
                 const uint32_t old = atomicCAS(&tab->key[h], kLineFree, line);
                 if (old == kLineFree || old == line) {
-                    lds_add4(tab->val + (row & 3u) * 4 * kLinePitch + h, v);
                     placed = true;
                     break;
                 }
                 h = (h + 1) & (kLineSlots - 1);
             }
+            if (placed) lds_add4(tab->val + (row & 3u) * 4 * kLinePitch + h, v);
         }
         // The rest goes to memory now, regrouped so that the four floats of a
         // row leave from neighbouring lanes of one instruction (one request a
         // row; one lane sending its four floats would make four).
-        const uint64_t all = __ballot(want);
         const uint64_t out = __ballot(want && !placed);
-        wanted += __popcll(all);
         if (out == 0) return;
         const int n = __popcll(out);
         spilled += n;
@@ -765,9 +791,9 @@ struct LineAcc {
             tab->key[lane] = kLineFree;
             tab->key[lane + 64] = kLineFree;
             wave_lds_fence();
-            if (spilled * 2 > wanted) rest = kLineRest;
+            // more rows went past the table than it has lines
+            if (spilled > kLineSlots) rest = kLineRest;
         }
-        wanted = 0;
         spilled = 0;
     }
 };
