@@ -803,14 +803,23 @@ struct LineAcc {
 // what it selects -- a row number, an axis term -- must come out of registers
 // by conditional moves: an indexed access would move the whole array to
 // scratch memory.  To keep the compiler from building that indexed access
-// itself, both operands of every ?: pass through an empty asm statement, which
-// makes them values without an origin in memory (between two loads from one
-// object the compiler would select the address instead).
+// itself, both operands of every select pass through an empty asm statement,
+// which makes them values without an origin in memory (between two loads from
+// one object the compiler would select the address instead).
 template <typename V>
 __device__ __forceinline__ V in_register(V x) {
     static_assert(sizeof(V) == 4, "one 32-bit register");
     asm("" : "+v"(x));
     return x;
+}
+
+// Both operands are laundered before the select, so that the select stays one
+// conditional move (an asm statement inside an arm of ?: would make it a branch).
+template <typename V>
+__device__ __forceinline__ V pick(bool second, V a, V b) {
+    const V x = in_register(a);
+    const V y = in_register(b);
+    return second ? y : x;
 }
 
 struct Rows8 {
@@ -820,13 +829,13 @@ struct Rows8 {
         for (int i = 0; i < 8; ++i) r[i] = row[i];
     }
     __device__ __forceinline__ uint32_t at(int c) const {
-        const uint32_t a = (c & 1) ? in_register(r[1]) : in_register(r[0]);
-        const uint32_t b = (c & 1) ? in_register(r[3]) : in_register(r[2]);
-        const uint32_t d = (c & 1) ? in_register(r[5]) : in_register(r[4]);
-        const uint32_t e = (c & 1) ? in_register(r[7]) : in_register(r[6]);
-        const uint32_t ab = (c & 2) ? in_register(b) : in_register(a);
-        const uint32_t de = (c & 2) ? in_register(e) : in_register(d);
-        return (c & 4) ? in_register(de) : in_register(ab);
+        const uint32_t a = pick((c & 1) != 0, r[0], r[1]);
+        const uint32_t b = pick((c & 1) != 0, r[2], r[3]);
+        const uint32_t d = pick((c & 1) != 0, r[4], r[5]);
+        const uint32_t e = pick((c & 1) != 0, r[6], r[7]);
+        const uint32_t ab = pick((c & 2) != 0, a, b);
+        const uint32_t de = pick((c & 2) != 0, d, e);
+        return pick((c & 4) != 0, ab, de);
     }
 };
 
@@ -843,18 +852,18 @@ struct AxisValues {
           d2a(t.dw[2][0]), d2b(t.dw[2][1]) {}
     __device__ __forceinline__ float weight(int c) const {
         float w = 1.0f;
-        w *= (c & 1) ? in_register(w0b) : in_register(w0a);
-        w *= (c & 2) ? in_register(w1b) : in_register(w1a);
-        w *= (c & 4) ? in_register(w2b) : in_register(w2a);
+        w *= pick((c & 1) != 0, w0a, w0b);
+        w *= pick((c & 2) != 0, w1a, w1b);
+        w *= pick((c & 4) != 0, w2a, w2b);
         return w;
     }
     __device__ __forceinline__ void weight_grad(int c, float (&g)[3]) const {
-        const float w0 = (c & 1) ? in_register(w0b) : in_register(w0a);
-        const float w1 = (c & 2) ? in_register(w1b) : in_register(w1a);
-        const float w2 = (c & 4) ? in_register(w2b) : in_register(w2a);
-        const float d0 = (c & 1) ? in_register(d0b) : in_register(d0a);
-        const float d1 = (c & 2) ? in_register(d1b) : in_register(d1a);
-        const float d2 = (c & 4) ? in_register(d2b) : in_register(d2a);
+        const float w0 = pick((c & 1) != 0, w0a, w0b);
+        const float w1 = pick((c & 2) != 0, w1a, w1b);
+        const float w2 = pick((c & 4) != 0, w2a, w2b);
+        const float d0 = pick((c & 1) != 0, d0a, d0b);
+        const float d1 = pick((c & 2) != 0, d1a, d1b);
+        const float d2 = pick((c & 4) != 0, d2a, d2b);
         g[0] = d0 * w1 * w2;
         g[1] = w0 * d1 * w2;
         g[2] = w0 * w1 * d2;
