@@ -101,8 +101,8 @@ MEASURED_COUNTERS = {
     "cfg3_forward_smooth_step": (3_519_000_000 + 282_000_000, 0.171, 0),
     "cfg4_forward": (369_000_000 + 67_000_000, 0.258, 0),
     # kernel only: the zero fill of the dense gradient adds 1.64 GB written
-    "cfg4_backward": (431_000_000 + 311_000_000 + 1_638_400_000, 0.078, 7_589_000),
-    "cfg4_double_backward": (478_000_000 + 328_000_000 + 1_638_400_000, 0.087, 7_589_000),
+    "cfg4_backward": (431_000_000 + 149_000_000 + 1_638_400_000, 0.093, 2_344_000),
+    "cfg4_double_backward": (486_000_000 + 197_000_000 + 1_638_400_000, 0.163, 2_344_000),
     "cfg4_grid_query": (71_000_000 + 122_000_000, 0.399, 0),
 }
 
@@ -193,8 +193,9 @@ def measure_ceilings(torch, ash, dev, table_bytes, n):
     """What this device's memory system delivers for the two access patterns
     that bound the table kernels, measured with the probes of bench_probes.hip on a
     buffer of the table's size: random 128-byte line reads (a probe) and random
-    line read + compare-and-swap + dword store (an insert); plus a plain
-    device-to-device copy for the streaming rate."""
+    line read + compare-and-swap + dword store (an insert); float adds without
+    a result, alone and sixteen to a 64-byte half-line (gradient accumulation);
+    plus a plain device-to-device copy for the streaming rate."""
     lib = load_probes()
     stream = torch.cuda.current_stream(dev).cuda_stream
     buf = torch.empty(table_bytes // 128 * 128, dtype=torch.uint8, device=dev).fill_(255)
@@ -212,6 +213,21 @@ def measure_ceilings(torch, ash, dev, table_bytes, n):
                 timer(call)
         ms = timer.mean_ms()
         out[name] = {"Glines_per_s": round(n / ms / 1e6, 2), "ms": round(ms, 4)}
+    # float adds without a result: one lane per line against sixteen lanes per
+    # 64-byte half-line -- the memory side charges per request, not per float
+    for mode, name, lanes in ((3, "float_adds_one_lane_per_line", 1),
+                              (4, "float_adds_16_lanes_per_half_line", 16)):
+        timer = EventTimer(torch)
+        for it in range(6):
+            call = lambda: lib.bench_probe_random_lines(
+                mode, buf.data_ptr(), buf.numel(), n, sink.data_ptr(), 7919 * it, stream)
+            if it == 0:
+                assert call() == 0, lib.bench_probe_last_error().decode()
+            else:
+                timer(call)
+        ms = timer.mean_ms()
+        out[name] = {"Grequests_per_s": round(n / lanes / ms / 1e6, 2),
+                     "Gfloats_per_s": round(n / ms / 1e6, 2), "ms": round(ms, 4)}
     src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
     dst = torch.empty_like(src)
     timer = EventTimer(torch)
@@ -474,10 +490,10 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         "cfg4_forward": roofline_entry(
             "query_forward_kernel<f32,E4>", fwd_bytes(4) * n_live + (29 + 16) * masked, t_f.mean_ms()),
         "cfg4_backward": roofline_entry(
-            "zero16 + query_backward_forward_kernel<f32,E4>",
+            "zero16 + query_backward_forward_vec_kernel (E=4)",
             bwd_bytes(4) * n_live + (29 + 12) * masked + dense, t_b.mean_ms()),
         "cfg4_double_backward": roofline_entry(
-            "zero16 + query_backward_backward_kernel<f32,E4>",
+            "zero16 + query_backward_backward_vec_kernel (E=4)",
             bwd2_bytes(4) * n_live + (29 + 16) * masked + dense, t_bb.mean_ms()),
     }
     for name, e in entries.items():

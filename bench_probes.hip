@@ -96,6 +96,24 @@ __global__ __launch_bounds__(kBlock) void probe_line_updates(
     if (t < n) sink[t] = static_cast<uint32_t>(old);
 }
 
+// Float adds without a result, the accumulation of a gradient: every group of
+// GROUP neighbouring lanes adds to GROUP consecutive floats of one
+// pseudo-random aligned piece of a 64-byte line (GROUP = 1: a lone float,
+// GROUP = 16: a whole line).  Shows what the memory side charges for: the
+// float, or the request one instruction sends to one line.
+template <int GROUP>
+__global__ __launch_bounds__(kBlock) void probe_float_adds(
+        float* __restrict__ buf, uint32_t nlines, uint64_t seed) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const uint64_t h = mix64(static_cast<uint64_t>(t / GROUP) + seed);
+    const uint32_t line = __umulhi(static_cast<uint32_t>(h >> 32), nlines);
+    const uint32_t piece = (static_cast<uint32_t>(h) % (16u / GROUP)) * GROUP;
+    // half-lines of 64 bytes: line numbers count 128-byte lines
+    float* p = buf + static_cast<size_t>(line) * 32 + (static_cast<uint32_t>(h >> 8) & 1u) * 16 +
+               piece + static_cast<uint32_t>(t % GROUP);
+    __hip_atomic_fetch_add(p, 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 }  // namespace
 
 extern "C" const char* bench_probe_last_error(void) { return g_error.c_str(); }
@@ -108,7 +126,11 @@ extern "C" const char* bench_probe_last_error(void) { return g_error.c_str(); }
 //   mode 1: per line one 64-bit read, one 64-bit compare-and-swap and one
 //           32-bit store (the accesses of an insert); modifies `buf`;
 //   mode 2: `n` pseudo-random aligned 64-byte halves of lines, each read by 4
-//           lanes x 16 bytes (what a table of 64-byte buckets would fetch).
+//           lanes x 16 bytes (what a table of 64-byte buckets would fetch);
+//   mode 3: `n` float adds (no result), every lane to a float of a line of
+//           its own; modifies `buf`, `sink` is not written;
+//   mode 4: `n` float adds, 16 neighbouring lanes to the 16 floats of one
+//           64-byte half-line (n / 16 half-lines).
 extern "C" int bench_probe_random_lines(int mode, void* buf, int64_t buf_bytes,
                                      int64_t n, uint32_t* sink, uint64_t seed,
                                      void* stream) {
@@ -134,6 +156,10 @@ extern "C" int bench_probe_random_lines(int mode, void* buf, int64_t buf_bytes,
     } else if (mode == 2) {
         probe_half_line_reads<<<g, kBlock, 0, s>>>(static_cast<const uint4*>(buf),
                                                    nlines, n, sink, seed);
+    } else if (mode == 3) {
+        probe_float_adds<1><<<g, kBlock, 0, s>>>(static_cast<float*>(buf), nlines, seed);
+    } else if (mode == 4) {
+        probe_float_adds<16><<<g, kBlock, 0, s>>>(static_cast<float*>(buf), nlines, seed);
     } else {
         PROBE_FAIL("unknown probe mode");
     }
