@@ -297,8 +297,13 @@ def bench_hash(torch, ash, workloads, args, dev):
     workspace = torch.empty(max(ws_bytes.value, 256), dtype=torch.uint8, device=dev)
     t_bulk, t_bulk_keys = EventTimer(torch), EventTimer(torch)
 
-    t_clear, t_insert, t_insert_keys, t_find, t_items, t_erase = (
-        EventTimer(torch) for _ in range(6))
+    t_clear, t_insert, t_insert_keys, t_find, t_items, t_erase, t_erase_bulk = (
+        EventTimer(torch) for _ in range(7))
+    erase_bytes, erase_worthwhile = ctypes.c_int64(0), ctypes.c_int(0)
+    check(lib.ash_map_erase_bulk_query(
+        handle, n, ctypes.byref(erase_bytes), ctypes.byref(erase_worthwhile)))
+    erase_ws = (torch.empty(erase_bytes.value, dtype=torch.uint8, device=dev)
+                if erase_bytes.value > 0 else None)
 
     def settle():
         check(lib.ash_map_find(handle, queries.data_ptr(), 1, idx_out.data_ptr(),
@@ -330,6 +335,11 @@ def bench_hash(torch, ash, workloads, args, dev):
         run(t_items, lambda: check(lib.ash_map_items(
             handle, items_keys.data_ptr(), items_idx.data_ptr(), n, stream)))
         run(t_erase, lambda: check(lib.ash_map_erase(handle, keys.data_ptr(), n, stream)))
+        if erase_ws is not None:
+            # the same erase through the streaming path, on a map filled again
+            check(lib.ash_map_insert_keys(handle, keys.data_ptr(), n, stream))
+            run(t_erase_bulk, lambda: check(lib.ash_map_erase_bulk(
+                handle, keys.data_ptr(), n, erase_ws.data_ptr(), erase_ws.numel(), stream)))
     assert int(mask_out.sum()) == hits
     assert backend.status()["size"] == 0   # a fresh read: the launches above went past the shim
     c_count = (ctypes.c_int64 * k)(args.capacity, args.capacity)
@@ -371,10 +381,18 @@ def bench_hash(torch, ash, workloads, args, dev):
             kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
             kernels[name]["workspace_bytes"] = ws_bytes.value
     kernels["api_insert_path"] = "insert_values_bulk" if api_uses_bulk else "insert_values"
+    if erase_ws is not None:
+        kernels["erase_bulk"] = roofline_entry(
+            "split_keys_kernel<3> + split_records_kernel + erase_range_kernel "
+            "(ash_map_erase_bulk, every key stored)", INSERT_KEY_BYTES * n, t_erase_bulk.mean_ms())
+        kernels["erase_bulk"]["Mkeys_per_s"] = round(n / kernels["erase_bulk"]["ms"] / 1e3, 1)
+    kernels["api_erase_path"] = (
+        "erase_bulk" if erase_ws is not None and erase_worthwhile.value
+        and ash.common.BULK_ERASE != "never" else "erase")
     for name in ("insert_values", "insert_keys", "find", "erase"):
         kernels[name]["Mkeys_per_s"] = round(n / kernels[name]["ms"] / 1e3, 1)
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
-    del hm, w, workspace
+    del hm, w, workspace, erase_ws
     torch.cuda.empty_cache()
     return ms_per_step, hits, kernels
 

@@ -278,6 +278,21 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
  * batch erase once. */
 int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n, void* stream);
 
+/* Streaming variant of ash_map_erase for batches of the order of the table
+ * (same reference function, ash/src/hashmap_gpu.cuh:316-351, same resulting
+ * map): the batch is split by bucket range as for ash_map_insert_bulk, and each
+ * range of 512 buckets is taken into LDS by one workgroup, which frees the
+ * slots of its keys there and writes the range back; the heap counter moves
+ * once per workgroup instead of one global compare-and-swap per key.
+ *   ash_map_erase_bulk_query: *bytes = size of the device workspace for `n`
+ *   keys (0 when the path does not apply, as for ash_map_bulk_workspace_bytes
+ *   without value rows); *worthwhile (optional) = 1 when n is large enough
+ *   relative to the table for this path to be the faster one.
+ *   ash_map_erase_bulk: workspace as for ash_map_insert_bulk. */
+int ash_map_erase_bulk_query(ash_map_t* map, int64_t n, int64_t* bytes, int* worthwhile);
+int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+
 /* Replaces `HashMap::clear` (ash/src/hashmap_gpu.cuh:354-358,
  * ash/src/hashmap_impl.h:26-33).  Counters, heap and the second region are
  * reset on `stream` at once (the heap array is rewritten to 0..capacity-1 only

@@ -145,6 +145,10 @@ _SIGNATURES = {
         ],
     ),
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
+    "ash_map_erase_bulk_query": (
+        ctypes.c_int, [_PTR, _I64, ctypes.POINTER(_I64), ctypes.POINTER(ctypes.c_int)]
+    ),
+    "ash_map_erase_bulk": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR, _I64, _PTR]),
     "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
     "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_status_staged": (ctypes.c_int, [_PTR, _PTR, ctypes.POINTER(_I64), _PTR]),
@@ -234,11 +238,12 @@ ACTIVATE_STATIC_MAX = 1 << 20
 # Deferred activations between two looks at the table's counters.
 DEFERRED_UPKEEP_EVERY = 64
 
-# Which inserts take the streaming (partition + build in LDS) path of the
-# library instead of the per-key kernel: "auto" = when the library says the
-# batch is large enough relative to the table, "always" = whenever the path
-# applies, "never".
+# Which inserts (and erases) take the streaming path of the library (batch split
+# by bucket range, ranges handled in LDS) instead of the per-key kernel:
+# "auto" = when the library says the batch is large enough relative to the
+# table, "always" = whenever the path applies, "never".
 BULK_INSERT = os.environ.get("ASH_BULK_INSERT", "auto")
+BULK_ERASE = os.environ.get("ASH_BULK_ERASE", "auto")
 _DTYPE = {torch.float32: 0, torch.float64: 1}
 
 
@@ -1325,12 +1330,30 @@ class _HashMap:
         self._maybe_tombstones = True
         self._status_after_insert = None
         self.version = next(_VERSIONS)
-        with torch.cuda.device(self._device):
+        n = keys.shape[0]
+        workspace = None
+        if BULK_ERASE != "never":
+            nbytes, worthwhile = _I64(0), ctypes.c_int(0)
             self._check(
-                self._lib.ash_map_erase(
-                    self._handle, keys.data_ptr(), keys.shape[0], self._stream()
+                self._lib.ash_map_erase_bulk_query(
+                    self._handle, n, ctypes.byref(nbytes), ctypes.byref(worthwhile)
                 )
             )
+            if nbytes.value and (worthwhile.value or BULK_ERASE == "always"):
+                workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=self._device)
+        self.last_erase_path = "per-key" if workspace is None else "streaming"
+        with torch.cuda.device(self._device):
+            if workspace is not None:
+                self._check(
+                    self._lib.ash_map_erase_bulk(
+                        self._handle, keys.data_ptr(), n, workspace.data_ptr(),
+                        workspace.numel(), self._stream(),
+                    )
+                )
+            else:
+                self._check(
+                    self._lib.ash_map_erase(self._handle, keys.data_ptr(), n, self._stream())
+                )
 
     def clear(self) -> None:
         with torch.cuda.device(self._device):

@@ -1001,17 +1001,23 @@ __global__ __launch_bounds__(kBlock) void ray_compact_kernel(
 // one update of each counter per workgroup 0.85 ms.
 constexpr int kEraseBlock = 1024;
 
-template <int DIM>
-__global__ __launch_bounds__(kEraseBlock) void erase_kernel(
-        MapDev m, const int32_t* __restrict__ keys, int64_t n) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kEraseBlock + threadIdx.x;
+// One key per thread, every thread of the workgroup calls this together.
+// CODES: `keys` holds packed 64-bit codes instead of int32[DIM] rows.
+template <int DIM, bool CODES>
+__device__ __forceinline__ void erase_one(const MapDev& m, const int32_t* __restrict__ keys,
+                                          int64_t i, bool active) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const bool active = i < n;
-    int32_t k[DIM];
-    load_key<DIM>(keys, i, active, k);
+    int32_t k[DIM] = {};
     uint64_t code;
-    const bool fits = pack_key<DIM>(k, code);
+    bool fits;
+    if constexpr (CODES) {
+        code = active ? reinterpret_cast<const uint64_t*>(keys)[i] : 0ull;
+        fits = true;
+    } else {
+        load_key<DIM>(keys, i, active, k);
+        fits = pack_key<DIM>(k, code);
+    }
     bool pend = active && fits;
     uint32_t b = bucket_of(code, m.nb);
     uint32_t steps = 0;
@@ -1083,6 +1089,29 @@ __global__ __launch_bounds__(kEraseBlock) void erase_kernel(
         const int pos = s_base - 1 - below;
         if (pos >= 0 && pos < m.capacity) m.heap[pos] = idx;
         m.klog[idx] = kEmpty;
+    }
+}
+
+template <int DIM>
+__global__ __launch_bounds__(kEraseBlock) void erase_kernel(
+        MapDev m, const int32_t* __restrict__ keys, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kEraseBlock + threadIdx.x;
+    erase_one<DIM, false>(m, keys, i, i < n);
+}
+
+// The same erase over a selection made on the device (see
+// insert_selected_kernel): thread t handles key sel[t], t < *nsel.
+template <int DIM, bool CODES>
+__global__ __launch_bounds__(kEraseBlock) void erase_selected_kernel(
+        MapDev m, const int32_t* __restrict__ keys, const int32_t* __restrict__ sel,
+        const int32_t* __restrict__ nsel) {
+    const int64_t total = *nsel;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * kEraseBlock; base < total;
+         base += static_cast<int64_t>(gridDim.x) * kEraseBlock) {
+        const int64_t t = base + threadIdx.x;
+        const bool active = t < total;
+        erase_one<DIM, CODES>(m, keys, active ? sel[t] : 0, active);
+        __syncthreads();   // the counters in LDS are free again
     }
 }
 
@@ -1592,6 +1621,32 @@ int check_batch(const ash_map* map, const void* keys, int64_t n) {
     if (n < 0) ASH_FAIL("negative key count");
     if (n > 0 && keys == nullptr) ASH_FAIL("null keys pointer");
     if (n > (int64_t{1} << 31) - kHeapBlock) ASH_FAIL("too many keys in one call");
+    return 0;
+}
+
+int erase_selected(ash_map* map, bool codes, const void* keys, const int32_t* sel,
+                   const int32_t* nsel, hipStream_t s) {
+    const int32_t* k = static_cast<const int32_t*>(keys);
+    constexpr unsigned g = 64;   // the selection is empty or short as a rule
+    if (codes) {
+        erase_selected_kernel<1, true><<<g, kEraseBlock, 0, s>>>(map->d, k, sel, nsel);
+    } else {
+        switch (map->key_dim) {
+            case 1:
+                erase_selected_kernel<1, false><<<g, kEraseBlock, 0, s>>>(map->d, k, sel, nsel);
+                break;
+            case 2:
+                erase_selected_kernel<2, false><<<g, kEraseBlock, 0, s>>>(map->d, k, sel, nsel);
+                break;
+            case 3:
+                erase_selected_kernel<3, false><<<g, kEraseBlock, 0, s>>>(map->d, k, sel, nsel);
+                break;
+            default:
+                erase_selected_kernel<4, false><<<g, kEraseBlock, 0, s>>>(map->d, k, sel, nsel);
+                break;
+        }
+    }
+    ASH_LAUNCH_CHECK();
     return 0;
 }
 

@@ -143,6 +143,11 @@ int insert_selected(ash_map* map, bool codes, const void* keys,
                     const int32_t* sel, const int32_t* nsel,
                     const ValueArgs& va, hipStream_t s);
 
+// Erases the selected keys with the per-key kernel; arguments as for
+// insert_selected.
+int erase_selected(ash_map* map, bool codes, const void* keys, const int32_t* sel,
+                   const int32_t* nsel, hipStream_t s);
+
 int check_batch(const ash_map* map, const void* keys, int64_t n);
 // Fills the bucket array if a clear() left that to the next user of the table.
 int settle_table(ash_map* map, hipStream_t s);
