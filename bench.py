@@ -92,6 +92,9 @@ MEASURED_COUNTERS = {
     "insert_keys": (2_304_000_000 + 1_691_000_000, 0.243, 16_465_000),
     "find": (2_230_000_000 + 146_000_000, 0.064, 0),
     "erase": (2_234_000_000 + 1_217_000_000, 0.447, 16_031_000),
+    # the two keys-only split passes and the range pass
+    "erase_bulk": (192_000_000 + 128_000_000 + 641_000_000
+                   + 139_000_000 + 134_000_000 + 1_092_000_000, 0.21, 66_000),
     "items": (128_000_000 + 320_000_000, 0.417, 1_954),
     "items_values": (528_000_000 + 256_000_000, 0.247, 0),
     # sums over the split, build and row-copy kernels
