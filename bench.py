@@ -96,7 +96,7 @@ MEASURED_COUNTERS = {
     "erase_bulk": (192_000_000 + 128_000_000 + 641_000_000
                    + 139_000_000 + 134_000_000 + 1_092_000_000, 0.21, 66_000),
     "items": (128_000_000 + 320_000_000, 0.417, 1_954),
-    "items_values": (528_000_000 + 256_000_000, 0.247, 0),
+    "items_values_by_index": (528_000_000 + 256_000_000, 0.247, 0),
     # sums over the split, build and row-copy kernels
     "insert_values_bulk": (834_000_000 + 1_330_000_000, 0.390, 47_000),
     "insert_keys_bulk": (449_000_000 + 914_000_000, 0.411, 59_000),
@@ -356,16 +356,30 @@ def bench_hash(torch, ash, workloads, args, dev):
             t_gather(fn)
         else:
             fn()
+    # what HashMap.items(return_values=True) does while the listing is in index
+    # order (nothing erased or loaded since the clear): the first n rows, copied
+    t_rows = EventTimer(torch)
+    for it in range(args.warmup + args.steps):
+        fn = lambda: [v[:n].clone() for v in (hm.color, hm.depth)]
+        if it >= args.warmup:
+            t_rows(fn)
+        else:
+            fn()
     kernels = {
         "insert_values": roofline_entry(
             "insert_kernel<3,fused>", (INSERT_KEY_BYTES + VALUE_ROW_BYTES) * n, t_insert.mean_ms()),
         "insert_keys": roofline_entry("insert_kernel<3,keys>", INSERT_KEY_BYTES * n, t_insert_keys.mean_ms()),
         "find": roofline_entry("find_kernel<3>", FIND_BYTES * n, t_find.mean_ms()),
         # the heap is in its initial order when items() runs here: n indices scanned
-        "items": roofline_entry("items_kernel<3>", items_bytes(n, n), t_items.mean_ms()),
-        # value rows of the enumerated entries: index in, 16 B read and written
-        "items_values": roofline_entry("gather_rows_kernel (color + depth by items() index)",
-                                       (8 + VALUE_ROW_BYTES) * n, t_gather.mean_ms()),
+        "items": roofline_entry("items_dense_kernel<3>", items_bytes(n, n), t_items.mean_ms()),
+        # value rows of the enumerated entries while the listing is in index
+        # order: 16 B read and written per entry (two device copies)
+        "items_values": roofline_entry("copy of the first n rows of color and depth",
+                                       VALUE_ROW_BYTES * n, t_rows.mean_ms()),
+        # ... and by index (after an erase or a load): index in, 16 B read and written
+        "items_values_by_index": roofline_entry(
+            "gather_rows_kernel (color + depth by items() index)",
+            (8 + VALUE_ROW_BYTES) * n, t_gather.mean_ms()),
         # the heap array is rewritten only after an erase or a load wrote to it;
         # none did before the clear timed here
         "clear": roofline_entry("reset counters + deferred fill16 (+ a one-key find)",

@@ -332,6 +332,17 @@ int ash_map_size(ash_map_t* map, int64_t* size, void* stream);
 int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
                   int64_t n_expected, void* stream);
 
+/* Whether the next ash_map_items lists entry i under index i (*dense = 1):
+ * while nothing has been erased or loaded since the map was created or
+ * cleared and no key lives in the second region, the indices in use are
+ * 0 .. size-1 (a new key takes heap[counter++], ash/src/hashmap_gpu.cuh:226-231,
+ * from a heap in its initial order, ash/src/hashmap_impl.h:26-33), and the
+ * listing follows them.  A binding can then take the value rows of the listed
+ * entries as the first `size` rows of every value tensor instead of gathering
+ * them by index (`values[name][indices]`, ash/hashmap.py:138-146).  Host-side
+ * state only, no synchronisation.  No counterpart in the reference. */
+int ash_map_items_in_index_order(ash_map_t* map, int* dense);
+
 /* Replaces `HashMap::load_states` (ash/src/hashmap_gpu.cuh:407-450): the map
  * is emptied, then (keys[i] -> indices[i]) are stored, size := n and the heap
  * := heap_src (skipped when heap_src is NULL or already the map's heap). */

@@ -147,6 +147,57 @@ def test_gather_rows_equals_torch_indexing(gpu_ash):
     assert torch.equal(order[0], sort_rows(keys)[0])
 
 
+def test_listing_in_index_order_while_nothing_was_erased(gpu_ash):
+    """While nothing has been erased or loaded since the clear (and no key
+    lives in the second region) entry i of items() is index i and the value
+    rows of the listing are the first rows of the value tensors, copied; after
+    an erase, with a key that does not pack, or after a load the listing goes
+    by the key log and the rows are gathered.  Either way:
+    values[name][indices] (ash/hashmap.py:138-146)."""
+    g = torch.Generator().manual_seed(77)
+    hm = gpu_ash.HashMap(3, {"color": 3, "depth": 1}, 60_000, DEV)
+    backend = hm.engine.backend
+    keys = torch.unique(torch.randint(-40, 40, (50_000, 3), generator=g, dtype=torch.int32), dim=0)
+    keys = keys[torch.randperm(len(keys), generator=g)].to(DEV)
+    first, second = keys[:20_000], keys[20_000:45_000]
+
+    def check(expect_dense, stored):
+        k, i, v = hm.items(return_indices=True, return_values=True)
+        assert backend.last_items_in_index_order == expect_dense
+        if expect_dense:
+            assert torch.equal(i, torch.arange(len(i), device=DEV))
+        assert torch.equal(v["color"], hm.color[i]) and torch.equal(v["depth"], hm.depth[i])
+        assert v["color"].data_ptr() != hm.color.data_ptr()   # a copy, not a view
+        assert torch.equal(sort_rows(k)[0], sort_rows(stored)[0])
+        masks, idx = hm.find(k)
+        assert bool(masks.all()) and torch.equal(idx, i)
+        # a second listing may come in another order; every row belongs to its key
+        k2, v2 = hm.items(return_indices=False, return_values=True)
+        assert torch.equal(v2["color"], k2.float()) and torch.equal(v2["depth"], k2[:, :1].float() * 0.5)
+
+    def rows(k):
+        return {"color": k.float(), "depth": k[:, :1].float() * 0.5}
+
+    hm.insert(first, rows(first))
+    check(True, first)
+    hm.insert(torch.cat([second, first[:500]]), rows(torch.cat([second, first[:500]])))
+    check(True, torch.cat([first, second]))
+    hm.erase(first[:3_000])
+    check(False, torch.cat([first[3_000:], second]))
+    hm.clear()
+    hm.insert(second, rows(second))
+    check(True, second)
+    odd = torch.tensor([[2**30, -(2**30), 5]], dtype=torch.int32, device=DEV)
+    hm.insert(odd, rows(odd))
+    check(False, torch.cat([second, odd]))
+    state = hm.state_dict()
+    other = gpu_ash.HashMap(3, {"color": 3, "depth": 1}, 60_000, DEV)
+    other.load_state_dict(state)
+    k, i, v = other.items(return_indices=True, return_values=True)
+    assert not other.engine.backend.last_items_in_index_order
+    assert torch.equal(v["color"], other.color[i])
+
+
 def test_state_with_duplicate_keys_is_refused(gpu_ash):
     """A saved state whose active keys repeat a key (the reference prints
     "should never reach here", ash/src/hashmap_gpu.cuh:420-422, and goes on

@@ -144,6 +144,7 @@ _SIGNATURES = {
             _PTR,
         ],
     ),
+    "ash_map_items_in_index_order": (ctypes.c_int, [_PTR, ctypes.POINTER(ctypes.c_int)]),
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_erase_bulk_query": (
         ctypes.c_int, [_PTR, _I64, ctypes.POINTER(_I64), ctypes.POINTER(ctypes.c_int)]
@@ -1366,6 +1367,11 @@ class _HashMap:
         n = self.size()
         keys = torch.empty((n, self.key_dim), dtype=torch.int32, device=self._device)
         indices = torch.empty(n, dtype=torch.int64, device=self._device)
+        # whether entry i is listed under index i: the value rows of the listing
+        # are then the first n rows of every value tensor (HashMap.items)
+        dense = ctypes.c_int(0)
+        self._check(self._lib.ash_map_items_in_index_order(self._handle, ctypes.byref(dense)))
+        self.last_items_in_index_order = bool(dense.value)
         if n > 0:
             with torch.cuda.device(self._device):
                 self._check(

@@ -161,6 +161,13 @@ class HashMap(ASHModule):
     def items(self, return_indices: bool = True, return_values: bool = False) -> Tuple:
         """(keys[, indices][, values]) of the stored entries."""
         keys, indices = self.engine.items()
+        if return_values and getattr(self.engine.backend, "last_items_in_index_order", False):
+            # entry i sits under index i: values[name][indices] (ash/hashmap.py:138-146)
+            # is a copy of the first rows
+            assert return_indices or return_values
+            n = indices.shape[0]
+            rows = self._layout.declared({name: v[:n].clone() for name, v in self.values.items()})
+            return (keys, indices, rows) if return_indices else (keys, rows)
         return self._answer(keys, indices, return_indices, return_values)
 
     def keys(self) -> torch.Tensor:

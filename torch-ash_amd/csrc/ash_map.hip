@@ -1130,6 +1130,23 @@ constexpr int kItemsBlock = 1024;
 constexpr int kItemsRounds = 8;
 constexpr int kItemsSpan = kItemsBlock * kItemsRounds;   // indices per workgroup
 
+// items() while the heap is in its initial order and no key lives in the
+// second region: the indices in use are 0 .. n-1, every one of them, so entry
+// i of the output is index i and its key comes from log entry i -- no ranks,
+// no cursor, and the value rows of the listed entries are the first n rows of
+// every value tensor.
+template <int DIM>
+__global__ __launch_bounds__(kBlock) void items_dense_kernel(
+        MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= n) return;
+    int32_t k[DIM];
+    unpack_key<DIM>(m.klog[i], k);
+#pragma unroll
+    for (int d = 0; d < DIM; ++d) keys_out[i * DIM + d] = k[d];
+    idx_out[i] = i;
+}
+
 template <int DIM>
 __global__ __launch_bounds__(kItemsBlock) void items_kernel(
         MapDev m, int32_t* __restrict__ keys_out, int64_t* __restrict__ idx_out,
@@ -2266,10 +2283,30 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
+    const int identity = map->heap_dirty ? 0 : 1;
+    if (identity && !map->general_attached) {
+        const int64_t n = n_expected < map->capacity ? n_expected : map->capacity;
+        const unsigned gd = grid_for(n);
+        switch (map->key_dim) {
+            case 1:
+                items_dense_kernel<1><<<gd, kBlock, 0, s>>>(map->d, keys_out, indices_out, n);
+                break;
+            case 2:
+                items_dense_kernel<2><<<gd, kBlock, 0, s>>>(map->d, keys_out, indices_out, n);
+                break;
+            case 3:
+                items_dense_kernel<3><<<gd, kBlock, 0, s>>>(map->d, keys_out, indices_out, n);
+                break;
+            default:
+                items_dense_kernel<4><<<gd, kBlock, 0, s>>>(map->d, keys_out, indices_out, n);
+                break;
+        }
+        ASH_LAUNCH_CHECK();
+        return 0;
+    }
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrCursor, 0);
     ASH_LAUNCH_CHECK();
     const unsigned g = grid_for(map->capacity, kItemsSpan);
-    const int identity = map->heap_dirty ? 0 : 1;
     switch (map->key_dim) {
         case 1:
             items_kernel<1><<<g, kItemsBlock, 0, s>>>(map->d, keys_out, indices_out,
@@ -2352,6 +2389,13 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
     ValueArgs va = {};
     return launch_insert<kInsertLoad>(map, keys_scratch, n, va, nullptr,
                                       indices_scratch, s);
+}
+
+int ash_map_items_in_index_order(ash_map_t* map, int* dense) {
+    if (check_map(map)) return 1;
+    if (dense == nullptr) ASH_FAIL("null output pointer");
+    *dense = (!map->heap_dirty && !map->general_attached) ? 1 : 0;
+    return 0;
 }
 
 int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
