@@ -273,6 +273,24 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
                         const int64_t* row_bytes, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* ash_map_insert_bulk for a caller that reads the table's counters after every
+ * insert and does not want to wait for the whole insert to do so.  The only
+ * counter that decides what the caller does next -- keys that need the second
+ * region, out[3] of ash_map_status -- can only be non-zero when the first
+ * split pass handed keys over to the per-key kernel (unpackable keys are among
+ * them).  Their number is written to `handed_over` (one int32 of page-locked
+ * host memory that the device can write to) right after that pass and
+ * `handed_over_event` (a hipEvent_t of the caller's, may be NULL) is recorded
+ * behind it, about a quarter into the call's work: zero means that no key of
+ * this batch is waiting for the second region, and the other counters can be
+ * fetched without blocking (ash_map_status_begin).  No counterpart in the
+ * reference. */
+int ash_map_insert_bulk_early(ash_map_t* map, const int32_t* keys, int64_t n,
+                              int n_values, const void* const* src, void* const* dst,
+                              const int64_t* row_bytes, void* workspace,
+                              int64_t workspace_bytes, int32_t* handed_over,
+                              void* handed_over_event, void* stream);
+
 /* Replaces `HashMap::erase` (ash/src/hashmap_gpu.cuh:316-351): found keys are
  * removed and their indices pushed back on the heap; duplicates inside the
  * batch erase once. */
@@ -321,6 +339,15 @@ int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
  * insert.  out[5] is the number of rows the latest ash_grid_collect_touched
  * listed.  No counterpart in the reference. */
 int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[6], void* stream);
+
+/* ash_map_status_staged in two halves: ash_map_status_begin queues the copy of
+ * the counters into `staging` (eight int32 of page-locked host memory) on
+ * `stream` and records `event` (a hipEvent_t of the caller's, may be NULL)
+ * behind it, without waiting; once the event or the stream has completed,
+ * ash_map_status_decode turns the staging area into the six values of
+ * ash_map_status_staged.  No counterpart in the reference. */
+int ash_map_status_begin(ash_map_t* map, int32_t* staging, void* event, void* stream);
+int ash_map_status_decode(const int32_t* staging, int64_t out[6]);
 
 /* Replaces `HashMap::size` (ash/src/hashmap_gpu.cuh:157); synchronises. */
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream);

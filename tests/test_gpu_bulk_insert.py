@@ -394,3 +394,52 @@ def test_streaming_insert_refuses_a_pending_fill_under_capture(gpu_ash):
     assert rc == 0, lib.ash_last_error().decode()
     assert backend.status()["size"] == len(keys)
     assert bool(engine.find(keys)[1].all())
+
+
+def test_streaming_insert_returns_before_its_counters_are_read(bulk_ash, oracle):
+    """A streaming insert whose first pass hands no key to the per-key kernel
+    returns without waiting for the table's counters; they are looked at when
+    somebody asks (size, items, the next insert) and dropped when an erase or a
+    clear makes them stale.  A batch with an unpackable key takes the waiting
+    path (the key has to be re-issued into the second region before anything
+    else looks at the map).  Two maps at once: each has its own landing place."""
+    dim, capacity = 3, 120_000
+    rng = np.random.default_rng(990)
+    a, b = bulk_ash.ASHEngine(dim, capacity, DEV), bulk_ash.ASHEngine(dim, capacity, DEV)
+    oa, ob = _oracle_map(oracle, dim, capacity), _oracle_map(oracle, dim, capacity)
+    ka, kb = _random_keys(rng, 90_000, dim, 30), _random_keys(rng, 70_000, dim, 28)
+    a.insert_keys(ka.to(DEV))
+    b.insert_keys(kb.to(DEV))
+    assert a.backend._status_pending and b.backend._status_pending
+    # look-ups do not need the counters
+    _, mask = a.find(ka[:1000].to(DEV))
+    assert bool(mask.all()) and a.backend._status_pending
+    oa.insert_keys(ka)
+    ob.insert_keys(kb)
+    assert b.size() == ob.size() and not b.backend._status_pending
+    assert a.size() == oa.size() and not a.backend._status_pending
+    # an erase makes queued counters stale
+    a.insert_keys(_random_keys(rng, 10_000, dim, 31).to(DEV))
+    assert a.backend._status_pending
+    gone = ka[:5_000]
+    a.erase(gone.to(DEV))
+    assert not a.backend._status_pending
+    oa2 = _oracle_map(oracle, dim, capacity)
+    k_now, _ = a.items()
+    oa2.insert_keys(k_now.cpu())
+    assert a.size() == oa2.size()
+    _, mask = a.find(gone.to(DEV))
+    left = set(map(tuple, k_now.cpu().tolist()))
+    assert mask.cpu().tolist() == [tuple(k) in left for k in gone.tolist()]
+    # a batch with a key that does not pack waits and re-issues
+    odd = torch.tensor([[2**30, 5, -(2**30)]], dtype=torch.int32)
+    batch = torch.cat([_random_keys(rng, 8_000, dim, 29), odd])
+    b.insert_keys(batch.to(DEV))
+    assert not b.backend._status_pending
+    ob.insert_keys(batch)
+    _assert_same_map(b, ob, torch.cat([batch, kb[:2000]]).to(DEV))
+    # with the second region attached an unpackable key still takes the waiting path
+    b.insert_keys(torch.cat([_random_keys(rng, 6_000, dim, 27), odd + 1]).to(DEV))
+    assert not b.backend._status_pending
+    b.insert_keys(_random_keys(rng, 6_000, dim, 27).to(DEV))
+    assert b.backend._status_pending and b.size() <= capacity

@@ -145,6 +145,12 @@ _SIGNATURES = {
         ],
     ),
     "ash_map_items_in_index_order": (ctypes.c_int, [_PTR, ctypes.POINTER(ctypes.c_int)]),
+    "ash_map_insert_bulk_early": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _PTR, _PTR],
+    ),
+    "ash_map_status_begin": (ctypes.c_int, [_PTR, _PTR, _PTR, _PTR]),
+    "ash_map_status_decode": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64)]),
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_erase_bulk_query": (
         ctypes.c_int, [_PTR, _I64, ctypes.POINTER(_I64), ctypes.POINTER(ctypes.c_int)]
@@ -924,6 +930,16 @@ class _HashMap:
         self._table = torch.empty(table_bytes.value, dtype=torch.uint8, device=self._device)
         self._general = None
         self._maybe_tombstones = False
+        # a read-back of the counters that has been queued behind an insert and
+        # not looked at yet (_finish_streaming_insert): page-locked landing
+        # places and events of this map's own
+        self._status_pending = False
+        self._early = None
+        # a new map is empty and every counter is zero
+        self._status_after_insert = {
+            "size": 0, "dropped": 0, "tombstones": 0,
+            "exotic_pending": 0, "load_duplicates": 0, "touched": 0,
+        }
         # counts the calls that may have changed the stored keys; lets callers
         # keep results derived from the key set (orderings, tables) while it stands
         self.version = next(_VERSIONS)
@@ -968,6 +984,7 @@ class _HashMap:
         """Before an insert: if earlier erases or refused keys may have left
         tombstones, look at the counters and re-place the live entries into a
         cleared table when too few empty slots remain."""
+        self._resolve_status()
         if not self._maybe_tombstones:
             return
         st = self.status()
@@ -987,6 +1004,58 @@ class _HashMap:
                 )
             )
         self._maybe_tombstones = False
+
+    def _deferred(self):
+        """(handed-over count int32[1], counters int32[8], two events), made on
+        first use: page-locked memory the device writes to."""
+        if self._early is None:
+            self._early = torch.zeros(1, dtype=torch.int32, pin_memory=True)
+            self._late = torch.zeros(8, dtype=torch.int32, pin_memory=True)
+            stream = torch.cuda.current_stream(self._device)
+            self._early_event, self._late_event = torch.cuda.Event(), torch.cuda.Event()
+            # an event has a handle once it has been recorded
+            self._early_event.record(stream)
+            self._late_event.record(stream)
+        return self._early, self._late, self._early_event, self._late_event
+
+    def _finish_streaming_insert(self) -> bool:
+        """After ash_map_insert_bulk_early has been queued.  Waits for the first
+        split pass only: when it handed no key to the per-key kernel, no key of
+        the batch can be waiting for the second region, so nothing has to be
+        re-issued and the counters are fetched behind the insert without
+        waiting for them (True).  Otherwise the caller reads them now (False)."""
+        early, late, early_event, late_event = self._deferred()
+        early_event.synchronize()
+        if int(early[0]) != 0:
+            return False
+        self._check(
+            self._lib.ash_map_status_begin(
+                self._handle, late.data_ptr(), late_event.cuda_event, self._stream()
+            )
+        )
+        self._status_pending = True
+        self._status_after_insert = None
+        self.version = next(_VERSIONS)
+        return True
+
+    def _resolve_status(self) -> None:
+        """Looks at a read-back that an insert left queued."""
+        if not self._status_pending:
+            return
+        self._status_pending = False
+        _, late, _, late_event = self._deferred()
+        late_event.synchronize()
+        out = (_I64 * 6)()
+        self._check(self._lib.ash_map_status_decode(late.data_ptr(), out))
+        st = {
+            "size": out[0], "dropped": out[1], "tombstones": out[2],
+            "exotic_pending": out[3], "load_duplicates": out[4], "touched": out[5],
+        }
+        if st["exotic_pending"] != 0:
+            raise RuntimeError("internal error: unpackable keys pending after a streaming insert")
+        self._status_after_insert = st
+        if st["dropped"] > 0 or st["tombstones"] > 0:
+            self._maybe_tombstones = True
 
     def _attach_general_if_needed(self) -> bool:
         """After an insert/load: keys that need the second region are counted by
@@ -1014,6 +1083,7 @@ class _HashMap:
         return self._device
 
     def status(self) -> Dict[str, int]:
+        self._status_pending = False   # this read is newer
         out = (_I64 * 6)()
         staging = _status_staging()
         with torch.cuda.device(self._device):
@@ -1034,12 +1104,21 @@ class _HashMap:
     def status_after_insert(self) -> Dict[str, int]:
         """The counters as read back at the end of the latest insert (every
         insert reads them once); saves the caller a second read-back."""
+        self._resolve_status()
         st = getattr(self, "_status_after_insert", None)
         return st if st is not None else self.status()
+
+    def known_size(self) -> Optional[int]:
+        """The size if it is known on the host (from the latest read-back, or
+        zero after a clear), else None; never asks the device for it."""
+        self._resolve_status()
+        st = getattr(self, "_status_after_insert", None)
+        return None if st is None else st["size"]
 
     def size(self) -> int:
         # every insert / load / activation ends with one read-back of the
         # counters; until the next erase or clear that read-back still holds
+        self._resolve_status()
         st = getattr(self, "_status_after_insert", None)
         if st is not None:
             return st["size"]
@@ -1212,6 +1291,7 @@ class _HashMap:
                 )
             )
         self._status_after_insert = None
+        self._status_pending = False
         self.version = next(_VERSIONS)
         # Keys refused for lack of capacity leave tombstones behind and are
         # only visible in the counters: every DEFERRED_UPKEEP_EVERY-th call the
@@ -1246,12 +1326,16 @@ class _HashMap:
         for _ in range(2):
             with torch.cuda.device(self._device):
                 if workspace is not None:
+                    early, _, early_event, _ = self._deferred()
                     self._check(
-                        self._lib.ash_map_insert_bulk(
+                        self._lib.ash_map_insert_bulk_early(
                             self._handle, keys.data_ptr(), n, 0, None, None, None,
-                            workspace.data_ptr(), workspace.numel(), self._stream(),
+                            workspace.data_ptr(), workspace.numel(), early.data_ptr(),
+                            early_event.cuda_event, self._stream(),
                         )
                     )
+                    if self._finish_streaming_insert():
+                        return
                 else:
                     self._check(
                         self._lib.ash_map_insert_keys(
@@ -1303,12 +1387,16 @@ class _HashMap:
         for _ in range(2):
             with torch.cuda.device(self._device):
                 if workspace is not None:
+                    early, _, early_event, _ = self._deferred()
                     self._check(
-                        self._lib.ash_map_insert_bulk(
+                        self._lib.ash_map_insert_bulk_early(
                             self._handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows,
-                            workspace.data_ptr(), workspace.numel(), self._stream(),
+                            workspace.data_ptr(), workspace.numel(), early.data_ptr(),
+                            early_event.cuda_event, self._stream(),
                         )
                     )
+                    if self._finish_streaming_insert():
+                        return
                 else:
                     self._check(
                         self._lib.ash_map_insert(
@@ -1330,6 +1418,7 @@ class _HashMap:
         keys = self._keys(keys)
         self._maybe_tombstones = True
         self._status_after_insert = None
+        self._status_pending = False
         self.version = next(_VERSIONS)
         n = keys.shape[0]
         workspace = None
@@ -1360,7 +1449,12 @@ class _HashMap:
         with torch.cuda.device(self._device):
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
         self._maybe_tombstones = False
-        self._status_after_insert = None
+        # clear zeroes every counter, so they are known without a read-back
+        self._status_after_insert = {
+            "size": 0, "dropped": 0, "tombstones": 0,
+            "exotic_pending": 0, "load_duplicates": 0, "touched": 0,
+        }
+        self._status_pending = False
         self.version = next(_VERSIONS)
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -135,8 +135,10 @@ class ASHEngine(nn.Module):
             warnings.warn("empty keys")
             return
         dropped_before = self._dropped()
+        room = self._room_known()
         self.backend.insert_keys(self._prepare(keys))
-        self._warn_if_overfull(keys.shape[0], dropped_before)
+        if not self._surely_stored(keys.shape[0], room):
+            self._warn_if_overfull(keys.shape[0], dropped_before)
 
     def insert(
         self,
@@ -154,8 +156,28 @@ class ASHEngine(nn.Module):
         for rows in values.values():
             assert rows.shape[0] == keys.shape[0]
         dropped_before = self._dropped()
+        room = self._room_known()
         self.backend.insert(self._prepare(keys), values, external_values)
-        self._warn_if_overfull(keys.shape[0], dropped_before)
+        if not self._surely_stored(keys.shape[0], room):
+            self._warn_if_overfull(keys.shape[0], dropped_before)
+
+    def _room_known(self) -> Optional[int]:
+        """Free indices before an insert, if the backend knows the size without
+        asking the device."""
+        known = getattr(self.backend, "known_size", None)
+        size = known() if known is not None else None
+        return None if size is None else self.capacity - size
+
+    def _surely_stored(self, inserted: int, room: Optional[int]) -> bool:
+        """Whether the overflow check can be left out: the backend has returned
+        from a streaming insert without reading its counters, and the batch
+        fitted the free indices, so no key was refused for lack of room.  The
+        counters are looked at by the next call that needs them."""
+        return (
+            room is not None
+            and inserted <= room
+            and getattr(self.backend, "_status_pending", False)
+        )
 
     def _dropped(self) -> int:
         # kept on the host: the count only changes inside insert calls

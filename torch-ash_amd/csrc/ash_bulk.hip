@@ -982,6 +982,15 @@ __global__ __launch_bounds__(kListThreads) void settle_rows_kernel(
     }
 }
 
+// Leaves one word of the workspace header where the host can read it (`out` is
+// page-locked host memory the device can write to).
+__global__ void publish_word_kernel(const int32_t* __restrict__ word, int32_t* out) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        *out = *word;
+        __threadfence_system();
+    }
+}
+
 int check_values(int n_values, const void* const* src, void* const* dst,
                  const int64_t* row_bytes) {
     if (n_values < 0) ASH_FAIL("negative value count");
@@ -1074,10 +1083,15 @@ int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
     return 0;
 }
 
-int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
-                        int n_values, const void* const* src, void* const* dst,
-                        const int64_t* row_bytes, void* workspace,
-                        int64_t workspace_bytes, void* stream) {
+namespace {
+
+// `early`: where to leave, right after the first split pass, the number of keys
+// that pass handed to the per-key kernel; `early_event` is recorded behind it.
+int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
+                int n_values, const void* const* src, void* const* dst,
+                const int64_t* row_bytes, void* workspace,
+                int64_t workspace_bytes, int32_t* early, hipEvent_t early_event,
+                void* stream) {
     if (check_batch(map, keys, n)) return 1;
     if (check_values(n_values, src, dst, row_bytes)) return 1;
     if (workspace == nullptr) ASH_FAIL("null bulk workspace");
@@ -1118,8 +1132,16 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
+    auto publish = [&]() -> int {
+        if (early == nullptr) return 0;
+        publish_word_kernel<<<1, 64, 0, s>>>(pl.hdr + kHdrSpillKeys, early);
+        ASH_LAUNCH_CHECK();
+        if (early_event != nullptr) ASH_HIP(hipEventRecord(early_event, s));
+        return 0;
+    };
     if (n_values == 0) {
         if (launch_split_keys<false>(map, pl, keys, identity, s)) return 1;
+        if (publish()) return 1;
         split_records_kernel<false><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
         ASH_LAUNCH_CHECK();
         build_kernel<false><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
@@ -1131,6 +1153,7 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
         return insert_selected(map, true, pl.codes_a, pl.spill_a, pl.hdr + kHdrSpillA, none, s);
     }
     if (launch_split_keys<true>(map, pl, keys, identity, s)) return 1;
+    if (publish()) return 1;
     split_records_kernel<true><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
     build_kernel<true><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
@@ -1144,6 +1167,26 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     ASH_LAUNCH_CHECK();
     if (launch_settle_rows(map, pl, keys, user, identity, s)) return 1;
     return insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys, user, s);
+}
+
+}  // namespace
+
+int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
+                        int n_values, const void* const* src, void* const* dst,
+                        const int64_t* row_bytes, void* workspace,
+                        int64_t workspace_bytes, void* stream) {
+    return insert_bulk(map, keys, n, n_values, src, dst, row_bytes, workspace, workspace_bytes,
+                       nullptr, nullptr, stream);
+}
+
+int ash_map_insert_bulk_early(ash_map_t* map, const int32_t* keys, int64_t n,
+                              int n_values, const void* const* src, void* const* dst,
+                              const int64_t* row_bytes, void* workspace,
+                              int64_t workspace_bytes, int32_t* handed_over,
+                              void* handed_over_event, void* stream) {
+    if (handed_over == nullptr) ASH_FAIL("null pointer for the early count");
+    return insert_bulk(map, keys, n, n_values, src, dst, row_bytes, workspace, workspace_bytes,
+                       handed_over, static_cast<hipEvent_t>(handed_over_event), stream);
 }
 
 int ash_map_erase_bulk_query(ash_map_t* map, int64_t n, int64_t* bytes, int* worthwhile) {

@@ -2230,6 +2230,29 @@ int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], int64_t* touch
 
 }  // namespace
 
+int ash_map_status_begin(ash_map_t* map, int32_t* staging, void* event, void* stream) {
+    if (check_map(map)) return 1;
+    if (staging == nullptr) ASH_FAIL("null staging buffer");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    ASH_HIP(hipMemcpyAsync(staging, map->d.ctr, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    if (event != nullptr) ASH_HIP(hipEventRecord(static_cast<hipEvent_t>(event), s));
+    return 0;
+}
+
+int ash_map_status_decode(const int32_t* staging, int64_t out[6]) {
+    if (staging == nullptr) ASH_FAIL("null staging buffer");
+    if (out == nullptr) ASH_FAIL("null status output");
+    out[0] = staging[kCtrSize];
+    out[1] = staging[kCtrDropped];
+    out[2] = staging[kCtrTombs];
+    out[3] = staging[kCtrExotic];
+    out[4] = staging[kCtrLoadDup];
+    out[5] = staging[kCtrTouched];
+    return 0;
+}
+
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
     return read_status(map, nullptr, out, nullptr, stream);
 }
