@@ -94,7 +94,7 @@ def test_streaming_erase_equals_per_key_kernel(gpu_ash, monkeypatch):
         results.append((sort_rows(left)[0], engine.size(), engine.backend.status()["tombstones"]))
     assert torch.equal(results[0][0], results[1][0])
     assert results[0][1] == results[1][1]
-    assert abs(results[0][2] - results[1][2]) <= 0.05 * results[0][2] + 10
+    assert abs(results[0][2] - results[1][2]) <= 0.25 * max(results[0][2], results[1][2]) + 50
 
 
 def test_streaming_erase_piles_unpackable_keys_and_values(streaming, oracle):
