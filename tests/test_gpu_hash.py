@@ -577,6 +577,29 @@ def test_config2_full_size_properties(gpu_ash):
     assert bool(found.all()) and torch.equal(lookup, idx_out)
 
 
+def test_config2_full_size_against_oracle(gpu_ash, oracle):
+    """Configuration 2 at its full size against the oracle on the same keys,
+    rows and queries: the same masks, the same value rows under the indices
+    found, the same key set listed with the same rows."""
+    num, capacity = 16_000_000, 24_000_000
+    w, hm = _run_config2(gpu_ash, num, capacity)
+    omap = _oracle_map(oracle, 3, capacity)
+    stores = {"color": torch.zeros(capacity, 3), "depth": torch.zeros(capacity, 1)}
+    omap.insert(w["keys"].cpu(), {"color": w["color"].cpu(), "depth": w["depth"].cpu()}, stores)
+    assert hm.size() == omap.size() == num
+    masks, indices, values = hm.find(w["query_keys"], return_values=True)
+    idx_cpu, masks_cpu = omap.find(w["query_keys"].cpu())
+    assert torch.equal(masks.cpu(), masks_cpu)
+    for name in ("color", "depth"):
+        assert torch.equal(values[name][masks].cpu(), stores[name][idx_cpu][masks_cpu])
+    del values, masks, indices
+    keys_out, idx_out, vals_out = hm.items(return_values=True)
+    k_cpu, i_cpu = omap.items()
+    s_gpu = sort_rows(keys_out, vals_out["color"], vals_out["depth"])
+    s_cpu = sort_rows(k_cpu, stores["color"][i_cpu], stores["depth"][i_cpu])
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(s_gpu, s_cpu))
+
+
 def test_config5_fusion_reduced_against_oracle(gpu_ash, oracle, monkeypatch):
     """Configuration 5 at reduced size (160x120 frames, three views): per frame
     unproject -> activate blocks with a one-block dilation through the hash map

@@ -934,6 +934,7 @@ class _HashMap:
         # not looked at yet (_finish_streaming_insert): page-locked landing
         # places and events of this map's own
         self._status_pending = False
+        self._late_in_flight = False   # a copy into _late may still be under way
         self._early = None
         # a new map is empty and every counter is zero
         self._status_after_insert = {
@@ -961,6 +962,13 @@ class _HashMap:
 
     def __del__(self):
         handle, self._handle = getattr(self, "_handle", None), None
+        if getattr(self, "_late_in_flight", False):
+            # the device may still owe a write into this map's page-locked
+            # landing place; it must arrive before that memory is given back
+            try:
+                self._late_event.synchronize()
+            except Exception:
+                pass
         if handle:
             self._lib.ash_map_destroy(handle)
 
@@ -1028,6 +1036,11 @@ class _HashMap:
         early_event.synchronize()
         if int(early[0]) != 0:
             return False
+        if self._late_in_flight:
+            # an earlier read-back that nobody looked at (an erase or a clear
+            # made it stale) must have landed before the next one is queued
+            late_event.synchronize()
+        self._late_in_flight = True
         self._check(
             self._lib.ash_map_status_begin(
                 self._handle, late.data_ptr(), late_event.cuda_event, self._stream()
@@ -1045,6 +1058,7 @@ class _HashMap:
         self._status_pending = False
         _, late, _, late_event = self._deferred()
         late_event.synchronize()
+        self._late_in_flight = False
         out = (_I64 * 6)()
         self._check(self._lib.ash_map_status_decode(late.data_ptr(), out))
         st = {
