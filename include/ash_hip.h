@@ -316,7 +316,9 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
  * reset on `stream` at once (the heap array is rewritten to 0..capacity-1 only
  * when ash_map_erase or ash_map_load has written to it since it was last in
  * that state: inserts only read it, and nothing but this library may write to
- * it while the map lives); the fill of the bucket array runs with the next
+ * it while the map lives; while it is in that state listings read the log of
+ * stored keys only below the size, so the log is left as it is and emptied
+ * beyond the size by the first erase); the fill of the bucket array runs with the next
  * call that reads or updates the table, on that call's stream, and not at all
  * when that call is an ash_map_insert_bulk, which rewrites every bucket.  A
  * call whose stream is being captured refuses to run that pending fill (the

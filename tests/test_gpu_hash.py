@@ -577,6 +577,50 @@ def test_config2_full_size_properties(gpu_ash):
     assert bool(found.all()) and torch.equal(lookup, idx_out)
 
 
+def test_listing_after_clears_that_left_the_key_log(gpu_ash, oracle):
+    """clear() does not touch the log of stored keys while nothing was ever
+    erased (a listing then reads no entry beyond the size); what earlier, larger
+    fillings left there must be gone once an erase or a load makes listings
+    read all of it."""
+    dim, capacity = 3, 50_000
+    rng = np.random.default_rng(77)
+
+    def fresh(n, shift):
+        k = torch.from_numpy(rng.integers(-40, 40, size=(n * 2, dim)).astype(np.int32))
+        return (torch.unique(k, dim=0)[:n] + shift).to(DEV)
+
+    engine = gpu_ash.ASHEngine(dim, capacity, DEV)
+    for n in (30_001, 12_345, 20_000):           # fillings of different sizes
+        engine.insert_keys(fresh(n, 0))
+        engine.clear()
+    keys = fresh(7_777, 1000)
+    engine.insert_keys(keys)
+    listed, idx = engine.items()
+    assert torch.equal(sort_rows(listed)[0], sort_rows(keys)[0])
+    assert torch.equal(torch.sort(idx)[0].cpu(), torch.arange(7_777))
+    engine.erase(keys[:1_111])                  # an odd number of keys stays
+    listed, idx = engine.items()
+    assert torch.equal(sort_rows(listed)[0], sort_rows(keys[1_111:])[0])
+    found, mask = engine.find(listed)
+    assert bool(mask.all()) and torch.equal(found, idx)
+    # once more, ending with a load instead of an erase
+    engine.clear()
+    engine.insert_keys(fresh(25_000, 0))
+    engine.clear()
+    engine.insert_keys(keys[:3_333])
+    k_saved, i_saved = engine.items()
+    other = gpu_ash.ASHEngine(dim, capacity, DEV)
+    for n in (9_999, 28_000):
+        other.insert_keys(fresh(n, 0))
+        other.clear()
+    other.insert_keys(fresh(5_001, -1000))
+    other.load_state_dict(engine.state_dict())
+    listed, idx = other.items()
+    got, want = sort_rows(listed, idx), sort_rows(k_saved, i_saved)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    assert other.size() == 3_333
+
+
 def test_config2_full_size_against_oracle(gpu_ash, oracle):
     """Configuration 2 at its full size against the oracle on the same keys,
     rows and queries: the same masks, the same value rows under the indices

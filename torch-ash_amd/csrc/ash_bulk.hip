@@ -1221,7 +1221,7 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
-    map->heap_dirty = true;   // freed indices go back onto the heap
+    if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);

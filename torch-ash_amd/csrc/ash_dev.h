@@ -65,6 +65,7 @@ enum Counter {
     kCtrCursor = 5,    // output cursor of items()
     kCtrTouched = 6,   // blocks listed by the latest ash_grid_collect_touched
     kCtrTicket = 7,    // workgroups of a running ash_grid_collect_touched that have read their input
+    kCtrLogHigh = 8,   // log entries at or beyond the size and below this index may hold keys of an earlier filling
     kNumCounters = 64
 };
 constexpr int64_t kHeaderBytes = 256;
@@ -130,4 +131,9 @@ struct ash_map {
     // the heap array may differ from 0, 1, 2, ... (an erase or a load has
     // written to it since it was last reset): clear() rewrites it only then
     bool heap_dirty;
+    // a clear() has left the key log as it was (while the heap is in its
+    // initial order only entries below the size are read): entries between
+    // the size and the counter kCtrLogHigh are emptied before the order of
+    // the heap is given up (give_up_heap_order)
+    bool log_stale;
 };

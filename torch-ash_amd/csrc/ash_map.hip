@@ -1251,7 +1251,8 @@ __global__ __launch_bounds__(kBlock) void fill16_kernel(uint4* __restrict__ p,
 }
 
 // klog[0 .. limit) := free, limit = the capacity or (prefix_only) the size
-// counter rounded up to whole 16-byte units.  The log's allocation is a
+// counter -- or, if larger, the index below which an earlier clear left its
+// entries standing -- rounded up to whole 16-byte units.  The log's allocation is a
 // multiple of 16 bytes plus slack (256-byte aligned workspace regions), so the
 // last unit of an odd capacity is written whole.
 __global__ __launch_bounds__(kBlock) void empty_log_kernel(
@@ -1259,7 +1260,8 @@ __global__ __launch_bounds__(kBlock) void empty_log_kernel(
         int prefix_only) {
     int64_t entries = capacity;
     if (prefix_only) {
-        const int64_t used = ctr[kCtrSize];
+        const int64_t size = ctr[kCtrSize], high = ctr[kCtrLogHigh];
+        const int64_t used = size > high ? size : high;
         entries = used < capacity ? used : capacity;
     }
     const int64_t n16 = (entries + 1) / 2;
@@ -1271,12 +1273,36 @@ __global__ __launch_bounds__(kBlock) void empty_log_kernel(
     }
 }
 
+// klog[size .. kCtrLogHigh) := free (8-byte stores: an odd size shares its
+// 16 bytes with an entry in use).
+__global__ __launch_bounds__(kBlock) void empty_log_tail_kernel(
+        uint64_t* __restrict__ klog, int64_t capacity, const int32_t* __restrict__ ctr) {
+    const int64_t from = ctr[kCtrSize] < 0 ? 0 : ctr[kCtrSize];
+    const int64_t high = ctr[kCtrLogHigh];
+    const int64_t to = high < capacity ? high : capacity;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    for (int64_t i = from + static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < to;
+         i += stride) {
+        klog[i] = kEmpty;
+    }
+}
+
+// `keep_log`: the key log is left as it is; the counter kCtrLogHigh then
+// remembers how far it may hold entries (the size so far, or what an earlier
+// call remembered).
 __global__ __launch_bounds__(kBlock) void reset_heap_kernel(
         int32_t* __restrict__ heap, int64_t capacity, int32_t* __restrict__ ctr,
-        int32_t size_value, bool write_heap) {
+        int32_t size_value, bool write_heap, bool keep_log) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (write_heap && i < capacity) heap[i] = static_cast<int32_t>(i);
-    if (i < kNumCounters) ctr[i] = (i == kCtrSize) ? size_value : 0;
+    if (i < kNumCounters) {
+        // (one wavefront: every lane has read before any lane writes)
+        const int32_t size = ctr[kCtrSize], high = ctr[kCtrLogHigh];
+        int32_t v = 0;
+        if (i == kCtrSize) v = size_value;
+        if (i == kCtrLogHigh && keep_log) v = size > high ? size : high;
+        ctr[i] = v;
+    }
 }
 
 __global__ void set_counter_kernel(int32_t* ctr, int which, int32_t value) {
@@ -1524,6 +1550,7 @@ int fill_buckets(ash_map* map, hipStream_t s) {
 }
 
 // `lazy`: leave the bucket array to the next call that needs it (settle_table).
+// `lazy` also leaves the key log while the heap is in its initial order.
 int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool lazy = false) {
     if (lazy) {
         map->table_stale = true;
@@ -1537,26 +1564,47 @@ int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool
         ASH_LAUNCH_CHECK();
     }
     // The key log: every index is free again.  While nothing has written to the
-    // heap since its last reset the indices in use are 0 .. size-1, and only
-    // that part of the log (the size is read on the device, before the counters
-    // are reset below) needs clearing.
-    {
+    // heap since its last reset the indices in use are 0 .. size-1 and nothing
+    // reads the log beyond the size: a lazy clear leaves the log alone and only
+    // notes how far it holds entries (reset_heap_kernel); otherwise that part
+    // of the log (read on the device, before the counters are reset below) is
+    // emptied, or all of it once the heap has been written to.
+    const bool keep_log = lazy && !map->heap_dirty;
+    if (keep_log) {
+        map->log_stale = true;
+    } else {
         const int64_t n16 = (map->capacity + 1) / 2;
         empty_log_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
                 reinterpret_cast<uint4*>(map->d.klog), map->capacity, map->d.ctr,
                 map->heap_dirty ? 0 : 1);
         ASH_LAUNCH_CHECK();
+        map->log_stale = false;
     }
     // Inserts only read the heap; while nothing has written to it since the
     // last reset it still is 0, 1, 2, ... and only the counters are reset.
     const bool rewrite = write_heap && map->heap_dirty;
     int64_t span = rewrite && map->capacity > kNumCounters ? map->capacity : kNumCounters;
     reset_heap_kernel<<<grid_for(span), kBlock, 0, s>>>(
-            map->d.heap, map->capacity, map->d.ctr, size, rewrite);
+            map->d.heap, map->capacity, map->d.ctr, size, rewrite, keep_log);
     ASH_LAUNCH_CHECK();
     if (rewrite) map->heap_dirty = false;
     return 0;
 }
+
+}  // namespace
+
+int give_up_heap_order(ash_map* map, hipStream_t s) {
+    if (map->heap_dirty) return 0;
+    map->heap_dirty = true;
+    if (!map->log_stale) return 0;
+    empty_log_tail_kernel<<<capped_grid(map->capacity), kBlock, 0, s>>>(
+            map->d.klog, map->capacity, map->d.ctr);
+    ASH_LAUNCH_CHECK();
+    map->log_stale = false;
+    return 0;
+}
+
+namespace {
 
 template <int MODE>
 int launch_insert(ash_map* map, const int32_t* keys, int64_t n,
@@ -1720,6 +1768,7 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->general_attached = false;
     map->table_stale = false;
     map->heap_dirty = true;   // the caller's buffer holds anything
+    map->log_stale = false;
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
@@ -2177,7 +2226,7 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
-    map->heap_dirty = true;   // freed indices go back onto the heap
+    if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
     const unsigned g = grid_for(n, kEraseBlock);
     switch (map->key_dim) {
         case 1:

@@ -151,5 +151,9 @@ int erase_selected(ash_map* map, bool codes, const void* keys, const int32_t* se
 int check_batch(const ash_map* map, const void* keys, int64_t n);
 // Fills the bucket array if a clear() left that to the next user of the table.
 int settle_table(ash_map* map, hipStream_t s);
+// Before the first call that writes to the heap (an erase; a load brings a
+// heap of its own): from here on items() reads the whole key log, so what a
+// clear() left in it beyond the size is emptied now.
+int give_up_heap_order(ash_map* map, hipStream_t s);
 
 }  // namespace ash
