@@ -565,40 +565,52 @@ __device__ __forceinline__ T dpp(T v) {
 constexpr int kRowShl = 0x100;  // lane i takes lane i + n of its row of 16 (0 beyond it)
 constexpr int kRowShr = 0x110;  // lane i takes lane i - n
 
-// One step of the segmented sum: adds what lies `D` lanes below, unless a run
-// starts in between.
-template <int D>
-__device__ __forceinline__ void run_step(float (&v)[4], int& f, int g) {
-    const int fu = dpp_int<kRowShr + D>(f);
-    const bool take = g >= D && !f;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const float vu = dpp<kRowShr + D>(v[k]);
-        if (take) v[k] += vu;
-    }
-    if (take) f |= fu;
-}
-
 constexpr int kRowBcast15 = 0x142;  // every lane of a row takes lane 15 of the row before
 
-// Sums `v` over runs of consecutive lanes with equal `id`; returns whether this
-// lane ends its run and holds the total.  Every lane of the wavefront must take
-// part.  The sums run inside the rows of 16 lanes; a run that goes on in the
-// next row hands its part over: lane 15 keeps quiet and the lane that ends the
-// run in the next row adds what lane 15 had.  (A run that fills a whole row
-// and still goes on is not handed over a second time; its parts meet in the
-// table of lines.)
-__device__ __forceinline__ bool merge_runs(uint32_t id, float (&v)[4], int lane) {
+// Runs of consecutive lanes whose queries lie in the same cell.  Two queries
+// meet in the same row at a corner only when they lie in the same cell, and
+// then at every corner, so the runs are found once per tile, from the row of the
+// cell itself, and the sums over them are taken corner by corner (sum_runs).
+// The sums run inside the rows of 16 lanes; a run that goes on in the next row
+// hands its part over: lane 15 keeps quiet and the lane that ends the run in
+// the next row adds what lane 15 had.  (A run that fills a whole row and still
+// goes on is not handed over a second time; its parts meet in the table of
+// lines.)
+struct Runs {
+    bool any;         // some lane continues the run of the lane before it (the same for all lanes)
+    bool take[4];     // step 1, 2, 4, 8 of the segmented sum adds what lies that far below
+    bool takes_offer; // adds what lane 15 of the row before holds
+    bool tail;        // this lane ends its run and holds the total
+};
+
+// `id`: the row of the query's cell, or for a lane without a query a number no
+// neighbour shares.  Every lane of the wavefront must take part.
+__device__ __forceinline__ Runs find_runs(uint32_t id, int lane) {
+    Runs r;
     const int g = lane & 15;
     const uint32_t prev = dpp<kRowShr + 1>(id);
     const uint32_t next = dpp<kRowShl + 1>(id);
+    const bool joins = g > 0 && prev == id;
+    r.any = __ballot(joins) != 0;
     const bool starts = g > 0 && prev != id;   // a run starts here, inside the row
-    int f = (g == 0 || starts) ? 1 : 0;
+    int f = (g == 0 || starts) ? 1 : 0;        // a run starts at or below this lane, as far as summed
+    {
+        const int fu = dpp_int<kRowShr + 1>(f);
+        r.take[0] = g >= 1 && !f;
+        if (r.take[0]) f |= fu;
+    }
+    {
+        const int fu = dpp_int<kRowShr + 2>(f);
+        r.take[1] = g >= 2 && !f;
+        if (r.take[1]) f |= fu;
+    }
+    {
+        const int fu = dpp_int<kRowShr + 4>(f);
+        r.take[2] = g >= 4 && !f;
+        if (r.take[2]) f |= fu;
+    }
+    r.take[3] = g >= 8 && !f;
     bool tail = g == 15 || next != id;
-    run_step<1>(v, f, g);
-    run_step<2>(v, f, g);
-    run_step<4>(v, f, g);
-    run_step<8>(v, f, g);
     // in the first run of its row: no run starts between the row's first lane and here
     const uint64_t started = __ballot(starts);
     const uint64_t upto = (2ull << lane) - 1ull;
@@ -608,20 +620,38 @@ __device__ __forceinline__ bool merge_runs(uint32_t id, float (&v)[4], int lane)
     const int offers = (g == 15 && !first_run) ? 1 : 0;
     const int offered = dpp_int<kRowBcast15>(offers);
     const uint32_t offered_id = dpp<kRowBcast15>(id);
-    float part[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) part[k] = dpp<kRowBcast15>(v[k]);
-    if (lane >= 16 && tail && first_run && offered != 0 && offered_id == id) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) v[k] += part[k];
-    }
+    r.takes_offer = lane >= 16 && tail && first_run && offered != 0 && offered_id == id;
     // ... and keeps quiet when the next row takes the offer
     const uint32_t id16 = __builtin_amdgcn_readlane(id, 16);
     const uint32_t id32 = __builtin_amdgcn_readlane(id, 32);
     const uint32_t id48 = __builtin_amdgcn_readlane(id, 48);
     const uint32_t over = lane < 16 ? id16 : lane < 32 ? id32 : id48;
     if (offers != 0 && lane < 48 && over == id) tail = false;
-    return tail;
+    r.tail = tail;
+    return r;
+}
+
+template <int D>
+__device__ __forceinline__ void run_step(float (&v)[4], bool take) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float vu = dpp<kRowShr + D>(v[k]);
+        if (take) v[k] += vu;
+    }
+}
+
+// Sums `v` over the runs; the lanes with r.tail hold the totals afterwards.
+// Every lane of the wavefront must take part.
+__device__ __forceinline__ void sum_runs(const Runs& r, float (&v)[4]) {
+    run_step<1>(v, r.take[0]);
+    run_step<2>(v, r.take[1]);
+    run_step<4>(v, r.take[2]);
+    run_step<8>(v, r.take[3]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float part = dpp<kRowBcast15>(v[k]);
+        if (r.takes_offer) v[k] += part;
+    }
 }
 
 constexpr int kLineSlots = 128;   // lines per wavefront's table
@@ -798,88 +828,22 @@ struct LineAcc {
     }
 };
 
-// The loop over the corners that scatters is not unrolled (one copy of the
-// code, fewer registers), so the corner number is a run-time value there, and
-// what it selects -- a row number, an axis term -- must come out of registers
-// by conditional moves: an indexed access would move the whole array to
-// scratch memory.  To keep the compiler from building that indexed access
-// itself, both operands of every select pass through an empty asm statement,
-// which makes them values without an origin in memory (between two loads from
-// one object the compiler would select the address instead).
-template <typename V>
-__device__ __forceinline__ V in_register(V x) {
-    static_assert(sizeof(V) == 4, "one 32-bit register");
-    asm("" : "+v"(x));
-    return x;
-}
-
-// Both operands are laundered before the select, so that the select stays one
-// conditional move (an asm statement inside an arm of ?: would make it a branch).
-template <typename V>
-__device__ __forceinline__ V pick(bool second, V a, V b) {
-    const V x = in_register(a);
-    const V y = in_register(b);
-    return second ? y : x;
-}
-
-struct Rows8 {
-    uint32_t r[8];
-    __device__ __forceinline__ explicit Rows8(const uint32_t (&row)[8]) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = row[i];
-    }
-    __device__ __forceinline__ uint32_t at(int c) const {
-        const uint32_t a = pick((c & 1) != 0, r[0], r[1]);
-        const uint32_t b = pick((c & 1) != 0, r[2], r[3]);
-        const uint32_t d = pick((c & 1) != 0, r[4], r[5]);
-        const uint32_t e = pick((c & 1) != 0, r[6], r[7]);
-        const uint32_t ab = pick((c & 2) != 0, a, b);
-        const uint32_t de = pick((c & 2) != 0, d, e);
-        return pick((c & 4) != 0, ab, de);
-    }
-};
-
-// Corner weights for a corner number known at run time.
-struct AxisValues {
-    float w0a, w0b, w1a, w1b, w2a, w2b;
-    float d0a, d0b, d1a, d1b, d2a, d2b;
-    __device__ __forceinline__ explicit AxisValues(const AxisTerms<float>& t)
-        : w0a(t.w[0][0]), w0b(t.w[0][1]),
-          w1a(t.w[1][0]), w1b(t.w[1][1]),
-          w2a(t.w[2][0]), w2b(t.w[2][1]),
-          d0a(t.dw[0][0]), d0b(t.dw[0][1]),
-          d1a(t.dw[1][0]), d1b(t.dw[1][1]),
-          d2a(t.dw[2][0]), d2b(t.dw[2][1]) {}
-    __device__ __forceinline__ float weight(int c) const {
-        float w = 1.0f;
-        w *= pick((c & 1) != 0, w0a, w0b);
-        w *= pick((c & 2) != 0, w1a, w1b);
-        w *= pick((c & 4) != 0, w2a, w2b);
-        return w;
-    }
-    __device__ __forceinline__ void weight_grad(int c, float (&g)[3]) const {
-        const float w0 = pick((c & 1) != 0, w0a, w0b);
-        const float w1 = pick((c & 2) != 0, w1a, w1b);
-        const float w2 = pick((c & 4) != 0, w2a, w2b);
-        const float d0 = pick((c & 1) != 0, d0a, d0b);
-        const float d1 = pick((c & 2) != 0, d1a, d1b);
-        const float d2 = pick((c & 4) != 0, d2a, d2b);
-        g[0] = d0 * w1 * w2;
-        g[1] = w0 * d1 * w2;
-        g[2] = w0 * w1 * d2;
-    }
-};
-
 // grad_emb[row, 0..3] += v for the lanes that are `on`; every lane of the
-// wavefront must take part.
+// wavefront must take part.  `runs`: find_runs of this tile.
 __device__ __forceinline__ void accumulate_row4(LineAcc& acc, float* __restrict__ grad_emb,
-                                                uint32_t row, bool on, float (&v)[4],
-                                                int lane) {
-    // lanes that are off get a row number no neighbour shares
-    const uint32_t id = on ? row : (kNoRow - static_cast<uint32_t>(lane & 1));
-    if (!on) v[0] = v[1] = v[2] = v[3] = 0.f;
-    const bool tail = merge_runs(id, v, lane);
+                                                uint32_t row, bool on, const Runs& runs,
+                                                float (&v)[4], int lane) {
+    bool tail = true;
+    if (runs.any) {   // (samples cells apart, scattered points: nothing to join)
+        sum_runs(runs, v);
+        tail = runs.tail;
+    }
     acc.add4(grad_emb, on && tail, row, v, lane);
+}
+
+// The runs of a tile: lanes without a query get a number no neighbour shares.
+__device__ __forceinline__ Runs tile_runs(uint32_t cell_row, bool on, int lane) {
+    return find_runs(on ? cell_row : (kNoRow - static_cast<uint32_t>(lane & 1)), lane);
 }
 
 __device__ __forceinline__ LineTable* line_table(unsigned char* smem, const QDev& a,
@@ -947,15 +911,12 @@ query_backward_forward_vec_kernel(
             }
         }
         if constexpr (want_emb) {
-            // one copy of the scatter code, not eight: fewer registers and a
-            // loop that stays in the instruction cache
-            const AxisValues tv(t);
-            const Rows8 rows(row);
-#pragma unroll 1
+            const Runs runs = tile_runs(row[0], on, lane);
+#pragma unroll
             for (int c = 0; c < 8; ++c) {
-                const float w = tv.weight(c);
+                const float w = corner_weight<float>(t, c);
                 float v[4] = {w * z4.x, w * z4.y, w * z4.z, w * z4.w};
-                accumulate_row4(acc, grad_emb, rows.at(c), on, v, lane);
+                accumulate_row4(acc, grad_emb, row[c], on, runs, v, lane);
             }
             acc.flush(grad_emb, lane);
         }
@@ -1023,15 +984,14 @@ query_backward_backward_vec_kernel(
             }
         }
         if constexpr (want_emb) {
-            const AxisValues tv(t);
-            const Rows8 rows(row);
-#pragma unroll 1
+            const Runs runs = tile_runs(row[0], on, lane);
+#pragma unroll
             for (int c = 0; c < 8; ++c) {
                 float gw[3];
-                tv.weight_grad(c, gw);
+                corner_weight_grad<float>(t, c, gw);
                 const float d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
                 float v[4] = {d * z4.x, d * z4.y, d * z4.z, d * z4.w};
-                accumulate_row4(acc, grad_emb, rows.at(c), on, v, lane);
+                accumulate_row4(acc, grad_emb, row[c], on, runs, v, lane);
             }
             acc.flush(grad_emb, lane);
         }
