@@ -196,24 +196,44 @@ struct TileWalk {
     }
 };
 
+// What a query brings.  The mask, the indices and the offsets are asked for
+// together (one trip to memory, not two); what a masked query has there is read
+// and dropped.
+struct QueryInputs {
+    // low dwords of the int64 indices: a row of the block table is below 2^31
+    // and "none" is -1, a cell is below 2^31 too
+    int32_t gi, ci;
+    float o[3];
+    uint8_t m;   // 0: masked out or beyond the last query
+};
+
+__device__ __forceinline__ QueryInputs load_inputs(const QDev& a, int64_t q) {
+    QueryInputs in;
+    in.gi = in.ci = 0;
+    in.o[0] = in.o[1] = in.o[2] = 0.f;
+    in.m = 0;
+    if (q < a.N) {
+        in.m = a.mask[q];
+        in.gi = reinterpret_cast<const int32_t*>(a.gidx)[q * 2];
+        in.ci = reinterpret_cast<const int32_t*>(a.cidx)[q * 2];
+        in.o[0] = a.off[q * 3 + 0];
+        in.o[1] = a.off[q * 3 + 1];
+        in.o[2] = a.off[q * 3 + 2];
+    }
+    return in;
+}
+
 // Phase 1 for one query: the 8 corner rows (kNoRow in row[0] when the query is
 // masked out, out of range, or misses a neighbour block) and the offsets.
 template <bool LDS>
 __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
-                                             int64_t q, uint32_t (&row)[8],
+                                             const QueryInputs& in, uint32_t (&row)[8],
                                              float (&o)[3]) {
-    bool valid = q < a.N && a.mask[q] != 0;
-    int64_t gi = 0, ci = 0;
-    o[0] = o[1] = o[2] = 0.f;
-    if (valid) {
-        gi = a.gidx[q];
-        ci = a.cidx[q];
-        o[0] = a.off[q * 3 + 0];
-        o[1] = a.off[q * 3 + 1];
-        o[2] = a.off[q * 3 + 2];
-        valid = gi >= 0 && gi < a.B;
-        ci = ci < 0 ? 0 : (ci >= a.M ? a.M - 1 : ci);
-    }
+    bool valid = in.m != 0 && static_cast<uint32_t>(in.gi) < static_cast<uint32_t>(a.B);
+    const int64_t gi = valid ? in.gi : 0;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) o[d] = valid ? in.o[d] : 0.f;
+    const int64_t ci = in.ci < 0 ? 0 : (in.ci >= a.M ? a.M - 1 : in.ci);
     // Block indices are below 2^31 and a missing block is -1, so the low
     // dword of each int64 table entry carries everything.
     const int32_t* lut_g32 = reinterpret_cast<const int32_t*>(a.lut_g) + gi * 16;
@@ -238,6 +258,13 @@ __device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
         }
     }
     if (!valid) row[0] = kNoRow;
+}
+
+template <bool LDS>
+__device__ __forceinline__ void resolve_rows(const QDev& a, const CellLut& lut,
+                                             int64_t q, uint32_t (&row)[8],
+                                             float (&o)[3]) {
+    resolve_rows<LDS>(a, lut, load_inputs(a, q), row, o);
 }
 
 // Runs phase 1 for the tile and hands every thread the rows / offsets of the
@@ -873,7 +900,8 @@ query_backward_forward_vec_kernel(
         uint32_t row[8];
         float o[3];
         const int64_t q = tile * kBlock + threadIdx.x;
-        resolve_rows<LDS>(a, lut, q, row, o);
+        const QueryInputs in = load_inputs(a, q);
+        resolve_rows<LDS>(a, lut, in, row, o);
         const bool on = row[0] != kNoRow;
         float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
         if (on) z4 = *reinterpret_cast<const float4*>(z + q * 4);
@@ -944,7 +972,8 @@ query_backward_backward_vec_kernel(
         uint32_t row[8];
         float o[3];
         const int64_t q = tile * kBlock + threadIdx.x;
-        resolve_rows<LDS>(a, lut, q, row, o);
+        const QueryInputs in = load_inputs(a, q);
+        resolve_rows<LDS>(a, lut, in, row, o);
         const bool on = row[0] != kNoRow;
         float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
         float gg[3] = {0.f, 0.f, 0.f};
