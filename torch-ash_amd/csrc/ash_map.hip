@@ -1504,7 +1504,22 @@ inline unsigned grid_for(int64_t n, int per_block = kBlock) {
     return static_cast<unsigned>((n + per_block - 1) / per_block);
 }
 
+// One unit per thread as far as a launch goes (the kernels loop beyond that):
+// workgroups that are handed out one after the other walk through memory in
+// order, which the memory side rewards (a 1.6 GB fill: 6.8 TB/s, against 5.7
+// with 16 384 workgroups that stride through it and 4.5 with 4096).
 inline unsigned capped_grid(int64_t n) {
+    int64_t g = (n + kBlock - 1) / kBlock;
+    const int64_t cap = 0x7FFFFFFF;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return static_cast<unsigned>(g);
+}
+
+// For the kernels that move rows by index (random on one side): 8192
+// workgroups that loop (one unit per thread: 0.23 against 0.185 ms for the 16 M
+// rows of two value tensors).
+inline unsigned looping_grid(int64_t n) {
     int64_t g = (n + kBlock - 1) / kBlock;
     const int64_t cap = 256 * 32;
     if (g > cap) g = cap;
@@ -2121,16 +2136,16 @@ int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
                             static_cast<uintptr_t>(row_bytes);
     if (align % 16 == 0) {
         const int64_t upr = row_bytes / 16;
-        scatter_rows_kernel<uint4><<<capped_grid(n * upr), kBlock, 0, s>>>(
+        scatter_rows_kernel<uint4><<<looping_grid(n * upr), kBlock, 0, s>>>(
                 static_cast<const uint4*>(src), static_cast<uint4*>(dst),
                 assigned, n, upr);
     } else if (align % 4 == 0) {
         const int64_t upr = row_bytes / 4;
-        scatter_rows_kernel<uint32_t><<<capped_grid(n * upr), kBlock, 0, s>>>(
+        scatter_rows_kernel<uint32_t><<<looping_grid(n * upr), kBlock, 0, s>>>(
                 static_cast<const uint32_t*>(src), static_cast<uint32_t*>(dst),
                 assigned, n, upr);
     } else {
-        scatter_rows_kernel<uint8_t><<<capped_grid(n * row_bytes), kBlock, 0,
+        scatter_rows_kernel<uint8_t><<<looping_grid(n * row_bytes), kBlock, 0,
                                        s>>>(static_cast<const uint8_t*>(src),
                                             static_cast<uint8_t*>(dst),
                                             assigned, n, row_bytes);
@@ -2169,7 +2184,7 @@ int ash_gather_rows(int n_values, const void* const* src, void* const* dst,
     }
     PointerGuard guard;
     ASH_HIP(guard.enter_for(indices));
-    gather_rows_kernel<<<capped_grid(most), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
+    gather_rows_kernel<<<looping_grid(most), kBlock, 0, static_cast<hipStream_t>(stream)>>>(
             a, indices, n);
     ASH_LAUNCH_CHECK();
     return 0;

@@ -1909,8 +1909,10 @@ int zero_fill(void* ptr, int64_t bytes, hipStream_t s) {
     }
     const int64_t n16 = (bytes - head) / 16;
     if (n16 > 0) {
+        // one store per thread: workgroups handed out one after the other walk
+        // through memory in order (6.8 TB/s; 5.7 with 16 384 workgroups striding)
         int64_t g = (n16 + kBlock - 1) / kBlock;
-        if (g > 256 * 64) g = 256 * 64;
+        if (g > 0x7FFFFFFF) g = 0x7FFFFFFF;
         zero16_kernel<<<static_cast<unsigned>(g), kBlock, 0, s>>>(
                 reinterpret_cast<uint4*>(p + head), n16);
         ASH_LAUNCH_CHECK();
