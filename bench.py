@@ -102,10 +102,10 @@ MEASURED_COUNTERS = {
     "insert_keys_bulk": (449_000_000 + 914_000_000, 0.411, 59_000),
     "cfg3_forward_linear": (3_519_000_000 + 282_000_000, 0.171, 0),
     "cfg3_forward_smooth_step": (3_519_000_000 + 282_000_000, 0.171, 0),
-    "cfg4_forward": (369_000_000 + 67_000_000, 0.258, 0),
+    "cfg4_forward": (376_000_000 + 67_000_000, 0.259, 0),
     # kernel only: the zero fill of the dense gradient adds 1.64 GB written
-    "cfg4_backward": (431_000_000 + 149_000_000 + 1_638_400_000, 0.093, 2_344_000),
-    "cfg4_double_backward": (486_000_000 + 197_000_000 + 1_638_400_000, 0.163, 2_344_000),
+    "cfg4_backward": (438_000_000 + 149_000_000 + 1_638_400_000, 0.097, 2_344_000),
+    "cfg4_double_backward": (485_000_000 + 166_000_000 + 1_638_400_000, 0.108, 2_344_000),
     "cfg4_grid_query": (71_000_000 + 122_000_000, 0.399, 0),
 }
 

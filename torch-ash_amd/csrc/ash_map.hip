@@ -1589,7 +1589,9 @@ int clear_table(ash_map* map, hipStream_t s, bool write_heap, int32_t size, bool
         map->log_stale = true;
     } else {
         const int64_t n16 = (map->capacity + 1) / 2;
-        empty_log_kernel<<<capped_grid(n16), kBlock, 0, s>>>(
+        // (a prefix of unknown length: few workgroups that loop, not one per
+        // 4 KB of the capacity, most of which would start only to leave)
+        empty_log_kernel<<<map->heap_dirty ? capped_grid(n16) : looping_grid(n16), kBlock, 0, s>>>(
                 reinterpret_cast<uint4*>(map->d.klog), map->capacity, map->d.ctr,
                 map->heap_dirty ? 0 : 1);
         ASH_LAUNCH_CHECK();
@@ -1612,7 +1614,7 @@ int give_up_heap_order(ash_map* map, hipStream_t s) {
     if (map->heap_dirty) return 0;
     map->heap_dirty = true;
     if (!map->log_stale) return 0;
-    empty_log_tail_kernel<<<capped_grid(map->capacity), kBlock, 0, s>>>(
+    empty_log_tail_kernel<<<looping_grid(map->capacity), kBlock, 0, s>>>(
             map->d.klog, map->capacity, map->d.ctr);
     ASH_LAUNCH_CHECK();
     map->log_stale = false;
