@@ -418,6 +418,8 @@ enum { ASH_F32 = 0, ASH_F64 = 1 };
  *   embeddings   scalar[B, M, E]   (M = cells per block, E <= 16)
  *   offsets      float32[N, 3]     (always fp32, ash/src/grid.cu:71)
  *   grid_indices int64[N], cell_indices int64[N], masks uint8/bool[N]
+ *                (B and M are below 2^31 and only the low 32 bits of an index
+ *                are read; what a masked query holds there is read and dropped)
  *   lut_grid_nb2grid_idx int64[B, 8]  (-1 = missing neighbour block)
  *   lut_cell_nb2cell_idx int64[M, 8], lut_cell_nb2grid_nb int64[M, 8] */
 typedef struct ash_query_args {
