@@ -410,20 +410,20 @@ def test_streaming_insert_returns_before_its_counters_are_read(bulk_ash, oracle)
     ka, kb = _random_keys(rng, 90_000, dim, 30), _random_keys(rng, 70_000, dim, 28)
     a.insert_keys(ka.to(DEV))
     b.insert_keys(kb.to(DEV))
-    assert a.backend._status_pending and b.backend._status_pending
+    assert a.backend.counters_queued and b.backend.counters_queued
     # look-ups do not need the counters
     _, mask = a.find(ka[:1000].to(DEV))
-    assert bool(mask.all()) and a.backend._status_pending
+    assert bool(mask.all()) and a.backend.counters_queued
     oa.insert_keys(ka)
     ob.insert_keys(kb)
-    assert b.size() == ob.size() and not b.backend._status_pending
-    assert a.size() == oa.size() and not a.backend._status_pending
+    assert b.size() == ob.size() and not b.backend.counters_queued
+    assert a.size() == oa.size() and not a.backend.counters_queued
     # an erase makes queued counters stale
     a.insert_keys(_random_keys(rng, 10_000, dim, 31).to(DEV))
-    assert a.backend._status_pending
+    assert a.backend.counters_queued
     gone = ka[:5_000]
     a.erase(gone.to(DEV))
-    assert not a.backend._status_pending
+    assert not a.backend.counters_queued
     oa2 = _oracle_map(oracle, dim, capacity)
     k_now, _ = a.items()
     oa2.insert_keys(k_now.cpu())
@@ -435,11 +435,11 @@ def test_streaming_insert_returns_before_its_counters_are_read(bulk_ash, oracle)
     odd = torch.tensor([[2**30, 5, -(2**30)]], dtype=torch.int32)
     batch = torch.cat([_random_keys(rng, 8_000, dim, 29), odd])
     b.insert_keys(batch.to(DEV))
-    assert not b.backend._status_pending
+    assert not b.backend.counters_queued
     ob.insert_keys(batch)
     _assert_same_map(b, ob, torch.cat([batch, kb[:2000]]).to(DEV))
     # with the second region attached an unpackable key still takes the waiting path
     b.insert_keys(torch.cat([_random_keys(rng, 6_000, dim, 27), odd + 1]).to(DEV))
-    assert not b.backend._status_pending
+    assert not b.backend.counters_queued
     b.insert_keys(_random_keys(rng, 6_000, dim, 27).to(DEV))
-    assert b.backend._status_pending and b.size() <= capacity
+    assert b.backend.counters_queued and b.size() <= capacity

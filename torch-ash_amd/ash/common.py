@@ -1122,6 +1122,12 @@ class _HashMap:
         st = getattr(self, "_status_after_insert", None)
         return st if st is not None else self.status()
 
+    @property
+    def counters_queued(self) -> bool:
+        """Whether the latest insert returned with the read-back of the
+        counters still queued behind it (see _finish_streaming_insert)."""
+        return self._status_pending
+
     def known_size(self) -> Optional[int]:
         """The size if it is known on the host (from the latest read-back, or
         zero after a clear), else None; never asks the device for it."""

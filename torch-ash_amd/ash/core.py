@@ -176,7 +176,7 @@ class ASHEngine(nn.Module):
         return (
             room is not None
             and inserted <= room
-            and getattr(self.backend, "_status_pending", False)
+            and getattr(self.backend, "counters_queued", False)
         )
 
     def _dropped(self) -> int:
