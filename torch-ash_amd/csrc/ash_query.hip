@@ -376,46 +376,64 @@ query_forward_kernel(
 }
 
 // ------------------------------------------------- run merge for atomics
-// Inclusive segmented sum over the query groups of a wavefront: `head` marks
-// the first group of a run of equal rows; afterwards the last group of every
-// run holds the run's total.
-template <typename T, int LPQ>
-__device__ __forceinline__ T run_sum(T v, bool head, int lane) {
-    constexpr int kGroups = 64 / LPQ;
+// Runs of consecutive queries of a wavefront that lie in the same cell.  Two
+// queries meet in the same row at a corner only when they lie in the same
+// cell, and then at every corner, so the runs are found once per pass, from
+// the row of the cell itself, and the sums over them are taken corner by
+// corner: one lane exchange per step and corner.  Query groups are LPQ lanes
+// wide (one lane per channel); a lane talks to the lanes of its own channel.
+template <int LPQ>
+struct GroupRuns {
+    static constexpr int kGroups = 64 / LPQ;
+    static constexpr int kSteps = kGroups > 32 ? 6 : kGroups > 16 ? 5 : kGroups > 8 ? 4
+                                  : kGroups > 4 ? 3 : kGroups > 2 ? 2 : 1;
+    bool any;            // some group continues the run of the group before it (the same for all lanes)
+    bool take[kSteps];   // step k of the segmented sum adds what lies 2^k groups below
+    bool tail;           // the last group of its run: holds the total afterwards
+};
+
+// `on`: the lane has a query and a channel.  Every lane of the wavefront must
+// take part.
+template <int LPQ>
+__device__ __forceinline__ GroupRuns<LPQ> find_group_runs(uint32_t cell_row, bool on, int lane) {
+    using R = GroupRuns<LPQ>;
+    R r;
     const int grp = lane / LPQ;
+    // lanes that are off get a row number no neighbour shares
+    const uint32_t id = on ? cell_row : (kNoRow - static_cast<uint32_t>(grp & 1));
+    const uint32_t prev = __shfl_up(id, LPQ);
+    const uint32_t next = __shfl_down(id, LPQ);
+    const bool head = (grp == 0) || (prev != id) || !on;
+    r.tail = (grp == R::kGroups - 1) || (next != id);
+    r.any = __ballot(!head) != 0;
     int f = head ? 1 : 0;
 #pragma unroll
-    for (int d = 1; d < kGroups; d <<= 1) {
-        const T vu = __shfl_up(v, d * LPQ);
+    for (int k = 0; k < R::kSteps; ++k) {
+        const int d = 1 << k;
         const int fu = __shfl_up(f, d * LPQ);
-        if (grp >= d && !f) {
-            v += vu;
-            f |= fu;
-        }
+        r.take[k] = grp >= d && !f;
+        if (r.take[k]) f |= fu;
     }
-    return v;
+    return r;
 }
 
-// Adds v to grad_emb[row, ch] for the lanes that are `on`.
+// Adds v to grad_emb[row, ch] for the lanes that are `on`; with `runs` the
+// last group of every run adds the run's sum (runs.any false: every lane for
+// itself).  Every lane of the wavefront must take part.
 template <typename T, int LPQ>
 __device__ __forceinline__ void accumulate_row(T* __restrict__ grad_emb,
                                                uint32_t row, int E, int ch,
-                                               bool on, T v, int lane,
-                                               int merge) {
-    if (merge) {
-        constexpr int kGroups = 64 / LPQ;
-        const int grp = lane / LPQ;
-        // lanes that are off get a row number no neighbour shares
-        const uint32_t id = on ? row : (kNoRow - static_cast<uint32_t>(grp & 1));
-        const uint32_t prev = __shfl_up(id, LPQ);
-        const uint32_t next = __shfl_down(id, LPQ);
-        const bool head = (grp == 0) || (prev != id) || !on;
-        const bool tail = (grp == kGroups - 1) || (next != id);
-        v = run_sum<T, LPQ>(on ? v : T(0), head, lane);
-        if (on && tail) {
-            unsafeAtomicAdd(grad_emb + static_cast<int64_t>(row) * E + ch, v);
+                                               bool on, T v, const GroupRuns<LPQ>& runs) {
+    bool last = true;
+    if (runs.any) {   // (the same for all lanes)
+#pragma unroll
+        for (int k = 0; k < GroupRuns<LPQ>::kSteps; ++k) {
+            const T vu = __shfl_up(v, (1 << k) * LPQ);
+            if (runs.take[k]) v += vu;
         }
-    } else if (on) {
+        last = runs.tail;
+    }
+    if (on && last) {
         unsafeAtomicAdd(grad_emb + static_cast<int64_t>(row) * E + ch, v);
     }
 }
@@ -453,6 +471,9 @@ query_backward_forward_kernel(
             const bool valid = row[0] != kNoRow;
             const bool on = valid && chv;
             const T zk = on ? z[q * a.E + ch] : T(0);
+            GroupRuns<LPQ> runs;
+            runs.any = false;
+            if (want_emb && a.merge) runs = find_group_runs<LPQ>(row[0], on, lane);
             T e[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
@@ -467,8 +488,7 @@ query_backward_forward_kernel(
             for (int c = 0; c < 8; ++c) {
                 if constexpr (want_emb) {
                     const T w = corner_weight<T>(t, c);
-                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk,
-                                           lane, a.merge);
+                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, w * zk, runs);
                 }
                 if constexpr (want_off) {
                     T gw[3];
@@ -522,6 +542,9 @@ query_backward_backward_kernel(
             const bool valid = row[0] != kNoRow;
             const bool on = valid && chv;
             const T zk = on ? z[q * a.E + ch] : T(0);
+            GroupRuns<LPQ> runs;
+            runs.any = false;
+            if (want_emb && a.merge) runs = find_group_runs<LPQ>(row[0], on, lane);
             T gg[3] = {T(0), T(0), T(0)};
             if (valid) {
                 gg[0] = gg_off[q * 3 + 0];
@@ -544,8 +567,7 @@ query_backward_backward_kernel(
                 corner_weight_grad<T>(t, c, gw);
                 const T d = gw[0] * gg[0] + gw[1] * gg[1] + gw[2] * gg[2];
                 if constexpr (want_emb) {
-                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk,
-                                           lane, a.merge);
+                    accumulate_row<T, LPQ>(grad_emb, row[c], a.E, ch, on, d * zk, runs);
                 }
                 gz += d * e[c];
             }
