@@ -322,7 +322,7 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
             rank[k] = atomicAdd(&sh.cnt[bin[k]], 1);
             if constexpr (PROV) {
                 pl.flags[i] = 0;
-                if (identity) m.klog[heap_base + i] = code[k];
+                if (identity) __builtin_nontemporal_store(code[k], m.klog + heap_base + i);
             }
         } else if (active) {
             // unpackable, or beyond what the heap can still give: left to the
@@ -620,8 +620,16 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
         }
         __syncthreads();
     }
-    for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
-        gl[t] = tab[staged(t >> 3, t & 7)];
+    // (stores marked as not to be kept in the caches: nothing reads the range,
+    // the value rows or the log entries again before a later call does; the
+    // insert with values of 16 M keys: 0.588 -> 0.570 ms)
+    {
+        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+        for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
+            const uint4 x = tab[staged(t >> 3, t & 7)];
+            v4u y = {x.x, x.y, x.z, x.w};
+            __builtin_nontemporal_store(y, reinterpret_cast<v4u*>(gl) + t);
+        }
     }
     if constexpr (PROV) {
         if (tid == 0 && s_losers) atomicAdd(pl.hdr + kHdrLosers, s_losers);
@@ -793,7 +801,12 @@ __device__ __forceinline__ void copy_plane(const MapDev& m, const BulkPlan& pl,
             for (int64_t r = lo; r <= hi; ++r) all = all && pl.flags[r] == 0;
         }
         if (all) {
-            reinterpret_cast<uint4*>(to)[t] = reinterpret_cast<const uint4*>(src)[t];
+            {
+                typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+                const uint4 x = reinterpret_cast<const uint4*>(src)[t];
+                v4u y = {x.x, x.y, x.z, x.w};
+                __builtin_nontemporal_store(y, reinterpret_cast<v4u*>(to) + t);
+            }
         } else {
             for (int q = 0; q < 4; ++q) move_word(4 * t + q);
         }
