@@ -391,8 +391,10 @@ __global__ __launch_bounds__(kSplitThreads) void split_records_kernel(MapDev m, 
         code[k] = 0;
         aux[k] = j;
         if (start + j < cnt) {
-            code[k] = pl.codes_a[abase + j];
-            if constexpr (PROV) aux[k] = pl.rows_a[abase + j];
+            // (records are read once: loads marked as not to be kept in the
+            // caches, here and in the range passes; 3 % of an insert)
+            code[k] = __builtin_nontemporal_load(pl.codes_a + abase + j);
+            if constexpr (PROV) aux[k] = __builtin_nontemporal_load(pl.rows_a + abase + j);
             bin[k] = static_cast<int>((bucket_of(code[k], m.nb) >> kPartShift) & fmask);
             rank[k] = atomicAdd(&sh.cnt[bin[k]], 1);
         }
@@ -518,8 +520,8 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
 #pragma unroll
     for (int k = 0; k < kBuildRecs; ++k) {
         const int r = k * kBuildThreads + tid;
-        codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
-        if constexpr (PROV) rows[k] = r < cnt ? pl.rows_b[bbase + r] : 0;
+        codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
+        if constexpr (PROV) rows[k] = r < cnt ? __builtin_nontemporal_load(pl.rows_b + bbase + r) : 0;
     }
     for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
         tab[staged(t >> 3, t & 7)] =
@@ -541,8 +543,8 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
 #pragma unroll
             for (int k = 0; k < kBuildRecs; ++k) {
                 const int r = rb + k * kBuildThreads + tid;
-                codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
-                if constexpr (PROV) rows[k] = r < cnt ? pl.rows_b[bbase + r] : 0;
+                codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
+                if constexpr (PROV) rows[k] = r < cnt ? __builtin_nontemporal_load(pl.rows_b + bbase + r) : 0;
             }
         }
 #pragma unroll
@@ -667,7 +669,7 @@ __global__ __launch_bounds__(kBuildThreads) void erase_range_kernel(MapDev m, Bu
 #pragma unroll
     for (int k = 0; k < kBuildRecs; ++k) {
         const int r = k * kBuildThreads + tid;
-        codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
+        codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
     }
     for (int t = tid; t < nbk * kGroup; t += kBuildThreads) tab[staged(t >> 3, t & 7)] = gl[t];
     if (tid == 0) s_tombs = 0;
@@ -681,7 +683,7 @@ __global__ __launch_bounds__(kBuildThreads) void erase_range_kernel(MapDev m, Bu
 #pragma unroll
             for (int k = 0; k < kBuildRecs; ++k) {
                 const int r = rb + k * kBuildThreads + tid;
-                codes[k] = r < cnt ? pl.codes_b[bbase + r] : 0ull;
+                codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
             }
         }
         int32_t freed[kBuildRecs];
@@ -803,7 +805,8 @@ __device__ __forceinline__ void copy_plane(const MapDev& m, const BulkPlan& pl,
         if (all) {
             {
                 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-                const uint4 x = reinterpret_cast<const uint4*>(src)[t];
+                const v4u xl = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(src) + t);
+                const uint4 x = make_uint4(xl.x, xl.y, xl.z, xl.w);
                 v4u y = {x.x, x.y, x.z, x.w};
                 __builtin_nontemporal_store(y, reinterpret_cast<v4u*>(to) + t);
             }
