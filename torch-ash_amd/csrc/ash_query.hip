@@ -198,7 +198,9 @@ struct TileWalk {
 
 // What a query brings.  The mask, the indices and the offsets are asked for
 // together (one trip to memory, not two); what a masked query has there is read
-// and dropped.
+// and dropped.  They are read once, like z, and the per-query outputs are
+// written once: those loads and stores carry the non-temporal hint, which
+// leaves the caches to the embedding rows (forward, E = 4: 0.129 -> 0.117 ms).
 struct QueryInputs {
     // low dwords of the int64 indices: a row of the block table is below 2^31
     // and "none" is -1, a cell is below 2^31 too
@@ -213,12 +215,12 @@ __device__ __forceinline__ QueryInputs load_inputs(const QDev& a, int64_t q) {
     in.o[0] = in.o[1] = in.o[2] = 0.f;
     in.m = 0;
     if (q < a.N) {
-        in.m = a.mask[q];
-        in.gi = reinterpret_cast<const int32_t*>(a.gidx)[q * 2];
-        in.ci = reinterpret_cast<const int32_t*>(a.cidx)[q * 2];
-        in.o[0] = a.off[q * 3 + 0];
-        in.o[1] = a.off[q * 3 + 1];
-        in.o[2] = a.off[q * 3 + 2];
+        in.m = __builtin_nontemporal_load(a.mask + q);
+        in.gi = __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(a.gidx) + q * 2);
+        in.ci = __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(a.cidx) + q * 2);
+        in.o[0] = __builtin_nontemporal_load(a.off + q * 3 + 0);
+        in.o[1] = __builtin_nontemporal_load(a.off + q * 3 + 1);
+        in.o[2] = __builtin_nontemporal_load(a.off + q * 3 + 2);
     }
     return in;
 }
@@ -368,8 +370,14 @@ query_forward_kernel(
                 }
             }
             if (q < a.N && chv) {
-                *reinterpret_cast<V*>(out + q * a.E + ch0) =
-                        *reinterpret_cast<const V*>(acc);
+                if constexpr (sizeof(V) == 16) {
+                    typedef float v4f __attribute__((ext_vector_type(4)));
+                    const v4f r4 = {static_cast<float>(acc[0]), static_cast<float>(acc[VEC > 1 ? 1 : 0]),
+                                    static_cast<float>(acc[VEC > 2 ? 2 : 0]), static_cast<float>(acc[VEC > 3 ? 3 : 0])};
+                    __builtin_nontemporal_store(r4, reinterpret_cast<v4f*>(out + q * a.E + ch0));
+                } else {
+                    __builtin_nontemporal_store(acc[0], out + q * a.E + ch0);
+                }
             }
         }
     }
@@ -926,7 +934,11 @@ query_backward_forward_vec_kernel(
         resolve_rows<LDS>(a, lut, in, row, o);
         const bool on = row[0] != kNoRow;
         float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (on) z4 = *reinterpret_cast<const float4*>(z + q * 4);
+        if (on) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f zl = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(z + q * 4));
+            z4 = make_float4(zl.x, zl.y, zl.z, zl.w);
+        }
         AxisTerms<float> t;
         axis_terms<float, true>(o, a.smooth, t);
         // the gathered rows are used up before the scatter starts, which keeps
@@ -955,9 +967,9 @@ query_backward_forward_vec_kernel(
                 go[2] += dot * gw[2];
             }
             if (q < a.N) {
-                grad_off[q * 3 + 0] = on ? go[0] : 0.f;
-                grad_off[q * 3 + 1] = on ? go[1] : 0.f;
-                grad_off[q * 3 + 2] = on ? go[2] : 0.f;
+                __builtin_nontemporal_store(on ? go[0] : 0.f, grad_off + q * 3 + 0);
+                __builtin_nontemporal_store(on ? go[1] : 0.f, grad_off + q * 3 + 1);
+                __builtin_nontemporal_store(on ? go[2] : 0.f, grad_off + q * 3 + 2);
             }
         }
         if constexpr (want_emb) {
@@ -1000,10 +1012,12 @@ query_backward_backward_vec_kernel(
         float4 z4 = make_float4(0.f, 0.f, 0.f, 0.f);
         float gg[3] = {0.f, 0.f, 0.f};
         if (on) {
-            z4 = *reinterpret_cast<const float4*>(z + q * 4);
-            gg[0] = gg_off[q * 3 + 0];
-            gg[1] = gg_off[q * 3 + 1];
-            gg[2] = gg_off[q * 3 + 2];
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f zl = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(z + q * 4));
+            z4 = make_float4(zl.x, zl.y, zl.z, zl.w);
+            gg[0] = __builtin_nontemporal_load(gg_off + q * 3 + 0);
+            gg[1] = __builtin_nontemporal_load(gg_off + q * 3 + 1);
+            gg[2] = __builtin_nontemporal_load(gg_off + q * 3 + 2);
         }
         AxisTerms<float> t;
         axis_terms<float, true>(o, a.smooth, t);
@@ -1029,9 +1043,9 @@ query_backward_backward_vec_kernel(
                 gz[3] += d * e[c].w;
             }
             if (q < a.N) {
-                *reinterpret_cast<float4*>(grad_z + q * 4) =
-                        on ? make_float4(gz[0], gz[1], gz[2], gz[3])
-                           : make_float4(0.f, 0.f, 0.f, 0.f);
+                typedef float v4f __attribute__((ext_vector_type(4)));
+                const v4f g4 = {on ? gz[0] : 0.f, on ? gz[1] : 0.f, on ? gz[2] : 0.f, on ? gz[3] : 0.f};
+                __builtin_nontemporal_store(g4, reinterpret_cast<v4f*>(grad_z + q * 4));
             }
         }
         if constexpr (want_emb) {
