@@ -360,7 +360,7 @@ def bench_hash(torch, ash, workloads, args, dev):
     # order (nothing erased or loaded since the clear): the first n rows, copied
     t_rows = EventTimer(torch)
     for it in range(args.warmup + args.steps):
-        fn = lambda: [v[:n].clone() for v in (hm.color, hm.depth)]
+        fn = lambda: check(lib.ash_gather_rows(k, c_dst, c_out, c_rows, c_count, None, n, stream))
         if it >= args.warmup:
             t_rows(fn)
         else:
@@ -373,8 +373,8 @@ def bench_hash(torch, ash, workloads, args, dev):
         # the heap is in its initial order when items() runs here: n indices scanned
         "items": roofline_entry("items_dense_kernel<3>", items_bytes(n, n), t_items.mean_ms()),
         # value rows of the enumerated entries while the listing is in index
-        # order: 16 B read and written per entry (two device copies)
-        "items_values": roofline_entry("copy of the first n rows of color and depth",
+        # order: 16 B read and written per entry (one launch for both tensors)
+        "items_values": roofline_entry("copy_first_rows_kernel (first n rows of color and depth)",
                                        VALUE_ROW_BYTES * n, t_rows.mean_ms()),
         # ... and by index (after an erase or a load): index in, 16 B read and written
         "items_values_by_index": roofline_entry(

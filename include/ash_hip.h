@@ -404,7 +404,9 @@ int ash_scatter_rows(const void* src, void* dst, const int32_t* assigned,
  * launch per tensor): dst[v][i] = src[v][indices[i]] for up to four tensors in
  * one launch.  Rows of tensor v are row_bytes[v] bytes (a multiple of 4), the
  * source has src_rows[v] rows; an index outside the source gives a zero row.
- * dst[v] holds n rows.  Runs on the device that holds `indices`. */
+ * dst[v] holds n rows.  indices == NULL stands for 0, 1, .., n-1 (what a
+ * listing holds while ash_map_items_in_index_order says so): the first n rows
+ * are copied.  Runs on the device that holds the first source tensor. */
 int ash_gather_rows(int n_values, const void* const* src, void* const* dst,
                     const int64_t* row_bytes, const int64_t* src_rows,
                     const int64_t* indices, int64_t n, void* stream);

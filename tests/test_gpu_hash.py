@@ -577,6 +577,30 @@ def test_config2_full_size_properties(gpu_ash):
     assert bool(found.all()) and torch.equal(lookup, idx_out)
 
 
+def test_first_rows_copy_equals_indexing(gpu_ash):
+    """ash_gather_rows without indices copies the first n rows of every tensor
+    (what a listing in index order asks for): equal to table[:n] for rows of
+    4 to 64 bytes, tensors that do not start on a 16-byte boundary, n = 0, 1,
+    odd and full."""
+    backend = gpu_ash.core.backend
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    base = torch.rand(7 + 1001 * 16, generator=gen).to(DEV)
+    tables = {
+        "a": torch.rand(1001, 3, generator=gen).to(DEV),
+        "b": torch.rand(1001, 1, generator=gen).to(DEV),
+        "c": torch.rand(1001, 4, 4, generator=gen).to(DEV),
+        "d": base[3:3 + 1001 * 5].view(1001, 5),          # starts 12 bytes into its storage
+        "e": torch.arange(1001 * 2, dtype=torch.int32, device=DEV).view(1001, 2),
+    }
+    for n in (0, 1, 2, 333, 1000, 1001):
+        got = backend.gather_rows(tables, None, first=n)
+        for name, table in tables.items():
+            assert got[name].shape == (n,) + tuple(table.shape[1:])
+            assert torch.equal(got[name], table[:n]), (name, n)
+            if n:
+                assert got[name].data_ptr() != table.data_ptr()
+
+
 def test_listing_after_clears_that_left_the_key_log(gpu_ash, oracle):
     """clear() does not touch the log of stored keys while nothing was ever
     erased (a listing then reads no entry beyond the size); what earlier, larger

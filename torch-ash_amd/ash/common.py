@@ -613,28 +613,33 @@ class _Backend:
                 )
 
     # -- value rows by index (ash/hashmap.py:87-95,138-146) -------------------
-    def gather_rows(self, tables: Dict[str, torch.Tensor], indices: torch.Tensor) -> Dict[str, torch.Tensor]:
+    def gather_rows(self, tables: Dict[str, torch.Tensor], indices: Optional[torch.Tensor],
+                    first: int = 0) -> Dict[str, torch.Tensor]:
         """{name: table[indices]} for value tables on a HIP device, four tables
-        per launch.  Tables the kernel does not take (rows that are not a
-        multiple of 4 bytes, non-contiguous storage) are indexed by torch."""
+        per launch; with indices None, {name: copy of table[:first]}.  Tables
+        the kernel does not take (rows that are not a multiple of 4 bytes,
+        non-contiguous storage) are indexed by torch."""
         out: Dict[str, torch.Tensor] = {}
         batch = []
-        indices = indices.reshape(-1)
-        n = indices.shape[0]
+        if indices is not None:
+            indices = indices.reshape(-1)
+        n = indices.shape[0] if indices is not None else int(first)
         for name, table in tables.items():
             row_bytes = (table.numel() // max(table.shape[0], 1)) * table.element_size()
             fits = (table.is_cuda and table.is_contiguous() and table.shape[0] > 0
-                    and row_bytes % 4 == 0 and row_bytes > 0 and indices.device == table.device
-                    and indices.dtype == torch.int64 and not table.requires_grad)
+                    and row_bytes % 4 == 0 and row_bytes > 0 and not table.requires_grad
+                    and (indices is None
+                         or (indices.device == table.device and indices.dtype == torch.int64)))
             if not fits:
-                out[name] = table[indices]
+                out[name] = table[indices] if indices is not None else table[:n].clone()
                 continue
             out[name] = torch.empty((n,) + tuple(table.shape[1:]), dtype=table.dtype,
                                     device=table.device)
             batch.append((table, out[name], row_bytes))
-        indices = indices.contiguous()
-        for first in range(0, len(batch), 4):
-            part = batch[first:first + 4]
+        if indices is not None:
+            indices = indices.contiguous()
+        for start in range(0, len(batch), 4):
+            part = batch[start:start + 4]
             if n == 0:
                 break
             k = len(part)
@@ -644,8 +649,9 @@ class _Backend:
             c_count = (_I64 * k)(*[t.shape[0] for t, _, _ in part])
             dev = part[0][0].device
             with torch.cuda.device(dev):
-                self.check(self.lib.ash_gather_rows(k, c_src, c_dst, c_rows, c_count,
-                                                    indices.data_ptr(), n, _stream_of(dev)))
+                self.check(self.lib.ash_gather_rows(
+                    k, c_src, c_dst, c_rows, c_count,
+                    indices.data_ptr() if indices is not None else None, n, _stream_of(dev)))
         return {name: out[name] for name in tables}
 
     # -- trilinear queries (ash/src/pybind.cpp:25-29) ---------------------

@@ -166,7 +166,11 @@ class HashMap(ASHModule):
             # is a copy of the first rows
             assert return_indices or return_values
             n = indices.shape[0]
-            rows = self._layout.declared({name: v[:n].clone() for name, v in self.values.items()})
+            gather = getattr(core.backend, "gather_rows", None)
+            if gather is not None:
+                rows = self._layout.declared(gather(self.values, None, first=n))   # one launch
+            else:
+                rows = self._layout.declared({name: v[:n].clone() for name, v in self.values.items()})
             return (keys, indices, rows) if return_indices else (keys, rows)
         return self._answer(keys, indices, return_indices, return_values)
 
