@@ -1352,7 +1352,7 @@ __device__ __forceinline__ void gather_plane(const uint32_t* __restrict__ src,
         const uint32_t q = static_cast<uint32_t>(t - row * rd);
         const int64_t from = indices[row];
         // an index outside the source reads as zero instead of faulting
-        dst[t] = (from >= 0 && from < src_rows) ? src[from * rd + q] : 0u;
+        __builtin_nontemporal_store((from >= 0 && from < src_rows) ? src[from * rd + q] : 0u, dst + t);
     }
 }
 
