@@ -671,7 +671,13 @@ __global__ __launch_bounds__(kBuildThreads) void erase_range_kernel(MapDev m, Bu
         const int r = k * kBuildThreads + tid;
         codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
     }
-    for (int t = tid; t < nbk * kGroup; t += kBuildThreads) tab[staged(t >> 3, t & 7)] = gl[t];
+    {
+        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+        for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
+            const v4u x = __builtin_nontemporal_load(reinterpret_cast<const v4u*>(gl) + t);
+            tab[staged(t >> 3, t & 7)] = make_uint4(x.x, x.y, x.z, x.w);
+        }
+    }
     if (tid == 0) s_tombs = 0;
     __syncthreads();
 
@@ -752,7 +758,14 @@ __global__ __launch_bounds__(kBuildThreads) void erase_range_kernel(MapDev m, Bu
         __syncthreads();
     }
     if (!__syncthreads_or(changed ? 1 : 0)) return;
-    for (int t = tid; t < nbk * kGroup; t += kBuildThreads) gl[t] = tab[staged(t >> 3, t & 7)];
+    {
+        typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+        for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
+            const uint4 x = tab[staged(t >> 3, t & 7)];
+            const v4u y = {x.x, x.y, x.z, x.w};
+            __builtin_nontemporal_store(y, reinterpret_cast<v4u*>(gl) + t);
+        }
+    }
     if (tid == 0 && s_tombs) atomicAdd(m.ctr + kCtrTombs, s_tombs);
 }
 
