@@ -5,6 +5,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
 from ash import common
@@ -44,9 +45,10 @@ def _error(lib):
 def test_workspace_sizes(lib):
     table, general = ctypes.c_int64(0), ctypes.c_int64(0)
     assert lib.ash_map_workspace_bytes(3, 24_000_000, ctypes.byref(table), ctypes.byref(general)) == 0
-    # 256-byte header + one 128-byte bucket per 6 entries of capacity + the key
-    # log (8 bytes per entry, in 16-byte units, 256-byte aligned)
-    assert table.value == 256 + 4_000_000 * 128 + 24_000_000 * 8
+    # 256-byte header + one 128-byte bucket per 6 entries of capacity, rounded up
+    # to whole probe ranges of 512 buckets, + the key log (8 bytes per entry, in
+    # 16-byte units, 256-byte aligned)
+    assert table.value == 256 + 4_000_256 * 128 + 24_000_000 * 8
     assert general.value == 2**26 * 20  # next power of two >= 2 * capacity, 20 B per slot
     assert lib.ash_map_workspace_bytes(1, 1, ctypes.byref(table), ctypes.byref(general)) == 0
     assert table.value == 256 + 2 * 128 + 16
@@ -55,6 +57,52 @@ def test_workspace_sizes(lib):
         assert "key_dim" in _error(lib)
     assert lib.ash_map_workspace_bytes(3, 0, ctypes.byref(table), ctypes.byref(general)) != 0
     assert "capacity" in _error(lib)
+
+
+def _buckets(lib, capacity):
+    table = ctypes.c_int64(0)
+    assert lib.ash_map_workspace_bytes(3, capacity, ctypes.byref(table), None) == 0
+    log_bytes = (capacity + 1) // 2 * 16
+    return (table.value - log_bytes - 256) // 128   # (the log starts 256-byte aligned)
+
+
+def _mix64(h):
+    h = h ^ (h >> np.uint64(33))
+    h = h * np.uint64(0xFF51AFD7ED558CCD)
+    h = h ^ (h >> np.uint64(33))
+    h = h * np.uint64(0xC4CEB9FE1A85EC53)
+    return h ^ (h >> np.uint64(33))
+
+
+@pytest.mark.parametrize("capacity", [3078, 6150, 122_886, 1_000_000])
+def test_tables_of_several_probe_ranges_have_whole_ranges(lib, capacity):
+    """A probe never leaves its aligned range of 512 buckets, and the hash
+    spreads keys evenly over all buckets: a short last range (capacity 3078 used
+    to get 513 buckets, i.e. a last range of one bucket) would overflow while
+    the heap still has indices.  The bucket count is a multiple of 512 beyond
+    one range, and with the table's hash no range of a map filled to capacity
+    with distinct keys comes near its 5120 slots."""
+    nb = _buckets(lib, capacity)
+    assert nb >= (capacity + 5) // 6
+    assert nb % 512 == 0
+    worst = 0
+    with np.errstate(over="ignore"):
+        for seed in range(20):
+            rng = np.random.default_rng(seed)
+            codes = np.unique(rng.integers(0, 1 << 62, size=capacity + capacity // 8,
+                                           dtype=np.uint64))[:capacity]
+            rng.shuffle(codes)
+            # bucket = high 32 bits of (high 32 bits of the mixed code x nb)
+            bucket = ((_mix64(codes) >> np.uint64(32)) * np.uint64(nb)) >> np.uint64(32)
+            per_range = np.bincount((bucket >> np.uint64(9)).astype(np.int64), minlength=nb // 512)
+            worst = max(worst, int(per_range.max()))
+    assert worst <= 3072 + 10 * 56 < 5120
+
+
+def test_small_tables_are_one_probe_range(lib):
+    for capacity in (1, 100, 3072):
+        assert _buckets(lib, capacity) in (max(2, (capacity + 5) // 6), max(2, (capacity + 5) // 6) + 1)
+        assert _buckets(lib, capacity) <= 513
 
 
 def test_create_rejects_bad_buffers_without_a_device(lib):

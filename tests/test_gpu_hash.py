@@ -433,6 +433,28 @@ def test_overflow_drops_and_warns(gpu_ash):
     assert bool(engine.find(keys[~mask][:300])[1].all())
 
 
+@pytest.mark.parametrize("capacity", [3078, 6150, 122_886])
+def test_maps_just_beyond_whole_probe_ranges_fill_to_capacity(gpu_ash, monkeypatch, capacity):
+    """Capacities whose bucket count is one bucket (or a few) beyond a multiple
+    of the probe range: every distinct key up to the capacity is stored, as in
+    the reference, whose map holds `capacity` keys.  Per-key and streaming
+    insert, several key sets."""
+    for seed, policy in ((0, "never"), (1, "never"), (2, "always"), (3, "always")):
+        g = torch.Generator().manual_seed(900 + seed)
+        keys = torch.unique(torch.randint(-2000, 2000, (capacity * 2, 3), generator=g,
+                                          dtype=torch.int32), dim=0)
+        keys = keys[torch.randperm(len(keys), generator=g)][:capacity].to(DEV)
+        assert len(keys) == capacity
+        engine = gpu_ash.ASHEngine(3, capacity, DEV)
+        monkeypatch.setattr(gpu_ash.common, "BULK_INSERT", policy)
+        engine.insert_keys(keys)
+        status = engine.backend.status()
+        assert status["dropped"] == 0 and status["size"] == capacity, (capacity, seed, status)
+        idx, mask = engine.find(keys)
+        assert bool(mask.all())
+        assert_is_bijection_into(idx, capacity)
+
+
 def test_erase_insert_cycles_at_full_load(gpu_ash, oracle):
     """Buckets that have been full keep tombstones; lookups of keys pushed to a
     following bucket must keep working through many cycles."""

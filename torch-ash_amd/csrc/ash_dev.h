@@ -49,9 +49,10 @@ constexpr uint64_t kTomb = ~0ull - 1ull;
 // The streaming insert builds one such range per workgroup in LDS, and a range
 // is what a key's neighbours in the table share in the caches.  At the table's
 // load (six entries per ten-slot bucket at capacity) a range that is full is
-// out of reach (its 5120 slots against a mean of 3072 entries with a standard
-// deviation of 55); a key that finds its range full is refused and counted
-// like a key that finds the heap exhausted.
+// out of reach (its 5120 slots against a mean of at most 3072 entries with a
+// standard deviation of 55; every range of a table with several is a whole
+// one, see num_buckets); a key that finds its range full is refused and
+// counted like a key that finds the heap exhausted.
 constexpr int kPartShift = 9;
 constexpr uint32_t kPartBuckets = 1u << kPartShift;
 
@@ -93,9 +94,17 @@ struct MapDev {
     int32_t capacity;
 };
 
+// A table of more than one probe range consists of whole ranges: a short last
+// range would receive a full bucket's share of the keys per bucket like every
+// other and, having few slots, could fill up (and refuse keys) while the heap
+// still has indices.  A table of at most kPartBuckets buckets is one range.
 inline int64_t num_buckets(int64_t capacity) {
     int64_t nb = (capacity + kTargetFill - 1) / kTargetFill;
-    return nb < 2 ? 2 : nb;
+    if (nb < 2) nb = 2;
+    if (nb > static_cast<int64_t>(kPartBuckets)) {
+        nb = (nb + kPartBuckets - 1) & ~static_cast<int64_t>(kPartBuckets - 1);
+    }
+    return nb;
 }
 
 // Byte offset of the key log inside the table workspace.

@@ -74,8 +74,8 @@ __device__ __forceinline__ uint32_t bucket_of(uint64_t code, uint32_t nb) {
 }
 
 // The bucket after b in b's probe sequence: the next one of b's aligned range
-// of kPartBuckets buckets, wrapping inside that range (the table's last range
-// may be shorter).  A sequence visits at most kPartBuckets buckets.
+// of kPartBuckets buckets, wrapping inside that range (a table of fewer
+// buckets is one shorter range).  A sequence visits at most kPartBuckets buckets.
 __device__ __forceinline__ uint32_t next_bucket(uint32_t b, uint32_t nb) {
     const uint32_t n = b + 1;
     return ((n & (kPartBuckets - 1)) == 0 || n == nb) ? (b & ~(kPartBuckets - 1)) : n;
