@@ -110,7 +110,42 @@ MEASURED_COUNTERS = {
 }
 
 
-def attach_counters(kernels):
+# The figures above were not measured by the run that prints them: they come
+# from separate rocprofv3 --pmc runs (counters cannot be collected together with
+# timings) whose summaries are the files below, taken on the kernel sources with
+# the fingerprint below.  A run on other kernel sources, or at other sizes, does
+# not attach them (`traffic` is then null).
+COUNTERS_SOURCE = {
+    "profiles": ["profiles/bench_hbm_traffic_pmc.md",
+                 "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
+    "csrc_sha256": "unset",
+}
+
+
+def csrc_fingerprint() -> str:
+    """SHA-256 over the kernel sources of libash_hip.so (names and contents)."""
+    import hashlib
+
+    csrc = os.path.join(ROOT, "torch-ash_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def attach_counters(kernels, default_sizes: bool):
+    """Adds the separately collected counter figures to the kernel entries when
+    they describe this run; returns what the JSON line says about them."""
+    current = csrc_fingerprint()
+    note = dict(COUNTERS_SOURCE, measured_in_this_run=False, csrc_sha256_of_this_run=current)
+    note["attached"] = bool(default_sizes and current == COUNTERS_SOURCE["csrc_sha256"])
+    if not note["attached"]:
+        note["why_not"] = ("other sizes than the counters were collected at" if not default_sizes
+                           else "the kernel sources changed since the counters were collected")
+        return note
     for name, (traffic, hit_rate, atomics) in MEASURED_COUNTERS.items():
         entry = kernels.get(name)
         if not isinstance(entry, dict) or "ms" not in entry:
@@ -118,7 +153,8 @@ def attach_counters(kernels):
         entry["traffic"] = traffic
         entry["l2_hit_rate"] = hit_rate
         entry["atomic_requests"] = atomics
-        entry["atomic_requests_per_s"] = round(atomics / (entry["ms"] * 1e-3)) if entry["ms"] else 0
+        entry["counters_from"] = "separate rocprofv3 --pmc runs, see `counters`"
+    return note
 
 
 def items_bytes(scanned: int, n: int) -> int:
@@ -152,6 +188,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-keys", type=int, default=0,
                     help="CPU baseline size (0 = the configuration itself: --keys into --capacity)")
+    ap.add_argument("--csrc-fingerprint", action="store_true",
+                    help="print the fingerprint of the kernel sources (COUNTERS_SOURCE) and exit")
     ap.add_argument("--calibrate", action="store_true",
                     help="run a 1 GiB device copy first (reference point for HBM counters)")
     return ap.parse_args()
@@ -271,6 +309,29 @@ def bench_hash(torch, ash, workloads, args, dev):
     assert keys_out.shape[0] == n
     hits = int(masks.sum())
     ms_per_step = elapsed / args.steps * 1e3
+
+    # The same step with one key erased and put back after the insert: the
+    # heap is no longer 0, 1, 2, ..., so the listing goes by ranks, the value
+    # rows are gathered by index and the next clear rewrites heap and key log
+    # -- the general case of which the step above is the best one.
+    def step_after_erase():
+        hm.clear()
+        hm.insert(w["keys"], values)
+        hm.erase(w["keys"][:1])
+        hm.insert(w["keys"][:1], {name: rows[:1] for name, rows in values.items()})
+        masks, indices = hm.find(w["query_keys"])
+        return hm.items(return_indices=True, return_values=True)
+
+    for _ in range(args.warmup):
+        step_after_erase()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        keys_out, _, _ = step_after_erase()
+    torch.cuda.synchronize()
+    ms_per_step_after_erase = (time.perf_counter() - t0) / args.steps * 1e3
+    assert keys_out.shape[0] == n and not hm.engine.backend.last_items_in_index_order
+    hm.clear()
 
     # Kernel-only timings through the raw C ABI (no host read-back inside).
     backend = hm.engine.backend
@@ -413,6 +474,7 @@ def bench_hash(torch, ash, workloads, args, dev):
     kernels["items"]["Mkeys_per_s"] = round(n / kernels["items"]["ms"] / 1e3, 1)
     del hm, w, workspace, erase_ws
     torch.cuda.empty_cache()
+    kernels["step_after_erase_ms"] = round(ms_per_step_after_erase, 3)
     return ms_per_step, hits, kernels
 
 
@@ -439,7 +501,7 @@ def bench_config1(torch, ash, workloads, dev, reps=5):
         run(t_find, lambda: lib.ash_map_find(handle, queries.data_ptr(), n_q, idx.data_ptr(),
                                              msk.data_ptr(), stream))
     ms_i, ms_f = t_ins.mean_ms(), t_find.mean_ms()
-    unique = hs.size()
+    unique = backend.status()["size"]   # from the device: the launches above went past the shim
     # 38 B per input key: 12 + 16 for every key, 16 + 4 more for the unique half
     out = {
         "insert_keys": roofline_entry("insert_kernel<3,keys> 1 M keys, 50 % duplicates",
@@ -601,33 +663,55 @@ def bench_trilinear(torch, ash, workloads, args, dev):
     out["cfg4_isosurface_points"] = e
     del field, ones, box
 
+    # the module's forward, grid(x): positions -> features in one kernel
+    # (ash_grid_forward); 12 B position + 16 B slot + 8 rows + 1 row out + mask
+    # per live query -- the same 29 + 36 E as the operand-level forward; with
+    # the operands of a backward pass written as well: + 28 B per query
+    t_inf, t_trn = EventTimer(torch), EventTimer(torch)
+    xg = x.clone().requires_grad_(True)
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        with torch.no_grad():
+            run(t_inf, lambda: grid(x, "smooth_step"))
+        run(t_trn, lambda: grid(xg, "smooth_step"))
+    for name, timer, extra in (("cfg4_module_forward", t_inf, 0),
+                               ("cfg4_module_forward_for_training", t_trn, 28)):
+        e = roofline_entry("grid_forward_kernel<f32,E4> (SparseDenseGrid.forward, smooth_step)",
+                           (fwd_bytes(4) + extra) * n_live + (29 + 16 + extra) * masked,
+                           timer.mean_ms())
+        e["Mqueries_per_s"] = round(n4 / e["ms"] / 1e3, 1)
+        out[name] = e
+    del xg
+
     # module-level training step: value loss + gradient-norm loss
+    # (demo/train_scene_recon.py:326-341)
     xq = x.clone().requires_grad_(True)
 
-    def train_step():
+    def train_step(contract):
         grid.embeddings.grad = None
         feats, _ = grid(xq, "smooth_step")
         (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
         loss = (feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
-        loss.backward()
+        if contract:
+            with ash.dense_grad(grid):
+                loss.backward()
+        else:
+            loss.backward()
 
-    # as shipped every backward node fills a dense gradient of its own (the
-    # reference's behaviour); ash.grid_query.SHARE_DENSE_GRADIENT lets the nodes
-    # of one pass share one
-    step_ms = {}
-    for label, share in (("", False), ("_shared_gradient", True)):
-        ash.grid_query.SHARE_DENSE_GRADIENT = share
+    # plain backward(): every backward node fills a dense gradient of its own
+    # and autograd adds them (the reference's behaviour); inside
+    # `with ash.dense_grad(grid):` the nodes add to embeddings.grad directly
+    for label, contract in (("", False), ("_dense_grad", True)):
         for _ in range(2):
-            train_step()
+            train_step(contract)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(reps):
-            train_step()
+            train_step(contract)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / reps * 1e3
         out["cfg4_module_train_step" + label] = {
             "ms": round(ms, 3), "Mqueries_per_s": round(n4 / ms / 1e3, 1)}
-    ash.grid_query.SHARE_DENSE_GRADIENT = False
     if not args.no_cpu:
         # The CPU baseline runs after every section that is timed with the wall
         # clock: its OpenMP workers keep spinning for a while after a parallel
@@ -780,6 +864,9 @@ def cpu_trilinear(cops, zc, uc, n_sample):
 
 def main():
     args = parse_args()
+    if args.csrc_fingerprint:
+        print(csrc_fingerprint())
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this build has one GPU and the path "
               "has no multi-GPU part; run with --gpus 1", file=sys.stderr)
@@ -812,8 +899,8 @@ def main():
     kernels["cfg1_hashset"] = bench_config1(torch, ash, workloads, dev)
     if not args.no_fusion:
         kernels["cfg5_fusion"] = bench_fusion(torch, ash, workloads, args, dev)
-    if args.keys == 16_000_000 and args.capacity == 24_000_000:
-        attach_counters(kernels)
+    counters_note = attach_counters(
+        kernels, args.keys == 16_000_000 and args.capacity == 24_000_000)
     dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
     table_bytes = (args.capacity + 5) // 6 * 128
@@ -832,6 +919,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3),
+        # the same step once the map has seen an erase (plus one erase and one
+        # one-key insert per step): listing by ranks, value rows by index
+        "ms_per_step_after_erase": kernels.pop("step_after_erase_ms"),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -846,6 +936,7 @@ def main():
             "capacity": args.capacity,
         },
         "roofline": roof,
+        "counters": counters_note,
         "kernels": kernels,
         "ceilings": ceilings,
     }

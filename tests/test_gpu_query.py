@@ -347,26 +347,29 @@ def test_accumulating_gradient_calls(gpu_ash, oracle, dtype):
                                         accumulate_into=start.to(torch.float16))
 
 
-def test_training_step_shares_one_dense_gradient(gpu_ash, oracle, monkeypatch):
+def test_training_step_with_one_dense_gradient(gpu_ash, oracle):
     """In a pass that reaches the embeddings through the first- and the
-    second-order backward, the second node adds to the first one's gradient
-    (ash_query_backward_*_accumulate) instead of filling a dense tensor of its
-    own: same .grad as two separate passes, one accumulating call per pass,
-    also on a second pass into an existing .grad.  Both sides add up the same
-    terms in another order, so they may differ by the rounding of those sums:
-    K_ROUND * eps * sum|terms|, the terms being those of the recorded calls."""
+    second-order backward every node fills a dense gradient of its own, as in
+    the reference (ash/grid_query.py:86-129,209-283); inside
+    `with ash.dense_grad(grid):` both nodes add to `embeddings.grad`
+    (ash_query_backward_*_accumulate) and hand autograd nothing.  Same .grad as
+    two separate passes, also on a second pass into an existing .grad and with
+    a hook that keeps the query node's gradients while a weight-decay term
+    contributes as well (the step of demo/train_scene_recon.py:326-341 with a
+    regulariser).  Both sides add up the same terms in another order, so they
+    may differ by the rounding of those sums: K_ROUND * eps * sum|terms|, the
+    terms being those of the recorded calls."""
     grid = _make_grid(gpu_ash, 4, 4, 2, seed=41, holes=5)
     x = _queries(4, 2, 20_000, seed=42)
     backend = gpu_ash.grid_query.backend
-    monkeypatch.setattr(gpu_ash.grid_query, "SHARE_DENSE_GRADIENT", True)
-    shared_calls, recorded = [], []
+    in_place_calls, recorded = [], []
     reals = {name: getattr(backend, name)
              for name in ("query_backward_forward", "query_backward_backward")}
 
     def spy(name):
         def call(*args, **kwargs):
             if kwargs.get("accumulate_into") is not None:
-                shared_calls.append(name)
+                in_place_calls.append(name)
             if kwargs.get("need_embeddings", True):
                 recorded.append((name, [a.detach().clone() if torch.is_tensor(a) else a for a in args]))
             return reals[name](*args, **kwargs)
@@ -384,9 +387,11 @@ def test_training_step_shares_one_dense_gradient(gpu_ash, oracle, monkeypatch):
                 total += oracle.query_term_sums(u, z, *ops, 4, "smooth_step")["bb_embeddings"]
         return total
 
-    def losses():
+    def losses(hook=None):
         xq = x.clone().requires_grad_(True)
         feats, _ = grid(xq, "smooth_step")
+        if hook is not None:
+            feats.grad_fn.register_hook(hook)
         (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
         return (feats[:, 1:] ** 2).mean(), (gx.norm(dim=-1) - 1).abs().mean()
 
@@ -398,29 +403,70 @@ def test_training_step_shares_one_dense_gradient(gpu_ash, oracle, monkeypatch):
             grid.embeddings.grad = None
             losses()[which].backward()
             expected += grid.embeddings.grad
-        assert shared_calls == []
+        assert in_place_calls == []
         sums = term_sums(recorded)
         assert float(sums.sum()) > 0
         order = dict(rtol=0.0, atol=0.0, eps=2.0**-24)
+        # as shipped, outside a block: every node fills a dense gradient of its own
         grid.embeddings.grad = None
         value, eikonal = losses()
         (value + eikonal).backward()
-        assert len(shared_calls) == 1 and gpu_ash.grid_query.LAST_GRADIENT_PATH == "shared"
-        assert_close_sums(grid.embeddings.grad, expected, sums, what="one pass", **order)
-        value, eikonal = losses()
-        (value + eikonal).backward()
-        assert len(shared_calls) == 2
-        assert_close_sums(grid.embeddings.grad, 2 * expected, 2 * sums, what="two passes", **order)
-        # as shipped (switch off) every node fills a dense gradient of its own
-        monkeypatch.setattr(gpu_ash.grid_query, "SHARE_DENSE_GRADIENT", False)
+        assert in_place_calls == [] and gpu_ash.grid_query.LAST_GRADIENT_PATH == "own"
+        assert_close_sums(grid.embeddings.grad, expected, sums, what="plain", **order)
+        # inside the block: two in-place calls, one .grad tensor
         grid.embeddings.grad = None
-        value, eikonal = losses()
-        (value + eikonal).backward()
-        assert len(shared_calls) == 2 and gpu_ash.grid_query.LAST_GRADIENT_PATH == "own"
-        assert_close_sums(grid.embeddings.grad, expected, sums, what="switch off", **order)
+        with gpu_ash.dense_grad(grid):
+            value, eikonal = losses()
+            (value + eikonal).backward()
+            assert len(in_place_calls) == 2
+            assert gpu_ash.grid_query.LAST_GRADIENT_PATH == "contract"
+            assert_close_sums(grid.embeddings.grad, expected, sums, what="one pass", **order)
+            held = grid.embeddings.grad
+            value, eikonal = losses()
+            (value + eikonal).backward()
+            assert len(in_place_calls) == 4 and grid.embeddings.grad is held
+            assert_close_sums(grid.embeddings.grad, 2 * expected, 2 * sums, what="two passes",
+                              **order)
+        # a hook that keeps the node's gradients + a weight-decay term, inside
+        # the block and outside: the same total
+        decay = grid.embeddings.detach().cpu().double()
+        for inside in (False, True):
+            kept = []
+            grid.embeddings.grad = None
+            value, eikonal = losses(hook=lambda gin, gout: kept.append(gin))
+            loss = value + eikonal + 0.5 * (grid.embeddings ** 2).sum()
+            if inside:
+                with gpu_ash.dense_grad(grid):
+                    loss.backward()
+            else:
+                loss.backward()
+            assert len(kept) >= 1
+            assert len(in_place_calls) == (6 if inside else 4)
+            assert_close_sums(grid.embeddings.grad, expected.cpu().double() + decay,
+                              sums + decay.abs(), what=f"hook + decay, inside={inside}", **order)
     finally:
         for name in reals:
             delattr(backend, name)
+
+
+def test_gradient_paths_on_this_torch(gpu_ash):
+    """Which gradients a backward node computes is decided with one private
+    call of the autograd engine (torch._C._will_engine_execute_node); where it
+    is missing or means something else both gradients are produced (right, but
+    `autograd.grad(y, x, create_graph=True)` then fills and accumulates a dense
+    gradient of the whole parameter that nobody reads).  This pins the
+    behaviour on the torch that is installed."""
+    assert hasattr(torch._C, "_will_engine_execute_node"), torch.__version__
+    grid = _make_grid(gpu_ash, 4, 4, 1, seed=43)
+    xq = _queries(4, 1, 2000, seed=44).requires_grad_(True)
+    feats, _ = grid(xq, "smooth_step")
+    gpu_ash.grid_query.LAST_GRADIENT_PATH = None
+    (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+    assert gpu_ash.grid_query.LAST_GRADIENT_PATH == "skipped", torch.__version__
+    grid.embeddings.grad = None
+    ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()).backward()
+    assert gpu_ash.grid_query.LAST_GRADIENT_PATH == "own", torch.__version__
+    assert grid.embeddings.grad is not None and xq.grad is not None
 
 
 def _config_grid(gpu_ash, embedding_dim, num_blocks=3000, sparse=64):
@@ -480,19 +526,41 @@ def test_config4_full_size_against_oracle(gpu_ash, oracle):
     # each query's weights add up to 1 within a few eps; K_ROUND eps sum|z| covers
     # that and the accumulation
     assert bool(((got - total).abs() <= K_ROUND * 2.0**-24 * magnitude).all()), (got, total)
+    # the module's forward (one kernel from positions to features) at this size
+    y = gpu_ash.grid_query.backend.query_forward(*ops, 8, "smooth_step")
+    feats, masks = grid(x, "smooth_step")
+    assert torch.equal(masks, ops[4]) and torch.equal(feats, y)
 
 
-def test_full_size_forward_properties(gpu_ash):
-    """Configuration 3 at full size (200 k blocks, E = 16, 4.4 M queries),
-    through properties that need no oracle: linearity in the embeddings,
-    constants reproduced where all 8 corners exist, masked rows zero."""
+def test_config3_full_size_against_oracle(gpu_ash, oracle):
+    """Configuration 3 at full size (200 k blocks of 8^3 cells, E = 16: 1.64 G
+    embedding values, 4.4 M queries of which a tenth in empty space): forward
+    with both interpolations against the oracle (ash/src/grid.cu:68-132) at the
+    fp32 tolerance -- this is the shape at which row numbers times the row
+    width pass 2^31 elements -- the module's fused forward bit for bit against
+    the two calls, and properties that need no oracle: linearity in the
+    embeddings, constants reproduced where all 8 corners exist, masked rows
+    zero."""
     grid, _, _ = workloads.build_grid(gpu_ash, device=DEV)
     x = workloads.uniform_queries(grid)
+    assert grid.embeddings.shape == (200_000, 512, 16) and x.shape[0] == 4_400_000
     ops = list(_operands(grid, grid.transform_world_to_cell(x)))
+    assert int(ops[2].max()) * 512 * 16 > 2**31     # rows beyond 2^31 elements are addressed
     backend = gpu_ash.grid_query.backend
-    y1 = backend.query_forward(*ops, 8, "smooth_step")
+    cops = _to_cpu(ops)
     masks = ops[4]
-    assert float(y1[~masks].abs().sum()) == 0.0
+    assert 0.85 < float(masks.float().mean()) < 0.95
+    for interpolation in ("linear", "smooth_step"):
+        y = backend.query_forward(*ops, 8, interpolation)
+        y_ref = oracle.query_forward(*cops, 8, interpolation)
+        assert torch.allclose(y.cpu(), y_ref, rtol=RTOL32, atol=ATOL32), (
+            interpolation, float((y.cpu() - y_ref).abs().max()))
+        assert float(y[~masks].abs().sum()) == 0.0
+        feats, m2 = grid(x, interpolation)
+        assert torch.equal(m2, masks) and torch.equal(feats, y), interpolation
+        del y_ref, feats
+    del cops
+    y1 = backend.query_forward(*ops, 8, "smooth_step")
     emb = ops[0]
     ops[0] = emb * 3.0
     y3 = backend.query_forward(*ops, 8, "smooth_step")
@@ -504,6 +572,78 @@ def test_full_size_forward_properties(gpu_ash):
     assert bool((complete <= masks).all())
     assert float(complete.float().mean()) > 0.7
     assert torch.allclose(yc[complete], torch.ones_like(yc[complete]), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("grid_dim,embedding_dim", [(1, 3), (2, 1), (3, 5), (8, 4), (8, 8), (8, 16), (16, 2)])
+def test_fused_forward_equals_query_then_interpolation(gpu_ash, oracle, monkeypatch, dtype,
+                                                       grid_dim, embedding_dim):
+    """`SparseDenseGrid.forward` through ash_grid_forward (positions -> features
+    in one kernel) against `query` followed by `query_forward`
+    (ash/grid.py:201-238), bit for bit: features, masks and -- when a backward
+    pass will want them -- block indices, cell indices and offsets; positions
+    inside, outside and right on block boundaries, run-ordered and shuffled;
+    against the oracle at the stated tolerance; and the gradients that flow
+    through either formulation."""
+    grid = _make_grid(gpu_ash, grid_dim, embedding_dim, 2, dtype=dtype,
+                      seed=7 * grid_dim + embedding_dim, holes=9)
+    g = torch.Generator().manual_seed(70 + grid_dim)
+    span = grid_dim * 3.5
+    rand = (torch.rand(30_011, 3, generator=g) * 2 - 1) * span
+    # runs of positions inside one block, as samples along a ray come
+    walk = (torch.rand(300, 1, 3, generator=g) * 2 - 1) * span * 0.6 + \
+        torch.linspace(0, 1, 40).view(1, 40, 1) * (torch.rand(300, 1, 3, generator=g) - 0.5) * grid_dim
+    ints = torch.randint(-3 * grid_dim, 3 * grid_dim + 1, (1000, 3), generator=g).float()
+    edge = torch.tensor([[-1e-9, 0.0, 0.0], [-1e-9, -1e-9, -1e-9], [grid_dim - 1e-7, 0.5, 0.5],
+                         [-0.0, 0.0, -1e-30], [1e-7 - grid_dim, 0.25, 0.75]])
+    x = torch.cat([rand, walk.reshape(-1, 3), ints, edge]).to(DEV)
+    backend = gpu_ash.grid_query.backend
+    tables = (grid.lut_grid_nb2grid_idx, grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)
+    emb = grid.embeddings.detach()
+    gi, ci, off, masks = grid.query(x)
+    for interpolation in ("linear", "smooth_step"):
+        y = backend.query_forward(emb, off, gi, ci, masks, *tables, grid_dim, interpolation)
+        y_ref = oracle.query_forward(emb.cpu(), off.cpu(), gi.cpu(), ci.cpu(), masks.cpu(),
+                                     *[t.cpu() for t in tables], grid_dim, interpolation)
+        assert torch.allclose(y.cpu(), y_ref, **_tol(dtype))
+        # inference: nothing but features and masks is produced
+        f0, m0, none_gi, none_ci, none_off = backend.grid_forward(
+            grid.engine.backend, x, emb, *tables, grid_dim, interpolation, need_operands=False)
+        assert none_gi is None and none_ci is None and none_off is None
+        assert torch.equal(f0, y) and torch.equal(m0, masks)
+        # with the operands of the backward pass
+        f1, m1, gi1, ci1, off1 = backend.grid_forward(
+            grid.engine.backend, x, emb, *tables, grid_dim, interpolation)
+        assert torch.equal(f1, y) and torch.equal(m1, masks)
+        assert torch.equal(gi1, gi) and torch.equal(ci1, ci) and torch.equal(off1, off)
+        assert gi1.dtype == torch.int64 and off1.dtype == torch.float32 and m1.dtype == torch.bool
+        # through the module, with and without gradients, both formulations
+        results = {}
+        for fused in (True, False):
+            monkeypatch.setattr(gpu_ash.grid, "FUSED_FORWARD", fused)
+            with torch.no_grad():
+                f2, m2 = grid(x, interpolation)
+            assert torch.equal(f2, y) and torch.equal(m2, masks)
+            xq = x.clone().requires_grad_(True)
+            grid.embeddings.grad = None
+            feats, m3 = grid(xq, interpolation)
+            assert torch.equal(feats.detach(), y) and torch.equal(m3, masks)
+            assert not m3.requires_grad
+            weights = torch.linspace(0.5, 1.5, embedding_dim, device=DEV, dtype=dtype)
+            (gx,) = torch.autograd.grad((feats * weights).sum(), xq, create_graph=True)
+            ((feats ** 2).sum() + (gx ** 2).sum()).backward()
+            results[fused] = (gx.detach(), xq.grad.clone(), grid.embeddings.grad.clone())
+        assert torch.equal(results[True][0], results[False][0])
+        assert torch.equal(results[True][1], results[False][1])
+        # the dense gradients are the same sums, accumulated in an order of the
+        # device's own on either side
+        scale = results[False][2].abs().max()
+        assert torch.allclose(results[True][2], results[False][2], rtol=1e-4 if dtype == torch.float32 else 1e-10,
+                              atol=float(scale) * (1e-5 if dtype == torch.float32 else 1e-12))
+    with pytest.raises(RuntimeError, match="grid_dim"):
+        backend.grid_forward(grid.engine.backend, x, emb, *tables, grid_dim + 1, "linear")
+    with pytest.raises(RuntimeError, match="Unknown interpolation"):
+        backend.grid_forward(grid.engine.backend, x, emb, *tables, grid_dim, "cubic")
 
 
 @pytest.mark.parametrize("grid_dim", [1, 3, 8, 16])

@@ -241,15 +241,15 @@ def test_grid_gradcheck_through_autograd_functions(cpu_ash, embedding_dim, grid_
 
 def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
     """A value loss plus a gradient-norm loss reach the embeddings through the
-    first- and the second-order backward in one pass: the second node adds to
-    the first node's gradient instead of producing a dense tensor of its own,
-    and the result is what separate passes give -- also with another user of
-    the embeddings in the loss, on a second pass into an existing .grad, and
-    not at all while a graph of the backward is being recorded.  That is with
-    ash.grid_query.SHARE_DENSE_GRADIENT switched on; as shipped (off) every
-    node produces its own dense gradient, as in the reference, which is also
-    right when a hook keeps a node's gradients while a third contribution
-    arrives (the case the switch cannot see and is off for)."""
+    first- and the second-order backward in one pass.  As shipped every node
+    produces a dense gradient of its own and autograd adds them, as in the
+    reference.  Inside `with ash.dense_grad(grid):` both nodes add to
+    `embeddings.grad` directly and return no gradient: the result is what
+    separate passes give -- also with another user of the embeddings in the
+    loss while a hook keeps a node's gradients (the case an implicit sharing
+    cannot get right), on a second pass into an existing .grad, with a
+    caller's buffer, and not at all while a graph of the backward is being
+    recorded or for tensors that were not registered."""
     import ash.grid_query as gq
 
     torch.manual_seed(7)
@@ -262,13 +262,13 @@ def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
         grid.embeddings.copy_(torch.rand(grid.embeddings.shape) * 2 - 1)
     x = (torch.randint(high=g_dim * 2 - 1, size=(50, 3)) + torch.rand(50, 3).clamp(0.05, 0.95))
 
-    shared_calls = []
+    in_place_calls = []
     for name in ("query_backward_forward", "query_backward_backward"):
         real = getattr(oracle, name)
 
         def spy(*args, _real=real, _name=name, **kwargs):
             if kwargs.get("accumulate_into") is not None:
-                shared_calls.append(_name)
+                in_place_calls.append(_name)
             return _real(*args, **kwargs)
 
         monkeypatch.setattr(oracle, name, spy, raising=False)
@@ -286,81 +286,96 @@ def test_one_dense_gradient_per_backward_pass(cpu_ash, oracle, monkeypatch):
             total += grid.embeddings.grad
         return total
 
-    assert gq.SHARE_DENSE_GRADIENT is False          # as shipped
     expected = separate()
     grid.embeddings.grad = None
     value, eikonal = losses(x.clone().requires_grad_(True))
     (value + eikonal).backward()
-    assert shared_calls == [] and gq.LAST_GRADIENT_PATH == "own"
-    assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
-    # a hook that keeps the gradients of the query node + a third contribution
-    kept = []
-    grid.embeddings.grad = None
-    xq = x.clone().requires_grad_(True)
-    feats, _ = grid(xq, "smooth_step")
-    feats.grad_fn.register_hook(lambda grad_inputs, grad_outputs: kept.append(grad_inputs))
-    (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
-    ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
-     + 0.5 * (grid.embeddings ** 2).sum()).backward()
-    assert shared_calls == [] and len(kept) >= 1
-    assert torch.allclose(grid.embeddings.grad, expected + grid.embeddings.detach(),
-                          rtol=1e-5, atol=1e-6)
-
-    monkeypatch.setattr(gq, "SHARE_DENSE_GRADIENT", True)
-    expected = separate()
-    assert shared_calls == []          # one producer per pass: nothing to share
-
-    grid.embeddings.grad = None
-    value, eikonal = losses(x.clone().requires_grad_(True))
-    (value + eikonal).backward()
-    assert len(shared_calls) == 1 and gq.LAST_GRADIENT_PATH == "shared"
+    assert in_place_calls == [] and gq.LAST_GRADIENT_PATH == "own"
     assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
 
-    # a second pass adds to the existing .grad
-    value, eikonal = losses(x.clone().requires_grad_(True))
-    (value + eikonal).backward()
-    assert len(shared_calls) == 2
-    assert torch.allclose(grid.embeddings.grad, 2 * expected, rtol=1e-5, atol=1e-6)
+    def hooked_step(inside_block):
+        """A hook that keeps the gradients of the query node + a third
+        contribution to the parameter."""
+        kept = []
+        grid.embeddings.grad = None
+        xq = x.clone().requires_grad_(True)
+        feats, _ = grid(xq, "smooth_step")
+        feats.grad_fn.register_hook(lambda grad_inputs, grad_outputs: kept.append(grad_inputs))
+        (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+        loss = ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()
+                + 0.5 * (grid.embeddings ** 2).sum())
+        if inside_block:
+            with cpu_ash.dense_grad(grid):
+                loss.backward()
+        else:
+            loss.backward()
+        assert len(kept) >= 1
+        return grid.embeddings.grad.clone()
 
-    # a regulariser is a third contribution; whether autograd sums it into the
-    # shared tensor or into a new one (which ends the sharing), the total holds
-    grid.embeddings.grad = None
-    value, eikonal = losses(x.clone().requires_grad_(True))
-    (value + eikonal + 0.5 * (grid.embeddings ** 2).sum()).backward()
     want = expected + grid.embeddings.detach()
-    assert torch.allclose(grid.embeddings.grad, want, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(hooked_step(False), want, rtol=1e-5, atol=1e-6)
+    assert in_place_calls == []
+    assert torch.allclose(hooked_step(True), want, rtol=1e-5, atol=1e-6)
+    assert sorted(in_place_calls) == ["query_backward_backward", "query_backward_forward"]
+    assert gq._DENSE_TARGETS == {}          # the block has ended
 
-    # while a graph of the backward pass is recorded nothing is shared
-    before = len(shared_calls)
+    # the plain step inside the block; a second pass adds to the existing .grad
+    del in_place_calls[:]
+    grid.embeddings.grad = None
+    with cpu_ash.dense_grad(grid.embeddings):
+        value, eikonal = losses(x.clone().requires_grad_(True))
+        (value + eikonal).backward()
+        assert len(in_place_calls) == 2 and gq.LAST_GRADIENT_PATH == "contract"
+        assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
+        held = grid.embeddings.grad
+        value, eikonal = losses(x.clone().requires_grad_(True))
+        (value + eikonal).backward()
+        assert len(in_place_calls) == 4 and grid.embeddings.grad is held
+        assert torch.allclose(grid.embeddings.grad, 2 * expected, rtol=1e-5, atol=1e-6)
+
+    # a caller's buffer becomes .grad (zero-filled on entry) when there is none
+    mine = torch.full_like(grid.embeddings, 7.0)
+    grid.embeddings.grad = None
+    with cpu_ash.dense_grad(grid, buffers={grid.embeddings: mine}):
+        assert grid.embeddings.grad is mine and float(mine.abs().max()) == 0.0
+        value, eikonal = losses(x.clone().requires_grad_(True))
+        (value + eikonal).backward()
+    assert grid.embeddings.grad is mine
+    assert torch.allclose(mine, expected, rtol=1e-5, atol=1e-7)
+
+    # while a graph of the backward pass is recorded nothing is added in place
+    before = len(in_place_calls)
     grid.embeddings.grad = None
     value, eikonal = losses(x.clone().requires_grad_(True))
-    (got,) = torch.autograd.grad(value + eikonal, grid.embeddings, create_graph=True)
-    assert len(shared_calls) == before
+    with cpu_ash.dense_grad(grid):
+        (got,) = torch.autograd.grad(value + eikonal, grid.embeddings, create_graph=True)
+    assert len(in_place_calls) == before
     assert torch.allclose(got.detach(), expected, rtol=1e-5, atol=1e-7)
 
-    # two different leaves over the same storage are two consumers
+    # another leaf over the same storage, and a tensor computed from the
+    # parameter, are not the registered parameter: autograd gets their gradients
     grid.embeddings.grad = None
     alias = grid.embeddings.detach().requires_grad_(True)
     tables = (grid.lut_grid_nb2grid_idx, grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb, g_dim)
     gi, ci, off, masks = grid.query(x)
-    before = len(shared_calls)
+    before = len(in_place_calls)
     a = cpu_ash.SparseDenseGridQuery.apply(grid.embeddings, off, gi, ci, masks, *tables)
     b = cpu_ash.SparseDenseGridQuery.apply(alias, off, gi, ci, masks, *tables)
-    (a.sum() + 2 * b.sum()).backward()
-    assert len(shared_calls) == before
+    with cpu_ash.dense_grad(grid):
+        (a.sum() + 2 * b.sum()).backward()
+    assert len(in_place_calls) == before + 1
     assert torch.allclose(alias.grad, 2 * grid.embeddings.grad)
 
-    # a consumer that is not the accumulation node of a leaf is never shared with
     scaled = grid.embeddings * 1.0
-    gi, ci, off, masks = grid.query(x)
     xq = x.clone().requires_grad_(True)
     gi, ci, off, masks = grid.query(xq)
     feats = cpu_ash.SparseDenseGridQuery.apply(scaled, off, gi, ci, masks, *tables, "smooth_step")
     (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
     grid.embeddings.grad = None
-    before = len(shared_calls)
-    ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()).backward()
-    assert len(shared_calls) == before and gq.LAST_GRADIENT_PATH == "own"
+    before = len(in_place_calls)
+    with cpu_ash.dense_grad(grid):
+        ((feats[:, 1:] ** 2).mean() + (gx.norm(dim=-1) - 1).abs().mean()).backward()
+    assert len(in_place_calls) == before and gq.LAST_GRADIENT_PATH == "own"
     assert torch.allclose(grid.embeddings.grad, expected, rtol=1e-5, atol=1e-7)
 
 

@@ -10,7 +10,7 @@ from .embedding import HashEmbedding
 from . import fusion
 from .grid import BoundedSparseDenseGrid, SparseDenseGrid, UnBoundedSparseDenseGrid
 from .grid_nns import enumerate_neighbor_coord_offsets
-from .grid_query import SparseDenseGridQuery, SparseDenseGridQueryBackward
+from .grid_query import SparseDenseGridQuery, SparseDenseGridQueryBackward, dense_grad
 from .hashmap import HashMap, HashSet
 
 __all__ = [
@@ -25,6 +25,7 @@ __all__ = [
     "SparseDenseGridQuery",
     "SparseDenseGridQueryBackward",
     "UnBoundedSparseDenseGrid",
+    "dense_grad",
     "enumerate_neighbor_coord_offsets",
     "fusion",
 ]

@@ -71,6 +71,10 @@ _SIGNATURES = {
         ctypes.c_int,
         [_PTR, _PTR, _I64, ctypes.c_int, _PTR, _PTR, _PTR, _PTR, _PTR],
     ),
+    "ash_grid_forward": (
+        ctypes.c_int,
+        [_PTR, _PTR, ctypes.c_int, ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR, _PTR, _PTR],
+    ),
     "ash_grid_activate": (
         ctypes.c_int,
         [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -740,6 +744,69 @@ class _Backend:
                 self.lib.ash_query_forward(ctypes.byref(args), out.data_ptr(), _stream_of(dev))
             )
         return out
+
+    def grid_forward(
+        self,
+        hashmap,
+        x,
+        embeddings,
+        lut_grid_nb2grid_idx,
+        lut_cell_nb2cell_idx,
+        lut_cell_nb2grid_nb,
+        grid_dim,
+        interpolation,
+        need_operands: bool = True,
+    ):
+        """`SparseDenseGrid.query` and `query_forward` in one kernel: positions x
+        (float32 (N, 3), cell units) -> (features (N, E), masks (N,),
+        grid_indices, cell_indices, offsets).  The last three are what a
+        backward pass needs; with need_operands False they are not produced
+        (None)."""
+        if interpolation not in _INTERPOLATION:
+            raise RuntimeError(f"Unknown interpolation functor: {interpolation}")
+        if embeddings.dtype not in _DTYPE:
+            raise RuntimeError(f"embeddings must be float32 or float64, got {embeddings.dtype}")
+        if embeddings.dim() != 3 or not embeddings.is_contiguous():
+            raise RuntimeError("embeddings must be contiguous (num_embeddings, cells_per_grid, dim)")
+        _require_hip(embeddings, "embeddings")
+        dev = embeddings.device
+        if hashmap.device() != dev:
+            raise RuntimeError(f"the map is on {hashmap.device()}, embeddings on {dev}")
+        if x.dim() != 2 or x.shape[1] != 3 or x.dtype != torch.float32 or x.device != dev:
+            raise RuntimeError("positions must be float32 (N, 3) on the device of the embeddings")
+        x = x.contiguous()
+        b, m, e = embeddings.shape
+        n = x.shape[0]
+
+        def table(t, shape, name):
+            if t.device != dev or t.dtype != torch.int64 or tuple(t.shape) != shape:
+                raise RuntimeError(f"{name} must be int64 {shape} on {dev}")
+            return t.contiguous()
+
+        held = [table(lut_grid_nb2grid_idx, (b, 8), "lut_grid_nb2grid_idx"),
+                table(lut_cell_nb2cell_idx, (m, 8), "lut_cell_nb2cell_idx"),
+                table(lut_cell_nb2grid_nb, (m, 8), "lut_cell_nb2grid_nb")]
+        args = _QueryArgs(embeddings.data_ptr(), None, None, None, None,
+                          *[t.data_ptr() for t in held], n, b, m, e,
+                          _INTERPOLATION[interpolation], _DTYPE[embeddings.dtype])
+        out = torch.empty((n, e), dtype=embeddings.dtype, device=dev)
+        masks = torch.empty(n, dtype=torch.bool, device=dev)
+        grid_indices = cell_indices = offsets = None
+        if need_operands:
+            grid_indices = torch.empty(n, dtype=torch.int64, device=dev)
+            cell_indices = torch.empty(n, dtype=torch.int64, device=dev)
+            offsets = torch.empty((n, 3), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            self.check(
+                self.lib.ash_grid_forward(
+                    hashmap._handle, x.data_ptr(), int(grid_dim), ctypes.byref(args),
+                    out.data_ptr(), masks.data_ptr(),
+                    grid_indices.data_ptr() if need_operands else None,
+                    cell_indices.data_ptr() if need_operands else None,
+                    offsets.data_ptr() if need_operands else None, _stream_of(dev),
+                )
+            )
+        return out, masks, grid_indices, cell_indices, offsets
 
     def query_backward_forward(
         self,

@@ -14,7 +14,7 @@ import torch.nn as nn
 from .common import _get_c_extension
 from .core import ASHEngine, ASHModule
 from .grid_nns import enumerate_neighbor_coord_offsets
-from .grid_query import SparseDenseGridQuery
+from .grid_query import SparseDenseGridQuery, first_order_backward
 from .hashmap import HashSet
 
 backend = _get_c_extension()
@@ -45,6 +45,40 @@ class _FusedCellQuery(torch.autograd.Function):
     @staticmethod
     def backward(ctx, _grad_grid, _grad_cell, grad_offsets, _grad_masks):
         return grad_offsets, None, None
+
+
+# `SparseDenseGrid.forward` through the library's fused kernel (positions ->
+# features in one launch, the intermediate index / offset arrays written only
+# when a backward pass will read them); False = `query` and the interpolation
+# as two calls, as the reference has them.  Same numbers either way.
+FUSED_FORWARD = True
+
+
+class _FusedGridForward(torch.autograd.Function):
+    """(embeddings, x in cell units) -> (features, masks) in one kernel; the
+    operands of the backward pass (block / cell indices, offsets) come out of
+    the same kernel.  Differentiable like `query` followed by
+    `SparseDenseGridQuery`: with respect to the embeddings and, through the
+    offsets (unit Jacobian), to x; the backward is itself differentiable."""
+
+    @staticmethod
+    def forward(ctx, embeddings, x, table, lut_grid_nb2grid_idx, lut_cell_nb2cell_idx,
+                lut_cell_nb2grid_nb, grid_dim, interpolation):
+        features, masks, grid_indices, cell_indices, offsets = backend.grid_forward(
+            table, x, embeddings, lut_grid_nb2grid_idx, lut_cell_nb2cell_idx,
+            lut_cell_nb2grid_nb, grid_dim, interpolation, need_operands=True,
+        )
+        ctx.save_for_backward(embeddings, offsets, grid_indices, cell_indices, masks,
+                              lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb)
+        ctx.grid_dim = grid_dim
+        ctx.interpolation = interpolation
+        ctx.mark_non_differentiable(masks)
+        return features, masks
+
+    @staticmethod
+    def backward(ctx, z, _grad_masks):
+        grad_embeddings, grad_x = first_order_backward(ctx, z, ctx.saved_tensors, 0, 1)
+        return (grad_embeddings, grad_x) + (None,) * 6
 
 
 class SparseDenseGrid(ASHModule):
@@ -216,12 +250,37 @@ class SparseDenseGrid(ASHModule):
         """Embeddings at world positions x (N, 3): features (N, E) and the mask
         of positions that fall into an active block (ash/grid.py:201-238)."""
         x = self.transform_world_to_cell(x)
+        if interpolation not in ("nearest", "linear", "smooth_step"):
+            raise ValueError(f"Unknown interpolation: {interpolation}")
+        table = self.engine.backend
+        if (
+            FUSED_FORWARD
+            and interpolation != "nearest"
+            and hasattr(backend, "grid_forward")
+            and hasattr(table, "query_cells")
+            and x.dtype == torch.float32
+            and x.dim() == 2
+            and len(x) > 0
+            and self.embeddings.is_contiguous()
+        ):
+            if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
+                self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+            tables = (self.lut_grid_nb2grid_idx, self.lut_cell_nb2cell_idx,
+                      self.lut_cell_nb2grid_nb)
+            if torch.is_grad_enabled() and (x.requires_grad or self.embeddings.requires_grad):
+                return _FusedGridForward.apply(self.embeddings, x, table, *tables,
+                                               self.grid_dim, interpolation)
+            # nobody will ask for a gradient: the intermediate arrays are not
+            # even written
+            features, masks, _, _, _ = backend.grid_forward(
+                table, x.detach(), self.embeddings.detach(), *tables, self.grid_dim,
+                interpolation, need_operands=False)
+            return features, masks
+
         grid_indices, cell_indices, offsets, masks = self.query(x)
 
         if interpolation == "nearest":
             return self.embeddings[grid_indices, cell_indices], masks
-        if interpolation not in ("linear", "smooth_step"):
-            raise ValueError(f"Unknown interpolation: {interpolation}")
 
         if self.grid_coords is None or self.lut_grid_nb2grid_idx is None:
             self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)

@@ -3,7 +3,6 @@ backward.  Two chained Functions with the same operands and return
 conventions as the reference (ash/grid_query.py:10-283); each one is a single
 call into the HIP library.
 """
-import os
 import weakref
 from typing import Literal
 
@@ -20,87 +19,101 @@ _N_TABLE_ARGS = 8  # grid_indices .. interpolation: operands without gradients
 # and the second-order backward, and each zero-fills a dense gradient of the
 # whole parameter and leaves the sum of the two to autograd (two fills and an
 # add over the parameter: about a third of such a step), as in the reference.
+# `dense_grad` below is the way around that.
 #
-# SHARE_DENSE_GRADIENT (off unless the caller switches it on, here or with
-# ASH_SHARE_DENSE_GRADIENT=1) saves the second fill and the add: the first node
-# of a pass that produces the gradient for a leaf parameter leaves a note with
-# the parameter's accumulation node -- the graph task, the stream and a weak
-# reference to the tensor, in the node's own metadata dictionary, so that the
-# note lives and dies with the node -- and a later node of the same pass adds its
-# contribution to that tensor in place and returns no gradient of its own.
-#
-# Why it is a switch: the in-place addition is only right while the tensor the
-# first node returned still is what the autograd engine holds for the
-# parameter.  The engine replaces it by a new tensor when a further gradient
-# for the same parameter arrives (a weight-decay term, say) while something
-# else still refers to the first one -- a hook on this function's grad_fn that
-# keeps its grad_inputs is enough -- and this code cannot see that; the later
-# contribution would then be lost.  Without such references the engine adds
-# in place (or autograd drops the tensor and the weak reference dies, and the
-# node falls back to a gradient of its own).  So: switch it on for training
-# loops that keep no references to intermediate gradients.
-#
-# Shared only: with the switch on, without create_graph (an in-place change
-# would be invisible to a graph recorded over the first gradient), towards the
-# accumulation node of a leaf, by nodes that run on the same stream.
-_NOTE = "ash_shared_gradient"
-SHARE_DENSE_GRADIENT = os.environ.get("ASH_SHARE_DENSE_GRADIENT", "0") not in ("", "0")
 # which way the embedding gradient of the latest backward node went: "own"
-# (a dense tensor of its own), "shared" (added to another node's), "skipped"
+# (a dense tensor of its own, handed to autograd), "contract" (added to the
+# parameter's .grad inside a dense_grad block), "skipped" (nobody asked for it)
 LAST_GRADIENT_PATH = None
 
 
-def _pass_id() -> int:
-    if not SHARE_DENSE_GRADIENT or torch.is_grad_enabled():
-        return -1
-    try:
-        return torch._C._current_graph_task_id()
-    except Exception:  # older torch
-        return -1
+# ---------------------------------------------------------------------------
+# One dense gradient per step, by contract.
+#
+#     optimizer.zero_grad()
+#     with ash.dense_grad(grid):          # or a Parameter, or several of either
+#         loss.backward()
+#     optimizer.step()
+#
+# Inside the block every backward node of the query adds its contribution for
+# a registered parameter straight into `parameter.grad` (the library's
+# `_accumulate` entries) and hands autograd no gradient for it: one zero fill
+# per step instead of one per node plus autograd's additions over the whole
+# parameter.  On entry a parameter whose `.grad` is None gets a zero-filled
+# one (filled once); an existing `.grad` is accumulated onto, as
+# `loss.backward()` would.  Nothing is handed to the engine and nothing is
+# learnt from it: `.grad` is looked up when a node runs, other contributions to
+# the parameter (a weight-decay term, say) reach the same tensor through
+# autograd's own in-place accumulation, and hooks on other nodes may keep
+# whatever they like.  What differs from plain `backward()`: hooks registered
+# on the parameter itself do not see the query's contributions (they bypass
+# its accumulation node), and under `create_graph=True` the block has no
+# effect (an in-place addition would be invisible to the recorded graph).
+# The block is for `loss.backward()`: a `torch.autograd.grad(..)` *with respect
+# to a registered parameter* inside it would find the query's share in `.grad`
+# and not in what it returns (gradients with respect to anything else, the
+# positions for instance, are not affected).
+_DENSE_TARGETS = {}   # id(parameter) -> (weak reference, nesting depth)
 
 
-def _notes(consumer):
-    """(graph task, dictionary of the consumer node, key) or None."""
-    task = _pass_id()
-    if task < 0 or consumer is None or consumer[0] is None:
+class dense_grad:
+    """Context manager: see the comment above.  `targets` are Parameters or
+    modules (every parameter of a module that is an `embeddings` operand of a
+    query is simply one of its parameters).  `buffers` maps a parameter to the
+    tensor to install as its `.grad` when it has none (default: a new one per
+    entry)."""
+
+    def __init__(self, *targets, buffers=None):
+        self.parameters = []
+        for t in targets:
+            if isinstance(t, torch.nn.Module):
+                self.parameters.extend(p for p in t.parameters() if p.requires_grad)
+            elif isinstance(t, torch.Tensor):
+                self.parameters.append(t)
+            else:
+                raise TypeError(f"dense_grad takes parameters or modules, got {type(t)}")
+        self.buffers = buffers or {}
+
+    def __enter__(self):
+        for p in self.parameters:
+            if p.grad is None:
+                given = self.buffers.get(p)
+                if given is not None:
+                    if given.shape != p.shape or given.dtype != p.dtype or given.device != p.device:
+                        raise RuntimeError("dense_grad: a buffer must be like its parameter")
+                    p.grad = given.zero_()
+                else:
+                    p.grad = torch.zeros_like(p, memory_format=torch.contiguous_format)
+            ref, depth = _DENSE_TARGETS.get(id(p), (weakref.ref(p), 0))
+            _DENSE_TARGETS[id(p)] = (ref, depth + 1)
+        return self
+
+    def __exit__(self, *exc):
+        for p in self.parameters:
+            ref, depth = _DENSE_TARGETS[id(p)]
+            if depth <= 1:
+                del _DENSE_TARGETS[id(p)]
+            else:
+                _DENSE_TARGETS[id(p)] = (ref, depth - 1)
+        return False
+
+
+def _dense_target(embeddings):
+    """The `.grad` tensor the running node is to add to, if `embeddings` is a
+    parameter registered by a `dense_grad` block that applies, else None."""
+    if not _DENSE_TARGETS or torch.is_grad_enabled():
         return None
-    node = consumer[0]
-    # only the accumulation node of a leaf: what it receives is added to .grad
-    # and goes nowhere else
-    if type(node).__name__ != "AccumulateGrad":
+    entry = _DENSE_TARGETS.get(id(embeddings))
+    if entry is None or entry[0]() is not embeddings:
         return None
-    try:
-        return task, node.metadata, (_NOTE, consumer[1])
-    except Exception:  # a node without metadata
+    grad = embeddings.grad
+    if grad is None:
+        # somebody dropped it inside the block: start a new one
+        grad = embeddings.grad = torch.zeros_like(embeddings, memory_format=torch.contiguous_format)
+    if (grad.shape != embeddings.shape or grad.dtype != embeddings.dtype
+            or grad.device != embeddings.device or not grad.is_contiguous()):
         return None
-
-
-def _stream_id(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream if t.is_cuda else 0
-
-
-def _shared_gradient(consumer):
-    """The gradient another node of the running pass already produced for
-    `consumer`, or None."""
-    notes = _notes(consumer)
-    if notes is None:
-        return None
-    task, where, key = notes
-    entry = where.get(key)
-    if entry is None or entry[0] != task:
-        return None
-    gradient = entry[2]()
-    if gradient is None or entry[1] != _stream_id(gradient):
-        return None
-    return gradient
-
-
-def _share_gradient(consumer, gradient) -> None:
-    notes = _notes(consumer)
-    if notes is None or gradient is None:
-        return
-    task, where, key = notes
-    where[key] = (task, _stream_id(gradient), weakref.ref(gradient))
+    return grad
 
 
 def _record_path(path: str) -> None:
@@ -165,38 +178,45 @@ class SparseDenseGridQuery(torch.autograd.Function):
     def backward(ctx, z: torch.Tensor):
         """Delegates to SparseDenseGridQueryBackward so that this step is itself
         differentiable (needed for gradient-norm losses)."""
-        need_embeddings, need_offsets = _grad_requested(ctx, 0), _grad_requested(ctx, 1)
-        if not (need_embeddings or need_offsets):
-            return (None,) * (2 + _N_TABLE_ARGS)
-        # The reference always produces both gradients (ash/grid_query.py:104-116);
-        # the dense embedding gradient (zero fill + atomics over the whole
-        # parameter) is skipped when nobody asked for it, e.g. in
-        # autograd.grad(y, x, create_graph=True).
-        consumer = ctx.next_functions[0] if need_embeddings else None
-        shared = _shared_gradient(consumer)
-        _record_path("shared" if shared is not None else "own" if need_embeddings else "skipped")
-        if shared is not None:
-            # no graph is being recorded: the library is called directly
-            _, grad_offsets = backend.query_backward_forward(
-                z.contiguous(),
-                *ctx.saved_tensors,
-                ctx.grid_dim,
-                ctx.interpolation,
-                need_embeddings=True,
-                need_offsets=need_offsets,
-                accumulate_into=shared,
-            )
-            return (None, grad_offsets) + (None,) * _N_TABLE_ARGS
-        grad_embeddings, grad_offsets = SparseDenseGridQueryBackward.apply(
+        return first_order_backward(ctx, z, ctx.saved_tensors) + (None,) * _N_TABLE_ARGS
+
+
+def first_order_backward(ctx, z, operands, embeddings_input: int = 0, offsets_input: int = 1):
+    """(grad_embeddings, grad_offsets) of a forward node whose inputs number
+    `embeddings_input` / `offsets_input` are the embeddings and (what the
+    offsets depend on with unit Jacobian:) the offsets or positions; `operands`
+    = (embeddings, offsets, grid_indices, cell_indices, masks, three tables)."""
+    need_embeddings = _grad_requested(ctx, embeddings_input)
+    need_offsets = _grad_requested(ctx, offsets_input)
+    if not (need_embeddings or need_offsets):
+        return None, None
+    # The reference always produces both gradients (ash/grid_query.py:104-116);
+    # the dense embedding gradient (zero fill + atomics over the whole
+    # parameter) is skipped when nobody asked for it, e.g. in
+    # autograd.grad(y, x, create_graph=True).
+    target = _dense_target(operands[0]) if need_embeddings else None
+    _record_path("contract" if target is not None else "own" if need_embeddings else "skipped")
+    if target is not None:
+        # no graph is being recorded: the library is called directly
+        _, grad_offsets = backend.query_backward_forward(
             z.contiguous(),
-            *ctx.saved_tensors,
+            *operands,
             ctx.grid_dim,
             ctx.interpolation,
-            need_embeddings,
-            need_offsets,
+            need_embeddings=True,
+            need_offsets=need_offsets,
+            accumulate_into=target,
         )
-        _share_gradient(consumer, grad_embeddings)
-        return (grad_embeddings, grad_offsets) + (None,) * _N_TABLE_ARGS
+        return None, grad_offsets
+    grad_embeddings, grad_offsets = SparseDenseGridQueryBackward.apply(
+        z.contiguous(),
+        *operands,
+        ctx.grid_dim,
+        ctx.interpolation,
+        need_embeddings,
+        need_offsets,
+    )
+    return grad_embeddings, grad_offsets
 
 
 class SparseDenseGridQueryBackward(torch.autograd.Function):
@@ -267,10 +287,9 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
         n_rest = _N_TABLE_ARGS + 3  # offsets, tables, grid_dim, interpolation, 2 flags
         if grad_grad_offsets is None or not (need_z or need_embeddings):
             return (None, None) + (None,) * n_rest
-        consumer = ctx.next_functions[1] if need_embeddings else None
-        shared = _shared_gradient(consumer)
-        _record_path("shared" if shared is not None else "own" if need_embeddings else "skipped")
-        if shared is not None:
+        target = _dense_target(ctx.saved_tensors[1]) if need_embeddings else None
+        _record_path("contract" if target is not None else "own" if need_embeddings else "skipped")
+        if target is not None:
             grad_z, _, _ = backend.query_backward_backward(
                 grad_grad_embeddings,
                 grad_grad_offsets,
@@ -279,7 +298,7 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
                 ctx.interpolation,
                 need_z=need_z,
                 need_embeddings=True,
-                accumulate_into=shared,
+                accumulate_into=target,
             )
             return (grad_z, None) + (None,) * n_rest
         if need_z and need_embeddings:
@@ -300,5 +319,4 @@ class SparseDenseGridQueryBackward(torch.autograd.Function):
                 need_z=need_z,
                 need_embeddings=need_embeddings,
             )
-        _share_gradient(consumer, grad_embeddings)
         return (grad_z, grad_embeddings) + (None,) * n_rest

@@ -18,6 +18,7 @@ OUT_DIR = os.path.join(HERE, "ash", "lib")
 OUT = os.path.join(OUT_DIR, "libash_hip.so")
 SOURCES = ["ash_map.hip", "ash_bulk.hip", "ash_query.hip", "ash_fusion.hip", "ash_mesh.hip"]
 HEADERS = [
+    os.path.join(CSRC, "ash_probe.h"),
     os.path.join(CSRC, "ash_dev.h"),
     os.path.join(CSRC, "ash_table.h"),
     os.path.join(CSRC, "ash_mc_table.h"),

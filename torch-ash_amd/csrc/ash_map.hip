@@ -20,7 +20,7 @@
 // (ash/src/hashmap_gpu.cuh:211-232,316-336): a new key takes heap[counter++],
 // an erased key stores its index at heap[--counter]; here the counter is
 // advanced once per 256-thread block instead of once per key.
-#include "ash_table.h"
+#include "ash_probe.h"
 
 #include "../../include/ash_hip.h"
 
@@ -55,18 +55,6 @@ __device__ __forceinline__ uint32_t spread8(uint32_t x) {
     x = (x | (x << 2)) & 0x3333u;
     x = (x | (x << 1)) & 0x5555u;
     return x;
-}
-
-__device__ __forceinline__ unsigned long long* slot_ptr(const MapDev& m,
-                                                        uint32_t b, int s) {
-    return reinterpret_cast<unsigned long long*>(
-            m.buckets + static_cast<size_t>(b) * kBucketQwords + s);
-}
-
-__device__ __forceinline__ int32_t* value_ptr(const MapDev& m, uint32_t b,
-                                              int s) {
-    return reinterpret_cast<int32_t*>(m.buckets) +
-           static_cast<size_t>(b) * kBucketDwords + kValDword0 + s;
 }
 
 // -------------------------------------------------- cooperative probe pass
@@ -151,53 +139,6 @@ __device__ __forceinline__ void probe_pass(const MapDev& m, uint64_t code,
 }
 
 // ------------------------------------------------ general (exotic) region
-template <int DIM>
-__device__ __forceinline__ uint32_t gen_home(const int32_t (&k)[DIM],
-                                             uint32_t gslots) {
-    uint64_t h = 0xcbf29ce484222325ull;
-#pragma unroll
-    for (int d = 0; d < DIM; ++d) {
-        h ^= static_cast<uint32_t>(k[d]);
-        h *= 0x100000001b3ull;
-    }
-    return static_cast<uint32_t>(mix64(h)) & (gslots - 1);
-}
-
-__device__ __forceinline__ int32_t gen_load(const int32_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-template <int DIM>
-__device__ __forceinline__ bool gen_key_equal(const MapDev& m, uint32_t p,
-                                              const int32_t (&k)[DIM]) {
-    bool eq = true;
-#pragma unroll
-    for (int d = 0; d < DIM; ++d) {
-        eq = eq && (gen_load(m.gkeys + static_cast<size_t>(p) * 4 + d) == k[d]);
-    }
-    return eq;
-}
-
-// Returns true and the stored index when the key is present.
-template <int DIM>
-__device__ bool gen_find(const MapDev& m, const int32_t (&k)[DIM],
-                         int32_t& idx, uint32_t& pos) {
-    if (m.gstate == nullptr) return false;
-    const uint32_t mask = m.gslots - 1;
-    uint32_t p = gen_home<DIM>(k, m.gslots);
-    for (uint32_t step = 0; step < m.gslots; ++step) {
-        const int32_t w = gen_load(m.gstate + p);
-        if (w == kGenEmpty) return false;
-        if (w >= 0 && gen_key_equal<DIM>(m, p, k)) {
-            idx = w;
-            pos = p;
-            return true;
-        }
-        p = (p + 1) & mask;
-    }
-    return false;
-}
-
 enum { kGenWon = 0, kGenDup = 1, kGenFull = 2, kGenNoRegion = 3 };
 
 // Claims a slot for an exotic key.  The slot word goes EMPTY -> LOCKED ->
@@ -355,56 +296,6 @@ __device__ __forceinline__ bool find_key_shared(const MapDev& m, const int32_t (
     return found;
 }
 
-// The same look-up by one lane on its own: it reads the ten codes of the key's
-// bucket itself (five 16-byte loads of one 128-byte line).  Far fewer vector
-// instructions per wavefront than the cooperative probe, at the price of one
-// line per lane and load instruction; for kernels whose table is small enough
-// to stay in the caches and that are bound by instructions, not by lines.
-template <int DIM>
-__device__ __forceinline__ bool find_key_alone(const MapDev& m, const int32_t (&k)[DIM],
-                                               bool active, int32_t& res) {
-    static_assert(kSlots == 10, "reads the codes as five 16-byte words");
-    uint64_t code;
-    const bool fits = pack_key<DIM>(k, code);
-    bool pend = active && fits;
-    uint32_t b = bucket_of(code, m.nb);
-    uint32_t steps = 0;
-    res = 0;
-    bool found = false;
-    while (pend) {
-        const uint4* line = reinterpret_cast<const uint4*>(
-                m.buckets + static_cast<size_t>(b) * kBucketQwords);
-        uint4 w[5];
-#pragma unroll
-        for (int r = 0; r < 5; ++r) w[r] = line[r];
-        int slot = -1;
-        bool empty = false;
-#pragma unroll
-        for (int r = 4; r >= 0; --r) {
-            const uint64_t qa = static_cast<uint64_t>(w[r].x) | (static_cast<uint64_t>(w[r].y) << 32);
-            const uint64_t qb = static_cast<uint64_t>(w[r].z) | (static_cast<uint64_t>(w[r].w) << 32);
-            empty = empty || qa == kEmpty || qb == kEmpty;
-            if (qb == code) slot = 2 * r + 1;
-            if (qa == code) slot = 2 * r;
-        }
-        if (slot >= 0) {
-            found = true;
-            res = *value_ptr(m, b, slot);
-            pend = false;
-        } else if (empty) {
-            pend = false;
-        } else {
-            b = next_bucket(b, m.nb);
-            if (++steps >= kPartBuckets) pend = false;
-        }
-    }
-    if (active && !fits) {
-        uint32_t pos;
-        found = gen_find<DIM>(m, k, res, pos);
-    }
-    return found;
-}
-
 template <int DIM>
 __global__ __launch_bounds__(kBlock) void find_kernel(
         MapDev m, const int32_t* __restrict__ keys, int64_t n,
@@ -422,20 +313,13 @@ __global__ __launch_bounds__(kBlock) void find_kernel(
 }
 
 // Fused front end of the sparse-dense grid query (ash/grid.py:183-199): splits a
-// position x (cell units) into block / cell / fractional part and looks the
-// block up, in one pass.  The arithmetic is the reference's torch expression
-// evaluated operation by operation in fp32 (no fused multiply-add, so the
-// results equal the elementwise torch formulation bit for bit):
-//   xs = floor(x / G); xd = x - xs * G; off = xd - floor(xd)
-// with two corrections at block boundaries, where fp32 rounding takes xd out
-// of [0, G): xd < 0 (x / G rounded up to an integer) steps back one block,
-// xd == G (tiny negative x) is cell 0 of the next block.
+// position x (cell units) into block / cell / fractional part (split_axis) and
+// looks the block up (find_block_by_runs), in one pass.
 __global__ __launch_bounds__(kBlock) void grid_query_kernel(
         MapDev m, const float* __restrict__ x, int64_t n, float g, int gi,
         int64_t* __restrict__ grid_idx, int64_t* __restrict__ cell_idx,
         float* __restrict__ off, uint8_t* __restrict__ mask_out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    const int lane = threadIdx.x & 63;
     const bool active = i < n;
     int32_t k[3];
     float o[3];
@@ -443,33 +327,13 @@ __global__ __launch_bounds__(kBlock) void grid_query_kernel(
     int64_t stride = 1;
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
-        const float xv = active ? x[i * 3 + d] : 0.f;
-        float xs = floorf(__fdiv_rn(xv, g));
-        float xd = __fsub_rn(xv, __fmul_rn(xs, g));
-        const float under = xd < 0.f ? 1.f : 0.f;
-        xs = __fsub_rn(xs, under);
-        xd = __fadd_rn(xd, __fmul_rn(under, g));
-        const float spill = xd >= g ? 1.f : 0.f;
-        xs = __fadd_rn(xs, spill);
-        xd = __fsub_rn(xd, __fmul_rn(spill, g));
-        o[d] = __fsub_rn(xd, floorf(xd));
-        k[d] = static_cast<int32_t>(xs);
-        cell += static_cast<int64_t>(static_cast<int32_t>(xd)) * stride;
+        int32_t c;
+        split_axis(active ? x[i * 3 + d] : 0.f, g, k[d], c, o[d]);
+        cell += static_cast<int64_t>(c) * stride;
         stride *= gi;
     }
-    // neighbouring positions (samples along a ray) often stand in the same
-    // block: the first lane of such a run looks the block up, by itself, and
-    // the others take its answer
-    int same = lane > 0;
-#pragma unroll
-    for (int d = 0; d < 3; ++d) same &= __shfl_up(k[d], 1) == k[d];
-    const bool head = !same;
     int32_t res = 0;
-    const bool asked = find_key_alone<3>(m, k, active && head, res);
-    const uint64_t heads = __ballot(head);
-    const int my_head = 63 - __builtin_clzll(heads & (~0ull >> (63 - lane)));
-    const bool found = __shfl(static_cast<int>(asked), my_head) != 0;
-    res = __shfl(res, my_head);
+    const bool found = find_block_by_runs(m, k, active, res);
     if (active) {
         grid_idx[i] = found ? static_cast<int64_t>(res) : 0;
         mask_out[i] = found ? 1 : 0;

@@ -24,7 +24,7 @@
 // are accumulated with hardware floating-point atomics; consecutive queries of
 // a wavefront that hit the same row are summed in registers first and issue
 // one atomic per run (ray-ordered samples produce long runs).
-#include "ash_table.h"
+#include "ash_probe.h"
 
 #include <type_traits>
 
@@ -280,7 +280,17 @@ struct TileStage {
                                                 int64_t tile, Tile* s,
                                                 uint32_t (&row)[8],
                                                 float (&o)[3]) {
-        resolve_rows<LDS>(a, lut, tile * kBlock + threadIdx.x, row, o);
+        fill_from(a, lut, load_inputs(a, tile * kBlock + threadIdx.x), s, row, o);
+    }
+
+    // `in`: what the calling thread's query of the tile brings (read from the
+    // operand arrays, or worked out from a position by the fused front end)
+    static __device__ __forceinline__ void fill_from(const QDev& a,
+                                                     const CellLut& lut,
+                                                     const QueryInputs& in, Tile* s,
+                                                     uint32_t (&row)[8],
+                                                     float (&o)[3]) {
+        resolve_rows<LDS>(a, lut, in, row, o);
         if constexpr (LPQ > 1) {
             __syncthreads();  // previous tile fully consumed
 #pragma unroll
@@ -326,6 +336,47 @@ struct VecOf<double, 1> {
 };
 
 // ------------------------------------------------------------- forward
+// Phase 2 of the forward pass for the query the calling thread serves in pass
+// p of the tile: gather of the eight corner rows, weighted sum, one store.
+template <typename T, int VEC, int LPQ>
+__device__ __forceinline__ void forward_rows(const QDev& a, const T* __restrict__ emb,
+                                             T* __restrict__ out, int64_t q,
+                                             const uint32_t (&row)[8], const float (&o)[3],
+                                             int ch0, bool chv) {
+    using V = typename VecOf<T, VEC>::type;
+    const bool valid = row[0] != kNoRow;
+    alignas(16) T acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = T(0);
+    if (valid && chv) {
+        V e[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            e[c] = *reinterpret_cast<const V*>(
+                    emb + static_cast<int64_t>(row[c]) * a.E + ch0);
+        }
+        AxisTerms<T> t;
+        axis_terms<T, false>(o, a.smooth, t);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const T w = corner_weight<T>(t, c);
+            const T* ev = reinterpret_cast<const T*>(&e[c]);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] += w * ev[v];
+        }
+    }
+    if (q < a.N && chv) {
+        if constexpr (sizeof(V) == 16) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f r4 = {static_cast<float>(acc[0]), static_cast<float>(acc[VEC > 1 ? 1 : 0]),
+                            static_cast<float>(acc[VEC > 2 ? 2 : 0]), static_cast<float>(acc[VEC > 3 ? 3 : 0])};
+            __builtin_nontemporal_store(r4, reinterpret_cast<v4f*>(out + q * a.E + ch0));
+        } else {
+            __builtin_nontemporal_store(acc[0], out + q * a.E + ch0);
+        }
+    }
+}
+
 template <typename T, int VEC, int LPQ, bool LDS>
 __global__ __launch_bounds__(kBlock, LPQ == 1 ? kWavesGather : kWavesWide) void
 query_forward_kernel(
@@ -335,7 +386,6 @@ query_forward_kernel(
     const CellLut lut =
             stage_cell_lut<LDS>(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
     using Stage = TileStage<LPQ, LDS>;
-    using V = typename VecOf<T, VEC>::type;
     const int ch0 = (threadIdx.x % LPQ) * VEC;
     const bool chv = ch0 < a.E;
     const T* __restrict__ emb = static_cast<const T*>(a.emb);
@@ -348,37 +398,84 @@ query_forward_kernel(
 #pragma unroll 1
         for (int p = 0; p < Stage::kPasses; ++p) {
             const int64_t q = Stage::fetch(tile, p, tile_s, row, o);
-            const bool valid = row[0] != kNoRow;
-            alignas(16) T acc[VEC];
+            forward_rows<T, VEC, LPQ>(a, emb, out, q, row, o, ch0, chv);
+        }
+    }
+}
+
+// ------------------------------------------------ forward from positions
+// The module-level forward (ash/grid.py:201-238: `query`, then the
+// interpolation) in one kernel: the front end of ash_grid_query (position ->
+// block / cell / fractional part -> look-up of the block, ash_probe.h) stands
+// where the forward kernel reads a query's operands, so the four intermediate
+// arrays are neither written nor read back on the way to the result -- they are
+// written (once) only for a caller that needs them afterwards: the mask always
+// (the module returns it), block index, cell index and offsets when a backward
+// pass will want them (AUX).
+struct FrontDev {
+    MapDev m;
+    const float* x;      // float32[N, 3], cell units
+    float g;             // cells per block edge
+    int gdim;
+    uint8_t* mask_out;   // [N]
+    int64_t* gidx_out;   // [N]    (AUX)
+    int64_t* cidx_out;   // [N]    (AUX)
+    float* off_out;      // [N, 3] (AUX)
+};
+
+template <bool AUX>
+__device__ __forceinline__ QueryInputs front_inputs(const QDev& a, const FrontDev& f, int64_t q) {
+    const bool active = q < a.N;
+    QueryInputs in;
+    int32_t k[3];
+    int32_t cell = 0, stride = 1;
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) acc[v] = T(0);
-            if (valid && chv) {
-                V e[8];
+    for (int d = 0; d < 3; ++d) {
+        int32_t c;
+        const float xv = active ? __builtin_nontemporal_load(f.x + q * 3 + d) : 0.f;
+        split_axis(xv, f.g, k[d], c, in.o[d]);
+        cell += c * stride;
+        stride *= f.gdim;
+    }
+    int32_t res = 0;
+    const bool found = find_block_by_runs(f.m, k, active, res);
+    in.gi = found ? res : 0;
+    in.ci = cell;
+    in.m = (active && found) ? 1 : 0;
+    if (active) {
+        __builtin_nontemporal_store(in.m, f.mask_out + q);
+        if constexpr (AUX) {
+            __builtin_nontemporal_store(static_cast<int64_t>(in.gi), f.gidx_out + q);
+            __builtin_nontemporal_store(static_cast<int64_t>(cell), f.cidx_out + q);
 #pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    e[c] = *reinterpret_cast<const V*>(
-                            emb + static_cast<int64_t>(row[c]) * a.E + ch0);
-                }
-                AxisTerms<T> t;
-                axis_terms<T, false>(o, a.smooth, t);
-#pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    const T w = corner_weight<T>(t, c);
-                    const T* ev = reinterpret_cast<const T*>(&e[c]);
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] += w * ev[v];
-                }
-            }
-            if (q < a.N && chv) {
-                if constexpr (sizeof(V) == 16) {
-                    typedef float v4f __attribute__((ext_vector_type(4)));
-                    const v4f r4 = {static_cast<float>(acc[0]), static_cast<float>(acc[VEC > 1 ? 1 : 0]),
-                                    static_cast<float>(acc[VEC > 2 ? 2 : 0]), static_cast<float>(acc[VEC > 3 ? 3 : 0])};
-                    __builtin_nontemporal_store(r4, reinterpret_cast<v4f*>(out + q * a.E + ch0));
-                } else {
-                    __builtin_nontemporal_store(acc[0], out + q * a.E + ch0);
-                }
-            }
+            for (int d = 0; d < 3; ++d) __builtin_nontemporal_store(in.o[d], f.off_out + q * 3 + d);
+        }
+    }
+    return in;
+}
+
+template <typename T, int VEC, int LPQ, bool LDS, bool AUX>
+__global__ __launch_bounds__(kBlock, LPQ == 1 ? kWavesGather : kWavesWide) void
+grid_forward_kernel(QDev a, FrontDev f, T* __restrict__ out) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    Tile* tile_s = reinterpret_cast<Tile*>(smem);
+    const CellLut lut =
+            stage_cell_lut<LDS>(a, smem + (LPQ > 1 ? sizeof(Tile) : 0));
+    using Stage = TileStage<LPQ, LDS>;
+    const int ch0 = (threadIdx.x % LPQ) * VEC;
+    const bool chv = ch0 < a.E;
+    const T* __restrict__ emb = static_cast<const T*>(a.emb);
+    const int64_t ntiles = (a.N + kBlock - 1) / kBlock;
+    TileWalk walk(ntiles);
+    for (int64_t tile = walk.next; tile < walk.end; tile += walk.step) {
+        uint32_t row[8];
+        float o[3];
+        Stage::fill_from(a, lut, front_inputs<AUX>(a, f, tile * kBlock + threadIdx.x), tile_s,
+                         row, o);
+#pragma unroll 1
+        for (int p = 0; p < Stage::kPasses; ++p) {
+            const int64_t q = Stage::fetch(tile, p, tile_s, row, o);
+            forward_rows<T, VEC, LPQ>(a, emb, out, q, row, o, ch0, chv);
         }
     }
 }
@@ -1966,7 +2063,9 @@ int zero_fill(void* ptr, int64_t bytes, hipStream_t s) {
 // ones); the kernels keep the plain variant as a template parameter.
 constexpr bool merge_enabled() { return true; }
 
-int check_args(const ash_query_args* a, QDev& d) {
+// `from_positions`: the per-query operand arrays are not read (the fused front
+// end works them out), so they may be NULL.
+int check_args(const ash_query_args* a, QDev& d, bool from_positions = false) {
     if (a == nullptr) ASH_FAIL("null query arguments");
     if (a->num_queries < 0) ASH_FAIL("negative query count");
     if (a->num_embeddings < 1 || a->cells_per_grid < 1) {
@@ -1988,7 +2087,7 @@ int check_args(const ash_query_args* a, QDev& d) {
         a->lut_cell_nb2cell_idx == nullptr || a->lut_cell_nb2grid_nb == nullptr) {
         ASH_FAIL("null table pointer");
     }
-    if (a->num_queries > 0 &&
+    if (a->num_queries > 0 && !from_positions &&
         (a->offsets == nullptr || a->grid_indices == nullptr ||
          a->cell_indices == nullptr || a->masks == nullptr)) {
         ASH_FAIL("null query pointer");
@@ -2061,6 +2160,25 @@ int launch_forward(const QDev& d, void* out, hipStream_t s) {
         query_forward_kernel<T, VEC, LPQ, false>
                 <<<g, kBlock, smem, s>>>(d, static_cast<T*>(out));
     }
+    ASH_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename T, int VEC, int LPQ>
+int launch_grid_forward(const QDev& d, const FrontDev& f, void* out, hipStream_t s) {
+    const size_t smem = smem_bytes(d, LPQ);
+    const unsigned g = persistent_grid((d.N + kBlock - 1) / kBlock, smem);
+    const bool aux = f.gidx_out != nullptr;
+#define ASH_GF(L, A)                                                          \
+    grid_forward_kernel<T, VEC, LPQ, L, A><<<g, kBlock, smem, s>>>(d, f, static_cast<T*>(out))
+    if (lut_in_lds(d)) {
+        if (aux) ASH_GF(true, true);
+        else ASH_GF(true, false);
+    } else {
+        if (aux) ASH_GF(false, true);
+        else ASH_GF(false, false);
+    }
+#undef ASH_GF
     ASH_LAUNCH_CHECK();
     return 0;
 }
@@ -2197,6 +2315,36 @@ int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
     }
 }
 
+// Same choice of variant as dispatch_forward, so that the fused kernel adds up
+// the corner rows in the same order as ash_query_forward on the same operands.
+template <typename T>
+int dispatch_grid_forward(const QDev& d, const FrontDev& f, void* out, hipStream_t s) {
+    if constexpr (sizeof(T) == 4) {
+        if (d.E % 4 == 0 && aligned16(d.emb) && aligned16(out)) {
+            switch (d.E / 4) {
+                case 1:
+                    return launch_grid_forward<float, 4, 1>(d, f, out, s);
+                case 2:
+                    return launch_grid_forward<float, 4, 2>(d, f, out, s);
+                default:
+                    return launch_grid_forward<float, 4, 4>(d, f, out, s);
+            }
+        }
+    }
+    switch (pow2_ceil(d.E)) {
+        case 1:
+            return launch_grid_forward<T, 1, 1>(d, f, out, s);
+        case 2:
+            return launch_grid_forward<T, 1, 2>(d, f, out, s);
+        case 4:
+            return launch_grid_forward<T, 1, 4>(d, f, out, s);
+        case 8:
+            return launch_grid_forward<T, 1, 8>(d, f, out, s);
+        default:
+            return launch_grid_forward<T, 1, 16>(d, f, out, s);
+    }
+}
+
 template <typename T>
 int dispatch_bwd_fwd(const QDev& d, const void* z, void* ge, void* go,
                      hipStream_t s) {
@@ -2256,6 +2404,42 @@ int ash_query_forward(const ash_query_args* a, void* output, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     return a->dtype == ASH_F64 ? dispatch_forward<double>(d, output, s)
                                : dispatch_forward<float>(d, output, s);
+}
+
+int ash_grid_forward(ash_map_t* map, const float* x, int grid_dim,
+                     const ash_query_args* tables, void* output, uint8_t* masks,
+                     int64_t* grid_indices, int64_t* cell_indices, float* offsets,
+                     void* stream) {
+    if (map == nullptr) ASH_FAIL("null map handle");
+    if (map->key_dim != 3) ASH_FAIL("grid queries need a map with 3-d keys");
+    if (grid_dim < 1 || grid_dim > 1024) ASH_FAIL("grid_dim must be in 1..1024");
+    QDev d;
+    if (check_args(tables, d, true)) return 1;
+    if (d.M != static_cast<int64_t>(grid_dim) * grid_dim * grid_dim) {
+        ASH_FAIL("cells_per_grid must be grid_dim^3");
+    }
+    if (d.N > (int64_t{1} << 31) - kBlock) ASH_FAIL("too many positions in one call");
+    if (d.N == 0) return 0;
+    if (x == nullptr || output == nullptr || masks == nullptr) ASH_FAIL("null pointer");
+    const int given = (grid_indices != nullptr) + (cell_indices != nullptr) + (offsets != nullptr);
+    if (given != 0 && given != 3) {
+        ASH_FAIL("grid_indices, cell_indices and offsets are written together: pass all or none");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
+    FrontDev f;
+    f.m = map->d;
+    f.x = x;
+    f.g = static_cast<float>(grid_dim);
+    f.gdim = grid_dim;
+    f.mask_out = masks;
+    f.gidx_out = grid_indices;
+    f.cidx_out = cell_indices;
+    f.off_out = offsets;
+    return tables->dtype == ASH_F64 ? dispatch_grid_forward<double>(d, f, output, s)
+                                    : dispatch_grid_forward<float>(d, f, output, s);
 }
 
 namespace {
