@@ -536,8 +536,7 @@ def test_config3_full_size_against_oracle(gpu_ash, oracle):
     """Configuration 3 at full size (200 k blocks of 8^3 cells, E = 16: 1.64 G
     embedding values, 4.4 M queries of which a tenth in empty space): forward
     with both interpolations against the oracle (ash/src/grid.cu:68-132) at the
-    fp32 tolerance -- this is the shape at which row numbers times the row
-    width pass 2^31 elements -- the module's fused forward bit for bit against
+    fp32 tolerance -- 1.64 G elements, byte offsets beyond 32 bits -- the module's fused forward bit for bit against
     the two calls, and properties that need no oracle: linearity in the
     embeddings, constants reproduced where all 8 corners exist, masked rows
     zero."""
@@ -545,7 +544,7 @@ def test_config3_full_size_against_oracle(gpu_ash, oracle):
     x = workloads.uniform_queries(grid)
     assert grid.embeddings.shape == (200_000, 512, 16) and x.shape[0] == 4_400_000
     ops = list(_operands(grid, grid.transform_world_to_cell(x)))
-    assert int(ops[2].max()) * 512 * 16 > 2**31     # rows beyond 2^31 elements are addressed
+    assert int(ops[2].max()) * 512 * 16 * 4 > 2**32     # byte offsets beyond 32 bits are addressed
     backend = gpu_ash.grid_query.backend
     cops = _to_cpu(ops)
     masks = ops[4]
