@@ -447,10 +447,15 @@ typedef struct ash_query_args {
 int ash_query_forward(const ash_query_args* a, void* output, void* stream);
 
 /* Replaces the linear / smooth_step branch of `SparseDenseGrid.forward`
- * (ash/grid.py:201-238: `query`, ash/grid.py:183-199, then `query_forward`,
- * ash/src/grid.cu:68-175) in one kernel: x float32[N,3] positions in cell
- * units -> output scalar[N, E] and masks uint8/bool[N] (= block is active),
- * bit for bit what ash_grid_query followed by ash_query_forward give.  Of
+ * (ash/grid.py:201-238: world -> cell units, ash/grid.py:753,852, `query`,
+ * ash/grid.py:183-199, then `query_forward`, ash/src/grid.cu:68-175) in one
+ * kernel: x float32[N,3] positions -> output scalar[N, E] and masks
+ * uint8/bool[N] (= block is active).  Positions become cell units as
+ * (x - origin) * (1.0f / cell_size) in fp32 -- what torch computes on the
+ * device for `(x - origin) / cell_size` -- with origin float32[3] on the
+ * device or NULL for none; origin NULL and cell_size 1 leave x as it is, and
+ * the results are then bit for bit what ash_grid_query followed by
+ * ash_query_forward give.  Of
  * `tables` the embeddings, the three neighbour tables, the sizes (num_queries
  * = N, cells_per_grid = grid_dim^3), interpolation and dtype are used; its
  * per-query arrays are not read and may be NULL.  grid_indices int64[N],
@@ -458,8 +463,8 @@ int ash_query_forward(const ash_query_args* a, void* output, void* stream);
  * a later backward pass needs: pass all three to have them written, or three
  * NULLs to skip them (inference).  `map` must have 3-d keys and live on the
  * device of the embeddings. */
-int ash_grid_forward(ash_map_t* map, const float* x, int grid_dim,
-                     const ash_query_args* tables, void* output, uint8_t* masks,
+int ash_grid_forward(ash_map_t* map, const float* x, const float* origin, float cell_size,
+                     int grid_dim, const ash_query_args* tables, void* output, uint8_t* masks,
                      int64_t* grid_indices, int64_t* cell_indices, float* offsets,
                      void* stream);
 

@@ -645,6 +645,48 @@ def test_fused_forward_equals_query_then_interpolation(gpu_ash, oracle, monkeypa
         backend.grid_forward(grid.engine.backend, x, emb, *tables, grid_dim, "cubic")
 
 
+@pytest.mark.parametrize("kind", ["bounded", "unbounded", "user transform"])
+def test_fused_forward_applies_the_world_to_cell_transform(gpu_ash, monkeypatch, kind):
+    """World positions go through `transform_world_to_cell` (ash/grid.py:753,852:
+    `x / cell_size`, `(x - bbox_min) / cell_size`) before the query.  The fused
+    forward applies the class's own transform inside its kernel, with torch's
+    device arithmetic, and calls a transform that a user has assigned: features,
+    masks and the gradients with respect to the world positions equal the
+    formulation in separate calls bit for bit."""
+    if kind == "unbounded":
+        grid = gpu_ash.UnBoundedSparseDenseGrid(3, 4000, 4, 8, cell_size=0.0137, device=DEV)
+        pts = (torch.rand(3000, 3, generator=torch.Generator().manual_seed(3)) * 2 - 1).to(DEV)
+    else:
+        grid = gpu_ash.BoundedSparseDenseGrid(
+            3, 4000, 4, 8, sparse_grid_dim=24,
+            bbox_min=torch.tensor([-0.9, -1.1, -0.7]), bbox_max=torch.tensor([1.3, 0.8, 1.0]),
+            device=DEV)
+        pts = (torch.rand(3000, 3, generator=torch.Generator().manual_seed(4)) * 1.4 - 0.6).to(DEV)
+    if kind == "user transform":
+        grid.transform_world_to_cell = lambda x: (x - grid.bbox_min) * (1.0 / grid.cell_size) + 0.25
+    grid.spatial_init_(pts, dilation=1, bidirectional=True)
+    with torch.no_grad():
+        grid.embeddings.copy_(torch.rand(grid.embeddings.shape, device=DEV) * 2 - 1)
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    assert (grid._world_to_cell_affine(pts) is None) == (kind == "user transform")
+    x = torch.cat([pts + 0.003, pts * 1.7, (torch.rand(5000, 3, device=DEV) * 2 - 1) * 1.2])
+    results = {}
+    for fused in (True, False):
+        monkeypatch.setattr(gpu_ash.grid, "FUSED_FORWARD", fused)
+        with torch.no_grad():
+            f0, m0 = grid(x, "smooth_step")
+        xq = x.clone().requires_grad_(True)
+        grid.embeddings.grad = None
+        feats, masks = grid(xq, "smooth_step")
+        (gx,) = torch.autograd.grad(feats[:, 0].sum(), xq, create_graph=True)
+        ((feats ** 2).sum() + (gx ** 2).sum()).backward()
+        assert torch.equal(f0, feats.detach()) and torch.equal(m0, masks)
+        results[fused] = (f0, m0, gx.detach(), xq.grad.clone())
+    assert 0.2 < float(results[True][1].float().mean()) < 1.0
+    for a, b in zip(results[True], results[False]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("grid_dim", [1, 3, 8, 16])
 def test_fused_cell_query_equals_elementwise_chain(gpu_ash, grid_dim):
     """`SparseDenseGrid.query` through the fused kernel against the reference's

@@ -73,7 +73,8 @@ _SIGNATURES = {
     ),
     "ash_grid_forward": (
         ctypes.c_int,
-        [_PTR, _PTR, ctypes.c_int, ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR, _PTR, _PTR, _PTR],
+        [_PTR, _PTR, _PTR, ctypes.c_float, ctypes.c_int, ctypes.POINTER(_QueryArgs), _PTR, _PTR, _PTR,
+         _PTR, _PTR, _PTR],
     ),
     "ash_grid_activate": (
         ctypes.c_int,
@@ -756,9 +757,12 @@ class _Backend:
         grid_dim,
         interpolation,
         need_operands: bool = True,
+        origin: Optional[torch.Tensor] = None,
+        cell_size: float = 1.0,
     ):
         """`SparseDenseGrid.query` and `query_forward` in one kernel: positions x
-        (float32 (N, 3), cell units) -> (features (N, E), masks (N,),
+        (float32 (N, 3); cell units = (x - origin) / cell_size, evaluated as
+        torch does on the device) -> (features (N, E), masks (N,),
         grid_indices, cell_indices, offsets).  The last three are what a
         backward pass needs; with need_operands False they are not produced
         (None)."""
@@ -775,6 +779,10 @@ class _Backend:
         if x.dim() != 2 or x.shape[1] != 3 or x.dtype != torch.float32 or x.device != dev:
             raise RuntimeError("positions must be float32 (N, 3) on the device of the embeddings")
         x = x.contiguous()
+        if origin is not None:
+            if origin.device != dev or origin.dtype != torch.float32 or origin.numel() != 3:
+                raise RuntimeError("origin must be three float32 on the device of the embeddings")
+            origin = origin.contiguous()
         b, m, e = embeddings.shape
         n = x.shape[0]
 
@@ -799,7 +807,9 @@ class _Backend:
         with torch.cuda.device(dev):
             self.check(
                 self.lib.ash_grid_forward(
-                    hashmap._handle, x.data_ptr(), int(grid_dim), ctypes.byref(args),
+                    hashmap._handle, x.data_ptr(),
+                    origin.data_ptr() if origin is not None else None, float(cell_size),
+                    int(grid_dim), ctypes.byref(args),
                     out.data_ptr(), masks.data_ptr(),
                     grid_indices.data_ptr() if need_operands else None,
                     cell_indices.data_ptr() if need_operands else None,

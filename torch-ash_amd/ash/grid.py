@@ -63,22 +63,27 @@ class _FusedGridForward(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, embeddings, x, table, lut_grid_nb2grid_idx, lut_cell_nb2cell_idx,
-                lut_cell_nb2grid_nb, grid_dim, interpolation):
+                lut_cell_nb2grid_nb, grid_dim, interpolation, origin, cell_size):
         features, masks, grid_indices, cell_indices, offsets = backend.grid_forward(
             table, x, embeddings, lut_grid_nb2grid_idx, lut_cell_nb2cell_idx,
             lut_cell_nb2grid_nb, grid_dim, interpolation, need_operands=True,
+            origin=origin, cell_size=cell_size,
         )
         ctx.save_for_backward(embeddings, offsets, grid_indices, cell_indices, masks,
                               lut_grid_nb2grid_idx, lut_cell_nb2cell_idx, lut_cell_nb2grid_nb)
         ctx.grid_dim = grid_dim
         ctx.interpolation = interpolation
+        ctx.cell_size = cell_size
         ctx.mark_non_differentiable(masks)
         return features, masks
 
     @staticmethod
     def backward(ctx, z, _grad_masks):
         grad_embeddings, grad_x = first_order_backward(ctx, z, ctx.saved_tensors, 0, 1)
-        return (grad_embeddings, grad_x) + (None,) * 6
+        if grad_x is not None and ctx.cell_size != 1.0:
+            # d cell / d x of x -> (x - origin) / cell_size, as autograd has it
+            grad_x = grad_x / ctx.cell_size
+        return (grad_embeddings, grad_x) + (None,) * 8
 
 
 class SparseDenseGrid(ASHModule):
@@ -104,6 +109,7 @@ class SparseDenseGrid(ASHModule):
 
         self.transform_world_to_cell = lambda x: x
         self.transform_cell_to_world = lambda x: x
+        self._remember_world_to_cell(lambda: (None, 1.0))
 
         self.in_dim = in_dim
         self.num_embeddings = num_embeddings
@@ -249,7 +255,6 @@ class SparseDenseGrid(ASHModule):
     ) -> Tuple[torch.Tensor, torch.Tensor]:
         """Embeddings at world positions x (N, 3): features (N, E) and the mask
         of positions that fall into an active block (ash/grid.py:201-238)."""
-        x = self.transform_world_to_cell(x)
         if interpolation not in ("nearest", "linear", "smooth_step"):
             raise ValueError(f"Unknown interpolation: {interpolation}")
         table = self.engine.backend
@@ -267,15 +272,27 @@ class SparseDenseGrid(ASHModule):
                 self.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
             tables = (self.lut_grid_nb2grid_idx, self.lut_cell_nb2cell_idx,
                       self.lut_cell_nb2grid_nb)
-            if torch.is_grad_enabled() and (x.requires_grad or self.embeddings.requires_grad):
+            # world -> cell units inside the kernel when the transform is the
+            # class's own affine one, else by calling it
+            affine = self._world_to_cell_affine(x)
+            if affine is None:
+                x = self.transform_world_to_cell(x)
+                affine = (None, 1.0)
+            if (
+                x.dtype == torch.float32 and torch.is_grad_enabled()
+                and (x.requires_grad or self.embeddings.requires_grad)
+            ):
                 return _FusedGridForward.apply(self.embeddings, x, table, *tables,
-                                               self.grid_dim, interpolation)
-            # nobody will ask for a gradient: the intermediate arrays are not
-            # even written
-            features, masks, _, _, _ = backend.grid_forward(
-                table, x.detach(), self.embeddings.detach(), *tables, self.grid_dim,
-                interpolation, need_operands=False)
-            return features, masks
+                                               self.grid_dim, interpolation, *affine)
+            if x.dtype == torch.float32:
+                # nobody will ask for a gradient: the intermediate arrays are
+                # not even written
+                features, masks, _, _, _ = backend.grid_forward(
+                    table, x.detach(), self.embeddings.detach(), *tables, self.grid_dim,
+                    interpolation, need_operands=False, origin=affine[0], cell_size=affine[1])
+                return features, masks
+        else:
+            x = self.transform_world_to_cell(x)
 
         grid_indices, cell_indices, offsets, masks = self.query(x)
 
@@ -366,6 +383,30 @@ class SparseDenseGrid(ASHModule):
         """Inclusive range of block coordinates `grids_in_bound` lets through
         (all of int32 short of the dilation range when unbounded)."""
         return -(2**31) + 64, 2**31 - 65
+
+    def _remember_world_to_cell(self, affine) -> None:
+        """Notes that `transform_world_to_cell`, as it stands now, is
+        x -> (x - origin) / cell_size with (origin, cell_size) = affine(); while
+        the attribute still holds that function the fused forward applies the
+        transform inside its kernel.  A transform assigned later by a user is
+        simply called."""
+        self._world_to_cell_known = (self.transform_world_to_cell, affine)
+
+    def _world_to_cell_affine(self, like: torch.Tensor):
+        """(origin float32[3] on the device or None, cell_size) if the fused
+        kernel can apply `transform_world_to_cell` to `like` itself, else None."""
+        fn, affine = self._world_to_cell_known
+        if self.transform_world_to_cell is not fn:
+            return None
+        origin, cell_size = affine()
+        if origin is not None and (
+            not torch.is_tensor(origin) or origin.dtype != torch.float32
+            or origin.device != like.device or origin.numel() != 3 or origin.requires_grad
+        ):
+            return None
+        if torch.is_tensor(cell_size) or not (0.0 < float(cell_size) < float("inf")):
+            return None
+        return origin, float(cell_size)
 
     def _cell_to_world_affine(self) -> Tuple[float, Optional[torch.Tensor]]:
         """`transform_cell_to_world` as (scale, origin): world = cell * scale
@@ -715,6 +756,7 @@ class UnBoundedSparseDenseGrid(SparseDenseGrid):
         self.cell_size = cell_size
         self.transform_world_to_cell = lambda x: x / self.cell_size
         self.transform_cell_to_world = lambda x: x * self.cell_size
+        self._remember_world_to_cell(lambda: (None, self.cell_size))
         self._cell_to_world_affine = lambda: (self.cell_size, None)
         self.bbox_min = None
         self.bbox_max = None
@@ -769,6 +811,7 @@ class BoundedSparseDenseGrid(SparseDenseGrid):
         self.cell_size = (extent / (sparse_grid_dim * grid_dim - 1)).min().item()
         self.transform_world_to_cell = lambda x: (x - self.bbox_min) / self.cell_size
         self.transform_cell_to_world = lambda x: x * self.cell_size + self.bbox_min
+        self._remember_world_to_cell(lambda: (self.bbox_min, self.cell_size))
         self._cell_to_world_affine = lambda: (self.cell_size, self.bbox_min)
 
     def grids_in_bound(self, grid_coords: torch.Tensor) -> torch.Tensor:

@@ -30,6 +30,7 @@
 
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
+#include <cmath>
 #include <cstdlib>
 
 #include "../../include/ash_hip.h"
@@ -414,7 +415,9 @@ query_forward_kernel(
 // pass will want them (AUX).
 struct FrontDev {
     MapDev m;
-    const float* x;      // float32[N, 3], cell units
+    const float* x;      // float32[N, 3]; cell units = (x - origin) * inv_cell
+    const float* origin; // float32[3] on the device, or nullptr for none
+    float inv_cell;      // 1 / cell size, rounded to fp32 once
     float g;             // cells per block edge
     int gdim;
     uint8_t* mask_out;   // [N]
@@ -432,7 +435,11 @@ __device__ __forceinline__ QueryInputs front_inputs(const QDev& a, const FrontDe
 #pragma unroll
     for (int d = 0; d < 3; ++d) {
         int32_t c;
-        const float xv = active ? __builtin_nontemporal_load(f.x + q * 3 + d) : 0.f;
+        float xv = active ? __builtin_nontemporal_load(f.x + q * 3 + d) : 0.f;
+        // world -> cell units the way torch evaluates `(x - origin) / cell_size`
+        // on the device: a subtraction, then a multiplication by the fp32
+        // reciprocal of the size (both exact no-ops for origin 0 and size 1)
+        xv = __fmul_rn(__fsub_rn(xv, f.origin != nullptr ? f.origin[d] : 0.f), f.inv_cell);
         split_axis(xv, f.g, k[d], c, in.o[d]);
         cell += c * stride;
         stride *= f.gdim;
@@ -2406,13 +2413,14 @@ int ash_query_forward(const ash_query_args* a, void* output, void* stream) {
                                : dispatch_forward<float>(d, output, s);
 }
 
-int ash_grid_forward(ash_map_t* map, const float* x, int grid_dim,
-                     const ash_query_args* tables, void* output, uint8_t* masks,
+int ash_grid_forward(ash_map_t* map, const float* x, const float* origin, float cell_size,
+                     int grid_dim, const ash_query_args* tables, void* output, uint8_t* masks,
                      int64_t* grid_indices, int64_t* cell_indices, float* offsets,
                      void* stream) {
     if (map == nullptr) ASH_FAIL("null map handle");
     if (map->key_dim != 3) ASH_FAIL("grid queries need a map with 3-d keys");
     if (grid_dim < 1 || grid_dim > 1024) ASH_FAIL("grid_dim must be in 1..1024");
+    if (!(cell_size > 0.f) || !(cell_size < INFINITY)) ASH_FAIL("cell_size must be positive and finite");
     QDev d;
     if (check_args(tables, d, true)) return 1;
     if (d.M != static_cast<int64_t>(grid_dim) * grid_dim * grid_dim) {
@@ -2432,6 +2440,8 @@ int ash_grid_forward(ash_map_t* map, const float* x, int grid_dim,
     FrontDev f;
     f.m = map->d;
     f.x = x;
+    f.origin = origin;
+    f.inv_cell = 1.0f / cell_size;
     f.g = static_cast<float>(grid_dim);
     f.gdim = grid_dim;
     f.mask_out = masks;
