@@ -474,20 +474,101 @@ __device__ __forceinline__ int place_code(uint4* tab, uint64_t code, int lb, int
     return kFull;
 }
 
+// Among the first n slots of local bucket lb (n <= kSlots, all of them
+// written), empties every slot that holds the code of a lower slot; `dropped`
+// is told the slot before it is emptied.  Every lane of the wavefront calls
+// this (n = 0: nothing to look at).
+template <typename Dropped>
+__device__ __forceinline__ void drop_repeats(uint4* tab, int lb, int n, Dropped dropped) {
+    uint64_t c[kSlots];
+#pragma unroll
+    for (int q = 0; q < kSlots / 2; ++q) {
+        const uint4 w = n > 2 * q ? tab[staged(lb, q)] : make_uint4(0u, 0u, 0u, 0u);
+        c[2 * q] = static_cast<uint64_t>(w.x) | (static_cast<uint64_t>(w.y) << 32);
+        c[2 * q + 1] = static_cast<uint64_t>(w.z) | (static_cast<uint64_t>(w.w) << 32);
+    }
+    // low words first: two slots hold the same code only if they agree there,
+    // which is rare enough to let whole wavefronts skip the full comparison
+    // (slots from n on get low words of their own)
+    uint32_t lo[kSlots];
+#pragma unroll
+    for (int j = 0; j < kSlots; ++j) lo[j] = j < n ? static_cast<uint32_t>(c[j]) : 0x80000000u + j;
+    bool maybe = false;
+#pragma unroll
+    for (int j = 1; j < kSlots; ++j) {
+#pragma unroll
+        for (int i = 0; i < j; ++i) maybe = maybe || lo[i] == lo[j];
+    }
+    if (!__ballot(maybe)) return;
+    uint32_t repeat = 0;
+#pragma unroll
+    for (int j = 1; j < kSlots; ++j) {
+#pragma unroll
+        for (int i = 0; i < j; ++i) {
+            // (a slot emptied by an earlier look is not a copy of another such slot)
+            if (lo[i] == lo[j] && c[i] == c[j] && j < n && c[j] != kEmpty) repeat |= 1u << j;
+        }
+    }
+    unsigned long long* tab64 = reinterpret_cast<unsigned long long*>(tab);
+    while (repeat) {
+        const int j = __builtin_ctz(repeat);
+        dropped(j);
+        tab64[staged(lb, j >> 1) * 2 + (j & 1)] = kEmpty;
+        repeat &= repeat - 1;
+    }
+}
+
 // Pass 3: one workgroup per partition builds its 512 buckets in LDS.
 // `stale`: the bucket array holds leftovers of a table that has been cleared
 // since (the clear left the fill to its successor): every partition is then
 // written, those without records as empty ones.  `identity`: the heap is
 // 0, 1, 2, ... (nothing has written to it since it was last reset), so
 // position p holds index p and need not be read.
+//
+// Into a range that starts empty (the map was empty on entry) records are
+// placed by counting: a record draws a number in its bucket (one LDS atomic)
+// and, while that number is below the bucket's ten slots, simply writes its
+// code there -- no read of the bucket, no compare-and-swap.  Copies of one key
+// draw different numbers in the same bucket: after a barrier one thread per
+// bucket compares the codes written so far and empties every slot that repeats
+// a lower one (a wavefront reads 64 whole buckets per instruction; a look by
+// every record at the slots below its own costs as many LDS instructions as
+// the probing path).  When a record's index is known as it draws (provisional
+// scheme, heap in its initial order) it is stored with the code and tells the
+// comparing thread which row lost; otherwise, after another barrier, a record
+// that no longer finds its code in its slot has lost.  Records whose number is ten or more (a
+// crowded bucket, or many copies of few keys) wait until every record of the
+// partition has drawn and are then placed by the probing path, which first
+// looks into the home bucket like any probe.  That path alone serves a range
+// that holds entries already.
+enum { kRecIdle = 0, kRecPlaced = 1, kRecLost = 2 };
+constexpr int kWaitList = 128;
+
 template <bool PROV>
 __global__ __launch_bounds__(kBuildThreads) void build_kernel(
         MapDev m, BulkPlan pl, int stale, int identity) {
+    // Records per thread and round.  With rows the partitions of a batch of the
+    // order of the table take one round of five (16 M keys into 24 M: 2048 +- 45
+    // records per partition; with four, half of the partitions went through
+    // every phase twice, 162 against 139 us); keys only, a fifth record costs
+    // more in the ranking of the winners than the second round (262 against
+    // 185 us).
+    constexpr int kRecs = PROV ? 5 : kBuildRecs;
+    constexpr int kRound = kBuildThreads * kRecs;
+    constexpr int kCountedRounds = 32 / kRecs;   // one bit per record of a thread
+    constexpr int kRecSlots = kRecs + 1;
     __shared__ uint4 tab[kPartBuckets * kGroup];
     // winners per (record slot k, wavefront), then their exclusive prefix
-    __shared__ int s_wcnt[kBuildRecs * (kBuildThreads / 64)];
+    __shared__ int s_wcnt[kRecSlots * (kBuildThreads / 64)];
     __shared__ int s_base;
     __shared__ int s_losers;
+    __shared__ int s_drawn[kPartBuckets];   // numbers drawn per bucket (range that starts empty)
+    __shared__ int s_seen[kPartBuckets];    // of which drop_repeats has compared this many
+    // records that wait for the probing path: the first kWaitList of them here,
+    // the others are read again from the partition's records
+    __shared__ uint64_t s_wait_code[kWaitList];
+    __shared__ int32_t s_wait_row[kWaitList];
+    __shared__ int s_nwait;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -510,22 +591,37 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
         return;
     }
     const bool was_empty = pl.hdr[kHdrWasEmpty] != 0;
+    const bool counted = was_empty && cnt <= kCountedRounds * kRound;
     const int32_t heap_base = pl.hdr[kHdrBase];
     const int64_t bbase = static_cast<int64_t>(p) * pl.cap_part;
-    if (tid == 0) s_losers = 0;
+    if (tid == 0) {
+        s_losers = 0;
+        s_nwait = 0;
+    }
+    // (slot kRecs: a record taken from the waiting list, last round only)
+    uint64_t codes[kRecSlots] = {};
+    int32_t rows[kRecSlots] = {};
+    // records rb + k * kBuildThreads + tid, k < kRecs; with `only`, just
+    // those whose bit is set
+    auto load_round = [&](int rb, uint32_t only) {
+#pragma unroll
+        for (int k = 0; k < kRecs; ++k) {
+            const int r = rb + k * kBuildThreads + tid;
+            const bool take = r < cnt && ((only >> k) & 1u);
+            codes[k] = take ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
+            if constexpr (PROV) rows[k] = take ? __builtin_nontemporal_load(pl.rows_b + bbase + r) : 0;
+        }
+    };
     // The first round's records are requested before the table range is
     // staged, so that both latencies overlap.
-    uint64_t codes[kBuildRecs];
-    int32_t rows[kBuildRecs];
-#pragma unroll
-    for (int k = 0; k < kBuildRecs; ++k) {
-        const int r = k * kBuildThreads + tid;
-        codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
-        if constexpr (PROV) rows[k] = r < cnt ? __builtin_nontemporal_load(pl.rows_b + bbase + r) : 0;
-    }
+    load_round(0, ~0u);
     for (int t = tid; t < nbk * kGroup; t += kBuildThreads) {
         tab[staged(t >> 3, t & 7)] =
                 was_empty ? make_uint4(~0u, ~0u, ~0u, ~0u) : gl[t];
+    }
+    for (int t = tid; t < static_cast<int>(kPartBuckets); t += kBuildThreads) {
+        s_drawn[t] = 0;
+        s_seen[t] = 0;
     }
     __syncthreads();
 
@@ -536,27 +632,18 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
         const int ws = where & 15;
         tab32[staged(wlb, (kValDword0 + ws) >> 2) * 4 + (ws & 3)] = idx;
     };
+    auto code_at = [&](int where) -> unsigned long long& {
+        return tab64[staged(where >> 4, (where & 15) >> 1) * 2 + (where & 1)];
+    };
 
-    for (int rb = 0; rb < cnt; rb += kBuildThreads * kBuildRecs) {
-        int wslot[kBuildRecs];
-        if (rb > 0) {
+    // Indices for the records of a round that hold a slot (state kRecPlaced,
+    // slot in wslot); rows of the provisional scheme that did not get one
+    // (kRecLost) are given up.  Every thread calls this the same number of times.
+    auto settle_round = [&](const int (&state)[kRecSlots], const int (&wslot)[kRecSlots]) {
+        if constexpr (PROV) {
 #pragma unroll
-            for (int k = 0; k < kBuildRecs; ++k) {
-                const int r = rb + k * kBuildThreads + tid;
-                codes[k] = r < cnt ? __builtin_nontemporal_load(pl.codes_b + bbase + r) : 0ull;
-                if constexpr (PROV) rows[k] = r < cnt ? __builtin_nontemporal_load(pl.rows_b + bbase + r) : 0;
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < kBuildRecs; ++k) {
-            const int r = rb + k * kBuildThreads + tid;
-            wslot[k] = -1;
-            if (r >= cnt) continue;
-            const int lb = static_cast<int>(bucket_of(codes[k], m.nb) - b0);
-            const int how = place_code(tab, codes[k], lb, nbk, wslot[k]);
-            if (how == kFull) atomicAdd(m.ctr + kCtrDropped, 1);   // refused
-            if constexpr (PROV) {
-                if (how == kPlaced) {
+            for (int k = 0; k < kRecSlots; ++k) {
+                if (state[k] == kRecPlaced) {
                     // the promised position; re-pointed later if it turns out
                     // to lie beyond the last position in use
                     const int32_t pos = heap_base + rows[k];
@@ -567,25 +654,24 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
                         store_index(wslot[k], idx);
                         m.klog[idx] = codes[k];
                     }
-                } else {
+                } else if (state[k] == kRecLost) {
                     give_up_row(pl, rows[k], &s_losers, false);
                 }
             }
-        }
-        if constexpr (!PROV) {
+        } else {
             // Winners are ranked in record order, so that consecutive lanes
             // take consecutive heap entries.
-            int wrank[kBuildRecs];
+            int wrank[kRecSlots];
 #pragma unroll
-            for (int k = 0; k < kBuildRecs; ++k) {
-                const uint64_t wm = __ballot(wslot[k] >= 0);
+            for (int k = 0; k < kRecSlots; ++k) {
+                const uint64_t wm = __ballot(state[k] == kRecPlaced);
                 wrank[k] = __popcll(wm & ((1ull << lane) - 1ull));
                 if (lane == 0) s_wcnt[k * (kBuildThreads / 64) + wave] = __popcll(wm);
             }
             __syncthreads();
             if (tid == 0) {
                 int tot = 0;
-                for (int q = 0; q < kBuildRecs * (kBuildThreads / 64); ++q) {
+                for (int q = 0; q < kRecSlots * (kBuildThreads / 64); ++q) {
                     const int c = s_wcnt[q];
                     s_wcnt[q] = tot;
                     tot += c;
@@ -604,8 +690,8 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
             }
             __syncthreads();
 #pragma unroll
-            for (int k = 0; k < kBuildRecs; ++k) {
-                if (wslot[k] < 0) continue;
+            for (int k = 0; k < kRecSlots; ++k) {
+                if (state[k] != kRecPlaced) continue;
                 const int top = s_base + s_wcnt[k * (kBuildThreads / 64) + wave] + wrank[k];
                 if (top < m.capacity) {
                     const int32_t idx = identity ? top : m.heap[top];
@@ -613,14 +699,128 @@ __global__ __launch_bounds__(kBuildThreads) void build_kernel(
                     m.klog[idx] = codes[k];
                 } else {
                     // Heap exhausted: give the slot up again.
-                    const int wlb = wslot[k] >> 4;
-                    const int ws = wslot[k] & 15;
-                    tab64[staged(wlb, ws >> 1) * 2 + (ws & 1)] = kTomb;
+                    code_at(wslot[k]) = kTomb;
                     atomicAdd(m.ctr + kCtrTombs, 1);
                 }
             }
         }
         __syncthreads();
+    };
+    // The probing path for the records of a round whose bit is set in `which`.
+    auto probe_round = [&](uint32_t which, int (&state)[kRecSlots], int (&wslot)[kRecSlots]) {
+#pragma unroll
+        for (int k = 0; k < kRecSlots; ++k) {
+            state[k] = kRecIdle;
+            wslot[k] = -1;
+            if (!((which >> k) & 1u)) continue;
+            const int lb = static_cast<int>(bucket_of(codes[k], m.nb) - b0);
+            const int how = place_code(tab, codes[k], lb, nbk, wslot[k]);
+            if (how == kFull) atomicAdd(m.ctr + kCtrDropped, 1);   // refused
+            state[k] = how == kPlaced ? kRecPlaced : kRecLost;
+        }
+    };
+
+    // the index of a record is known when it draws its number
+    const bool direct = PROV && identity != 0;
+    uint32_t waiting = 0;   // bit round * kRecs + k: that record drew a number beyond the slots
+    int round = 0;
+    for (int rb = 0; rb < cnt; rb += kRound, ++round) {
+        int wslot[kRecSlots];
+        int state[kRecSlots];
+        if (rb > 0) load_round(rb, ~0u);
+        state[kRecs] = kRecIdle;
+        wslot[kRecs] = -1;
+        uint32_t live = 0;
+#pragma unroll
+        for (int k = 0; k < kRecs; ++k) {
+            if (rb + k * kBuildThreads + tid < cnt) live |= 1u << k;
+        }
+        if (!counted) {
+            probe_round(live, state, wslot);
+        } else {
+#pragma unroll
+            for (int k = 0; k < kRecs; ++k) {
+                state[k] = kRecIdle;
+                wslot[k] = -1;
+                if (!((live >> k) & 1u)) continue;
+                const int lb = static_cast<int>(bucket_of(codes[k], m.nb) - b0);
+                const int number = atomicAdd(&s_drawn[lb], 1);
+                if (number < kSlots) {
+                    wslot[k] = lb * kBucketQwords + number;
+                    code_at(wslot[k]) = codes[k];
+                    state[k] = kRecPlaced;
+                    if (direct) {
+                        store_index(wslot[k], heap_base + rows[k]);
+                        state[k] = kRecIdle;   // nothing left to do for it
+                    }
+                } else {
+                    const int at = atomicAdd(&s_nwait, 1);
+                    if (at < kWaitList) {
+                        s_wait_code[at] = codes[k];
+                        s_wait_row[at] = rows[k];
+                    } else {
+                        waiting |= 1u << (round * kRecs + k);
+                    }
+                }
+            }
+            __syncthreads();
+            for (int first = 0; first < nbk; first += kBuildThreads) {
+                const int lb = first + tid;
+                int drawn = 0;
+                if (lb < nbk) {
+                    drawn = s_drawn[lb] < kSlots ? s_drawn[lb] : kSlots;
+                    // (numbers drawn in earlier rounds have been looked at)
+                    const bool news = drawn >= 2 && drawn > s_seen[lb];
+                    s_seen[lb] = drawn;
+                    if (!news) drawn = 0;
+                }
+                drop_repeats(tab, lb < nbk ? lb : 0, drawn, [&](int j) {
+                    if constexpr (PROV) {
+                        if (direct) {
+                            const int32_t idx = tab32[staged(lb, (kValDword0 + j) >> 2) * 4 + (j & 3)];
+                            give_up_row(pl, idx - heap_base, &s_losers, false);
+                        }
+                    }
+                });
+            }
+            const bool last = rb + kRound >= cnt && s_nwait > 0;
+            if (!direct || last) __syncthreads();
+            if (!direct) {
+#pragma unroll
+                for (int k = 0; k < kRecs; ++k) {
+                    if (state[k] == kRecPlaced && code_at(wslot[k]) != codes[k]) state[k] = kRecLost;
+                }
+            }
+            if (last) {
+                // the last round: every record has drawn, so the listed
+                // waiting records take the probing path now and get their
+                // indices with this round's
+                const int listed = s_nwait < kWaitList ? s_nwait : kWaitList;
+                if (tid < listed) {
+                    constexpr int x = kRecs;
+                    codes[x] = s_wait_code[tid];
+                    rows[x] = s_wait_row[tid];
+                    const int lb = static_cast<int>(bucket_of(codes[x], m.nb) - b0);
+                    const int how = place_code(tab, codes[x], lb, nbk, wslot[x]);
+                    if (how == kFull) atomicAdd(m.ctr + kCtrDropped, 1);   // refused
+                    state[x] = how == kPlaced ? kRecPlaced : kRecLost;
+                }
+            }
+        }
+        settle_round(state, wslot);
+    }
+    // (s_nwait is final: every round ends with a barrier)
+    if (counted && s_nwait > kWaitList) {
+        round = 0;
+        for (int rb = 0; rb < cnt; rb += kRound, ++round) {
+            const uint32_t mine = (waiting >> (round * kRecs)) & ((1u << kRecs) - 1u);
+            if (!__syncthreads_or(mine != 0)) continue;
+            int wslot[kRecSlots];
+            int state[kRecSlots];
+            load_round(rb, mine);
+            probe_round(mine, state, wslot);
+            settle_round(state, wslot);
+        }
     }
     // (stores marked as not to be kept in the caches: nothing reads the range,
     // the value rows or the log entries again before a later call does; the
