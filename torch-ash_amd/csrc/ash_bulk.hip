@@ -73,13 +73,19 @@ struct BulkPlan {
     uint32_t parts;        // partitions of kPartBuckets buckets
     uint32_t bins;         // coarse bins of (1 << fine_shift) partitions
     uint32_t fine_shift;
-    uint32_t cap_bin;      // records per coarse bin
+    // A coarse bin's buffer consists of 1 << lane_shift lanes with a cursor
+    // each; workgroup w of pass 1 appends to lane w mod lanes.  Every chunk of
+    // pass 1 reserves a run in every bin, and updates of one address serialise
+    // (about 7 ns each): with one cursor per bin the 3906 chunks of 16 M keys
+    // queued for 27 us at each, a quarter of the pass.
+    uint32_t lane_shift;
+    uint32_t cap_bin;      // records per lane of a coarse bin
     uint32_t cap_part;     // records per partition
-    uint32_t chunks;       // split chunks per coarse bin
+    uint32_t chunks;       // split chunks per lane of a coarse bin
     int32_t* hdr;
-    int32_t* cursor_bin;   // bins
+    int32_t* cursor_bin;   // bins << lane_shift
     int32_t* cursor_part;  // bins << fine_shift
-    uint64_t* codes_a;     // bins * cap_bin
+    uint64_t* codes_a;     // (bins << lane_shift) * cap_bin
     uint64_t* codes_b;     // parts * cap_part
     // keys only
     int32_t* spill_keys;   // n input row numbers (also the one list of the provisional scheme)
@@ -113,15 +119,21 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
     const int64_t bins = (parts + (1ll << fine_shift) - 1) >> fine_shift;
     if (bins > kMaxBins) return 0;
     const double per_bucket = static_cast<double>(n) / static_cast<double>(nb);
-    const double mean_bin = per_bucket * kPartBuckets * static_cast<double>(1ll << fine_shift);
+    double mean_bin = per_bucket * kPartBuckets * static_cast<double>(1ll << fine_shift);
     const double mean_part = per_bucket * kPartBuckets;
+    // lanes per bin: as many (up to eight) as leave a lane two chunks of pass 2
+    uint32_t lane_shift = 0;
+    while (lane_shift < 3 && mean_bin >= 4.0 * kSplitChunk) {
+        ++lane_shift;
+        mean_bin *= 0.5;
+    }
     int64_t cap_bin = static_cast<int64_t>(mean_bin + 10.0 * std::sqrt(mean_bin)) + 256;
     int64_t cap_part = static_cast<int64_t>(mean_part + 10.0 * std::sqrt(mean_part)) + 64;
     if (cap_bin > n) cap_bin = n;
     if (cap_part > n) cap_part = n;
     cap_bin = (cap_bin + 15) & ~int64_t{15};
     cap_part = (cap_part + 15) & ~int64_t{15};
-    const int64_t na = bins * cap_bin;
+    const int64_t na = (bins << lane_shift) * cap_bin;
     const int64_t nbp = parts * cap_part;
     if (na >= (int64_t{1} << 31) || nbp >= (int64_t{1} << 31)) return 0;
 
@@ -129,6 +141,7 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
     pl.parts = static_cast<uint32_t>(parts);
     pl.bins = static_cast<uint32_t>(bins);
     pl.fine_shift = fine_shift;
+    pl.lane_shift = lane_shift;
     pl.cap_bin = static_cast<uint32_t>(cap_bin);
     pl.cap_part = static_cast<uint32_t>(cap_part);
     pl.chunks = static_cast<uint32_t>((cap_bin + kSplitChunk - 1) / kSplitChunk);
@@ -140,7 +153,7 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
         return p;
     };
     pl.hdr = reinterpret_cast<int32_t*>(take(kHdrWords * 4));
-    pl.cursor_bin = reinterpret_cast<int32_t*>(take(bins * 4));
+    pl.cursor_bin = reinterpret_cast<int32_t*>(take((bins << lane_shift) * 4));
     pl.cursor_part = reinterpret_cast<int32_t*>(take((bins << fine_shift) * 4));
     pl.codes_a = reinterpret_cast<uint64_t*>(take(na * 8));
     pl.codes_b = reinterpret_cast<uint64_t*>(take(nbp * 8));
@@ -163,7 +176,7 @@ int64_t make_plan(const ash_map* map, int64_t n, int n_values,
 __global__ void bulk_init_kernel(MapDev m, BulkPlan pl, int ncursors) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     // cursor_bin and cursor_part are zeroed separately: they are not adjacent
-    if (t < static_cast<int>(pl.bins)) pl.cursor_bin[t] = 0;
+    if (t < static_cast<int>(pl.bins << pl.lane_shift)) pl.cursor_bin[t] = 0;
     if (t < ncursors) pl.cursor_part[t] = 0;
     if (t < kHdrWords) {
         int32_t v = 0;
@@ -201,8 +214,9 @@ struct SplitShared {
     uint64_t stage[kSplitChunk];   // sorted position -> code
 };
 
+// `shift`, `lane`: the cursor of bin b is cursors[(b << shift) + lane].
 __device__ __forceinline__ int reserve_runs(SplitShared& sh, int32_t* cursors,
-                                            int nbins) {
+                                            int nbins, int shift = 0, int lane_of_bin = 0) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     int v = 0, incl = 0;
@@ -221,7 +235,7 @@ __device__ __forceinline__ int reserve_runs(SplitShared& sh, int32_t* cursors,
         int off = 0;
         for (int w = 0; w < (tid >> 6); ++w) off += sh.wave_total[w];
         sh.start[tid] = off + incl - v;
-        sh.base[tid] = (v && tid < nbins) ? atomicAdd(cursors + tid, v) : 0;
+        sh.base[tid] = (v && tid < nbins) ? atomicAdd(cursors + (tid << shift) + lane_of_bin, v) : 0;
     }
     __syncthreads();
     int total = 0;
@@ -337,7 +351,9 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
         sh.spill_first = atomicAdd(pl.hdr + kHdrSpillKeys, sh.nspill);
         if constexpr (PROV) sh.losers = sh.nspill;
     }
-    const int total = reserve_runs(sh, pl.cursor_bin, static_cast<int>(pl.bins));
+    const int my_lane = static_cast<int>(blockIdx.x & ((1u << pl.lane_shift) - 1u));
+    const int total = reserve_runs(sh, pl.cursor_bin, static_cast<int>(pl.bins),
+                                   static_cast<int>(pl.lane_shift), my_lane);
 #pragma unroll
     for (int k = 0; k < kSplitKeys; ++k) {
         if (spill_rank[k] >= 0) {
@@ -347,7 +363,10 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
     }
     move_chunk<PROV>(
             sh, total, code, aux, bin, rank, pl.codes_a, pl.rows_a, pl.cap_bin,
-            [&](int b) { return static_cast<int64_t>(b) * pl.cap_bin; },
+            [&](int b) {
+                return static_cast<int64_t>((static_cast<uint32_t>(b) << pl.lane_shift) + my_lane) *
+                       pl.cap_bin;
+            },
             [&](int32_t a) {
                 if constexpr (PROV) {
                     give_up_row(pl, a, &sh.losers, true);
@@ -362,22 +381,23 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
     }
 }
 
-// Pass 2: coarse bin -> partitions.  Workgroup (bin, chunk) takes 4096 records
-// of its bin.
+// Pass 2: coarse bin -> partitions.  Workgroup (bin, lane, chunk) takes 4096
+// records of its lane of the bin.
 template <bool PROV>
 __global__ __launch_bounds__(kSplitThreads) void split_records_kernel(MapDev m, BulkPlan pl) {
     __shared__ SplitShared sh;
     const int tid = threadIdx.x;
-    const uint32_t c = blockIdx.x / pl.chunks;
+    const uint32_t lane_of_bin = blockIdx.x / pl.chunks;   // (bin << lane_shift) + lane
     const uint32_t chunk = blockIdx.x % pl.chunks;
-    int cnt = pl.cursor_bin[c];
+    const uint32_t c = lane_of_bin >> pl.lane_shift;
+    int cnt = pl.cursor_bin[lane_of_bin];
     if (cnt > static_cast<int>(pl.cap_bin)) cnt = static_cast<int>(pl.cap_bin);
     const int start = static_cast<int>(chunk) * kSplitChunk;
     if (start >= cnt) return;
     if (tid < kMaxBins) sh.cnt[tid] = 0;
     if (tid == 0) sh.losers = 0;
     __syncthreads();
-    const int64_t abase = static_cast<int64_t>(c) * pl.cap_bin + start;
+    const int64_t abase = static_cast<int64_t>(lane_of_bin) * pl.cap_bin + start;
     const uint32_t fmask = (1u << pl.fine_shift) - 1u;
     uint64_t code[kSplitKeys];
     int32_t aux[kSplitKeys];
@@ -1357,7 +1377,7 @@ int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     const int stale = map->table_stale ? 1 : 0;
     const int identity = map->heap_dirty ? 0 : 1;
 
-    const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);
+    const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
@@ -1371,7 +1391,7 @@ int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     if (n_values == 0) {
         if (launch_split_keys<false>(map, pl, keys, identity, s)) return 1;
         if (publish()) return 1;
-        split_records_kernel<false><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
+        split_records_kernel<false><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
         ASH_LAUNCH_CHECK();
         build_kernel<false><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
         ASH_LAUNCH_CHECK();
@@ -1383,7 +1403,7 @@ int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     }
     if (launch_split_keys<true>(map, pl, keys, identity, s)) return 1;
     if (publish()) return 1;
-    split_records_kernel<true><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
+    split_records_kernel<true><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
     build_kernel<true><<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl, stale, identity);
     ASH_LAUNCH_CHECK();
@@ -1451,12 +1471,12 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
-    const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);
+    const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
     if (launch_split_keys<false>(map, pl, keys, 0, s)) return 1;
-    split_records_kernel<false><<<pl.bins * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
+    split_records_kernel<false><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
     erase_range_kernel<<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
