@@ -405,7 +405,7 @@ def bench_hash(torch, ash, workloads, args, dev):
             run(t_erase_bulk, lambda: check(lib.ash_map_erase_bulk(
                 handle, keys.data_ptr(), n, erase_ws.data_ptr(), erase_ws.numel(), stream)))
     assert int(mask_out.sum()) == hits
-    assert backend.status()["size"] == 0   # a fresh read: the launches above went past the shim
+    assert backend.size() == 0
     c_count = (ctypes.c_int64 * k)(args.capacity, args.capacity)
     gathered = [torch.empty((n, 3), device=dev), torch.empty((n, 1), device=dev)]
     c_out = (ctypes.c_void_p * k)(gathered[0].data_ptr(), gathered[1].data_ptr())
@@ -501,7 +501,7 @@ def bench_config1(torch, ash, workloads, dev, reps=5):
         run(t_find, lambda: lib.ash_map_find(handle, queries.data_ptr(), n_q, idx.data_ptr(),
                                              msk.data_ptr(), stream))
     ms_i, ms_f = t_ins.mean_ms(), t_find.mean_ms()
-    unique = backend.status()["size"]   # from the device: the launches above went past the shim
+    unique = backend.size()   # (the handle follows the raw launches above as well)
     # 38 B per input key: 12 + 16 for every key, 16 + 4 more for the unique half
     out = {
         "insert_keys": roofline_entry("insert_kernel<3,keys> 1 M keys, 50 % duplicates",

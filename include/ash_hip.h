@@ -140,7 +140,7 @@ int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
 /* After ash_grid_activate: the rows whose flag is set in `touched`, in
  * ascending order, to out_indices int64[capacity] and their block coordinates
  * to out_coords int32[capacity, 3]; the flags are cleared and the count is left
- * in the table's counters (out[5] of ash_map_status_staged), so that the
+ * in the table's counters (out[5] of ash_map_counters), so that the
  * read-back that follows an activation anyway also sizes the result -- instead
  * of a `nonzero` over the flags with a read-back of its own.  Tables of up to
  * ASH_COLLECT_MAX_BLOCKS rows; `touched` 4-byte aligned.  No counterpart in the
@@ -273,24 +273,6 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
                         const int64_t* row_bytes, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
-/* ash_map_insert_bulk for a caller that reads the table's counters after every
- * insert and does not want to wait for the whole insert to do so.  The only
- * counter that decides what the caller does next -- keys that need the second
- * region, out[3] of ash_map_status -- can only be non-zero when the first
- * split pass handed keys over to the per-key kernel (unpackable keys are among
- * them).  Their number is written to `handed_over` (one int32 of page-locked
- * host memory that the device can write to) right after that pass and
- * `handed_over_event` (a hipEvent_t of the caller's, may be NULL) is recorded
- * behind it, about a quarter into the call's work: zero means that no key of
- * this batch is waiting for the second region, and the other counters can be
- * fetched without blocking (ash_map_status_begin).  No counterpart in the
- * reference. */
-int ash_map_insert_bulk_early(ash_map_t* map, const int32_t* keys, int64_t n,
-                              int n_values, const void* const* src, void* const* dst,
-                              const int64_t* row_bytes, void* workspace,
-                              int64_t workspace_bytes, int32_t* handed_over,
-                              void* handed_over_event, void* stream);
-
 /* Replaces `HashMap::erase` (ash/src/hashmap_gpu.cuh:316-351): found keys are
  * removed and their indices pushed back on the heap; duplicates inside the
  * batch erase once. */
@@ -311,6 +293,50 @@ int ash_map_erase_bulk_query(ash_map_t* map, int64_t n, int64_t* bytes, int* wor
 int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* workspace,
                        int64_t workspace_bytes, void* stream);
 
+/* `HashMap::insert_keys` / `HashMap::insert` (ash/src/hashmap_gpu.cuh:211-313)
+ * as one call that keeps the table in order by itself -- what a binding with
+ * the reference's nine methods (ash/src/pybind.cpp:9-23) calls:
+ *   1. if an erase or refused keys may have left tombstones, it looks at the
+ *      counters and re-places the entries when too few empty slots remain
+ *      (ash_map_should_rebuild / ash_map_rebuild);
+ *   2. it takes the streaming path (ash_map_insert_bulk) when the batch is large
+ *      enough relative to the table, else the per-key kernel, with `scratch` as
+ *      the workspace of either (`policy` overrides the choice);
+ *   3. it reads the counters, or -- streaming path, a landing place set with
+ *      ash_map_set_staging, no key of the batch handed to the per-key kernel --
+ *      queues their read-back behind the insert and returns without waiting
+ *      for it (ash_map_counters picks it up).
+ * Returns ASH_NEEDS_GENERAL (and inserts everything else) when keys of the
+ * batch do not fit the packed code and no second region is attached: attach
+ * one and issue the same call again.  n_values may be 0 (keys only).
+ * ash_map_insert_scratch_bytes gives the size of `scratch` (256-byte aligned
+ * device memory, free again when the call's work on `stream` has finished) for
+ * the call that follows it.  On a stream that is being captured the call only
+ * queues launches (no upkeep, no look at the counters): refused keys and keys
+ * waiting for the second region stay in the counters.  `staging` as for
+ * ash_map_counters. */
+enum { ASH_STREAMING_AUTO = 0, ASH_STREAMING_ALWAYS = 1, ASH_STREAMING_NEVER = 2 };
+enum { ASH_NEEDS_GENERAL = 2 };
+int ash_map_insert_scratch_bytes(ash_map_t* map, int64_t n, int n_values,
+                                 const int64_t* row_bytes, int policy, int64_t* bytes);
+int ash_map_insert_auto(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
+                        const void* const* src, void* const* dst, const int64_t* row_bytes,
+                        void* scratch, int64_t scratch_bytes, int policy, int32_t* staging,
+                        void* stream);
+
+/* `HashMap::erase` (ash/src/hashmap_gpu.cuh:316-351) with the choice between
+ * ash_map_erase and ash_map_erase_bulk made here; scratch as above. */
+int ash_map_erase_scratch_bytes(ash_map_t* map, int64_t n, int policy, int64_t* bytes);
+int ash_map_erase_auto(ash_map_t* map, const int32_t* keys, int64_t n, void* scratch,
+                       int64_t scratch_bytes, int policy, void* stream);
+
+/* Step 1 of ash_map_insert_auto on its own, for the entry points that insert
+ * without it (ash_grid_activate*): call it before them.  `scratch` is only
+ * needed by a map with a second region (ash_map_insert_scratch_bytes with
+ * n = 0 sizes it).  Does nothing on a stream that is being captured. */
+int ash_map_upkeep(ash_map_t* map, int64_t incoming, void* scratch, int64_t scratch_bytes,
+                   int32_t* staging, void* stream);
+
 /* Replaces `HashMap::clear` (ash/src/hashmap_gpu.cuh:354-358,
  * ash/src/hashmap_impl.h:26-33).  Counters, heap and the second region are
  * reset on `stream` at once (the heap array is rewritten to 0..capacity-1 only
@@ -325,31 +351,38 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
  * graph would empty the table at every replay). */
 int ash_map_clear(ash_map_t* map, void* stream);
 
-/* Host read-back of the device counters; synchronises `stream`.
+/* Host read-back of the device counters; always a copy from the device, which
+ * synchronises `stream`.
  *   out[0] size (= heap counter, ash/src/hashmap_gpu.cuh:157)
  *   out[1] keys dropped because the map was full (since the last clear)
  *   out[2] tombstoned slots
  *   out[3] keys that are waiting for ash_map_attach_general (re-issue the
  *          insert after attaching; the counter is reset by the attach)
- *   out[4] duplicate (key,index) pairs seen by ash_map_load */
+ *   out[4] pairs refused by ash_map_load: duplicate keys, indices or heap
+ *          entries outside 0 .. capacity-1 */
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream);
 
-/* ash_map_status through eight int32 of page-locked host memory of the
- * caller's (`staging`, e.g. one pinned tensor per host thread): the counters
- * are copied there directly instead of through the runtime's staging of
- * pageable memory, which halves the latency of the read-back that ends every
- * insert.  out[5] is the number of rows the latest ash_grid_collect_touched
- * listed.  No counterpart in the reference. */
-int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[6], void* stream);
-
-/* ash_map_status_staged in two halves: ash_map_status_begin queues the copy of
- * the counters into `staging` (eight int32 of page-locked host memory) on
- * `stream` and records `event` (a hipEvent_t of the caller's, may be NULL)
- * behind it, without waiting; once the event or the stream has completed,
- * ash_map_status_decode turns the staging area into the six values of
- * ash_map_status_staged.  No counterpart in the reference. */
-int ash_map_status_begin(ash_map_t* map, int32_t* staging, void* event, void* stream);
-int ash_map_status_decode(const int32_t* staging, int64_t out[6]);
+/* The same counters as the handle knows them, plus out[5] = rows listed by the
+ * latest ash_grid_collect_touched and out[6] = entries that live in the second
+ * region.  The handle follows every call that changes them: after a clear they
+ * are known to be zero, after ash_map_insert_auto they have been read (or are
+ * on their way, see there) -- only when neither holds are they copied from the
+ * device, which synchronises `stream`.  `staging`: eight int32 of page-locked
+ * host memory of the calling thread's for that copy, or NULL (pageable memory:
+ * about twice the latency).  No counterpart in the reference, whose `size()`
+ * synchronises every time (ash/src/hashmap_gpu.cuh:157). */
+int ash_map_counters(ash_map_t* map, int32_t* staging, int64_t out[7], void* stream);
+/* 1 while the read-back that a streaming ash_map_insert_auto queued has not
+ * been looked at yet. */
+int ash_map_counters_pending(ash_map_t* map);
+/* 1 and *size when the size is known without a copy from the device (waits for
+ * a queued read-back if there is one), 0 when it is not, -1 on failure. */
+int ash_map_known_size(ash_map_t* map, int64_t* size);
+/* Gives the map sixteen int32 of page-locked host memory of its own (NULL takes
+ * them away again): the landing place of the read-back that a streaming
+ * ash_map_insert_auto queues behind itself.  Must outlive the map or be taken
+ * away first. */
+int ash_map_set_staging(ash_map_t* map, int32_t* staging);
 
 /* Replaces `HashMap::size` (ash/src/hashmap_gpu.cuh:157); synchronises. */
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream);
@@ -383,10 +416,12 @@ int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
  * arithmetic only) says whether, with `size` live entries, `tombstones`
  * tombstones and `incoming` keys about to arrive, fewer than a fifth of the
  * slots would stay empty.  `ash_map_rebuild` then re-places the `n` = size live
- * (key, index) pairs into a cleared table; indices, heap and size are
- * untouched.  keys_scratch int32[n,key_dim] and indices_scratch int64[n] are
- * device temporaries.  No counterpart in the reference, whose container
- * recycles slots itself. */
+ * (key, index) pairs into an emptied table; indices, heap and size are
+ * untouched.  A map without a second region puts them back from its log of
+ * stored keys and needs no scratch (both pointers may be NULL); with one,
+ * keys_scratch int32[n,key_dim] and indices_scratch int64[n] are device
+ * temporaries.  ash_map_insert_auto / ash_map_upkeep do both by themselves.
+ * No counterpart in the reference, whose container recycles slots itself. */
 int ash_map_should_rebuild(ash_map_t* map, int64_t size, int64_t tombstones,
                            int64_t incoming);
 int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,

@@ -210,8 +210,12 @@ def test_clear_leaves_the_fill_to_the_next_call(gpu_ash, monkeypatch, policy):
     big.clear()
     sparse_batch = torch.unique(_random_keys(rng, 20_000, 3, 2000), dim=0).to(DEV)
     if policy == "always":
-        rows = (ctypes.c_int64 * 1)(8)
-        assert big.engine.backend._bulk_workspace(len(sparse_batch), 1, rows) is not None
+        # (the streaming path applies to this batch)
+        rows, nbytes = (ctypes.c_int64 * 1)(8), ctypes.c_int64(0)
+        backend = big.engine.backend
+        assert backend._lib.ash_map_insert_scratch_bytes(
+            backend._handle, len(sparse_batch), 1, rows, 1, ctypes.byref(nbytes)) == 0
+        assert nbytes.value > len(sparse_batch) * 20
     big.insert(sparse_batch, torch.zeros(len(sparse_batch), 2, device=DEV))
     keys, _ = big.items()
     assert torch.equal(sort_rows(keys)[0], sort_rows(sparse_batch)[0])

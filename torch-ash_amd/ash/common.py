@@ -150,12 +150,6 @@ _SIGNATURES = {
         ],
     ),
     "ash_map_items_in_index_order": (ctypes.c_int, [_PTR, ctypes.POINTER(ctypes.c_int)]),
-    "ash_map_insert_bulk_early": (
-        ctypes.c_int,
-        [_PTR, _PTR, _I64, ctypes.c_int, _PTR, _PTR, _PTR, _PTR, _I64, _PTR, _PTR, _PTR],
-    ),
-    "ash_map_status_begin": (ctypes.c_int, [_PTR, _PTR, _PTR, _PTR]),
-    "ash_map_status_decode": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64)]),
     "ash_map_erase": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR]),
     "ash_map_erase_bulk_query": (
         ctypes.c_int, [_PTR, _I64, ctypes.POINTER(_I64), ctypes.POINTER(ctypes.c_int)]
@@ -163,7 +157,24 @@ _SIGNATURES = {
     "ash_map_erase_bulk": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR, _I64, _PTR]),
     "ash_map_clear": (ctypes.c_int, [_PTR, _PTR]),
     "ash_map_status": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
-    "ash_map_status_staged": (ctypes.c_int, [_PTR, _PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_map_counters": (ctypes.c_int, [_PTR, _PTR, ctypes.POINTER(_I64), _PTR]),
+    "ash_map_counters_pending": (ctypes.c_int, [_PTR]),
+    "ash_map_known_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64)]),
+    "ash_map_set_staging": (ctypes.c_int, [_PTR, _PTR]),
+    "ash_map_insert_scratch_bytes": (
+        ctypes.c_int,
+        [_PTR, _I64, ctypes.c_int, ctypes.POINTER(_I64), ctypes.c_int, ctypes.POINTER(_I64)],
+    ),
+    "ash_map_insert_auto": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, ctypes.POINTER(_PTR), ctypes.POINTER(_PTR),
+         ctypes.POINTER(_I64), _PTR, _I64, ctypes.c_int, _PTR, _PTR],
+    ),
+    "ash_map_erase_scratch_bytes": (
+        ctypes.c_int, [_PTR, _I64, ctypes.c_int, ctypes.POINTER(_I64)]
+    ),
+    "ash_map_erase_auto": (ctypes.c_int, [_PTR, _PTR, _I64, _PTR, _I64, ctypes.c_int, _PTR]),
+    "ash_map_upkeep": (ctypes.c_int, [_PTR, _I64, _PTR, _I64, _PTR, _PTR]),
     "ash_grid_collect_touched": (ctypes.c_int, [_PTR] * 6),
     "ash_map_size": (ctypes.c_int, [_PTR, ctypes.POINTER(_I64), _PTR]),
     "ash_map_items": (ctypes.c_int, [_PTR, _PTR, _PTR, _I64, _PTR]),
@@ -247,15 +258,14 @@ COLLECT_MAX_BLOCKS = 1 << 20
 # Most positions per call of ash_grid_activate_static (the header's
 # ASH_ACTIVATE_STATIC_MAX_POSITIONS).
 ACTIVATE_STATIC_MAX = 1 << 20
-# Deferred activations between two looks at the table's counters.
-DEFERRED_UPKEEP_EVERY = 64
-
 # Which inserts (and erases) take the streaming path of the library (batch split
 # by bucket range, ranges handled in LDS) instead of the per-key kernel:
 # "auto" = when the library says the batch is large enough relative to the
 # table, "always" = whenever the path applies, "never".
 BULK_INSERT = os.environ.get("ASH_BULK_INSERT", "auto")
 BULK_ERASE = os.environ.get("ASH_BULK_ERASE", "auto")
+_POLICY = {"auto": 0, "always": 1, "never": 2}   # the header's ASH_STREAMING_*
+NEEDS_GENERAL = 2                                # the header's ASH_NEEDS_GENERAL
 _DTYPE = {torch.float32: 0, torch.float64: 1}
 
 
@@ -940,9 +950,10 @@ _STAGING: Dict[int, torch.Tensor] = {}
 
 
 def _status_staging() -> torch.Tensor:
-    """Page-locked landing place for the counters of a status read-back: one
-    per host thread for all maps (a read-back is complete when it returns, and
-    short-lived scratch sets would otherwise each allocate their own)."""
+    """Page-locked landing place for a copy of a map's counters that the caller
+    waits for: one per host thread for all maps (such a copy is complete when
+    the call returns, and short-lived scratch sets would otherwise each allocate
+    their own)."""
     key = threading.get_ident()
     staging = _STAGING.get(key)
     if staging is None:
@@ -984,9 +995,14 @@ class _HashMap:
 
     Owns the table workspace as torch tensors and a native handle.  `heap` is
     the caller's int32[capacity] buffer and is mutated in place by the kernels.
+    Which insert path a batch takes, the upkeep of the table and what is known
+    of its counters on the host are the library's business (ash_map_insert_auto,
+    ash_map_counters); this class allocates what the calls ask for.
     """
 
     _backend: "_Backend" = None
+    _COUNTERS = ("size", "dropped", "tombstones", "exotic_pending", "load_duplicates", "touched",
+                 "general_live")
 
     def __init__(self, key_dim: int, capacity: int, heap: torch.Tensor, device):
         device = torch.device(device)
@@ -1012,18 +1028,7 @@ class _HashMap:
         self._general_bytes = general_bytes.value
         self._table = torch.empty(table_bytes.value, dtype=torch.uint8, device=self._device)
         self._general = None
-        self._maybe_tombstones = False
-        # a read-back of the counters that has been queued behind an insert and
-        # not looked at yet (_finish_streaming_insert): page-locked landing
-        # places and events of this map's own
-        self._status_pending = False
-        self._late_in_flight = False   # a copy into _late may still be under way
-        self._early = None
-        # a new map is empty and every counter is zero
-        self._status_after_insert = {
-            "size": 0, "dropped": 0, "tombstones": 0,
-            "exotic_pending": 0, "load_duplicates": 0, "touched": 0,
-        }
+        self._landing = None   # page-locked int32[16] of this map's own, made on first use
         # counts the calls that may have changed the stored keys; lets callers
         # keep results derived from the key set (orderings, tables) while it stands
         self.version = next(_VERSIONS)
@@ -1045,14 +1050,8 @@ class _HashMap:
 
     def __del__(self):
         handle, self._handle = getattr(self, "_handle", None), None
-        if getattr(self, "_late_in_flight", False):
-            # the device may still owe a write into this map's page-locked
-            # landing place; it must arrive before that memory is given back
-            try:
-                self._late_event.synchronize()
-            except Exception:
-                pass
         if handle:
+            # (waits for a copy that is still on its way into `_landing`)
             self._lib.ash_map_destroy(handle)
 
     # -- helpers ---------------------------------------------------------
@@ -1071,99 +1070,12 @@ class _HashMap:
             keys = keys.to(torch.int32)
         return keys.contiguous()
 
-    def _make_room(self, incoming: int) -> None:
-        """Before an insert: if earlier erases or refused keys may have left
-        tombstones, look at the counters and re-place the live entries into a
-        cleared table when too few empty slots remain."""
-        self._resolve_status()
-        if not self._maybe_tombstones:
-            return
-        st = self.status()
-        self._maybe_tombstones = st["tombstones"] > 0
-        if not self._lib.ash_map_should_rebuild(
-            self._handle, st["size"], st["tombstones"], incoming
-        ):
-            return
-        n = st["size"]
-        keys = torch.empty((n, self.key_dim), dtype=torch.int32, device=self._device)
-        indices = torch.empty(n, dtype=torch.int64, device=self._device)
-        with torch.cuda.device(self._device):
-            self._check(
-                self._lib.ash_map_rebuild(
-                    self._handle, keys.data_ptr() if n else None,
-                    indices.data_ptr() if n else None, n, self._stream(),
-                )
-            )
-        self._maybe_tombstones = False
+    def _scratch(self, nbytes: int) -> Optional[torch.Tensor]:
+        return torch.empty(nbytes, dtype=torch.uint8, device=self._device) if nbytes else None
 
-    def _deferred(self):
-        """(handed-over count int32[1], counters int32[8], two events), made on
-        first use: page-locked memory the device writes to."""
-        if self._early is None:
-            self._early = torch.zeros(1, dtype=torch.int32, pin_memory=True)
-            self._late = torch.zeros(8, dtype=torch.int32, pin_memory=True)
-            stream = torch.cuda.current_stream(self._device)
-            self._early_event, self._late_event = torch.cuda.Event(), torch.cuda.Event()
-            # an event has a handle once it has been recorded
-            self._early_event.record(stream)
-            self._late_event.record(stream)
-        return self._early, self._late, self._early_event, self._late_event
-
-    def _finish_streaming_insert(self) -> bool:
-        """After ash_map_insert_bulk_early has been queued.  Waits for the first
-        split pass only: when it handed no key to the per-key kernel, no key of
-        the batch can be waiting for the second region, so nothing has to be
-        re-issued and the counters are fetched behind the insert without
-        waiting for them (True).  Otherwise the caller reads them now (False)."""
-        early, late, early_event, late_event = self._deferred()
-        early_event.synchronize()
-        if int(early[0]) != 0:
-            return False
-        if self._late_in_flight:
-            # an earlier read-back that nobody looked at (an erase or a clear
-            # made it stale) must have landed before the next one is queued
-            late_event.synchronize()
-        self._late_in_flight = True
-        self._check(
-            self._lib.ash_map_status_begin(
-                self._handle, late.data_ptr(), late_event.cuda_event, self._stream()
-            )
-        )
-        self._status_pending = True
-        self._status_after_insert = None
-        self.version = next(_VERSIONS)
-        return True
-
-    def _resolve_status(self) -> None:
-        """Looks at a read-back that an insert left queued."""
-        if not self._status_pending:
-            return
-        self._status_pending = False
-        _, late, _, late_event = self._deferred()
-        late_event.synchronize()
-        self._late_in_flight = False
-        out = (_I64 * 6)()
-        self._check(self._lib.ash_map_status_decode(late.data_ptr(), out))
-        st = {
-            "size": out[0], "dropped": out[1], "tombstones": out[2],
-            "exotic_pending": out[3], "load_duplicates": out[4], "touched": out[5],
-        }
-        if st["exotic_pending"] != 0:
-            raise RuntimeError("internal error: unpackable keys pending after a streaming insert")
-        self._status_after_insert = st
-        if st["dropped"] > 0 or st["tombstones"] > 0:
-            self._maybe_tombstones = True
-
-    def _attach_general_if_needed(self) -> bool:
-        """After an insert/load: keys that need the second region are counted by
-        the kernel; attach the region once and let the caller re-issue."""
-        st = self.status()
-        self._status_after_insert = st
-        self.version = next(_VERSIONS)
-        if st["dropped"] > 0 or st["tombstones"] > 0:
-            self._maybe_tombstones = True
-        if st["exotic_pending"] == 0:
-            return False
+    def _attach_general(self) -> None:
+        """Hands the table its second region (keys that do not fit the packed
+        code live there)."""
         if self._general is not None:
             raise RuntimeError("internal error: unpackable keys pending with region attached")
         self._general = torch.empty(self._general_bytes, dtype=torch.uint8, device=self._device)
@@ -1173,62 +1085,62 @@ class _HashMap:
                     self._handle, self._general.data_ptr(), self._general_bytes, self._stream()
                 )
             )
-        return True
+
+    def _upkeep(self, incoming: int) -> None:
+        """Before the entry points that insert without ash_map_insert_auto."""
+        nbytes = _I64(0)
+        self._check(self._lib.ash_map_insert_scratch_bytes(
+            self._handle, 0, 0, None, _POLICY["never"], ctypes.byref(nbytes)))
+        scratch = self._scratch(nbytes.value)
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_map_upkeep(
+                self._handle, incoming, scratch.data_ptr() if scratch is not None else None,
+                nbytes.value, _status_staging().data_ptr(), self._stream()))
 
     # -- pybind surface --------------------------------------------------
     def device(self) -> torch.device:
         return self._device
 
-    def status(self) -> Dict[str, int]:
-        self._status_pending = False   # this read is newer
-        out = (_I64 * 6)()
-        staging = _status_staging()
+    def counters(self) -> Dict[str, int]:
+        """The table's counters as the handle knows them; copied from the
+        device only when no earlier call has left them on the host."""
+        out = (_I64 * 7)()
         with torch.cuda.device(self._device):
-            self._check(
-                self._lib.ash_map_status_staged(
-                    self._handle, staging.data_ptr(), out, self._stream()
-                )
-            )
-        return {
-            "size": out[0],
-            "dropped": out[1],
-            "tombstones": out[2],
-            "exotic_pending": out[3],
-            "load_duplicates": out[4],
-            "touched": out[5],
-        }
+            self._check(self._lib.ash_map_counters(
+                self._handle, _status_staging().data_ptr(), out, self._stream()))
+        return dict(zip(self._COUNTERS, out))
+
+    def status(self) -> Dict[str, int]:
+        """The counters by a copy from the device, whatever the handle knows."""
+        out = (_I64 * 5)()
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_map_status(self._handle, out, self._stream()))
+        fresh = dict(zip(self._COUNTERS[:5], out))
+        fresh.update({k: v for k, v in self.counters().items() if k not in fresh})
+        return fresh
 
     def status_after_insert(self) -> Dict[str, int]:
-        """The counters as read back at the end of the latest insert (every
-        insert reads them once); saves the caller a second read-back."""
-        self._resolve_status()
-        st = getattr(self, "_status_after_insert", None)
-        return st if st is not None else self.status()
+        """The counters after the latest insert: every insert reads them (or
+        queues their read-back), which saves the caller a read-back of its own."""
+        return self.counters()
 
     @property
     def counters_queued(self) -> bool:
         """Whether the latest insert returned with the read-back of the
-        counters still queued behind it (see _finish_streaming_insert)."""
-        return self._status_pending
+        counters still queued behind it."""
+        return bool(self._lib.ash_map_counters_pending(self._handle))
 
     def known_size(self) -> Optional[int]:
         """The size if it is known on the host (from the latest read-back, or
         zero after a clear), else None; never asks the device for it."""
-        self._resolve_status()
-        st = getattr(self, "_status_after_insert", None)
-        return None if st is None else st["size"]
+        n = _I64(0)
+        rc = self._lib.ash_map_known_size(self._handle, ctypes.byref(n))
+        if rc < 0:
+            self._check(1)
+        return n.value if rc == 1 else None
 
     def size(self) -> int:
-        # every insert / load / activation ends with one read-back of the
-        # counters; until the next erase or clear that read-back still holds
-        self._resolve_status()
-        st = getattr(self, "_status_after_insert", None)
-        if st is not None:
-            return st["size"]
-        n = _I64(0)
-        with torch.cuda.device(self._device):
-            self._check(self._lib.ash_map_size(self._handle, ctypes.byref(n), self._stream()))
-        return n.value
+        return self.counters()["size"]
 
     def find(self, keys: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         keys = self._keys(keys)
@@ -1268,6 +1180,20 @@ class _HashMap:
             )
         return grid_indices, cell_indices, offsets, masks
 
+    def _activation_buffers(self, cells: torch.Tensor) -> torch.Tensor:
+        if self.key_dim != 3:
+            raise RuntimeError("block activation needs 3-d keys")
+        if cells.dim() != 2 or cells.shape[1] != 3 or cells.dtype != torch.float32:
+            raise RuntimeError("positions must be float32 (N, 3)")
+        if cells.device != self._device:
+            raise RuntimeError(f"positions are on {cells.device}, the map on {self._device}")
+        if getattr(self, "_touched", None) is None:
+            self._touched = torch.zeros(self.capacity, dtype=torch.uint8, device=self._device)
+            self._block_coords = torch.zeros(
+                (self.capacity, 3), dtype=torch.int32, device=self._device
+            )
+        return cells.contiguous()
+
     def activate_blocks(
         self,
         cells: torch.Tensor,
@@ -1280,19 +1206,8 @@ class _HashMap:
         """Fused body of `SparseDenseGrid.spatial_init_`: inserts the blocks
         around the positions `cells` (fp32, cell units) and returns the touched
         blocks as (grid_coords int32[n,3], grid_indices int64[n])."""
-        if self.key_dim != 3:
-            raise RuntimeError("block activation needs 3-d keys")
-        if cells.dim() != 2 or cells.shape[1] != 3 or cells.dtype != torch.float32:
-            raise RuntimeError("positions must be float32 (N, 3)")
-        if cells.device != self._device:
-            raise RuntimeError(f"positions are on {cells.device}, the map on {self._device}")
-        cells = cells.contiguous()
-        if getattr(self, "_touched", None) is None:
-            self._touched = torch.zeros(self.capacity, dtype=torch.uint8, device=self._device)
-            self._block_coords = torch.zeros(
-                (self.capacity, 3), dtype=torch.int32, device=self._device
-            )
-        self._make_room(cells.shape[0])
+        cells = self._activation_buffers(cells)
+        self._upkeep(cells.shape[0])
         heads = torch.empty(64 + 3 * cells.shape[0], dtype=torch.int32, device=self._device)
         # the touched rows are listed on the device and their count travels with
         # the read-back that ends the activation (tables beyond the listing
@@ -1318,10 +1233,14 @@ class _HashMap:
                             rows.data_ptr(), coords.data_ptr(), self._stream(),
                         )
                     )
-            if not self._attach_general_if_needed():
+            self.version = next(_VERSIONS)
+            counters = self.counters()
+            if counters["exotic_pending"] == 0:
                 break
+            # blocks beyond the packed range: they need the second region
+            self._attach_general()
         if listing:
-            n = self._status_after_insert["touched"]
+            n = counters["touched"]
             return coords[:n], rows[:n]
         grid_indices = self._touched.nonzero().view(-1)
         grid_coords = self._block_coords[grid_indices]
@@ -1342,24 +1261,15 @@ class _HashMap:
         grid_indices int64[capacity]) are returned whole -- how many of their
         rows the listing filled stays in the table's counters, where
         ash_grid_integrate_depth_touched reads it.  Nothing here waits for the
-        device; keys refused for lack of capacity show in the counters at the
-        next call that reads them (`status`, `size` after it, any insert).
-        Both tensors are reused by the next deferred activation of this map."""
-        if self.key_dim != 3:
-            raise RuntimeError("block activation needs 3-d keys")
-        if cells.dim() != 2 or cells.shape[1] != 3 or cells.dtype != torch.float32:
-            raise RuntimeError("positions must be float32 (N, 3)")
-        if cells.device != self._device:
-            raise RuntimeError(f"positions are on {cells.device}, the map on {self._device}")
+        device (every 64th call in a row looks at the counters for the table's
+        upkeep), so the launches can be captured into a graph; keys refused for
+        lack of capacity show in the counters at the next call that reads them
+        (`counters`, `size`, any insert).  Both tensors are reused by the next
+        deferred activation of this map."""
         if self.capacity > COLLECT_MAX_BLOCKS:
             raise RuntimeError("deferred activation lists at most 2^20 blocks")
-        cells = cells.contiguous()
+        cells = self._activation_buffers(cells)
         n = cells.shape[0]
-        if getattr(self, "_touched", None) is None:
-            self._touched = torch.zeros(self.capacity, dtype=torch.uint8, device=self._device)
-            self._block_coords = torch.zeros(
-                (self.capacity, 3), dtype=torch.int32, device=self._device
-            )
         if getattr(self, "_listing", None) is None:
             self._listing = (
                 torch.empty((self.capacity, 3), dtype=torch.int32, device=self._device),
@@ -1368,14 +1278,8 @@ class _HashMap:
         if self._general is None:
             # a key beyond the packed range would otherwise wait for a read-back
             # that this path does not make
-            self._general = torch.empty(self._general_bytes, dtype=torch.uint8, device=self._device)
-            with torch.cuda.device(self._device):
-                self._check(
-                    self._lib.ash_map_attach_general(
-                        self._handle, self._general.data_ptr(), self._general_bytes, self._stream()
-                    )
-                )
-        self._make_room(n)
+            self._attach_general()
+        self._upkeep(n)
         coords, rows = self._listing
         head = (self._handle, cells.data_ptr(), n, int(grid_dim), int(dilation),
                 int(bool(bidirectional)), int(bound_lo), int(bound_hi),
@@ -1393,60 +1297,11 @@ class _HashMap:
                     rows.data_ptr(), coords.data_ptr(), self._stream(),
                 )
             )
-        self._status_after_insert = None
-        self._status_pending = False
         self.version = next(_VERSIONS)
-        # Keys refused for lack of capacity leave tombstones behind and are
-        # only visible in the counters: every DEFERRED_UPKEEP_EVERY-th call the
-        # next insert looks at them (one read-back) and re-places the entries if
-        # tombstones have piled up.
-        self._deferred_calls = getattr(self, "_deferred_calls", 0) + 1
-        if self._deferred_calls >= DEFERRED_UPKEEP_EVERY:
-            self._deferred_calls = 0
-            self._maybe_tombstones = True
         return coords, rows
 
-    def _bulk_workspace(self, n: int, k: int, c_rows) -> Optional[torch.Tensor]:
-        """Workspace for the streaming insert path, or None when this batch goes
-        through the per-key kernel."""
-        if BULK_INSERT == "never":
-            return None
-        nbytes, worthwhile = _I64(0), ctypes.c_int(0)
-        self._check(
-            self._lib.ash_map_bulk_workspace_bytes(
-                self._handle, n, k, c_rows, ctypes.byref(nbytes), ctypes.byref(worthwhile)
-            )
-        )
-        if nbytes.value == 0 or not (worthwhile.value or BULK_INSERT == "always"):
-            return None
-        return torch.empty(nbytes.value, dtype=torch.uint8, device=self._device)
-
     def insert_keys(self, keys: torch.Tensor) -> None:
-        keys = self._keys(keys)
-        n = keys.shape[0]
-        self._make_room(n)
-        workspace = self._bulk_workspace(n, 0, None)
-        for _ in range(2):
-            with torch.cuda.device(self._device):
-                if workspace is not None:
-                    early, _, early_event, _ = self._deferred()
-                    self._check(
-                        self._lib.ash_map_insert_bulk_early(
-                            self._handle, keys.data_ptr(), n, 0, None, None, None,
-                            workspace.data_ptr(), workspace.numel(), early.data_ptr(),
-                            early_event.cuda_event, self._stream(),
-                        )
-                    )
-                    if self._finish_streaming_insert():
-                        return
-                else:
-                    self._check(
-                        self._lib.ash_map_insert_keys(
-                            self._handle, keys.data_ptr(), n, self._stream()
-                        )
-                    )
-            if not self._attach_general_if_needed():
-                break
+        self._insert(self._keys(keys), 0, None, None, None)
 
     def insert(
         self,
@@ -1476,88 +1331,57 @@ class _HashMap:
             src.append(v)
             dst.append(ext)
             row_bytes.append((v.numel() // max(n, 1)) * v.element_size() if n else 0)
+        k = len(names)
+        self._insert(keys, k, (_PTR * k)(*[t.data_ptr() for t in src]),
+                     (_PTR * k)(*[t.data_ptr() for t in dst]), (_I64 * k)(*row_bytes), held=src)
+
+    def _insert(self, keys, k, c_src, c_dst, c_rows, held=None) -> None:
+        """One ash_map_insert_auto (a second one after the second region has
+        been attached, the first time a key does not fit the packed code)."""
+        n = keys.shape[0]
         if n == 0:
             return
-        k = len(names)
-        c_rows = (_I64 * k)(*row_bytes)
-        c_src = (_PTR * k)(*[t.data_ptr() for t in src])
-        c_dst = (_PTR * k)(*[t.data_ptr() for t in dst])
-        assigned = None
-        if self._lib.ash_map_insert_needs_scratch(k, c_rows):
-            assigned = torch.empty(n, dtype=torch.int32, device=self._device)
-        self._make_room(n)
-        workspace = None if assigned is not None else self._bulk_workspace(n, k, c_rows)
+        policy = _POLICY[BULK_INSERT]
+        if self._landing is None and n >= (1 << 12):
+            # a batch that may take the streaming path: the map gets a landing
+            # place of its own for the read-back queued behind such an insert
+            self._landing = torch.zeros(16, dtype=torch.int32, pin_memory=True)
+            self._check(self._lib.ash_map_set_staging(self._handle, self._landing.data_ptr()))
         for _ in range(2):
+            nbytes = _I64(0)
+            self._check(self._lib.ash_map_insert_scratch_bytes(
+                self._handle, n, k, c_rows, policy, ctypes.byref(nbytes)))
+            scratch = self._scratch(nbytes.value)
             with torch.cuda.device(self._device):
-                if workspace is not None:
-                    early, _, early_event, _ = self._deferred()
-                    self._check(
-                        self._lib.ash_map_insert_bulk_early(
-                            self._handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows,
-                            workspace.data_ptr(), workspace.numel(), early.data_ptr(),
-                            early_event.cuda_event, self._stream(),
-                        )
-                    )
-                    if self._finish_streaming_insert():
-                        return
-                else:
-                    self._check(
-                        self._lib.ash_map_insert(
-                            self._handle,
-                            keys.data_ptr(),
-                            n,
-                            k,
-                            c_src,
-                            c_dst,
-                            c_rows,
-                            assigned.data_ptr() if assigned is not None else None,
-                            self._stream(),
-                        )
-                    )
-            if not self._attach_general_if_needed():
-                break
+                rc = self._lib.ash_map_insert_auto(
+                    self._handle, keys.data_ptr(), n, k, c_src, c_dst, c_rows,
+                    scratch.data_ptr() if scratch is not None else None, nbytes.value, policy,
+                    _status_staging().data_ptr(), self._stream())
+            self.version = next(_VERSIONS)
+            if rc != NEEDS_GENERAL:
+                return self._check(rc)
+            self._attach_general()
+        raise RuntimeError("internal error: unpackable keys pending with region attached")
 
     def erase(self, keys: torch.Tensor) -> None:
         keys = self._keys(keys)
-        self._maybe_tombstones = True
-        self._status_after_insert = None
-        self._status_pending = False
-        self.version = next(_VERSIONS)
         n = keys.shape[0]
-        workspace = None
-        if BULK_ERASE != "never":
-            nbytes, worthwhile = _I64(0), ctypes.c_int(0)
-            self._check(
-                self._lib.ash_map_erase_bulk_query(
-                    self._handle, n, ctypes.byref(nbytes), ctypes.byref(worthwhile)
-                )
-            )
-            if nbytes.value and (worthwhile.value or BULK_ERASE == "always"):
-                workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=self._device)
-        self.last_erase_path = "per-key" if workspace is None else "streaming"
+        policy = _POLICY[BULK_ERASE]
+        nbytes = _I64(0)
+        self._check(self._lib.ash_map_erase_scratch_bytes(
+            self._handle, n, policy, ctypes.byref(nbytes)))
+        scratch = self._scratch(nbytes.value)
+        self.last_erase_path = "per-key" if scratch is None else "streaming"
+        self.version = next(_VERSIONS)
         with torch.cuda.device(self._device):
-            if workspace is not None:
-                self._check(
-                    self._lib.ash_map_erase_bulk(
-                        self._handle, keys.data_ptr(), n, workspace.data_ptr(),
-                        workspace.numel(), self._stream(),
-                    )
-                )
-            else:
-                self._check(
-                    self._lib.ash_map_erase(self._handle, keys.data_ptr(), n, self._stream())
-                )
+            self._check(self._lib.ash_map_erase_auto(
+                self._handle, keys.data_ptr(), n,
+                scratch.data_ptr() if scratch is not None else None, nbytes.value, policy,
+                self._stream()))
 
     def clear(self) -> None:
         with torch.cuda.device(self._device):
             self._check(self._lib.ash_map_clear(self._handle, self._stream()))
-        self._maybe_tombstones = False
-        # clear zeroes every counter, so they are known without a read-back
-        self._status_after_insert = {
-            "size": 0, "dropped": 0, "tombstones": 0,
-            "exotic_pending": 0, "load_duplicates": 0, "touched": 0,
-        }
-        self._status_pending = False
         self.version = next(_VERSIONS)
 
     def items(self) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -1599,17 +1423,23 @@ class _HashMap:
                         self._stream(),
                     )
                 )
-            if not self._attach_general_if_needed():
+            self.version = next(_VERSIONS)
+            counters = self.counters()
+            if counters["exotic_pending"] == 0:
                 break
-        dup = self.status()["load_duplicates"]
-        if dup:
+            self._attach_general()
+        refused = counters["load_duplicates"]
+        if refused:
             # The reference prints "Error loading, should never reach here!"
-            # (ash/src/hashmap_gpu.cuh:420-422) and goes on with a heap counter
-            # that no longer matches the stored entries.  Here such a state is
-            # refused: the map is left empty.
+            # (ash/src/hashmap_gpu.cuh:420-422) for a repeated key and goes on
+            # with a heap counter that no longer matches the stored entries; an
+            # index or heap entry outside 0 .. capacity-1 makes its later calls
+            # write out of bounds.  Here such a state is refused: the map is
+            # left empty.
             self.clear()
             raise RuntimeError(
-                f"load_states: active_keys holds {dup} duplicate keys; nothing was loaded"
+                f"load_states: {refused} pairs were refused (duplicate keys, or indices / heap "
+                "entries outside the capacity); nothing was loaded"
             )
 
 

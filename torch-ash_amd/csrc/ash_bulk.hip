@@ -1332,15 +1332,15 @@ int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
     return 0;
 }
 
-namespace {
+}  // extern "C"
 
 // `early`: where to leave, right after the first split pass, the number of keys
 // that pass handed to the per-key kernel; `early_event` is recorded behind it.
-int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
-                int n_values, const void* const* src, void* const* dst,
-                const int64_t* row_bytes, void* workspace,
-                int64_t workspace_bytes, int32_t* early, hipEvent_t early_event,
-                void* stream) {
+int ash::insert_bulk(ash_map* map, const int32_t* keys, int64_t n,
+                     int n_values, const void* const* src, void* const* dst,
+                     const int64_t* row_bytes, void* workspace,
+                     int64_t workspace_bytes, int32_t* early, hipEvent_t early_event,
+                     void* stream) {
     if (check_batch(map, keys, n)) return 1;
     if (check_values(n_values, src, dst, row_bytes)) return 1;
     if (workspace == nullptr) ASH_FAIL("null bulk workspace");
@@ -1375,7 +1375,13 @@ int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     }
     const ValueArgs none = {};
     const int stale = map->table_stale ? 1 : 0;
-    const int identity = map->heap_dirty ? 0 : 1;
+    // (captured into a graph, the choice would be replayed whatever the heap
+    // holds then: a capture takes the variant that reads the heap)
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(s, &cap) == hipSuccess &&
+                           cap != hipStreamCaptureStatusNone;
+    const int identity = (map->heap_dirty || capturing) ? 0 : 1;
+    counters_changed(map, true);
 
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
@@ -1418,7 +1424,7 @@ int insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
     return insert_selected(map, false, keys, pl.spill_keys, pl.hdr + kHdrSpillKeys, user, s);
 }
 
-}  // namespace
+extern "C" {
 
 int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
                         int n_values, const void* const* src, void* const* dst,
@@ -1426,16 +1432,6 @@ int ash_map_insert_bulk(ash_map_t* map, const int32_t* keys, int64_t n,
                         int64_t workspace_bytes, void* stream) {
     return insert_bulk(map, keys, n, n_values, src, dst, row_bytes, workspace, workspace_bytes,
                        nullptr, nullptr, stream);
-}
-
-int ash_map_insert_bulk_early(ash_map_t* map, const int32_t* keys, int64_t n,
-                              int n_values, const void* const* src, void* const* dst,
-                              const int64_t* row_bytes, void* workspace,
-                              int64_t workspace_bytes, int32_t* handed_over,
-                              void* handed_over_event, void* stream) {
-    if (handed_over == nullptr) ASH_FAIL("null pointer for the early count");
-    return insert_bulk(map, keys, n, n_values, src, dst, row_bytes, workspace, workspace_bytes,
-                       handed_over, static_cast<hipEvent_t>(handed_over_event), stream);
 }
 
 int ash_map_erase_bulk_query(ash_map_t* map, int64_t n, int64_t* bytes, int* worthwhile) {
@@ -1471,6 +1467,7 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
+    counters_changed(map, false);
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);

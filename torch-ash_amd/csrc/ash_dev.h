@@ -62,13 +62,16 @@ enum Counter {
     kCtrDropped = 1,   // keys refused because the heap was exhausted
     kCtrTombs = 2,     // tombstoned slots (packed + general)
     kCtrExotic = 3,    // unpackable keys seen while no general region exists
-    kCtrLoadDup = 4,   // duplicate pairs met by load
-    kCtrCursor = 5,    // output cursor of items()
+    kCtrLoadDup = 4,   // pairs refused by load: duplicate keys, indices outside 0 .. capacity-1
+    kCtrGenLive = 5,   // entries that live in the general region
     kCtrTouched = 6,   // blocks listed by the latest ash_grid_collect_touched
     kCtrTicket = 7,    // workgroups of a running ash_grid_collect_touched that have read their input
+    // (the first eight are what a read-back of the counters copies to the host)
     kCtrLogHigh = 8,   // log entries at or beyond the size and below this index may hold keys of an earlier filling
+    kCtrCursor = 9,    // output cursor of items()
     kNumCounters = 64
 };
+constexpr int kHostCounters = 8;
 constexpr int64_t kHeaderBytes = 256;
 
 // General region: open addressing over 32-bit state words + 16-byte keys.
@@ -126,6 +129,11 @@ inline int64_t general_slots(int64_t capacity) {
 
 }  // namespace ash
 
+// What the host knows of the device counters (ash_map_counters).
+struct ash_counters {
+    int64_t size, dropped, tombstones, exotic_pending, load_refused, touched, general_live;
+};
+
 struct ash_map {
     int key_dim;
     int64_t capacity;
@@ -133,6 +141,20 @@ struct ash_map {
     ash::MapDev d;
     int64_t table_bytes;
     bool general_attached;
+    // --- bookkeeping of the counters on the host ------------------------
+    // page-locked int32[16] of the caller's (ash_map_set_staging) or null:
+    // [0, 8) landing place of a read-back, [8] the count a streaming insert
+    // publishes after its first pass
+    int32_t* staging;
+    hipEvent_t early_event, late_event;   // made on first use
+    bool late_in_flight;    // a copy into staging[0, 8) may still be under way
+    bool late_pending;      // ... and it is the latest state of the counters: nobody has looked at it yet
+    bool counters_known;    // `counters` is what the device holds
+    ash_counters counters;
+    // an erase, refused keys or a run of inserts whose counters nobody read
+    // may have left tombstones: the next managed insert looks at the counters
+    bool maybe_tombstones;
+    int unread_inserts;
     // clear() has reset the counters and the heap but left the bucket array as
     // it was: the next call that reads the table fills it first, a streaming
     // insert that rewrites every bucket does not need to

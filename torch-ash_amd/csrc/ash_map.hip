@@ -430,7 +430,25 @@ __device__ __forceinline__ void insert_key(
     const bool w = won || gwon;
     int32_t idx = -1;
     if constexpr (MODE == kInsertLoad) {
-        if (w) idx = static_cast<int32_t>(given[i]);
+        if (w) {
+            // the index comes with the key (`given` null: the key's own number,
+            // when the keys are the entries of the key log)
+            const int64_t g = given != nullptr ? given[i] : i;
+            if (g >= 0 && g < m.capacity) {
+                idx = static_cast<int32_t>(g);
+            } else {
+                // an index that addresses no row: the pair is refused (the
+                // slot goes back) and counted with the duplicates
+                if (won) {
+                    atomicExch(slot_ptr(m, wb, ws), kTomb);
+                } else {
+                    __hip_atomic_store(m.gstate + gp, kGenTomb, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                }
+                atomicAdd(m.ctr + kCtrTombs, 1);
+                atomicAdd(m.ctr + kCtrLoadDup, 1);
+            }
+        }
     } else {
         __shared__ int s_cnt[kHeapBlock / 64];
         __shared__ int s_base;
@@ -461,7 +479,11 @@ __device__ __forceinline__ void insert_key(
         if (w) {
             if (top < m.capacity) {
                 idx = m.heap[top];
-            } else {
+                // (a heap that a state dict brought may hold anything: an entry
+                // that addresses no row is treated like an exhausted heap)
+                if (static_cast<uint32_t>(idx) >= static_cast<uint32_t>(m.capacity)) idx = -1;
+            }
+            if (idx < 0) {
                 // Heap exhausted: give the slot up again.
                 if (won) {
                     atomicExch(slot_ptr(m, wb, ws), kTomb);
@@ -475,13 +497,15 @@ __device__ __forceinline__ void insert_key(
         }
     }
     if (idx >= 0) {
+        // (0 <= idx < capacity: heap entries are, loaded indices were checked)
         if (won) {
             *value_ptr(m, wb, ws) = idx;
-            if (idx < m.capacity) m.klog[idx] = code;   // (a loaded index may be anything)
+            m.klog[idx] = code;
         } else {
             __hip_atomic_store(m.gstate + gp, idx, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
-            if (idx < m.capacity) m.klog[idx] = kTomb;   // "stored in the general region"
+            m.klog[idx] = kTomb;   // "stored in the general region"
+            atomicAdd(m.ctr + kCtrGenLive, 1);
         }
         if constexpr (MODE == kInsertFused) {
 #pragma unroll
@@ -921,6 +945,7 @@ __device__ __forceinline__ void erase_one(const MapDev& m, const int32_t* __rest
                 won = true;
                 tomb = true;
                 idx = gi;
+                atomicSub(m.ctr + kCtrGenLive, 1);
             }
         }
     }
@@ -952,7 +977,7 @@ __device__ __forceinline__ void erase_one(const MapDev& m, const int32_t* __rest
         for (int q = 0; q < wave; ++q) below += s_cnt[q];
         const int pos = s_base - 1 - below;
         if (pos >= 0 && pos < m.capacity) m.heap[pos] = idx;
-        m.klog[idx] = kEmpty;
+        if (static_cast<uint32_t>(idx) < static_cast<uint32_t>(m.capacity)) m.klog[idx] = kEmpty;
     }
 }
 
@@ -1388,6 +1413,36 @@ __global__ __launch_bounds__(kCollectThreads) void collect_touched_kernel(
     if (threadIdx.x == 0) ctr[kCtrTicket] = 0;
 }
 
+// Puts the entries of the packed region back into an emptied bucket array:
+// entry i of the key log is the code stored under index i.  `identity`: only
+// the entries below the size are in use (see items_kernel).
+__global__ __launch_bounds__(kHeapBlock) void replace_from_log_kernel(MapDev m, int identity) {
+    const int64_t limit = identity ? static_cast<int64_t>(m.ctr[kCtrSize])
+                                   : static_cast<int64_t>(m.capacity);
+    const ValueArgs none = {};
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kHeapBlock;
+    for (int64_t first = static_cast<int64_t>(blockIdx.x) * kHeapBlock; first < limit;
+         first += stride) {
+        const int64_t i = first + threadIdx.x;
+        const uint64_t code = i < limit ? m.klog[i] : kEmpty;
+        const int32_t k[1] = {0};
+        insert_key<1, kInsertLoad>(m, k, code, true, i, code < kTomb, none, nullptr, nullptr);
+    }
+}
+
+// Entries of a heap that address no row, counted with the pairs a load refuses.
+__global__ __launch_bounds__(kBlock) void check_heap_kernel(const int32_t* __restrict__ heap,
+                                                           int64_t capacity,
+                                                           int32_t* __restrict__ ctr) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    int bad = 0;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < capacity;
+         i += stride) {
+        bad += static_cast<uint32_t>(heap[i]) >= static_cast<uint32_t>(capacity) ? 1 : 0;
+    }
+    if (bad) atomicAdd(ctr + kCtrLoadDup, bad);
+}
+
 // ---------------------------------------------------------------- host
 inline unsigned grid_for(int64_t n, int per_block = kBlock) {
     return static_cast<unsigned>((n + per_block - 1) / per_block);
@@ -1442,6 +1497,16 @@ int launch_ray_sample(ash_map_t* map, const float* origins, const float* directi
 int check_map(const ash_map* map) {
     if (map == nullptr) ASH_FAIL("null map handle");
     return 0;
+}
+
+// Whether a listing has entry i under index i: nothing has written to the heap
+// since it was last 0, 1, 2, ... (no erase, no load) and no entry lives in the
+// second region -- there is none, or the counters as the host knows them say
+// that it is empty.
+bool lists_in_index_order(const ash_map* map) {
+    if (map->heap_dirty) return false;
+    return !map->general_attached ||
+           (map->counters_known && map->counters.general_live == 0);
 }
 
 int fill_buckets(ash_map* map, hipStream_t s) {
@@ -1587,6 +1652,16 @@ int settle_table(ash_map* map, hipStream_t s) {
     return fill_buckets(map, s);
 }
 
+void counters_changed(ash_map* map, bool inserted) {
+    map->counters_known = false;
+    map->late_pending = false;   // what a queued read-back brings is out of date
+    if (inserted) {
+        ++map->unread_inserts;
+    } else {
+        map->maybe_tombstones = true;
+    }
+}
+
 int check_batch(const ash_map* map, const void* keys, int64_t n) {
     if (check_map(map)) return 1;
     if (n < 0) ASH_FAIL("negative key count");
@@ -1675,6 +1750,13 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->table_stale = false;
     map->heap_dirty = true;   // the caller's buffer holds anything
     map->log_stale = false;
+    map->staging = nullptr;
+    map->early_event = map->late_event = nullptr;
+    map->late_in_flight = map->late_pending = false;
+    map->counters_known = true;   // a new map is empty and every counter is zero
+    map->counters = {};
+    map->maybe_tombstones = false;
+    map->unread_inserts = 0;
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
@@ -1718,10 +1800,18 @@ int ash_map_attach_general(ash_map_t* map, void* general_ws,
     ASH_LAUNCH_CHECK();
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrExotic, 0);
     ASH_LAUNCH_CHECK();
+    if (map->counters_known) map->counters.exotic_pending = 0;
+    map->late_pending = false;
     return 0;
 }
 
 int ash_map_destroy(ash_map_t* map) {
+    if (map == nullptr) return 0;
+    // the device may still owe a write into the caller's page-locked landing
+    // place; it must have arrived before the caller gives that memory back
+    if (map->late_in_flight && map->late_event != nullptr) (void)hipEventSynchronize(map->late_event);
+    if (map->early_event != nullptr) (void)hipEventDestroy(map->early_event);
+    if (map->late_event != nullptr) (void)hipEventDestroy(map->late_event);
     delete map;
     return 0;
 }
@@ -1800,6 +1890,7 @@ int launch_activate(ash_map_t* map, const float* cells, int64_t n, int grid_dim,
                     int dilation, int bidirectional, int bound_lo, int bound_hi,
                     uint8_t* touched, int32_t* coords, int32_t* heads, hipStream_t s) {
     if (settle_table(map, s)) return 1;
+    counters_changed(map, true);
     const int lo = bidirectional ? -dilation : 0;
     const int width = dilation - lo + 1;
     const float g = static_cast<float>(grid_dim);
@@ -1999,6 +2090,7 @@ int ash_map_insert_keys(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
+    counters_changed(map, true);
     ValueArgs va = {};
     return launch_insert<kInsertKeys>(map, keys, n, va, nullptr, nullptr,
                                       static_cast<hipStream_t>(stream));
@@ -2107,6 +2199,7 @@ int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
+    counters_changed(map, true);
     ValueArgs va = {};
     if (!ash_map_insert_needs_scratch(n_values, row_bytes)) {
         va.n = n_values;
@@ -2141,6 +2234,7 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
+    counters_changed(map, false);
     const unsigned g = grid_for(n, kEraseBlock);
     switch (map->key_dim) {
         case 1:
@@ -2164,66 +2258,347 @@ int ash_map_clear(ash_map_t* map, void* stream) {
     if (check_map(map)) return 1;
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    return clear_table(map, static_cast<hipStream_t>(stream), true, 0, true);
+    if (clear_table(map, static_cast<hipStream_t>(stream), true, 0, true)) return 1;
+    // every counter is zero again: known without a read-back
+    map->counters_known = true;
+    map->counters = {};
+    map->late_pending = false;
+    map->maybe_tombstones = false;
+    map->unread_inserts = 0;
+    return 0;
 }
 
 namespace {
 
-// `staging`: eight int32 of page-locked host memory of the caller's, or NULL.
-// A copy into pageable memory goes through the runtime's own staging and
-// takes about twice as long (25 against 13 us on an idle device).
-int read_status(ash_map_t* map, int32_t* staging, int64_t out[5], int64_t* touched, void* stream) {
-    if (check_map(map)) return 1;
-    if (out == nullptr) ASH_FAIL("null status output");
-    DeviceGuard guard;
-    ASH_HIP(guard.enter(map->device));
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    int32_t pageable[8] = {0};
-    int32_t* host = staging != nullptr ? staging : pageable;
-    ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(pageable), hipMemcpyDeviceToHost, s));
-    ASH_HIP(hipStreamSynchronize(s));
-    out[0] = host[kCtrSize];
-    out[1] = host[kCtrDropped];
-    out[2] = host[kCtrTombs];
-    out[3] = host[kCtrExotic];
-    out[4] = host[kCtrLoadDup];
-    if (touched != nullptr) *touched = host[kCtrTouched];
+void decode_counters(const int32_t* host, ash_counters& c) {
+    c.size = host[kCtrSize];
+    c.dropped = host[kCtrDropped];
+    c.tombstones = host[kCtrTombs];
+    c.exotic_pending = host[kCtrExotic];
+    c.load_refused = host[kCtrLoadDup];
+    c.touched = host[kCtrTouched];
+    c.general_live = host[kCtrGenLive];
+}
+
+int ensure_events(ash_map* map) {
+    if (map->early_event == nullptr) {
+        ASH_HIP(hipEventCreateWithFlags(&map->early_event, hipEventDisableTiming));
+    }
+    if (map->late_event == nullptr) {
+        ASH_HIP(hipEventCreateWithFlags(&map->late_event, hipEventDisableTiming));
+    }
+    return 0;
+}
+
+// A copy into the map's own landing place that may still be under way has to
+// arrive before that memory is written or read for something else.
+int settle_landing_place(ash_map* map) {
+    if (map->late_in_flight) {
+        ASH_HIP(hipEventSynchronize(map->late_event));
+        map->late_in_flight = false;
+    }
+    return 0;
+}
+
+// Brings map->counters up to date (the map's device is current): they are
+// known already, or a read-back queued behind the latest insert brings them,
+// or they are copied now, which waits for `s`.  `staging`: eight int32 of
+// page-locked host memory of the calling thread's, or null -- a copy into
+// pageable memory goes through the runtime's own staging and takes about twice
+// as long (25 against 13 us on an idle device).
+int refresh_counters(ash_map* map, int32_t* staging, hipStream_t s) {
+    if (map->counters_known) return 0;
+    if (map->late_pending) {
+        if (settle_landing_place(map)) return 1;
+        map->late_pending = false;
+        decode_counters(map->staging, map->counters);
+    } else {
+        int32_t pageable[kHostCounters] = {0};
+        int32_t* host = staging != nullptr ? staging : pageable;
+        ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(pageable), hipMemcpyDeviceToHost, s));
+        ASH_HIP(hipStreamSynchronize(s));
+        decode_counters(host, map->counters);
+    }
+    map->counters_known = true;
+    map->unread_inserts = 0;
+    if (map->counters.dropped > 0 || map->counters.tombstones > 0) map->maybe_tombstones = true;
+    return 0;
+}
+
+bool is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+// Inserts whose counters nobody read (deferred activations) between two looks
+// at them for tombstone upkeep.
+constexpr int kUpkeepEvery = 64;
+
+int64_t rebuild_scratch_bytes(const ash_map* map) {
+    const int64_t keys = (map->capacity * map->key_dim * 4 + 255) & ~int64_t{255};
+    return keys + map->capacity * 8;
+}
+
+bool should_rebuild(const ash_map* map, int64_t size, int64_t tombstones, int64_t incoming) {
+    if (tombstones <= 0) return false;
+    int64_t room = map->capacity - size;
+    if (room < 0) room = 0;
+    const int64_t arriving = incoming < room ? incoming : room;
+    int64_t slots = static_cast<int64_t>(map->d.nb) * kSlots;
+    if (map->general_attached && map->d.gslots < slots) slots = map->d.gslots;
+    // keep at least a fifth of the slots truly empty
+    return (size + tombstones + arriving) * 5 > slots * 4;
+}
+
+// Before an insert of `incoming` keys (the map's device is current, `s` is not
+// being captured): if earlier erases or refused keys may have left
+// tombstones, looks at the counters and re-places the live entries into an
+// emptied table when too few empty slots would remain.
+int upkeep(ash_map* map, int64_t incoming, void* scratch, int64_t scratch_bytes,
+           int32_t* staging, hipStream_t s) {
+    if (map->late_pending && refresh_counters(map, staging, s)) return 1;
+    if (map->unread_inserts >= kUpkeepEvery) map->maybe_tombstones = true;
+    if (!map->maybe_tombstones) return 0;
+    if (refresh_counters(map, staging, s)) return 1;
+    const ash_counters& c = map->counters;
+    map->maybe_tombstones = c.tombstones > 0;
+    if (!should_rebuild(map, c.size, c.tombstones, incoming)) return 0;
+    int32_t* keys = nullptr;
+    int64_t* indices = nullptr;
+    if (map->general_attached && c.size > 0) {
+        // entries of the second region do not stand in the key log: the pairs
+        // are listed into the caller's scratch and put back from there
+        if (scratch == nullptr || scratch_bytes < rebuild_scratch_bytes(map)) {
+            ASH_FAIL("scratch too small to re-place the entries: size it with "
+                     "ash_map_insert_scratch_bytes before every insert");
+        }
+        keys = static_cast<int32_t*>(scratch);
+        indices = reinterpret_cast<int64_t*>(
+                static_cast<char*>(scratch) +
+                ((map->capacity * map->key_dim * 4 + 255) & ~int64_t{255}));
+    }
+    if (ash_map_rebuild(map, keys, indices, c.size, s)) return 1;
+    map->counters.tombstones = 0;
+    map->counters_known = true;
+    map->maybe_tombstones = false;
     return 0;
 }
 
 }  // namespace
 
-int ash_map_status_begin(ash_map_t* map, int32_t* staging, void* event, void* stream) {
+int ash_map_set_staging(ash_map_t* map, int32_t* staging) {
     if (check_map(map)) return 1;
-    if (staging == nullptr) ASH_FAIL("null staging buffer");
-    DeviceGuard guard;
-    ASH_HIP(guard.enter(map->device));
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    ASH_HIP(hipMemcpyAsync(staging, map->d.ctr, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
-    if (event != nullptr) ASH_HIP(hipEventRecord(static_cast<hipEvent_t>(event), s));
+    if (settle_landing_place(map)) return 1;
+    if (map->late_pending) {
+        // what the old landing place holds is the latest state of the counters
+        decode_counters(map->staging, map->counters);
+        map->counters_known = true;
+        map->late_pending = false;
+    }
+    map->staging = staging;
     return 0;
 }
 
-int ash_map_status_decode(const int32_t* staging, int64_t out[6]) {
-    if (staging == nullptr) ASH_FAIL("null staging buffer");
+int ash_map_counters(ash_map_t* map, int32_t* staging, int64_t out[7], void* stream) {
+    if (check_map(map)) return 1;
     if (out == nullptr) ASH_FAIL("null status output");
-    out[0] = staging[kCtrSize];
-    out[1] = staging[kCtrDropped];
-    out[2] = staging[kCtrTombs];
-    out[3] = staging[kCtrExotic];
-    out[4] = staging[kCtrLoadDup];
-    out[5] = staging[kCtrTouched];
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    if (refresh_counters(map, staging, static_cast<hipStream_t>(stream))) return 1;
+    const ash_counters& c = map->counters;
+    out[0] = c.size;
+    out[1] = c.dropped;
+    out[2] = c.tombstones;
+    out[3] = c.exotic_pending;
+    out[4] = c.load_refused;
+    out[5] = c.touched;
+    out[6] = c.general_live;
     return 0;
+}
+
+int ash_map_counters_pending(ash_map_t* map) {
+    return map != nullptr && map->late_pending ? 1 : 0;
+}
+
+int ash_map_known_size(ash_map_t* map, int64_t* size) {
+    if (check_map(map)) return -1;
+    if (size == nullptr) {
+        set_error("null size output");
+        return -1;
+    }
+    if (!map->counters_known) {
+        if (!map->late_pending) return 0;
+        DeviceGuard guard;
+        if (guard.enter(map->device) != hipSuccess || refresh_counters(map, nullptr, nullptr)) {
+            return -1;
+        }
+    }
+    *size = map->counters.size;
+    return 1;
 }
 
 int ash_map_status(ash_map_t* map, int64_t out[5], void* stream) {
-    return read_status(map, nullptr, out, nullptr, stream);
+    if (check_map(map)) return 1;
+    if (out == nullptr) ASH_FAIL("null status output");
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    // always a copy from the device
+    map->counters_known = false;
+    map->late_pending = false;
+    if (refresh_counters(map, nullptr, static_cast<hipStream_t>(stream))) return 1;
+    const ash_counters& c = map->counters;
+    out[0] = c.size;
+    out[1] = c.dropped;
+    out[2] = c.tombstones;
+    out[3] = c.exotic_pending;
+    out[4] = c.load_refused;
+    return 0;
 }
 
-int ash_map_status_staged(ash_map_t* map, int32_t* staging, int64_t out[6], void* stream) {
-    if (staging == nullptr) ASH_FAIL("null staging buffer");
-    if (out == nullptr) ASH_FAIL("null status output");
-    return read_status(map, staging, out, out + 5, stream);
+int ash_map_upkeep(ash_map_t* map, int64_t incoming, void* scratch, int64_t scratch_bytes,
+                   int32_t* staging, void* stream) {
+    if (check_map(map)) return 1;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (is_capturing(s)) return 0;
+    return upkeep(map, incoming, scratch, scratch_bytes, staging, s);
+}
+
+namespace {
+
+// Which path an insert of this batch takes; *bytes = device scratch it needs.
+enum { kPathPerKey = 0, kPathAssigned = 1, kPathStreaming = 2 };
+
+int plan_insert(ash_map_t* map, int64_t n, int n_values, const int64_t* row_bytes, int policy,
+                int* path, int64_t* bytes) {
+    if (policy < ASH_STREAMING_AUTO || policy > ASH_STREAMING_NEVER) ASH_FAIL("unknown policy");
+    if (n_values < 0) ASH_FAIL("negative value count");
+    if (n_values > 0 && row_bytes == nullptr) ASH_FAIL("null value tables");
+    *path = kPathPerKey;
+    *bytes = 0;
+    if (n_values > 0 && ash_map_insert_needs_scratch(n_values, row_bytes)) {
+        *path = kPathAssigned;
+        *bytes = n * 4;
+    } else if (policy != ASH_STREAMING_NEVER) {
+        int64_t ws = 0;
+        int worthwhile = 0;
+        if (ash_map_bulk_workspace_bytes(map, n, n_values, row_bytes, &ws, &worthwhile)) return 1;
+        if (ws > 0 && (worthwhile || policy == ASH_STREAMING_ALWAYS)) {
+            *path = kPathStreaming;
+            *bytes = ws;
+        }
+    }
+    // a map with a second region re-places its entries through the scratch
+    if (map->general_attached &&
+        (map->maybe_tombstones || map->unread_inserts >= kUpkeepEvery)) {
+        const int64_t r = rebuild_scratch_bytes(map);
+        if (r > *bytes) *bytes = r;
+    }
+    return 0;
+}
+
+}  // namespace
+
+int ash_map_insert_scratch_bytes(ash_map_t* map, int64_t n, int n_values,
+                                 const int64_t* row_bytes, int policy, int64_t* bytes) {
+    if (check_map(map)) return 1;
+    if (bytes == nullptr) ASH_FAIL("null output pointer");
+    if (n < 0) ASH_FAIL("negative key count");
+    int path = 0;
+    return plan_insert(map, n, n_values, row_bytes, policy, &path, bytes);
+}
+
+int ash_map_insert_auto(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
+                        const void* const* src, void* const* dst, const int64_t* row_bytes,
+                        void* scratch, int64_t scratch_bytes, int policy, int32_t* staging,
+                        void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n == 0) return 0;
+    int path = 0;
+    int64_t need = 0;
+    if (plan_insert(map, n, n_values, row_bytes, policy, &path, &need)) return 1;
+    if (need > 0 && (scratch == nullptr || scratch_bytes < need)) {
+        ASH_FAIL("insert scratch too small: size it with ash_map_insert_scratch_bytes");
+    }
+    if (need > 0 && reinterpret_cast<uintptr_t>(scratch) % 256 != 0) {
+        ASH_FAIL("insert scratch must be 256-byte aligned");
+    }
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool capturing = is_capturing(s);
+    // (a capture replays launches only: no look at the counters, no upkeep;
+    // refused keys stay in the counters for a later call to find)
+    if (!capturing && upkeep(map, n, scratch, scratch_bytes, staging, s)) return 1;
+    if (path == kPathStreaming) {
+        int32_t* early = nullptr;
+        if (!capturing && map->staging != nullptr) {
+            if (ensure_events(map) || settle_landing_place(map)) return 1;
+            early = map->staging + kHostCounters;
+        }
+        if (insert_bulk(map, keys, n, n_values, src, dst, row_bytes, scratch, scratch_bytes,
+                        early, early != nullptr ? map->early_event : nullptr, stream)) {
+            return 1;
+        }
+        if (capturing) return 0;
+        if (early != nullptr) {
+            // Only keys that the first pass hands to the per-key kernel can be
+            // waiting for the second region; their number arrives a quarter
+            // into the call's work.  None: the counters are fetched behind the
+            // insert without waiting for them.
+            ASH_HIP(hipEventSynchronize(map->early_event));
+            if (*early == 0) {
+                ASH_HIP(hipMemcpyAsync(map->staging, map->d.ctr, kHostCounters * sizeof(int32_t),
+                                       hipMemcpyDeviceToHost, s));
+                ASH_HIP(hipEventRecord(map->late_event, s));
+                map->late_in_flight = true;
+                map->late_pending = true;
+                map->unread_inserts = 0;
+                return 0;
+            }
+        }
+    } else {
+        if (ash_map_insert(map, keys, n, n_values, src, dst, row_bytes,
+                           path == kPathAssigned ? static_cast<int32_t*>(scratch) : nullptr,
+                           stream)) {
+            return 1;
+        }
+        if (capturing) return 0;
+    }
+    if (refresh_counters(map, staging, s)) return 1;
+    if (map->counters.exotic_pending > 0) {
+        set_error("keys that do not fit the packed code are waiting for the second region: "
+                  "attach it (ash_map_attach_general) and issue the insert again");
+        return ASH_NEEDS_GENERAL;
+    }
+    return 0;
+}
+
+int ash_map_erase_scratch_bytes(ash_map_t* map, int64_t n, int policy, int64_t* bytes) {
+    if (check_map(map)) return 1;
+    if (bytes == nullptr) ASH_FAIL("null output pointer");
+    if (policy < ASH_STREAMING_AUTO || policy > ASH_STREAMING_NEVER) ASH_FAIL("unknown policy");
+    *bytes = 0;
+    if (policy == ASH_STREAMING_NEVER) return 0;
+    int64_t ws = 0;
+    int worthwhile = 0;
+    if (ash_map_erase_bulk_query(map, n, &ws, &worthwhile)) return 1;
+    if (ws > 0 && (worthwhile || policy == ASH_STREAMING_ALWAYS)) *bytes = ws;
+    return 0;
+}
+
+int ash_map_erase_auto(ash_map_t* map, const int32_t* keys, int64_t n, void* scratch,
+                       int64_t scratch_bytes, int policy, void* stream) {
+    if (check_batch(map, keys, n)) return 1;
+    if (n == 0) return 0;
+    int64_t need = 0;
+    if (ash_map_erase_scratch_bytes(map, n, policy, &need)) return 1;
+    if (need == 0) return ash_map_erase(map, keys, n, stream);
+    if (scratch == nullptr || scratch_bytes < need) {
+        ASH_FAIL("erase scratch too small: size it with ash_map_erase_scratch_bytes");
+    }
+    return ash_map_erase_bulk(map, keys, n, scratch, scratch_bytes, stream);
 }
 
 int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* block_coords,
@@ -2242,6 +2617,8 @@ int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* bl
     if (groups > kCollectGroups) groups = kCollectGroups;
     const int words = static_cast<int>((map->capacity + groups * per_group - 1) / (groups * per_group));
     groups = (map->capacity + words * per_group - 1) / (words * per_group);   // no empty chunks
+    map->counters_known = false;   // the number of listed rows is one of them
+    map->late_pending = false;
     collect_touched_kernel<<<static_cast<unsigned>(groups), kCollectThreads, 0,
                              static_cast<hipStream_t>(stream)>>>(
             touched, block_coords, map->capacity, words, out_indices, out_coords, map->d.ctr);
@@ -2251,9 +2628,9 @@ int ash_grid_collect_touched(ash_map_t* map, uint8_t* touched, const int32_t* bl
 
 int ash_map_size(ash_map_t* map, int64_t* size, void* stream) {
     if (size == nullptr) ASH_FAIL("null size output");
-    int64_t st[5];
-    if (ash_map_status(map, st, stream)) return 1;
-    *size = st[0];
+    int64_t c[7];
+    if (ash_map_counters(map, nullptr, c, stream)) return 1;
+    *size = c[0];
     return 0;
 }
 
@@ -2270,7 +2647,9 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     const int identity = map->heap_dirty ? 0 : 1;
-    if (identity && !map->general_attached) {
+    const bool none_in_general = !map->general_attached ||
+                                 (map->counters_known && map->counters.general_live == 0);
+    if (lists_in_index_order(map)) {
         const int64_t n = n_expected < map->capacity ? n_expected : map->capacity;
         const unsigned gd = grid_for(n);
         switch (map->key_dim) {
@@ -2312,7 +2691,7 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
             break;
     }
     ASH_LAUNCH_CHECK();
-    if (map->general_attached) {
+    if (!none_in_general) {
         const unsigned gg = grid_for(map->d.gslots);
         switch (map->key_dim) {
             case 1:
@@ -2339,24 +2718,22 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
 
 int ash_map_should_rebuild(ash_map_t* map, int64_t size, int64_t tombstones,
                            int64_t incoming) {
-    if (map == nullptr || tombstones <= 0) return 0;
-    int64_t room = map->capacity - size;
-    if (room < 0) room = 0;
-    const int64_t arriving = incoming < room ? incoming : room;
-    int64_t slots = static_cast<int64_t>(map->d.nb) * kSlots;
-    if (map->general_attached && map->d.gslots < slots) slots = map->d.gslots;
-    // keep at least a fifth of the slots truly empty
-    return (size + tombstones + arriving) * 5 > slots * 4 ? 1 : 0;
+    if (map == nullptr) return 0;
+    return should_rebuild(map, size, tombstones, incoming) ? 1 : 0;
 }
 
 int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
                     int64_t* indices_scratch, int64_t n, void* stream) {
     if (check_map(map)) return 1;
     if (n < 0 || n > map->capacity) ASH_FAIL("rebuild: bad entry count");
-    if (n > 0 && (keys_scratch == nullptr || indices_scratch == nullptr)) {
+    // Without a second region every entry stands in the key log under its
+    // index and is put back from there; with one, the pairs are listed into the
+    // caller's scratch first.
+    const bool from_log = !map->general_attached;
+    if (!from_log && n > 0 && (keys_scratch == nullptr || indices_scratch == nullptr)) {
         ASH_FAIL("rebuild: null scratch pointer");
     }
-    if (n > 0 && ash_map_items(map, keys_scratch, indices_scratch, n, stream)) {
+    if (!from_log && n > 0 && ash_map_items(map, keys_scratch, indices_scratch, n, stream)) {
         return 1;
     }
     DeviceGuard guard;
@@ -2368,10 +2745,22 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
         fill16_kernel<<<capped_grid(g16), kBlock, 0, s>>>(
                 reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
         ASH_LAUNCH_CHECK();
+        set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrGenLive, 0);   // counted again below
+        ASH_LAUNCH_CHECK();
     }
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrTombs, 0);
     ASH_LAUNCH_CHECK();
+    map->counters_known = false;
+    map->late_pending = false;
     if (n == 0) return 0;
+    if (from_log) {
+        int64_t g = (map->capacity + kHeapBlock - 1) / kHeapBlock;
+        if (g > 256 * 16) g = 256 * 16;
+        replace_from_log_kernel<<<static_cast<unsigned>(g), kHeapBlock, 0, s>>>(
+                map->d, map->heap_dirty ? 0 : 1);
+        ASH_LAUNCH_CHECK();
+        return 0;
+    }
     ValueArgs va = {};
     return launch_insert<kInsertLoad>(map, keys_scratch, n, va, nullptr,
                                       indices_scratch, s);
@@ -2380,7 +2769,7 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
 int ash_map_items_in_index_order(ash_map_t* map, int* dense) {
     if (check_map(map)) return 1;
     if (dense == nullptr) ASH_FAIL("null output pointer");
-    *dense = (!map->heap_dirty && !map->general_attached) ? 1 : 0;
+    *dense = lists_in_index_order(map) ? 1 : 0;
     return 0;
 }
 
@@ -2394,11 +2783,20 @@ int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (clear_table(map, s, false, static_cast<int32_t>(n))) return 1;
     map->heap_dirty = true;   // the heap is the caller's from here on
+    map->counters_known = false;
+    map->late_pending = false;
+    map->maybe_tombstones = false;
+    map->unread_inserts = 0;
     if (heap_src != nullptr && heap_src != map->d.heap) {
         ASH_HIP(hipMemcpyAsync(map->d.heap, heap_src,
                                static_cast<size_t>(map->capacity) * 4,
                                hipMemcpyDeviceToDevice, s));
     }
+    // later inserts take their indices from this heap unchecked: entries that
+    // address no row are counted with the pairs the load refuses
+    check_heap_kernel<<<looping_grid(map->capacity), kBlock, 0, s>>>(map->d.heap, map->capacity,
+                                                                   map->d.ctr);
+    ASH_LAUNCH_CHECK();
     if (n == 0) return 0;
     ValueArgs va = {};
     return launch_insert<kInsertLoad>(map, keys, n, va, nullptr, indices, s);

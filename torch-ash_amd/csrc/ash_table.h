@@ -149,6 +149,16 @@ int erase_selected(ash_map* map, bool codes, const void* keys, const int32_t* se
                    const int32_t* nsel, hipStream_t s);
 
 int check_batch(const ash_map* map, const void* keys, int64_t n);
+// What the host keeps of the counters no longer holds: `inserted` for a call
+// that may have added entries (and ended without a look at the counters),
+// false for one that took entries away.
+void counters_changed(ash_map* map, bool inserted);
+// The streaming insert (ash_bulk.hip); `early`, `early_event` as for
+// ash_map_insert_bulk_early (both may be null).
+int insert_bulk(ash_map* map, const int32_t* keys, int64_t n, int n_values,
+                const void* const* src, void* const* dst, const int64_t* row_bytes,
+                void* workspace, int64_t workspace_bytes, int32_t* early,
+                hipEvent_t early_event, void* stream);
 // Fills the bucket array if a clear() left that to the next user of the table.
 int settle_table(ash_map* map, hipStream_t s);
 // Before the first call that writes to the heap (an erase; a load brings a
