@@ -762,6 +762,48 @@ def bench_fusion(torch, ash, workloads, args, dev, frames=100):
             "touched_blocks_per_frame": round(touched / frames),
         }
         del grid
+    # the same frames with the launches of a frame recorded once into a HIP
+    # graph and replayed (ash_map_insert-style calls only queue launches on a
+    # capturing stream): inputs are rewritten in place, the point lists padded
+    # to one length with copies of their last point
+    most = max(d[0].shape[0] for d in data)
+    for rep in range(2):
+        grid = ash.UnBoundedSparseDenseGrid(3, 80000, 2, 8, cell_size=0.015, device=dev)
+        pts = torch.empty((most, 3), device=dev)
+        depth, ext = torch.empty_like(data[0][1]), torch.empty_like(data[0][2])
+
+        def load(frame):
+            p = data[frame][0]
+            pts[: len(p)] = p
+            pts[len(p):] = p[-1]
+            depth.copy_(data[frame][1])
+            ext.copy_(data[frame][2])
+
+        load(0)
+        ash.fusion.fuse_frame(grid, pts, depth, intrinsic, ext, 0.04, 6.0, count_blocks=False)
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            ash.fusion.fuse_frame(grid, pts, depth, intrinsic, ext, 0.04, 6.0, count_blocks=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for frame in range(1, frames):
+            load(frame)
+            graph.replay()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        # the replays alone (inputs left as they are): what the graph costs
+        t_replay = EventTimer(torch)
+        for _ in range(20):
+            t_replay(graph.replay)
+        replay_ms = t_replay.mean_ms()
+    out["fused_graph_replay"] = {
+        "frames_per_s": round((frames - 1) / dt, 1),
+        "ms_per_frame": round(dt / (frames - 1) * 1e3, 3),
+        "ms_per_replay_alone": round(replay_ms, 4),
+        "active_blocks": grid.engine.size(),
+    }
+    del grid
     torch.cuda.empty_cache()
     return out
 

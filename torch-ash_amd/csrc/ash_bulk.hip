@@ -1355,15 +1355,11 @@ int ash::insert_bulk(ash_map* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (map->table_stale) {
+    if (map->table_stale && is_capturing(s)) {
         // A cleared table whose fill is still pending is rewritten whole by the
         // build pass.  Captured into a graph that decision would be replayed
         // against whatever the table holds then.
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &capturing) == hipSuccess &&
-            capturing != hipStreamCaptureStatusNone) {
-            ASH_FAIL("the table was cleared and not used since: run one call outside the capture first");
-        }
+        ASH_FAIL("the table was cleared and not used since: run one call outside the capture first");
     }
 
     ValueArgs user = {};
@@ -1375,13 +1371,10 @@ int ash::insert_bulk(ash_map* map, const int32_t* keys, int64_t n,
     }
     const ValueArgs none = {};
     const int stale = map->table_stale ? 1 : 0;
+    counters_changed(map, true, s);
     // (captured into a graph, the choice would be replayed whatever the heap
-    // holds then: a capture takes the variant that reads the heap)
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    const bool capturing = hipStreamIsCapturing(s, &cap) == hipSuccess &&
-                           cap != hipStreamCaptureStatusNone;
-    const int identity = (map->heap_dirty || capturing) ? 0 : 1;
-    counters_changed(map, true);
+    // holds then: a captured call takes the variant that reads the heap)
+    const int identity = heap_in_order(map) ? 1 : 0;
 
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
@@ -1467,7 +1460,7 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
-    counters_changed(map, false);
+    counters_changed(map, false, s);
     const int ncursors = static_cast<int>(pl.bins << pl.fine_shift);   // (>= bins << lane_shift)
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);

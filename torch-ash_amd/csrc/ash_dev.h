@@ -155,6 +155,12 @@ struct ash_map {
     // may have left tombstones: the next managed insert looks at the counters
     bool maybe_tombstones;
     int unread_inserts;
+    // A call that changes the map has been captured into a graph: replays
+    // change the device's state behind the host's back, so from then on nothing
+    // the host remembers of it is trusted -- the counters are copied from the
+    // device whenever they are asked for, the heap is read (never assumed to be
+    // 0, 1, 2, ...), listings go by ranks and a clear clears at once.
+    bool replayed;
     // clear() has reset the counters and the heap but left the bucket array as
     // it was: the next call that reads the table fills it first, a streaming
     // insert that rewrites every bucket does not need to

@@ -1194,6 +1194,16 @@ __global__ __launch_bounds__(kBlock) void reset_heap_kernel(
     }
 }
 
+// Keys counted as waiting for the second region although it is attached (a
+// graph captured before the attach still runs without it) cannot be issued
+// again by anybody: they are counted with the refused keys.
+__global__ void fold_waiting_keys_kernel(int32_t* ctr) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        ctr[kCtrDropped] += ctr[kCtrExotic];
+        ctr[kCtrExotic] = 0;
+    }
+}
+
 __global__ void set_counter_kernel(int32_t* ctr, int which, int32_t value) {
     if (threadIdx.x == 0 && blockIdx.x == 0) ctr[which] = value;
 }
@@ -1504,7 +1514,7 @@ int check_map(const ash_map* map) {
 // second region -- there is none, or the counters as the host knows them say
 // that it is empty.
 bool lists_in_index_order(const ash_map* map) {
-    if (map->heap_dirty) return false;
+    if (!heap_in_order(map)) return false;
     return !map->general_attached ||
            (map->counters_known && map->counters.general_live == 0);
 }
@@ -1652,7 +1662,8 @@ int settle_table(ash_map* map, hipStream_t s) {
     return fill_buckets(map, s);
 }
 
-void counters_changed(ash_map* map, bool inserted) {
+void counters_changed(ash_map* map, bool inserted, hipStream_t s) {
+    if (is_capturing(s)) map->replayed = true;
     map->counters_known = false;
     map->late_pending = false;   // what a queued read-back brings is out of date
     if (inserted) {
@@ -1757,6 +1768,7 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->counters = {};
     map->maybe_tombstones = false;
     map->unread_inserts = 0;
+    map->replayed = false;
     map->d.ctr = static_cast<int32_t*>(table_ws);
     map->d.buckets = reinterpret_cast<uint64_t*>(static_cast<char*>(table_ws) +
                                                  kHeaderBytes);
@@ -1890,7 +1902,7 @@ int launch_activate(ash_map_t* map, const float* cells, int64_t n, int grid_dim,
                     int dilation, int bidirectional, int bound_lo, int bound_hi,
                     uint8_t* touched, int32_t* coords, int32_t* heads, hipStream_t s) {
     if (settle_table(map, s)) return 1;
-    counters_changed(map, true);
+    counters_changed(map, true, s);
     const int lo = bidirectional ? -dilation : 0;
     const int width = dilation - lo + 1;
     const float g = static_cast<float>(grid_dim);
@@ -2090,7 +2102,7 @@ int ash_map_insert_keys(ash_map_t* map, const int32_t* keys, int64_t n,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     if (settle_table(map, static_cast<hipStream_t>(stream))) return 1;
-    counters_changed(map, true);
+    counters_changed(map, true, static_cast<hipStream_t>(stream));
     ValueArgs va = {};
     return launch_insert<kInsertKeys>(map, keys, n, va, nullptr, nullptr,
                                       static_cast<hipStream_t>(stream));
@@ -2199,7 +2211,7 @@ int ash_map_insert(ash_map_t* map, const int32_t* keys, int64_t n, int n_values,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
-    counters_changed(map, true);
+    counters_changed(map, true, s);
     ValueArgs va = {};
     if (!ash_map_insert_needs_scratch(n_values, row_bytes)) {
         va.n = n_values;
@@ -2234,7 +2246,7 @@ int ash_map_erase(ash_map_t* map, const int32_t* keys, int64_t n,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
     if (give_up_heap_order(map, s)) return 1;   // freed indices go back onto the heap
-    counters_changed(map, false);
+    counters_changed(map, false, s);
     const unsigned g = grid_for(n, kEraseBlock);
     switch (map->key_dim) {
         case 1:
@@ -2258,7 +2270,17 @@ int ash_map_clear(ash_map_t* map, void* stream) {
     if (check_map(map)) return 1;
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
-    if (clear_table(map, static_cast<hipStream_t>(stream), true, 0, true)) return 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (is_capturing(s)) map->replayed = true;
+    if (map->replayed) {
+        // what replays leave behind is unknown: everything is cleared now
+        if (settle_table(map, s)) return 1;
+        map->heap_dirty = true;
+        if (clear_table(map, s, true, 0, false)) return 1;
+        map->heap_dirty = true;   // (whatever the flag would say: see heap_in_order)
+    } else if (clear_table(map, s, true, 0, true)) {
+        return 1;
+    }
     // every counter is zero again: known without a read-back
     map->counters_known = true;
     map->counters = {};
@@ -2307,6 +2329,10 @@ int settle_landing_place(ash_map* map) {
 // pageable memory goes through the runtime's own staging and takes about twice
 // as long (25 against 13 us on an idle device).
 int refresh_counters(ash_map* map, int32_t* staging, hipStream_t s) {
+    if (map->replayed) {
+        if (settle_landing_place(map)) return 1;
+        map->counters_known = map->late_pending = false;
+    }
     if (map->counters_known) return 0;
     if (map->late_pending) {
         if (settle_landing_place(map)) return 1;
@@ -2323,11 +2349,6 @@ int refresh_counters(ash_map* map, int32_t* staging, hipStream_t s) {
     map->unread_inserts = 0;
     if (map->counters.dropped > 0 || map->counters.tombstones > 0) map->maybe_tombstones = true;
     return 0;
-}
-
-bool is_capturing(hipStream_t s) {
-    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
 }
 
 // Inserts whose counters nobody read (deferred activations) between two looks
@@ -2357,7 +2378,7 @@ bool should_rebuild(const ash_map* map, int64_t size, int64_t tombstones, int64_
 int upkeep(ash_map* map, int64_t incoming, void* scratch, int64_t scratch_bytes,
            int32_t* staging, hipStream_t s) {
     if (map->late_pending && refresh_counters(map, staging, s)) return 1;
-    if (map->unread_inserts >= kUpkeepEvery) map->maybe_tombstones = true;
+    if (map->unread_inserts >= kUpkeepEvery || map->replayed) map->maybe_tombstones = true;
     if (!map->maybe_tombstones) return 0;
     if (refresh_counters(map, staging, s)) return 1;
     const ash_counters& c = map->counters;
@@ -2426,6 +2447,7 @@ int ash_map_known_size(ash_map_t* map, int64_t* size) {
         set_error("null size output");
         return -1;
     }
+    if (map->replayed) return 0;
     if (!map->counters_known) {
         if (!map->late_pending) return 0;
         DeviceGuard guard;
@@ -2491,7 +2513,7 @@ int plan_insert(ash_map_t* map, int64_t n, int n_values, const int64_t* row_byte
     }
     // a map with a second region re-places its entries through the scratch
     if (map->general_attached &&
-        (map->maybe_tombstones || map->unread_inserts >= kUpkeepEvery)) {
+        (map->maybe_tombstones || map->unread_inserts >= kUpkeepEvery || map->replayed)) {
         const int64_t r = rebuild_scratch_bytes(map);
         if (r > *bytes) *bytes = r;
     }
@@ -2567,6 +2589,13 @@ int ash_map_insert_auto(ash_map_t* map, const int32_t* keys, int64_t n, int n_va
         if (capturing) return 0;
     }
     if (refresh_counters(map, staging, s)) return 1;
+    if (map->counters.exotic_pending > 0 && map->general_attached) {
+        fold_waiting_keys_kernel<<<1, 64, 0, s>>>(map->d.ctr);
+        ASH_LAUNCH_CHECK();
+        map->counters.dropped += map->counters.exotic_pending;
+        map->counters.exotic_pending = 0;
+        map->maybe_tombstones = true;
+    }
     if (map->counters.exotic_pending > 0) {
         set_error("keys that do not fit the packed code are waiting for the second region: "
                   "attach it (ash_map_attach_general) and issue the insert again");
@@ -2646,7 +2675,7 @@ int ash_map_items(ash_map_t* map, int32_t* keys_out, int64_t* indices_out,
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (settle_table(map, s)) return 1;
-    const int identity = map->heap_dirty ? 0 : 1;
+    const int identity = heap_in_order(map) ? 1 : 0;
     const bool none_in_general = !map->general_attached ||
                                  (map->counters_known && map->counters.general_live == 0);
     if (lists_in_index_order(map)) {
@@ -2757,7 +2786,7 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
         int64_t g = (map->capacity + kHeapBlock - 1) / kHeapBlock;
         if (g > 256 * 16) g = 256 * 16;
         replace_from_log_kernel<<<static_cast<unsigned>(g), kHeapBlock, 0, s>>>(
-                map->d, map->heap_dirty ? 0 : 1);
+                map->d, heap_in_order(map) ? 1 : 0);
         ASH_LAUNCH_CHECK();
         return 0;
     }
@@ -2781,6 +2810,7 @@ int ash_map_load(ash_map_t* map, const int32_t* keys, const int64_t* indices,
     DeviceGuard guard;
     ASH_HIP(guard.enter(map->device));
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (is_capturing(s)) ASH_FAIL("ash_map_load cannot be captured into a graph");
     if (clear_table(map, s, false, static_cast<int32_t>(n))) return 1;
     map->heap_dirty = true;   // the heap is the caller's from here on
     map->counters_known = false;

@@ -149,10 +149,19 @@ int erase_selected(ash_map* map, bool codes, const void* keys, const int32_t* se
                    const int32_t* nsel, hipStream_t s);
 
 int check_batch(const ash_map* map, const void* keys, int64_t n);
+inline bool is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+
+// Whether the heap array is known to be 0, 1, 2, ...
+inline bool heap_in_order(const ash_map* map) { return !map->heap_dirty && !map->replayed; }
+
 // What the host keeps of the counters no longer holds: `inserted` for a call
 // that may have added entries (and ended without a look at the counters),
 // false for one that took entries away.
-void counters_changed(ash_map* map, bool inserted);
+// `s`: the stream the call runs on (captured: see ash_map::replayed).
+void counters_changed(ash_map* map, bool inserted, hipStream_t s);
 // The streaming insert (ash_bulk.hip); `early`, `early_event` as for
 // ash_map_insert_bulk_early (both may be null).
 int insert_bulk(ash_map* map, const int32_t* keys, int64_t n, int n_values,
