@@ -67,8 +67,13 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap,
                    void* table_ws, int64_t table_bytes, int device,
                    void* stream, ash_map_t** out);
 
-/* Hands the map its second region (device buffer of >= general_bytes bytes).
- * Idempotent per handle: a second attach is an error. */
+/* Hands the map its second region: a 256-byte aligned device buffer of
+ * general_bytes bytes, 20 per slot.  ash_map_workspace_bytes' general_bytes is
+ * what `capacity` keys need at half load; a smaller buffer is taken as the
+ * largest power of two of slots that fits (at least 64) -- enough for a caller
+ * who attaches it ahead of time for keys that are not expected (a key that
+ * finds such a region full is refused and counted like a key that finds the
+ * map full).  Idempotent per handle: a second attach is an error. */
 int ash_map_attach_general(ash_map_t* map, void* general_ws,
                            int64_t general_bytes, void* stream);
 

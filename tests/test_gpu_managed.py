@@ -214,6 +214,39 @@ def test_listing_stays_in_index_order_with_an_empty_second_region(gpu_ash):
     assert not backend.last_items_in_index_order and len(k) == len(keys)
 
 
+def test_second_region_of_the_callers_size(gpu_ash, oracle):
+    """ash_map_attach_general takes a region smaller than what the capacity
+    would need (attached ahead of time for keys that are not expected): keys
+    that do not fit the packed code live there like in a full-sized one, and
+    when it is full further ones are refused and counted, like keys that find
+    the map full."""
+    rng = np.random.default_rng(4500)
+    wide = torch.from_numpy(rng.integers(2**22, 2**30, size=(300, 3)).astype(np.int32))
+    wide = torch.unique(wide, dim=0)
+    engine = gpu_ash.ASHEngine(3, 100_000, DEV)
+    engine.backend._attach_general(just_in_case=True)
+    assert engine.backend._general.numel() == 20 << 16 < engine.backend._general_bytes
+    omap = _oracle_map(oracle, 3, 100_000)
+    batch = torch.cat([_keys(rng, 20_000, 40), wide])
+    engine.insert_keys(batch.to(DEV))
+    omap.insert_keys(batch)
+    _assert_same_map(engine, omap, torch.cat([wide, wide + 1, batch[:3000]]).to(DEV))
+    assert engine.backend.counters()["general_live"] == len(wide)
+    engine.erase(wide[:100].to(DEV))
+    omap.erase(wide[:100])
+    _assert_same_map(engine, omap, wide.to(DEV))
+    # the smallest region: 64 slots
+    raw = RawMap(gpu_ash, 3, 10_000)
+    raw.general = torch.empty(64 * 20, dtype=torch.uint8, device=DEV)
+    raw.check(raw.lib.ash_map_attach_general(raw.handle, raw.general.data_ptr(), 64 * 20, raw.stream))
+    raw.insert(torch.cat([_keys(rng, 2000, 30), wide]), NEVER)
+    c = raw.counters()
+    assert c["general"] <= 64 and c["general"] + c["dropped"] == len(wide)
+    _, mask = raw.find(wide)
+    assert int(mask.sum()) == c["general"]
+    assert raw.lib.ash_map_attach_general(raw.handle, raw.general.data_ptr(), 63 * 20, raw.stream) != 0
+
+
 def test_states_that_address_no_row_are_refused(gpu_ash):
     """A state dict whose indices or heap entries lie outside 0 .. capacity-1
     would make later calls write outside the value rows and the key log

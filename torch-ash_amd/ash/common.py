@@ -255,6 +255,9 @@ RAY_STAGE_EXTRA = 2
 # Largest table whose touched rows ash_grid_collect_touched lists (the header's
 # ASH_COLLECT_MAX_BLOCKS).
 COLLECT_MAX_BLOCKS = 1 << 20
+# Size of a second region that is attached before any key has asked for it
+# (2^16 slots of 20 bytes).
+GENERAL_JUST_IN_CASE_BYTES = 20 << 16
 # Most positions per call of ash_grid_activate_static (the header's
 # ASH_ACTIVATE_STATIC_MAX_POSITIONS).
 ACTIVATE_STATIC_MAX = 1 << 20
@@ -1073,16 +1076,20 @@ class _HashMap:
     def _scratch(self, nbytes: int) -> Optional[torch.Tensor]:
         return torch.empty(nbytes, dtype=torch.uint8, device=self._device) if nbytes else None
 
-    def _attach_general(self) -> None:
+    def _attach_general(self, just_in_case: bool = False) -> None:
         """Hands the table its second region (keys that do not fit the packed
-        code live there)."""
+        code live there): sized for the capacity once such a key has shown up,
+        or -- `just_in_case`, ahead of time by a path that cannot come back for
+        it -- for a few thousand of them."""
         if self._general is not None:
             raise RuntimeError("internal error: unpackable keys pending with region attached")
-        self._general = torch.empty(self._general_bytes, dtype=torch.uint8, device=self._device)
+        nbytes = min(self._general_bytes, GENERAL_JUST_IN_CASE_BYTES) if just_in_case \
+            else self._general_bytes
+        self._general = torch.empty(nbytes, dtype=torch.uint8, device=self._device)
         with torch.cuda.device(self._device):
             self._check(
                 self._lib.ash_map_attach_general(
-                    self._handle, self._general.data_ptr(), self._general_bytes, self._stream()
+                    self._handle, self._general.data_ptr(), nbytes, self._stream()
                 )
             )
 
@@ -1278,7 +1285,7 @@ class _HashMap:
         if self._general is None:
             # a key beyond the packed range would otherwise wait for a read-back
             # that this path does not make
-            self._attach_general()
+            self._attach_general(just_in_case=True)
         self._upkeep(n)
         coords, rows = self._listing
         head = (self._handle, cells.data_ptr(), n, int(grid_dim), int(dilation),

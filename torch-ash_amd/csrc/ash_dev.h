@@ -65,10 +65,11 @@ enum Counter {
     kCtrLoadDup = 4,   // pairs refused by load: duplicate keys, indices outside 0 .. capacity-1
     kCtrGenLive = 5,   // entries that live in the general region
     kCtrTouched = 6,   // blocks listed by the latest ash_grid_collect_touched
-    kCtrTicket = 7,    // workgroups of a running ash_grid_collect_touched that have read their input
+    kCtrGenTombs = 7,  // of kCtrTombs, those in the general region
     // (the first eight are what a read-back of the counters copies to the host)
     kCtrLogHigh = 8,   // log entries at or beyond the size and below this index may hold keys of an earlier filling
     kCtrCursor = 9,    // output cursor of items()
+    kCtrTicket = 10,   // workgroups of a running ash_grid_collect_touched that have read their input
     kNumCounters = 64
 };
 constexpr int kHostCounters = 8;
@@ -121,8 +122,11 @@ inline int64_t table_workspace_bytes(int64_t capacity) {
     return klog_offset(capacity) + ((capacity + 1) / 2) * 16;
 }
 
+// Slots of a general region that can hold `capacity` keys at half load; a
+// caller may attach a smaller one (a power of two, at least kMinGeneralSlots).
+constexpr int64_t kMinGeneralSlots = 64;
 inline int64_t general_slots(int64_t capacity) {
-    int64_t s = 64;
+    int64_t s = kMinGeneralSlots;
     while (s < 2 * capacity) s <<= 1;
     return s;
 }
@@ -131,7 +135,8 @@ inline int64_t general_slots(int64_t capacity) {
 
 // What the host knows of the device counters (ash_map_counters).
 struct ash_counters {
-    int64_t size, dropped, tombstones, exotic_pending, load_refused, touched, general_live;
+    int64_t size, dropped, tombstones, exotic_pending, load_refused, touched, general_live,
+            general_tombstones;
 };
 
 struct ash_map {

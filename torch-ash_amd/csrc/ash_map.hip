@@ -444,6 +444,7 @@ __device__ __forceinline__ void insert_key(
                 } else {
                     __hip_atomic_store(m.gstate + gp, kGenTomb, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
+                    atomicAdd(m.ctr + kCtrGenTombs, 1);
                 }
                 atomicAdd(m.ctr + kCtrTombs, 1);
                 atomicAdd(m.ctr + kCtrLoadDup, 1);
@@ -491,6 +492,7 @@ __device__ __forceinline__ void insert_key(
                     __hip_atomic_store(m.gstate + gp, kGenTomb,
                                        __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
+                    atomicAdd(m.ctr + kCtrGenTombs, 1);
                 }
                 atomicAdd(m.ctr + kCtrTombs, 1);
             }
@@ -946,6 +948,7 @@ __device__ __forceinline__ void erase_one(const MapDev& m, const int32_t* __rest
                 tomb = true;
                 idx = gi;
                 atomicSub(m.ctr + kCtrGenLive, 1);
+                atomicAdd(m.ctr + kCtrGenTombs, 1);
             }
         }
     }
@@ -1792,10 +1795,12 @@ int ash_map_attach_general(ash_map_t* map, void* general_ws,
                            int64_t general_bytes, void* stream) {
     if (check_map(map)) return 1;
     if (map->general_attached) ASH_FAIL("general region already attached");
-    const int64_t slots = general_slots(map->capacity);
-    if (general_ws == nullptr || general_bytes < slots * 20) {
+    if (general_ws == nullptr || general_bytes < kMinGeneralSlots * 20) {
         ASH_FAIL("general workspace too small");
     }
+    // the largest power of two of slots that fits, up to what `capacity` keys need
+    int64_t slots = kMinGeneralSlots;
+    while (slots < general_slots(map->capacity) && slots * 2 * 20 <= general_bytes) slots <<= 1;
     if (reinterpret_cast<uintptr_t>(general_ws) % 256 != 0) {
         ASH_FAIL("general workspace must be 256-byte aligned");
     }
@@ -2300,6 +2305,7 @@ void decode_counters(const int32_t* host, ash_counters& c) {
     c.load_refused = host[kCtrLoadDup];
     c.touched = host[kCtrTouched];
     c.general_live = host[kCtrGenLive];
+    c.general_tombstones = host[kCtrGenTombs];
 }
 
 int ensure_events(ash_map* map) {
@@ -2360,15 +2366,19 @@ int64_t rebuild_scratch_bytes(const ash_map* map) {
     return keys + map->capacity * 8;
 }
 
-bool should_rebuild(const ash_map* map, int64_t size, int64_t tombstones, int64_t incoming) {
+// keep at least a fifth of the slots truly empty -- of the bucket array, and
+// of the second region on its own account (`general_used`: its entries and
+// tombstones; it may be much smaller than the table)
+bool should_rebuild(const ash_map* map, int64_t size, int64_t tombstones, int64_t incoming,
+                    int64_t general_used = 0, int64_t general_tombstones = 0) {
     if (tombstones <= 0) return false;
     int64_t room = map->capacity - size;
     if (room < 0) room = 0;
     const int64_t arriving = incoming < room ? incoming : room;
-    int64_t slots = static_cast<int64_t>(map->d.nb) * kSlots;
-    if (map->general_attached && map->d.gslots < slots) slots = map->d.gslots;
-    // keep at least a fifth of the slots truly empty
-    return (size + tombstones + arriving) * 5 > slots * 4;
+    const int64_t slots = static_cast<int64_t>(map->d.nb) * kSlots;
+    if ((size + tombstones + arriving) * 5 > slots * 4) return true;
+    return map->general_attached && general_tombstones > 0 &&
+           general_used * 5 > static_cast<int64_t>(map->d.gslots) * 4;
 }
 
 // Before an insert of `incoming` keys (the map's device is current, `s` is not
@@ -2383,7 +2393,10 @@ int upkeep(ash_map* map, int64_t incoming, void* scratch, int64_t scratch_bytes,
     if (refresh_counters(map, staging, s)) return 1;
     const ash_counters& c = map->counters;
     map->maybe_tombstones = c.tombstones > 0;
-    if (!should_rebuild(map, c.size, c.tombstones, incoming)) return 0;
+    if (!should_rebuild(map, c.size, c.tombstones, incoming,
+                        c.general_live + c.general_tombstones, c.general_tombstones)) {
+        return 0;
+    }
     int32_t* keys = nullptr;
     int64_t* indices = nullptr;
     if (map->general_attached && c.size > 0) {
@@ -2775,6 +2788,8 @@ int ash_map_rebuild(ash_map_t* map, int32_t* keys_scratch,
                 reinterpret_cast<uint4*>(map->d.gstate), g16, 0xFFFFFFFFu);
         ASH_LAUNCH_CHECK();
         set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrGenLive, 0);   // counted again below
+        ASH_LAUNCH_CHECK();
+        set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrGenTombs, 0);
         ASH_LAUNCH_CHECK();
     }
     set_counter_kernel<<<1, 64, 0, s>>>(map->d.ctr, kCtrTombs, 0);
