@@ -88,25 +88,27 @@ VALUE_ROW_BYTES = 2 * (12 + 4)               # color + depth, read and written
 #   atomic_requests: TCC_ATOMIC (all of them are forwarded to the memory side:
 #     TCC_EA0_ATOMIC reads the same).
 MEASURED_COUNTERS = {
-    "insert_values": (2_564_000_000 + 1_947_000_000, 0.343, 16_404_000),
-    "insert_keys": (2_304_000_000 + 1_691_000_000, 0.243, 16_465_000),
-    "find": (2_230_000_000 + 146_000_000, 0.064, 0),
-    "erase": (2_234_000_000 + 1_217_000_000, 0.447, 16_031_000),
+    "insert_values": (2_564_000_000 + 1_947_000_000, 0.343, 16_405_000),
+    "insert_keys": (2_336_000_000 + 1_688_000_000, 0.265, 16_422_000),
+    "find": (2_231_000_000 + 146_000_000, 0.064, 0),
+    "erase": (2_234_000_000 + 1_217_000_000, 0.448, 16_031_000),
     # the two keys-only split passes and the range pass
     "erase_bulk": (192_000_000 + 128_000_000 + 641_000_000
-                   + 139_000_000 + 134_000_000 + 1_092_000_000, 0.21, 66_000),
-    "items": (128_000_000 + 320_000_000, 0.417, 1_954),
+                   + 144_000_000 + 135_000_000 + 1_094_000_000, 0.212, 279_000),
+    "items": (128_000_000 + 320_000_000, 0.417, 0),
     "items_values_by_index": (528_000_000 + 256_000_000, 0.247, 0),
     # sums over the split, build and row-copy kernels
-    "insert_values_bulk": (834_000_000 + 1_330_000_000, 0.390, 47_000),
-    "insert_keys_bulk": (449_000_000 + 914_000_000, 0.411, 59_000),
-    "cfg3_forward_linear": (3_519_000_000 + 282_000_000, 0.171, 0),
-    "cfg3_forward_smooth_step": (3_519_000_000 + 282_000_000, 0.171, 0),
-    "cfg4_forward": (376_000_000 + 67_000_000, 0.259, 0),
+    "insert_values_bulk": (835_000_000 + 1_327_000_000, 0.413, 259_000),
+    "insert_keys_bulk": (449_000_000 + 920_000_000, 0.426, 271_000),
+    "cfg3_forward_linear": (3_508_000_000 + 282_000_000, 0.172, 0),
+    "cfg3_forward_smooth_step": (3_508_000_000 + 282_000_000, 0.172, 0),
+    "cfg4_forward": (377_000_000 + 67_000_000, 0.257, 0),
     # kernel only: the zero fill of the dense gradient adds 1.64 GB written
-    "cfg4_backward": (438_000_000 + 149_000_000 + 1_638_400_000, 0.097, 2_344_000),
-    "cfg4_double_backward": (485_000_000 + 166_000_000 + 1_638_400_000, 0.108, 2_344_000),
+    "cfg4_backward": (439_000_000 + 149_000_000 + 1_638_400_000, 0.098, 2_344_000),
+    "cfg4_double_backward": (486_000_000 + 166_000_000 + 1_638_400_000, 0.109, 2_344_000),
     "cfg4_grid_query": (71_000_000 + 122_000_000, 0.399, 0),
+    "cfg4_module_forward": (325_000_000 + 72_000_000, 0.398, 0),
+    "cfg4_module_forward_for_training": (325_000_000 + 190_000_000, 0.428, 0),
 }
 
 
@@ -118,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "unset",
+    "csrc_sha256": "aae38478b511ffab64b0b3bfeba81de7eae9d498caba61c7543ecdcf6901b60d",
 }
 
 
