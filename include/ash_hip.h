@@ -142,6 +142,22 @@ int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
                              int bound_lo, int bound_hi, uint8_t* touched,
                              int32_t* coords, void* stream);
 
+/* ash_grid_activate straight from world positions and without a scratch
+ * buffer: `positions` fp32[n,3] in world units, cell units = (position -
+ * origin) / cell_size evaluated as torch evaluates that expression on the
+ * device (a subtraction, then a multiplication by the fp32 reciprocal);
+ * `origin` fp32[3] ON THE DEVICE or NULL, cell_size 1 with a NULL origin for
+ * positions that are in cell units already.  Stands for
+ * `transform_world_to_cell` + the body of `spatial_init_` (ash/grid.py:121-159)
+ * in two launches: every workgroup finds the run heads among its own 128
+ * positions, so there is no list of heads, no counter to clear and nothing to
+ * allocate.  Same blocks, flags and coordinates as ash_grid_activate. */
+int ash_grid_activate_positions(ash_map_t* map, const float* positions, int64_t n,
+                                const float* origin, float cell_size, int grid_dim,
+                                int dilation, int bidirectional, int bound_lo,
+                                int bound_hi, uint8_t* touched, int32_t* coords,
+                                void* stream);
+
 /* After ash_grid_activate: the rows whose flag is set in `touched`, in
  * ascending order, to out_indices int64[capacity] and their block coordinates
  * to out_coords int32[capacity, 3]; the flags are cleared and the count is left
@@ -190,6 +206,22 @@ int ash_grid_integrate_depth_touched(ash_map_t* map, float* embeddings,
                                      int64_t num_embeddings, int grid_dim,
                                      int embedding_dim, const int64_t* grid_indices,
                                      const int32_t* grid_coords, float cell_size,
+                                     const float* origin, const float* intrinsic,
+                                     const float* extrinsic, const float* depth,
+                                     const float* color, int height, int width,
+                                     float trunc, float depth_max, void* stream);
+
+/* ash_grid_integrate_depth over every row whose flag an activation has set in
+ * `touched` (uint8[capacity]; block coordinates at coords[3*row..], as
+ * ash_grid_activate leaves them), without a listing in between: the kernel
+ * looks at the flags itself, takes them down and updates the cells of the
+ * flagged blocks.  With ash_grid_activate_positions a frame of a fusion loop
+ * is three launches, none of which waits for the host.  Same arithmetic as
+ * ash_grid_integrate_depth.  No counterpart in the reference. */
+int ash_grid_integrate_depth_flagged(ash_map_t* map, float* embeddings,
+                                     int64_t num_embeddings, int grid_dim,
+                                     int embedding_dim, uint8_t* touched,
+                                     const int32_t* coords, float cell_size,
                                      const float* origin, const float* intrinsic,
                                      const float* extrinsic, const float* depth,
                                      const float* color, int height, int width,

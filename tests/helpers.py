@@ -1,6 +1,7 @@
 """Shared helpers of the test-suite: an independent pure-torch statement of
 the trilinear query (used to pin the oracle through autograd), a dictionary
 model of the hash map, and comparison utilities."""
+import ctypes
 from typing import Dict, Tuple
 
 import numpy as np
@@ -155,3 +156,47 @@ def assert_is_bijection_into(indices: torch.Tensor, capacity: int):
     assert idx.numel() == idx.unique().numel(), "indices are not distinct"
     if idx.numel():
         assert int(idx.min()) >= 0 and int(idx.max()) < capacity
+
+
+class RawBlockMap:
+    """A 3-d map made through the C ABI, with the caller-owned arrays of a
+    block activation (flags and block coordinates per row)."""
+
+    def __init__(self, lib, capacity, device):
+        self.lib, self.capacity, self.device = lib, capacity, device
+        table, general = ctypes.c_int64(0), ctypes.c_int64(0)
+        assert lib.ash_map_workspace_bytes(3, capacity, ctypes.byref(table), ctypes.byref(general)) == 0
+        self.heap = torch.empty(capacity, dtype=torch.int32, device=device)
+        self.table = torch.empty(table.value, dtype=torch.uint8, device=device)
+        self.touched = torch.zeros(capacity, dtype=torch.uint8, device=device)
+        self.coords = torch.zeros((capacity, 3), dtype=torch.int32, device=device)
+        self.handle = ctypes.c_void_p()
+        self.stream = torch.cuda.current_stream(device).cuda_stream
+        rc = lib.ash_map_create(3, capacity, self.heap.data_ptr(), self.table.data_ptr(),
+                                table.value, device.index or 0, self.stream,
+                                ctypes.byref(self.handle))
+        assert rc == 0, lib.ash_last_error()
+
+    def close(self):
+        self.lib.ash_map_destroy(self.handle)
+
+    def touched_blocks(self):
+        """(sorted coordinates of the flagged rows, their rows); clears the flags."""
+        rows = self.touched.nonzero().view(-1)
+        out = sort_rows(self.coords[rows], rows)
+        self.touched.zero_()
+        return out
+
+    def size(self):
+        n = ctypes.c_int64(-1)
+        assert self.lib.ash_map_size(self.handle, ctypes.byref(n), self.stream) == 0
+        return n.value
+
+    def find(self, keys):
+        n = keys.shape[0]
+        idx = torch.empty(n, dtype=torch.int64, device=self.device)
+        mask = torch.empty(n, dtype=torch.bool, device=self.device)
+        rc = self.lib.ash_map_find(self.handle, keys.data_ptr(), n, idx.data_ptr(), mask.data_ptr(),
+                                   self.stream)
+        assert rc == 0, self.lib.ash_last_error()
+        return idx, mask

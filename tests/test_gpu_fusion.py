@@ -8,8 +8,11 @@ import numpy as np
 import pytest
 import torch
 
+import ctypes
+
 import workloads
-from helpers import sort_rows
+from ash import common
+from helpers import RawBlockMap, sort_rows
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -289,8 +292,13 @@ def test_frames_without_read_back_equal_counted_frames(gpu_ash):
         depth = scene.depth(ext)
         frames.append((scene.unproject(depth, ext).to(DEV), depth.to(DEV), ext.to(DEV)))
 
-    def run(count_blocks, capacity=30_000):
+    def run(count_blocks, capacity=30_000, listing=False):
         grid = gpu_ash.UnBoundedSparseDenseGrid(3, capacity, 2, 8, cell_size=0.015, device=DEV)
+        if listing:
+            # a transform of the user's: the frame cannot apply it inside its
+            # kernels and takes the activation that lists the touched rows
+            own = grid.transform_world_to_cell
+            grid.transform_world_to_cell = lambda x: own(x)
         with torch.no_grad():
             grid.embeddings.zero_()
         touched = [gpu_ash.fusion.fuse_frame(grid, p, d, intrinsic, e, 0.04, 6.0,
@@ -300,18 +308,125 @@ def test_frames_without_read_back_equal_counted_frames(gpu_ash):
         return grid, touched, order[0], grid.embeddings.detach()[order[1].to(DEV)].cpu()
 
     _, touched, keys_a, cells_a = run(True)
-    grid, nothing, keys_b, cells_b = run(False)
-    assert all(t > 100 for t in touched) and nothing == [None] * len(frames)
-    assert torch.equal(keys_a, keys_b) and len(keys_a) > 1000
-    assert torch.equal(cells_a, cells_b)
-    assert float(cells_a[..., 1].sum()) > 1e5
-    # the count of the last listing is still in the counters
-    assert grid.engine.backend.status()["touched"] == touched[-1]
+    assert all(t > 100 for t in touched) and float(cells_a[..., 1].sum()) > 1e5
+    for listing in (False, True):
+        grid, nothing, keys_b, cells_b = run(False, listing=listing)
+        assert nothing == [None] * len(frames)
+        assert torch.equal(keys_a, keys_b) and len(keys_a) > 1000
+        assert torch.equal(cells_a, cells_b)
+        table = grid.engine.backend
+        if listing:
+            # the count of the last listing is still in the counters
+            assert table.status()["touched"] == touched[-1]
+        # no flag is left standing either way
+        assert int(table._touched.sum()) == 0
     # too small a table: the frames run, the table is full, the next insert warns
     small, _, keys_c, _ = run(False, capacity=1500)
     assert small.engine.size() == 1500 and len(keys_c) == 1500
     with pytest.warns(UserWarning, match="exceeds the hash map capacity"):
         small.engine.insert_keys(torch.tensor([[900, 900, 900]], dtype=torch.int32, device=DEV))
+
+
+def test_activation_from_world_positions_equals_activation_from_cells(gpu_ash):
+    """ash_grid_activate_positions (world positions, run heads found per
+    workgroup, no scratch) against ash_grid_activate on torch's
+    (x - origin) / cell_size, through the C ABI on two identical maps, call
+    after call: same blocks stored, same rows' coordinates flagged, same
+    answers to look-ups.  Batches that end inside a workgroup's 128 positions,
+    every dilation, bounds that cut candidates off, positions in cell units."""
+    lib = common.load_library()
+    capacity = 60_000
+    plain, direct = RawBlockMap(lib, capacity, DEV), RawBlockMap(lib, capacity, DEV)
+    g = torch.Generator().manual_seed(77)
+    cases = (  # n, dilation, two-sided, origin, cell size, bounds
+        (40_001, 1, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),
+        (9_000, 2, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),
+        (5_003, 0, 0, None, 1.0, (-1000, 1000)),
+        (127, 1, 0, (0.5, 0.5, 0.5), 0.1, (-1000, 1000)),
+        (20_000, 1, 1, (-2.0, -2.0, -2.0), 0.02, (0, 11)),
+    )
+    try:
+        for n, dilation, two_sided, origin, cell_size, (lo, hi) in cases:
+            # image-like ordering: neighbouring rows are neighbouring positions
+            cells = ((torch.rand(n, 3, generator=g).cumsum(0) * 0.3) % 260.0) - 50.0
+            x = (cells * cell_size + (torch.tensor(origin) if origin else 0.0)).to(DEV).contiguous()
+            o = torch.tensor(origin, device=DEV) if origin else None
+            cells = ((x - o) / cell_size if origin else x / cell_size).contiguous()
+            heads = torch.empty(64 + 3 * n, dtype=torch.int32, device=DEV)
+            rc = lib.ash_grid_activate(plain.handle, cells.data_ptr(), n, 8, dilation, two_sided,
+                                       lo, hi, plain.touched.data_ptr(), plain.coords.data_ptr(),
+                                       heads.data_ptr(), plain.stream)
+            assert rc == 0, lib.ash_last_error()
+            rc = lib.ash_grid_activate_positions(
+                direct.handle, x.data_ptr(), n, o.data_ptr() if origin else None,
+                ctypes.c_float(cell_size), 8, dilation, two_sided, lo, hi,
+                direct.touched.data_ptr(), direct.coords.data_ptr(), direct.stream)
+            assert rc == 0, lib.ash_last_error()
+            torch.cuda.synchronize()
+            size = plain.size()
+            assert direct.size() == size and 20 < size < capacity
+            coords_p, rows_p = plain.touched_blocks()
+            coords_d, rows_d = direct.touched_blocks()
+            assert coords_p.shape[0] > 20 and torch.equal(coords_d, coords_p)
+            assert int(coords_p.min()) >= lo and int(coords_p.max()) <= hi
+            for m, rows in ((plain, rows_p), (direct, rows_d)):
+                idx, mask = m.find(coords_p.to(DEV))
+                assert bool(mask.all()) and torch.equal(idx.cpu(), rows.cpu())
+            probe = torch.cat([coords_p[::3] + 1, coords_p[::5]]).to(DEV).contiguous()
+            assert torch.equal(plain.find(probe)[1], direct.find(probe)[1])
+    finally:
+        plain.close()
+        direct.close()
+
+
+@pytest.mark.parametrize("grid_dim,e,bounded", [(8, 2, False), (8, 5, False), (4, 2, True), (8, 2, True)])
+def test_integration_by_flags_equals_integration_by_listing(gpu_ash, grid_dim, e, bounded):
+    """ash_grid_integrate_depth_flagged (after ash_grid_activate_positions)
+    against ash_grid_integrate_depth over the listing spatial_init_ returns, on
+    two grids from the same state, frame after frame: the same blocks and,
+    block by block, the same rows bit for bit; rows of untouched blocks keep
+    what they held; no flag is left standing.  Block edges of 8 with
+    distance + weight rows take kernels of their own; the others the general
+    ones."""
+    scene = workloads.FusionScene(width=320, height=240)
+    rnd = torch.Generator().manual_seed(5)
+    intrinsic = scene.intrinsic.to(DEV)
+    cell_size = 0.015 * 8 / grid_dim
+
+    def new_grid():
+        if bounded:
+            grid = gpu_ash.BoundedSparseDenseGrid(
+                3, 30_000, e, grid_dim=grid_dim, sparse_grid_dim=32,
+                bbox_min=-1.7 * torch.ones(3), bbox_max=1.7 * torch.ones(3), device=DEV)
+        else:
+            grid = gpu_ash.UnBoundedSparseDenseGrid(3, 30_000, e, grid_dim, cell_size=cell_size,
+                                                    device=DEV)
+        with torch.no_grad():
+            # (zeros: the two grids hand out their rows in different orders)
+            grid.embeddings.zero_()
+        return grid
+
+    listed, flagged = new_grid(), new_grid()
+    for frame in (0, 11, 22):
+        ext = scene.pose(frame)
+        depth = scene.depth(ext)
+        color = torch.rand(*depth.shape, 3, generator=rnd).to(DEV) if e >= 5 else None
+        pts = scene.unproject(depth, ext).to(DEV)
+        depth, ext = depth.to(DEV), ext.to(DEV)
+        gc, _, gi, _ = listed.spatial_init_(pts, dilation=1, bidirectional=True)
+        gpu_ash.fusion.integrate_depth(listed, gc, gi, depth, intrinsic, ext, 0.04, 6.0, color)
+        assert gpu_ash.fusion.fuse_frame(flagged, pts, depth, intrinsic, ext, 0.04, 6.0, color,
+                                         count_blocks=False) is None
+        keys_l, idx_l = sort_rows(*listed.engine.items())
+        keys_f, idx_f = sort_rows(*flagged.engine.items())
+        assert torch.equal(keys_l, keys_f) and len(gi) > 100
+        assert torch.equal(listed.embeddings.detach()[idx_l.to(DEV)],
+                           flagged.embeddings.detach()[idx_f.to(DEV)])
+        assert int(flagged.engine.backend._touched.sum()) == 0
+    # rows no block owns were not written
+    free = torch.ones(30_000, dtype=torch.bool, device=DEV)
+    free[idx_f.to(DEV)] = False
+    assert int(flagged.embeddings.detach()[free].count_nonzero()) == 0
 
 
 @pytest.mark.parametrize("capacity", [5, 1000, 80_000, 131_073, 200_000, 1_048_576])

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from ash import common
-from helpers import sort_rows
+from helpers import RawBlockMap
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -20,47 +20,8 @@ CAPACITY = 60_000
 GRID_DIM = 8
 
 
-class _Map:
-    """A map made through the C ABI, with the caller-owned arrays of an
-    activation."""
-
-    def __init__(self, lib):
-        self.lib = lib
-        table, general = ctypes.c_int64(0), ctypes.c_int64(0)
-        assert lib.ash_map_workspace_bytes(3, CAPACITY, ctypes.byref(table), ctypes.byref(general)) == 0
-        self.heap = torch.empty(CAPACITY, dtype=torch.int32, device=DEV)
-        self.table = torch.empty(table.value, dtype=torch.uint8, device=DEV)
-        self.touched = torch.zeros(CAPACITY, dtype=torch.uint8, device=DEV)
-        self.coords = torch.zeros((CAPACITY, 3), dtype=torch.int32, device=DEV)
-        self.handle = ctypes.c_void_p()
-        self.stream = torch.cuda.current_stream(DEV).cuda_stream
-        rc = lib.ash_map_create(3, CAPACITY, self.heap.data_ptr(), self.table.data_ptr(),
-                                table.value, 0, self.stream, ctypes.byref(self.handle))
-        assert rc == 0, lib.ash_last_error()
-
-    def close(self):
-        self.lib.ash_map_destroy(self.handle)
-
-    def touched_blocks(self):
-        """(sorted coordinates of the flagged rows, their rows); clears the flags."""
-        rows = self.touched.nonzero().view(-1)
-        out = sort_rows(self.coords[rows], rows)
-        self.touched.zero_()
-        return out
-
-    def size(self):
-        n = ctypes.c_int64(-1)
-        assert self.lib.ash_map_size(self.handle, ctypes.byref(n), self.stream) == 0
-        return n.value
-
-    def find(self, keys):
-        n = keys.shape[0]
-        idx = torch.empty(n, dtype=torch.int64, device=DEV)
-        mask = torch.empty(n, dtype=torch.bool, device=DEV)
-        rc = self.lib.ash_map_find(self.handle, keys.data_ptr(), n, idx.data_ptr(), mask.data_ptr(),
-                                   self.stream)
-        assert rc == 0, self.lib.ash_last_error()
-        return idx, mask
+def _Map(lib):
+    return RawBlockMap(lib, CAPACITY, DEV)
 
 
 def _positions(n, seed):

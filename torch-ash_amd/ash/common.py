@@ -86,6 +86,17 @@ _SIGNATURES = {
         [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
          _PTR, _PTR, _PTR],
     ),
+    "ash_grid_activate_positions": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, _PTR, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+         ctypes.c_int, ctypes.c_int, _PTR, _PTR, _PTR],
+    ),
+    "ash_grid_integrate_depth_flagged": (
+        ctypes.c_int,
+        [_PTR, _PTR, _I64, ctypes.c_int, ctypes.c_int, _PTR, _PTR, ctypes.c_float,
+         ctypes.POINTER(ctypes.c_float), _PTR, _PTR, _PTR, _PTR, ctypes.c_int, ctypes.c_int,
+         ctypes.c_float, ctypes.c_float, _PTR],
+    ),
     "ash_grid_integrate_depth": (
         ctypes.c_int,
         [_PTR, _I64, ctypes.c_int, ctypes.c_int, _PTR, _PTR, _I64, ctypes.c_float,
@@ -579,20 +590,29 @@ class _Backend:
         trunc: float,
         depth_max: float,
         counted_by=None,
+        flagged_by=None,
     ) -> None:
         """In-place TSDF update of the cells of the listed blocks.  With
         `counted_by` (a map whose latest deferred activation made the listing)
-        the number of listed blocks is read on the device."""
+        the number of listed blocks is read on the device; with `flagged_by` (a
+        map whose latest `activate_positions` left flags) there is no listing
+        and the kernel goes by the map's flags, which it takes down."""
         _require_hip(embeddings, "embeddings")
         dev = embeddings.device
         if embeddings.dtype != torch.float32 or not embeddings.is_contiguous():
             raise RuntimeError("embeddings must be contiguous float32")
         if embeddings.dim() != 3 or embeddings.shape[1] != grid_dim**3:
             raise RuntimeError("embeddings must be (num_embeddings, grid_dim^3, embedding_dim)")
-        grid_indices = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
-        grid_coords = grid_coords.reshape(-1, 3).to(dev, torch.int32).contiguous()
-        if grid_coords.shape[0] != grid_indices.shape[0]:
-            raise RuntimeError("one coordinate row per block index is needed")
+        if flagged_by is not None:
+            if flagged_by._device != dev or getattr(flagged_by, "_touched", None) is None:
+                raise RuntimeError("no activation has flagged rows of this map on this device")
+            if embeddings.shape[0] < flagged_by.capacity:
+                raise RuntimeError("one embedding row per index of the map is needed")
+        else:
+            grid_indices = grid_indices.reshape(-1).to(dev, torch.int64).contiguous()
+            grid_coords = grid_coords.reshape(-1, 3).to(dev, torch.int32).contiguous()
+            if grid_coords.shape[0] != grid_indices.shape[0]:
+                raise RuntimeError("one coordinate row per block index is needed")
         if counted_by is not None and grid_indices.shape[0] != counted_by.capacity:
             raise RuntimeError("a listing counted on the device has one row per block of the map")
         intrinsic = intrinsic.to(dev, torch.float32).contiguous()
@@ -613,7 +633,15 @@ class _Backend:
                 depth.data_ptr(), color.data_ptr() if color is not None else None,
                 depth.shape[0], depth.shape[1], float(trunc), float(depth_max), _stream_of(dev))
         with torch.cuda.device(dev):
-            if counted_by is not None:
+            if flagged_by is not None:
+                self.check(
+                    self.lib.ash_grid_integrate_depth_flagged(
+                        flagged_by._handle, embeddings.data_ptr(), embeddings.shape[0],
+                        int(grid_dim), embeddings.shape[2], flagged_by._touched.data_ptr(),
+                        flagged_by._block_coords.data_ptr(), *tail,
+                    )
+                )
+            elif counted_by is not None:
                 self.check(
                     self.lib.ash_grid_integrate_depth_touched(
                         counted_by._handle, embeddings.data_ptr(), embeddings.shape[0],
@@ -1215,7 +1243,6 @@ class _HashMap:
         blocks as (grid_coords int32[n,3], grid_indices int64[n])."""
         cells = self._activation_buffers(cells)
         self._upkeep(cells.shape[0])
-        heads = torch.empty(64 + 3 * cells.shape[0], dtype=torch.int32, device=self._device)
         # the touched rows are listed on the device and their count travels with
         # the read-back that ends the activation (tables beyond the listing
         # kernel's limit take torch's nonzero and a second read-back)
@@ -1225,12 +1252,13 @@ class _HashMap:
             coords = torch.empty((self.capacity, 3), dtype=torch.int32, device=self._device)
         for _ in range(2):
             with torch.cuda.device(self._device):
+                # (positions in cell units: no origin, cell size 1)
                 self._check(
-                    self._lib.ash_grid_activate(
-                        self._handle, cells.data_ptr(), cells.shape[0], int(grid_dim),
-                        int(dilation), int(bool(bidirectional)), int(bound_lo), int(bound_hi),
-                        self._touched.data_ptr(), self._block_coords.data_ptr(),
-                        heads.data_ptr(), self._stream(),
+                    self._lib.ash_grid_activate_positions(
+                        self._handle, cells.data_ptr(), cells.shape[0], None, 1.0,
+                        int(grid_dim), int(dilation), int(bool(bidirectional)), int(bound_lo),
+                        int(bound_hi), self._touched.data_ptr(), self._block_coords.data_ptr(),
+                        self._stream(),
                     )
                 )
                 if listing:
@@ -1306,6 +1334,41 @@ class _HashMap:
             )
         self.version = next(_VERSIONS)
         return coords, rows
+
+    def activate_positions(
+        self,
+        positions: torch.Tensor,
+        origin: Optional[torch.Tensor],
+        cell_size: float,
+        grid_dim: int,
+        dilation: int,
+        bidirectional: bool,
+        bound_lo: int,
+        bound_hi: int,
+    ) -> None:
+        """The activation of `activate_blocks` from world positions (cell units
+        = (positions - origin) / cell_size), two launches and nothing else: the
+        touched rows stay flagged in the map's own arrays for
+        `integrate_depth(flagged_by=map)`, which takes the flags down again.
+        Nothing waits for the device and nothing is allocated once the map's
+        arrays exist, so the launches can be captured into a graph; keys
+        refused for lack of capacity show in the counters at the next call that
+        reads them."""
+        positions = self._activation_buffers(positions)
+        n = positions.shape[0]
+        if self._general is None:
+            # a key beyond the packed range would otherwise wait for a read-back
+            # that this path does not make
+            self._attach_general(just_in_case=True)
+        self._upkeep(n)
+        with torch.cuda.device(self._device):
+            self._check(self._lib.ash_grid_activate_positions(
+                self._handle, positions.data_ptr(), n,
+                origin.data_ptr() if origin is not None else None, float(cell_size),
+                int(grid_dim), int(dilation), int(bool(bidirectional)), int(bound_lo),
+                int(bound_hi), self._touched.data_ptr(), self._block_coords.data_ptr(),
+                self._stream()))
+        self.version = next(_VERSIONS)
 
     def insert_keys(self, keys: torch.Tensor) -> None:
         self._insert(self._keys(keys), 0, None, None, None)

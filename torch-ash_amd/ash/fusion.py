@@ -31,13 +31,15 @@ def integrate_depth(
     depth_max: float,
     color: Optional[torch.Tensor] = None,
     counted_by=None,
+    flagged_by=None,
 ) -> None:
     """Projects every cell of the listed blocks into `depth` (H, W; metres, 0 =
     no reading) with the pinhole `intrinsic` (3, 3) and the world-to-camera
     `extrinsic` (4, 4) and folds the truncated signed distance (and `color`
     (H, W, 3), if given) into the grid's embedding rows.  `counted_by`: the
     table whose deferred activation made the listing (its length is then read
-    on the device)."""
+    on the device); `flagged_by`: the table whose `activate_positions` flagged
+    the blocks (no listing at all: pass None for the first two)."""
     scale, origin = grid._cell_to_world_affine()
     backend.integrate_depth(
         grid.embeddings.data,
@@ -53,6 +55,7 @@ def integrate_depth(
         trunc,
         depth_max,
         counted_by=counted_by,
+        flagged_by=flagged_by,
     )
 
 
@@ -77,6 +80,19 @@ def fuse_frame(
     its tensors, demo/rgbd_fusion.py:216-254; the kernels here read it where it
     is), the host only queues launches, and the reference's capacity warning
     comes with the next call that reads the table's counters."""
+    if not count_blocks and points.shape[0] > 0 and points.dtype == torch.float32:
+        affine = grid._world_to_cell_affine(points)
+        if affine is not None:
+            # three launches: the transform is applied inside the activation
+            # kernels, which flag the touched rows; the integration goes by the
+            # flags and takes them down
+            lo, hi = grid._block_bounds()
+            table = grid.engine.backend
+            table.activate_positions(points, affine[0], affine[1], grid.grid_dim, dilation, True,
+                                     lo, hi)
+            integrate_depth(grid, None, None, depth, intrinsic, extrinsic, trunc, depth_max,
+                            color, flagged_by=table)
+            return None
     if not count_blocks and points.shape[0] > 0 and grid.engine.capacity <= COLLECT_MAX_BLOCKS:
         cells = grid.transform_world_to_cell(points)
         if cells.dtype == torch.float32:

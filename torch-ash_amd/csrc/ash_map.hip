@@ -348,7 +348,8 @@ enum InsertMode {
     kInsertKeys = 0,    // allocate indices only
     kInsertFused = 1,   // + copy narrow value rows in the same kernel
     kInsertAssign = 2,  // + report the allocated index per input row
-    kInsertLoad = 3     // indices are given (state-dict load), heap untouched
+    kInsertLoad = 3,    // indices are given (state-dict load), heap untouched
+    kInsertReport = 4   // keys only; tells the caller the key's index when it is final
 };
 
 // The insert proper for a key held in registers (`code` is its packed form if
@@ -357,9 +358,12 @@ template <int DIM, int MODE>
 __device__ __forceinline__ void insert_key(
         const MapDev& m, const int32_t (&k)[DIM], uint64_t code, bool fits,
         int64_t i, bool active, const ValueArgs& va,
-        int32_t* __restrict__ assigned, const int64_t* __restrict__ given) {
+        int32_t* __restrict__ assigned, const int64_t* __restrict__ given,
+        int32_t* report = nullptr) {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    int32_t seen = -1;     // kInsertReport: the index read beside a key that was there
+    bool gdup = false;     // kInsertReport: the key stands in the general region
     bool pend = active && fits;
     uint32_t b = bucket_of(code, m.nb);
     uint32_t steps = 0;
@@ -380,6 +384,7 @@ __device__ __forceinline__ void insert_key(
                 if constexpr (MODE == kInsertLoad) {
                     atomicAdd(m.ctr + kCtrLoadDup, 1);
                 }
+                if constexpr (MODE == kInsertReport) seen = p.val;
             } else {
                 uint32_t em = p.emask;
                 while (em) {
@@ -422,6 +427,8 @@ __device__ __forceinline__ void insert_key(
             atomicAdd(m.ctr + kCtrExotic, 1);
         } else if constexpr (MODE == kInsertLoad) {
             atomicAdd(m.ctr + kCtrLoadDup, 1);
+        } else if constexpr (MODE == kInsertReport) {
+            gdup = true;
         }
     }
     if (refused) atomicAdd(m.ctr + kCtrDropped, 1);
@@ -523,6 +530,27 @@ __device__ __forceinline__ void insert_key(
     }
     if constexpr (MODE == kInsertAssign) {
         if (active) assigned[i] = idx;
+    }
+    if constexpr (MODE == kInsertReport) {
+        // The index of the key, if this thread can be sure of it: the one it
+        // was given just now, or the one read beside a key that was there --
+        // but a key that another thread is storing in this very launch shows
+        // before its index is written, and the word beside it still holds
+        // whatever an earlier tenant of the slot left.  The key log settles
+        // it: klog[index] names this key only if that index is the key's own.
+        // (-1 tells the caller that the thread storing the key will know.)
+        int32_t r = idx;
+        if (r < 0 && static_cast<uint32_t>(seen) < static_cast<uint32_t>(m.capacity) &&
+            m.klog[seen] == code) {
+            r = seen;
+        }
+        if (r < 0 && gdup) {
+            // (the general region shows an index only once it is final)
+            uint32_t at;
+            int32_t gi;
+            if (gen_find<DIM>(m, k, gi, at)) r = gi;
+        }
+        *report = r;
     }
 }
 
@@ -682,6 +710,152 @@ __global__ __launch_bounds__(kHeapBlock) void activate_kernel(
                 coords[static_cast<int64_t>(idx) * 3 + 1] = k[1];
                 coords[static_cast<int64_t>(idx) * 3 + 2] = k[2];
             }
+        }
+    }
+}
+
+// The same activation straight from world positions, without a list of run
+// heads in memory: a workgroup finds the heads among its own kRunPositions
+// positions (a position leads a run when the position before it lies in
+// another block, whichever workgroup that one belongs to), keeps them in LDS
+// and handles their (head, neighbour offset) pairs itself: no list to write
+// and read back, no counter to clear.
+// Positions are in world units: cell units = (x - origin) * inv_cell, evaluated
+// as torch evaluates `(x - origin) / cell_size` on the device (grid_forward's
+// front end does the same); origin null and inv_cell 1 leave them as they are.
+struct RunsArgs {
+    const float* x;        // float32[n, 3]
+    const float* origin;   // float32[3] on the device, or nullptr
+    float inv_cell;
+    float g;               // cells per block edge
+    int64_t n;
+    int off_lo, width;     // neighbour offsets off_lo .. off_lo + width - 1 per axis
+    int bound_lo, bound_hi;
+};
+
+__device__ __forceinline__ bool block_of_world(const RunsArgs& a, int64_t i,
+                                               int32_t (&base)[3]) {
+    bool inside = true;
+#pragma unroll
+    for (int d = 0; d < 3; ++d) {
+        const float o = a.origin != nullptr ? a.origin[d] : 0.f;
+        const float c = __fmul_rn(__fsub_rn(a.x[i * 3 + d], o), a.inv_cell);
+        base[d] = static_cast<int32_t>(floorf(__fdiv_rn(c, a.g)));
+        inside = inside && base[d] >= a.bound_lo && base[d] <= a.bound_hi;
+    }
+    return inside;
+}
+
+constexpr int kRunPositions = 256;
+static_assert(kRunPositions % 64 == 0 && kRunPositions <= kHeapBlock, "whole wavefronts of positions");
+constexpr int kCandChunk = 1024;         // candidates made distinct at a time
+constexpr int kDistinctSlots = 2048;     // two LDS slots per candidate of a chunk
+
+// One launch per batch: insert and flag.  The (head, neighbour offset)
+// candidates of a workgroup -- some 270 for 128 depth pixels at dilation 1 --
+// name every block twice on average (the neighbourhoods of neighbouring
+// blocks overlap in 18 of 27), so they are first made distinct in an LDS set,
+// which leaves one round of table work per workgroup as a rule.  The insert
+// reports the index of every key it can be sure of (insert_key, kInsertReport)
+// and the row is flagged at once; a key that another thread is storing at
+// that moment is flagged by that thread, which is handed the index.  No second
+// launch has to wait for the indices to settle.
+__global__ __launch_bounds__(kHeapBlock) void activate_runs_kernel(
+        MapDev m, RunsArgs a, uint8_t* __restrict__ touched, int32_t* __restrict__ coords) {
+    __shared__ unsigned long long s_set[kDistinctSlots];
+    __shared__ int32_t s_cand[kCandChunk * 3];
+    __shared__ int32_t s_heads[kRunPositions * 3];
+    __shared__ int s_wave[kRunPositions / 64];
+    __shared__ int s_ncand;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kRunPositions + threadIdx.x;
+    int32_t base[3] = {0, 0, 0};
+    bool lead = false;
+    if (threadIdx.x < kRunPositions && i < a.n) {
+        lead = block_of_world(a, i, base);
+        if (lead && i > 0) {
+            int32_t prev[3];
+            const bool pin = block_of_world(a, i - 1, prev);
+            lead = !pin || prev[0] != base[0] || prev[1] != base[1] || prev[2] != base[2];
+        }
+    }
+    const uint64_t lm = __ballot(lead);
+    if (lane == 0 && wave < kRunPositions / 64) s_wave[wave] = __popcll(lm);
+    __syncthreads();
+    int before = 0, nh = 0;
+#pragma unroll
+    for (int q = 0; q < kRunPositions / 64; ++q) {
+        const int c = s_wave[q];
+        if (q < wave) before += c;
+        nh += c;
+    }
+    if (lead) {
+        const int h = before + __popcll(lm & ((1ull << lane) - 1ull));
+        s_heads[h * 3 + 0] = base[0];
+        s_heads[h * 3 + 1] = base[1];
+        s_heads[h * 3 + 2] = base[2];
+    }
+    const int per_head = a.width * a.width * a.width;
+    const int total = nh * per_head;   // the same for every thread of the workgroup
+    const ValueArgs none = {};
+    for (int first = 0; first < total; first += kCandChunk) {
+        for (int q = threadIdx.x; q < kDistinctSlots; q += kHeapBlock) s_set[q] = kEmpty;
+        if (threadIdx.x == 0) s_ncand = 0;
+        __syncthreads();   // (also: s_heads is complete, the rounds below are over)
+        const int end = total - first < kCandChunk ? total : first + kCandChunk;
+        for (int t = first + threadIdx.x; t < end; t += kHeapBlock) {
+            const int h = t / per_head;
+            const int o = t - h * per_head;
+            int32_t c[3];
+            c[0] = s_heads[h * 3 + 0] + a.off_lo + o % a.width;
+            c[1] = s_heads[h * 3 + 1] + a.off_lo + (o / a.width) % a.width;
+            c[2] = s_heads[h * 3 + 2] + a.off_lo + o / (a.width * a.width);
+            bool keep = true;
+#pragma unroll
+            for (int d = 0; d < 3; ++d) keep = keep && c[d] >= a.bound_lo && c[d] <= a.bound_hi;
+            uint64_t code;
+            if (keep && pack_key<3>(c, code)) {   // (keys that do not pack are all kept)
+                uint32_t at = static_cast<uint32_t>(mix64(code)) & (kDistinctSlots - 1);
+                for (;;) {   // at most half of the slots are ever taken
+                    const unsigned long long old = atomicCAS(&s_set[at], kEmpty, code);
+                    if (old == kEmpty) break;
+                    if (old == code) {
+                        keep = false;
+                        break;
+                    }
+                    at = (at + 1) & (kDistinctSlots - 1);
+                }
+            }
+            if (keep) {
+                const int at = atomicAdd(&s_ncand, 1);
+                s_cand[at * 3 + 0] = c[0];
+                s_cand[at * 3 + 1] = c[1];
+                s_cand[at * 3 + 2] = c[2];
+            }
+        }
+        __syncthreads();
+        const int distinct = s_ncand;
+        for (int r0 = 0; r0 < distinct; r0 += kHeapBlock) {
+            const int t = r0 + threadIdx.x;
+            const bool ok = t < distinct;
+            int32_t k[3] = {0, 0, 0};
+            if (ok) {
+                k[0] = s_cand[t * 3 + 0];
+                k[1] = s_cand[t * 3 + 1];
+                k[2] = s_cand[t * 3 + 2];
+            }
+            uint64_t code;
+            const bool fits = pack_key<3>(k, code);
+            int32_t row = -1;
+            insert_key<3, kInsertReport>(m, k, code, fits, 0, ok, none, nullptr, nullptr, &row);
+            if (ok && row >= 0) {
+                touched[row] = 1;
+                coords[static_cast<int64_t>(row) * 3 + 0] = k[0];
+                coords[static_cast<int64_t>(row) * 3 + 1] = k[1];
+                coords[static_cast<int64_t>(row) * 3 + 2] = k[2];
+            }
+            __syncthreads();   // insert_key's own words are rewritten by the next round
         }
     }
 }
@@ -1984,6 +2158,39 @@ int ash_grid_activate_static(ash_map_t* map, const float* cells, int64_t n,
     if (scratch_on_current_device(map->device, &heads)) return 1;
     return launch_activate(map, cells, n, grid_dim, dilation, bidirectional, bound_lo, bound_hi,
                            touched, coords, heads, static_cast<hipStream_t>(stream));
+}
+
+int ash_grid_activate_positions(ash_map_t* map, const float* positions, int64_t n,
+                                const float* origin, float cell_size, int grid_dim,
+                                int dilation, int bidirectional, int bound_lo, int bound_hi,
+                                uint8_t* touched, int32_t* coords, void* stream) {
+    if (check_activate(map, positions, n, grid_dim, dilation, bound_lo, bound_hi, touched,
+                       coords)) {
+        return 1;
+    }
+    if (!(cell_size > 0.f) || !(cell_size < INFINITY)) ASH_FAIL("cell_size must be positive and finite");
+    if (n == 0) return 0;
+    DeviceGuard guard;
+    ASH_HIP(guard.enter(map->device));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (settle_table(map, s)) return 1;
+    counters_changed(map, true, s);
+    RunsArgs a;
+    a.x = positions;
+    a.origin = origin;
+    a.inv_cell = 1.0f / cell_size;
+    a.g = static_cast<float>(grid_dim);
+    a.n = n;
+    a.off_lo = bidirectional ? -dilation : 0;
+    a.width = dilation - a.off_lo + 1;
+    a.bound_lo = bound_lo;
+    a.bound_hi = bound_hi;
+    const int64_t groups = (n + kRunPositions - 1) / kRunPositions;
+    if (groups > 0x7FFFFFFFll) ASH_FAIL("too many positions in one call");
+    activate_runs_kernel<<<static_cast<unsigned>(groups), kHeapBlock, 0, s>>>(
+            map->d, a, touched, coords);
+    ASH_LAUNCH_CHECK();
+    return 0;
 }
 
 int ash_ray_find_near_far(ash_map_t* map, const float* ray_origins,
