@@ -332,8 +332,13 @@ def test_activation_from_world_positions_equals_activation_from_cells(gpu_ash):
     workgroup, no scratch) against ash_grid_activate on torch's
     (x - origin) / cell_size, through the C ABI on two identical maps, call
     after call: same blocks stored, same rows' coordinates flagged, same
-    answers to look-ups.  Batches that end inside a workgroup's 128 positions,
-    every dilation, bounds that cut candidates off, positions in cell units."""
+    answers to look-ups.  Batches that end inside a workgroup's share of the
+    positions, every dilation, bounds that cut candidates off, positions in
+    cell units; positions in no order at all (every workgroup then meets blocks
+    that others are storing at that moment, and has to leave their flags to
+    them) and, before the last batches, an erase of every second block, which
+    leaves tombstones and slots whose index word still names an earlier
+    tenant."""
     lib = common.load_library()
     capacity = 60_000
     plain, direct = RawBlockMap(lib, capacity, DEV), RawBlockMap(lib, capacity, DEV)
@@ -344,11 +349,22 @@ def test_activation_from_world_positions_equals_activation_from_cells(gpu_ash):
         (5_003, 0, 0, None, 1.0, (-1000, 1000)),
         (127, 1, 0, (0.5, 0.5, 0.5), 0.1, (-1000, 1000)),
         (20_000, 1, 1, (-2.0, -2.0, -2.0), 0.02, (0, 11)),
+        (30_000, 1, 1, (4.0, 4.0, 4.0), 0.015, (-1000, 1000)),     # shuffled, new ground
+        (30_000, 1, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),   # shuffled, after the erase
+        (40_001, 1, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),
     )
+    seen = []
     try:
-        for n, dilation, two_sided, origin, cell_size, (lo, hi) in cases:
+        for case, (n, dilation, two_sided, origin, cell_size, (lo, hi)) in enumerate(cases):
             # image-like ordering: neighbouring rows are neighbouring positions
             cells = ((torch.rand(n, 3, generator=g).cumsum(0) * 0.3) % 260.0) - 50.0
+            if case in (5, 6):
+                cells = cells[torch.randperm(n, generator=g)]
+            if case == 6:
+                stored = torch.unique(torch.cat(seen), dim=0)[::2].to(DEV).contiguous()
+                for m in (plain, direct):
+                    assert lib.ash_map_erase(m.handle, stored.data_ptr(), stored.shape[0], m.stream) == 0
+                assert plain.size() == direct.size()
             x = (cells * cell_size + (torch.tensor(origin) if origin else 0.0)).to(DEV).contiguous()
             o = torch.tensor(origin, device=DEV) if origin else None
             cells = ((x - o) / cell_size if origin else x / cell_size).contiguous()
@@ -374,6 +390,7 @@ def test_activation_from_world_positions_equals_activation_from_cells(gpu_ash):
                 assert bool(mask.all()) and torch.equal(idx.cpu(), rows.cpu())
             probe = torch.cat([coords_p[::3] + 1, coords_p[::5]]).to(DEV).contiguous()
             assert torch.equal(plain.find(probe)[1], direct.find(probe)[1])
+            seen.append(coords_p)
     finally:
         plain.close()
         direct.close()

@@ -21,7 +21,7 @@ namespace ash {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kFlaggedGroups = 16384;   // workgroups of the integration that goes by flags
+constexpr int kFlaggedGroups = 8192;    // workgroups of the integration that goes by flags
 
 struct IntegrateArgs {
     float* emb;                // [B, M, E]
