@@ -19,7 +19,8 @@
  *     temporaries are caller-owned buffers (the Python layer hands in torch
  *     tensors, so all device memory stays inside torch's caching allocator);
  *   - launches are asynchronous on `stream`; only `ash_map_status` /
- *     `ash_map_size` (which return host values) synchronise that stream;
+ *     `ash_map_size` / `ash_map_counters` (which return host values)
+ *     synchronise that stream, and are refused while it is being captured;
  *   - a map handle is not thread-safe; operations on one handle must be issued
  *     in order on one stream (as the reference issues them on the null stream);
  *   - calls on a map run on the map's device (ash_map_create's `device`); the

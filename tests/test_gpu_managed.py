@@ -324,6 +324,11 @@ def test_insert_and_find_replay_in_a_hip_graph(gpu_ash, oracle):
                 assert rc == 0, lib.ash_last_error().decode()
                 assert lib.ash_map_find(handle, probe.data_ptr(), n, idx.data_ptr(),
                                         mask.data_ptr(), side.cuda_stream) == 0
+                # a read of the counters would have to wait for the stream: it is
+                # refused, by name, and leaves the capture as it is
+                size = ctypes.c_int64(-1)
+                assert lib.ash_map_size(handle, ctypes.byref(size), side.cuda_stream) != 0
+                assert "being captured" in lib.ash_last_error().decode()
         torch.cuda.synchronize()
         assert engine.size() == omap.size()      # the capture itself inserted nothing
         for replay in range(3):

@@ -2552,6 +2552,9 @@ int refresh_counters(ash_map* map, int32_t* staging, hipStream_t s) {
         map->late_pending = false;
         decode_counters(map->staging, map->counters);
     } else {
+        if (is_capturing(s)) {
+            ASH_FAIL("the table's counters cannot be read while the stream is being captured");
+        }
         int32_t pageable[kHostCounters] = {0};
         int32_t* host = staging != nullptr ? staging : pageable;
         ASH_HIP(hipMemcpyAsync(host, map->d.ctr, sizeof(pageable), hipMemcpyDeviceToHost, s));
