@@ -269,9 +269,6 @@ COLLECT_MAX_BLOCKS = 1 << 20
 # Size of a second region that is attached before any key has asked for it
 # (2^16 slots of 20 bytes).
 GENERAL_JUST_IN_CASE_BYTES = 20 << 16
-# Most positions per call of ash_grid_activate_static (the header's
-# ASH_ACTIVATE_STATIC_MAX_POSITIONS).
-ACTIVATE_STATIC_MAX = 1 << 20
 # Which inserts (and erases) take the streaming path of the library (batch split
 # by bucket range, ranges handled in LDS) instead of the per-key kernel:
 # "auto" = when the library says the batch is large enough relative to the
@@ -1316,16 +1313,15 @@ class _HashMap:
             self._attach_general(just_in_case=True)
         self._upkeep(n)
         coords, rows = self._listing
-        head = (self._handle, cells.data_ptr(), n, int(grid_dim), int(dilation),
-                int(bool(bidirectional)), int(bound_lo), int(bound_hi),
-                self._touched.data_ptr(), self._block_coords.data_ptr())
         with torch.cuda.device(self._device):
-            if n <= ACTIVATE_STATIC_MAX:
-                # run heads in the library's own device array: no allocation
-                self._check(self._lib.ash_grid_activate_static(*head, self._stream()))
-            else:
-                heads = torch.empty(64 + 3 * n, dtype=torch.int32, device=self._device)
-                self._check(self._lib.ash_grid_activate(*head, heads.data_ptr(), self._stream()))
+            # (positions in cell units: no origin, cell size 1; no scratch)
+            self._check(
+                self._lib.ash_grid_activate_positions(
+                    self._handle, cells.data_ptr(), n, None, 1.0, int(grid_dim), int(dilation),
+                    int(bool(bidirectional)), int(bound_lo), int(bound_hi),
+                    self._touched.data_ptr(), self._block_coords.data_ptr(), self._stream(),
+                )
+            )
             self._check(
                 self._lib.ash_grid_collect_touched(
                     self._handle, self._touched.data_ptr(), self._block_coords.data_ptr(),

@@ -106,6 +106,26 @@ def fuse_frame(
                 color, counted_by=table,
             )
             return None
+    if (count_blocks and points.shape[0] > 0 and points.dtype == torch.float32
+            and grid.engine.capacity <= COLLECT_MAX_BLOCKS):
+        # the same launches as without the count (activation, listing on the
+        # device, integration over the listing), and one look at the table's
+        # counters behind them all -- not between activation and integration
+        engine = grid.engine
+        table = engine.backend
+        cells = grid.transform_world_to_cell(points)
+        lo, hi = grid._block_bounds()
+        dropped_before = engine._dropped()
+        grid_coords, grid_indices = table.activate_blocks_deferred(
+            cells, grid.grid_dim, dilation, True, lo, hi
+        )
+        integrate_depth(
+            grid, grid_coords, grid_indices, depth, intrinsic, extrinsic, trunc, depth_max,
+            color, counted_by=table,
+        )
+        touched = table.counters()["touched"]
+        engine._warn_if_overfull(points.shape[0], dropped_before)
+        return int(touched)
     grid_coords, _, grid_indices, _ = grid.spatial_init_(
         points, dilation=dilation, bidirectional=True
     )

@@ -193,14 +193,14 @@ __global__ __launch_bounds__(kBlock) void integrate_depth_flagged_kernel(
         if (threadIdx.x == 0) s_n = 0;
         __syncthreads();
         const int64_t row = first + static_cast<int64_t>(threadIdx.x) * stride;
-        if (row < a.n && row < a.rows) {
+        if (row < a.n) {
             // the coordinates are asked for with the flag, not after it
             const uint8_t flag = touched[row];
             const int32_t cx = a.grid_xyz[row * 3 + 0];
             const int32_t cy = a.grid_xyz[row * 3 + 1];
             const int32_t cz = a.grid_xyz[row * 3 + 2];
-            if (flag != 0) {
-                touched[row] = 0;
+            if (flag != 0) touched[row] = 0;
+            if (flag != 0 && row < a.rows) {   // (a flagged row without embeddings is let go)
                 const int at = atomicAdd(&s_n, 1);
                 s_rows[at * 4 + 0] = static_cast<int32_t>(row);
                 s_rows[at * 4 + 1] = cx;
