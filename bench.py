@@ -514,6 +514,25 @@ def bench_config1(torch, ash, workloads, dev, reps=5):
     }
     out["insert_keys"]["Mkeys_per_s"] = round(n_ins / ms_i / 1e3, 1)
     out["find"]["Mkeys_per_s"] = round(n_q / ms_f / 1e3, 1)
+    # the same insert through the API, HashSet.insert on the cleared set: the
+    # library chooses the path (a table that has not been used since it was
+    # emptied is written whole by the streaming passes, which saves its fill)
+    import ctypes
+    need = ctypes.c_int64(0)
+    assert lib.ash_map_clear(handle, stream) == 0
+    assert lib.ash_map_insert_scratch_bytes(handle, n_ins, 0, None, 0, ctypes.byref(need)) == 0
+    t_api = EventTimer(torch)
+    for it in range(2 + reps):
+        hs.clear()
+        (t_api if it >= 2 else (lambda fn: fn()))(lambda: hs.insert(keys))
+    assert backend.size() == unique
+    out["insert_api"] = {
+        "path": "streaming" if need.value > 0 else "per key",
+        "ms": round(t_api.mean_ms(), 4),
+        "Mkeys_per_s": round(n_ins / t_api.mean_ms() / 1e3, 1),
+        "includes": "all the call queues -- with the table fill a clear leaves behind when the "
+                    "per-key path runs -- and its look at the counters",
+    }
     del hs, w
     return out
 

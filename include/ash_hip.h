@@ -62,8 +62,11 @@ int ash_map_workspace_bytes(int key_dim, int64_t capacity,
  * free list (the `_heap` state-dict buffer, ash/core.py:72-74); the map aliases
  * and mutates it exactly like the reference does.  `table_ws` is a 256-byte
  * aligned device buffer of at least `table_bytes` bytes.  The table is cleared
- * (heap := 0..capacity-1, size := 0) before the call returns control of the
- * stream. */
+ * (heap := 0..capacity-1, size := 0) on `stream`; as after ash_map_clear, the
+ * fill of the bucket array itself runs with the first call that needs it (a
+ * streaming insert writes every bucket anyway and does not), so a new map,
+ * like a cleared one, takes one call outside a graph capture before look-ups
+ * on it can be captured. */
 int ash_map_create(int key_dim, int64_t capacity, int32_t* heap,
                    void* table_ws, int64_t table_bytes, int device,
                    void* stream, ash_map_t** out);

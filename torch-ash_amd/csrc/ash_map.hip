@@ -1957,7 +1957,9 @@ int ash_map_create(int key_dim, int64_t capacity, int32_t* heap, void* table_ws,
     map->d.nb = static_cast<uint32_t>(num_buckets(capacity));
     map->d.gslots = 0;
     map->d.capacity = static_cast<int32_t>(capacity);
-    if (clear_table(map, static_cast<hipStream_t>(stream), true, 0)) {
+    // (the fill of the bucket array is left to the first call that needs it: a
+    // streaming insert, which writes every bucket itself, does not)
+    if (clear_table(map, static_cast<hipStream_t>(stream), true, 0, true)) {
         delete map;
         return 1;
     }
