@@ -166,6 +166,42 @@ def test_two_calls_per_insert_keep_the_table_in_order(gpu_ash, oracle, policy):
         _same(raw, omap, torch.cat([odd, pool[: 4000]]))
 
 
+def test_first_filling_of_a_new_table_streams(gpu_ash, oracle):
+    """A table that has not been used since it was made (or emptied) still has
+    its bucket array to fill: the managed insert then streams from 2^18 keys,
+    where a table in use takes the per-key kernel at this size -- and either
+    way the map is the oracle's.  Duplicates inside the batch included."""
+    rng = np.random.default_rng(31)
+    capacity, n = 700_000, 300_000
+    raw, omap = RawMap(gpu_ash, 3, capacity), _oracle_map(oracle, 3, capacity)
+    nbytes = ctypes.c_int64(-1)
+
+    def wanted(count):
+        raw.check(raw.lib.ash_map_insert_scratch_bytes(raw.handle, count, 0, None, AUTO,
+                                                       ctypes.byref(nbytes)))
+        return nbytes.value
+
+    first = _keys(rng, n, 60)
+    first[1::3] = first[::3][: len(first[1::3])]        # a third of the batch repeats another third
+    probe = torch.cat([first[::7], _keys(rng, 50_000, 90)])
+    assert wanted(n) > 0                                  # new table: the streaming passes
+    assert wanted((1 << 18) - 1) == 0 and wanted(40 * capacity) == 0
+    raw.insert(first)
+    omap.insert_keys(first)
+    _same(raw, omap, probe)
+    assert wanted(n) == 0                                 # a table in use, and small: per key
+    second = _keys(rng, n, 75)
+    raw.insert(second)
+    omap.insert_keys(second)
+    _same(raw, omap, probe)
+    raw.check(raw.lib.ash_map_clear(raw.handle, raw.stream))
+    omap.clear()
+    assert wanted(n) > 0                                  # emptied and not used since: streams again
+    raw.insert(second)
+    omap.insert_keys(second)
+    _same(raw, omap, probe)
+
+
 def test_the_handle_follows_calls_that_go_past_the_managed_entries(gpu_ash):
     """The size the handle reports is the device's whoever made the launches:
     the fine-grained entries invalidate what the handle knows."""
