@@ -120,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "aae38478b511ffab64b0b3bfeba81de7eae9d498caba61c7543ecdcf6901b60d",
+    "csrc_sha256": "f91910e300a75a4367cced2445f69a17d71d5344c661aa7d9c73a2d59e255ede",
 }
 
 
