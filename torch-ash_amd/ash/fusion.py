@@ -4,9 +4,9 @@ the reference's demo (demo/rgbd_fusion.py:200-254) on two fused library calls.
 The reference activates blocks with `spatial_init_` and then updates
 `embeddings[grid_indices, cell_indices]` through torch expressions
 (`project_points_to_rgbd`, demo/rgbd_fusion.py:76-110, and the running weighted
-mean, :232-254).  Here `spatial_init_` runs as one activation kernel pair and
-the projection + update as one kernel that rewrites the embedding rows in
-place.  Row layout as in the demo: channel 0 signed distance, channels 1..3
+mean, :232-254).  Here the activation is one kernel (positions in, blocks
+inserted, their rows flagged) and the projection + update another that rewrites
+the embedding rows of the flagged blocks in place.  Row layout as in the demo: channel 0 signed distance, channels 1..3
 colour (only when a colour image is given), last channel weight.
 """
 from typing import Optional
