@@ -352,13 +352,14 @@ def test_activation_from_world_positions_equals_activation_from_cells(gpu_ash):
         (30_000, 1, 1, (4.0, 4.0, 4.0), 0.015, (-1000, 1000)),     # shuffled, new ground
         (30_000, 1, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),   # shuffled, after the erase
         (40_001, 1, 1, (-1.5, 0.25, 3.0), 0.015, (-1000, 1000)),
+        (12_000, 2, 1, (9.0, 9.0, 9.0), 0.015, (-1000, 1000)),     # shuffled, new ground, 125 each
     )
     seen = []
     try:
         for case, (n, dilation, two_sided, origin, cell_size, (lo, hi)) in enumerate(cases):
             # image-like ordering: neighbouring rows are neighbouring positions
             cells = ((torch.rand(n, 3, generator=g).cumsum(0) * 0.3) % 260.0) - 50.0
-            if case in (5, 6):
+            if case in (5, 6, 8):
                 cells = cells[torch.randperm(n, generator=g)]
             if case == 6:
                 stored = torch.unique(torch.cat(seen), dim=0)[::2].to(DEV).contiguous()
