@@ -120,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "f91910e300a75a4367cced2445f69a17d71d5344c661aa7d9c73a2d59e255ede",
+    "csrc_sha256": "7973acb1862ca153b2368a1171f145c5c3ae9255e3b004d833727e2ee6449821",
 }
 
 

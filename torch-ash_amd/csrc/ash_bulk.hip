@@ -66,6 +66,7 @@ enum { kHdrSpillKeys = 0, kHdrSpillA = 1, kHdrWasEmpty = 3,
        kHdrLosers = 5,    // rows that did not win a slot in the build pass
        kHdrHoles = 6,     // listed holes
        kHdrTaken = 7,     // holes handed to high winners
+       kHdrTicket = 8,    // workgroups of pass 1 that are done
        kHdrWords = 64 };
 
 struct BulkPlan {
@@ -302,7 +303,8 @@ __device__ __forceinline__ void give_up_row(const BulkPlan& pl, int32_t row, int
 // heap in another order the build pass writes it.
 template <int DIM, bool PROV>
 __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
-        MapDev m, BulkPlan pl, const int32_t* __restrict__ keys, int identity) {
+        MapDev m, BulkPlan pl, const int32_t* __restrict__ keys, int identity,
+        int32_t* __restrict__ early) {
     __shared__ SplitShared sh;
     const int tid = threadIdx.x;
     if (tid < kMaxBins) sh.cnt[tid] = 0;
@@ -378,6 +380,21 @@ __global__ __launch_bounds__(kSplitThreads) void split_keys_kernel(
     if constexpr (PROV) {
         __syncthreads();
         if (tid == 0 && sh.losers) atomicAdd(pl.hdr + kHdrLosers, sh.losers);
+    }
+    if (early != nullptr) {
+        // `early`: page-locked host memory.  The workgroup that finishes last
+        // leaves there how many rows this pass has handed to the per-key
+        // kernel, for a host that waits for nothing else of the call.  (Every
+        // update of that count has returned its value to the thread that made
+        // it before the barrier; no fence: one per wavefront would write the
+        // L2 back each time, which multiplied the duration of this pass.)
+        __syncthreads();
+        if (tid == 0 &&
+            atomicAdd(pl.hdr + kHdrTicket, 1) == static_cast<int32_t>(gridDim.x) - 1) {
+            __hip_atomic_store(early, atomicAdd(pl.hdr + kHdrSpillKeys, 0), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
+            __threadfence_system();
+        }
     }
 }
 
@@ -1231,15 +1248,6 @@ __global__ __launch_bounds__(kListThreads) void settle_rows_kernel(
     }
 }
 
-// Leaves one word of the workspace header where the host can read it (`out` is
-// page-locked host memory the device can write to).
-__global__ void publish_word_kernel(const int32_t* __restrict__ word, int32_t* out) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        *out = *word;
-        __threadfence_system();
-    }
-}
-
 int check_values(int n_values, const void* const* src, void* const* dst,
                  const int64_t* row_bytes) {
     if (n_values < 0) ASH_FAIL("negative value count");
@@ -1256,20 +1264,20 @@ int check_values(int n_values, const void* const* src, void* const* dst,
 
 template <bool PROV>
 int launch_split_keys(ash_map* map, const BulkPlan& pl, const int32_t* keys, int identity,
-                      hipStream_t s) {
+                      int32_t* early, hipStream_t s) {
     const unsigned g = static_cast<unsigned>((pl.n + kSplitChunk - 1) / kSplitChunk);
     switch (map->key_dim) {
         case 1:
-            split_keys_kernel<1, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            split_keys_kernel<1, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity, early);
             break;
         case 2:
-            split_keys_kernel<2, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            split_keys_kernel<2, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity, early);
             break;
         case 3:
-            split_keys_kernel<3, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            split_keys_kernel<3, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity, early);
             break;
         default:
-            split_keys_kernel<4, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity);
+            split_keys_kernel<4, PROV><<<g, kSplitThreads, 0, s>>>(map->d, pl, keys, identity, early);
             break;
     }
     ASH_LAUNCH_CHECK();
@@ -1391,15 +1399,13 @@ int ash::insert_bulk(ash_map* map, const int32_t* keys, int64_t n,
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
+    // (pass 1 leaves the early word itself; the event tells the host when)
     auto publish = [&]() -> int {
-        if (early == nullptr) return 0;
-        publish_word_kernel<<<1, 64, 0, s>>>(pl.hdr + kHdrSpillKeys, early);
-        ASH_LAUNCH_CHECK();
-        if (early_event != nullptr) ASH_HIP(hipEventRecord(early_event, s));
+        if (early != nullptr && early_event != nullptr) ASH_HIP(hipEventRecord(early_event, s));
         return 0;
     };
     if (n_values == 0) {
-        if (launch_split_keys<false>(map, pl, keys, identity, s)) return 1;
+        if (launch_split_keys<false>(map, pl, keys, identity, early, s)) return 1;
         if (publish()) return 1;
         split_records_kernel<false><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
         ASH_LAUNCH_CHECK();
@@ -1411,7 +1417,7 @@ int ash::insert_bulk(ash_map* map, const int32_t* keys, int64_t n,
         }
         return insert_selected(map, true, pl.codes_a, pl.spill_a, pl.hdr + kHdrSpillA, none, s);
     }
-    if (launch_split_keys<true>(map, pl, keys, identity, s)) return 1;
+    if (launch_split_keys<true>(map, pl, keys, identity, early, s)) return 1;
     if (publish()) return 1;
     split_records_kernel<true><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
@@ -1476,7 +1482,7 @@ int ash_map_erase_bulk(ash_map_t* map, const int32_t* keys, int64_t n, void* wor
     const int ninit = ncursors > kHdrWords ? ncursors : kHdrWords;
     bulk_init_kernel<<<(ninit + 255) / 256, 256, 0, s>>>(map->d, pl, ncursors);
     ASH_LAUNCH_CHECK();
-    if (launch_split_keys<false>(map, pl, keys, 0, s)) return 1;
+    if (launch_split_keys<false>(map, pl, keys, 0, nullptr, s)) return 1;
     split_records_kernel<false><<<(pl.bins << pl.lane_shift) * pl.chunks, kSplitThreads, 0, s>>>(map->d, pl);
     ASH_LAUNCH_CHECK();
     erase_range_kernel<<<pl.parts, kBuildThreads, 0, s>>>(map->d, pl);
