@@ -120,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "7973acb1862ca153b2368a1171f145c5c3ae9255e3b004d833727e2ee6449821",
+    "csrc_sha256": "7423550822a44250c202da61659f53a81d3722cff450c3ad48ff1de65fa01fa1",
 }
 
 

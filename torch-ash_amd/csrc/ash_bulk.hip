@@ -1340,7 +1340,7 @@ int ash_map_bulk_workspace_bytes(ash_map_t* map, int64_t n, int n_values,
         // every range anyway and saves that fill.  Measured for such tables:
         // the streaming path wins from 2^18 keys and a third of a key per
         // bucket (half with value rows): 1 M keys into a new table of capacity
-        // 2 M take 84 us instead of 144.  Not for batches far beyond what the
+        // 2 M take 77 us instead of 138.  Not for batches far beyond what the
         // table holds (piles of duplicates would queue on a few ranges).
         if (map->table_stale && n >= (int64_t{1} << 18) && n <= 12 * nb &&
             (n_values > 0 ? 2 * n >= nb : 3 * n >= nb)) {
