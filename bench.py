@@ -181,8 +181,8 @@ def bwd2_bytes(e: int) -> int:
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--keys", type=int, default=16_000_000, help="distinct keys (configuration 2)")
     ap.add_argument("--capacity", type=int, default=24_000_000)
     ap.add_argument("--no-trilinear", action="store_true", help="skip the trilinear kernel figures")
