@@ -833,3 +833,41 @@ def test_query_and_find_replay_in_a_hip_graph(gpu_ash, oracle):
         assert torch.allclose(captured[2], eager[2], rtol=1e-5, atol=1e-6)
         assert torch.equal(captured[3], eager[3]) and torch.equal(captured[4], eager[4])
         assert int(eager[4].sum()) > 100 and float(eager[1].abs().sum()) > 1.0
+
+
+def test_module_forward_replays_in_a_hip_graph(gpu_ash):
+    """SparseDenseGrid.forward on world positions is one launch that allocates
+    nothing of its own (ash_grid_forward): captured once under no_grad, every
+    replay equals the eager call on the positions and embeddings of that
+    replay, bit for bit, masks included."""
+    grid = gpu_ash.UnBoundedSparseDenseGrid(3, 400, 4, 4, cell_size=0.25, device=DEV)
+    g = torch.Generator().manual_seed(71)
+    r = torch.arange(-3, 4, dtype=torch.int32)
+    blocks = torch.stack(torch.meshgrid(r, r, r, indexing="ij"), dim=-1).view(-1, 3)
+    grid.engine.insert_keys(blocks[torch.randperm(len(blocks), generator=g)[5:]].to(DEV))
+    grid.construct_grid_neighbor_lut_(radius=1, bidirectional=False)
+    x = torch.zeros(30_000, 3, device=DEV)
+
+    def fill():
+        x.copy_(((torch.rand(x.shape, generator=g) * 9.0 - 4.0)).to(DEV))
+        with torch.no_grad():
+            grid.embeddings.copy_((torch.rand(grid.embeddings.shape, generator=g) * 2 - 1).to(DEV))
+
+    fill()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            grid(x, "smooth_step")                   # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = grid(x, "smooth_step")
+        for _ in range(3):
+            fill()
+            graph.replay()
+            torch.cuda.synchronize()
+            features, masks = grid(x, "smooth_step")
+            torch.cuda.synchronize()
+            assert torch.equal(captured[0], features) and torch.equal(captured[1], masks)
+            assert 1000 < int(masks.sum()) < x.shape[0] and float(features.abs().sum()) > 100.0
