@@ -537,6 +537,51 @@ def bench_config1(torch, ash, workloads, dev, reps=5):
     return out
 
 
+def demo_width_entry(torch, ash, workloads, x, radii, centres, reps, dev):
+    """The queries of configuration 4 on rows of five channels, the width of
+    the reference's demos (distance, colour, weight: demo/rgbd_fusion.py:283,
+    demo/train_scene_recon.py:41): kernel times of the three query functions
+    and the module forward, priced like the other widths."""
+    backend = ash.grid_query.backend
+    torch.cuda.empty_cache()
+    grid, _, _ = workloads.build_grid(ash, 200_000, 5, device=dev)
+    n = x.shape[0]
+    gi, ci, off, mk = grid.query(grid.transform_world_to_cell(x))
+    ops = (grid.embeddings.detach(), off, gi, ci, mk, grid.lut_grid_nb2grid_idx,
+           grid.lut_cell_nb2cell_idx, grid.lut_cell_nb2grid_nb)
+    n_live = int(mk.sum())
+    masked = n - n_live
+    z = torch.rand(n, 5, device=dev) - 0.5
+    u = torch.rand(n, 3, device=dev) - 0.5
+    dense = 4 * grid.embeddings.numel()
+    timers = [EventTimer(torch) for _ in range(4)]
+    for it in range(2 + reps):
+        run = (lambda timer, fn: timer(fn)) if it >= 2 else (lambda timer, fn: fn())
+        run(timers[0], lambda: backend.query_forward(*ops, 8, "smooth_step"))
+        run(timers[1], lambda: backend.query_backward_forward(z, *ops, 8, "smooth_step"))
+        run(timers[2], lambda: backend.query_backward_backward(None, u, z, *ops, 8, "smooth_step"))
+        with torch.no_grad():
+            run(timers[3], lambda: grid(x, "smooth_step"))
+    entry = {
+        "forward": roofline_entry("query_forward_kernel<f32,E5> (one lane per row)",
+                                  fwd_bytes(5) * n_live + (29 + 20) * masked, timers[0].mean_ms()),
+        "backward": roofline_entry("zero16 + query_backward_forward_kernel (E=5)",
+                                   bwd_bytes(5) * n_live + (29 + 12) * masked + dense,
+                                   timers[1].mean_ms()),
+        "double_backward": roofline_entry("zero16 + query_backward_backward_kernel (E=5)",
+                                          bwd2_bytes(5) * n_live + (29 + 20) * masked + dense,
+                                          timers[2].mean_ms()),
+        "module_forward": roofline_entry("grid_forward_kernel<f32,E5>",
+                                         fwd_bytes(5) * n_live + (29 + 20) * masked,
+                                         timers[3].mean_ms()),
+    }
+    for e in entry.values():
+        e["Mqueries_per_s"] = round(n / e["ms"] / 1e3, 1)
+    del grid, ops, z, u
+    torch.cuda.empty_cache()
+    return entry
+
+
 def bench_trilinear(torch, ash, workloads, args, dev):
     """Kernel figures of configurations 3 (E=16 forward) and 4 (E=4 forward,
     backward, double backward) plus the module-level autograd step of
@@ -733,6 +778,7 @@ def bench_trilinear(torch, ash, workloads, args, dev):
         ms = (time.perf_counter() - t0) / reps * 1e3
         out["cfg4_module_train_step" + label] = {
             "ms": round(ms, 3), "Mqueries_per_s": round(n4 / ms / 1e3, 1)}
+    out["cfg4_rows_of_five"] = demo_width_entry(torch, ash, workloads, x, radii, centres, reps, dev)
     if not args.no_cpu:
         # The CPU baseline runs after every section that is timed with the wall
         # clock: its OpenMP workers keep spinning for a while after a parallel

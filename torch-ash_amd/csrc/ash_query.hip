@@ -331,6 +331,25 @@ template <>
 struct VecOf<float, 1> {
     using type = float;
 };
+// Rows of two, three or five fp32 channels taken whole by one lane: a row is
+// only 4-byte aligned in general (rows of 12 or 20 bytes follow each other), which is
+// all a global load of several dwords asks for on this device.
+template <int N>
+struct alignas(4) FloatRow {
+    float v[N];
+};
+template <>
+struct VecOf<float, 2> {
+    using type = FloatRow<2>;
+};
+template <>
+struct VecOf<float, 3> {
+    using type = FloatRow<3>;
+};
+template <>
+struct VecOf<float, 5> {
+    using type = FloatRow<5>;
+};
 template <>
 struct VecOf<double, 1> {
     using type = double;
@@ -373,13 +392,16 @@ __device__ __forceinline__ void forward_rows(const QDev& a, const T* __restrict_
                             static_cast<float>(acc[VEC > 2 ? 2 : 0]), static_cast<float>(acc[VEC > 3 ? 3 : 0])};
             __builtin_nontemporal_store(r4, reinterpret_cast<v4f*>(out + q * a.E + ch0));
         } else {
-            __builtin_nontemporal_store(acc[0], out + q * a.E + ch0);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                __builtin_nontemporal_store(acc[v], out + q * a.E + ch0 + v);
+            }
         }
     }
 }
 
 template <typename T, int VEC, int LPQ, bool LDS>
-__global__ __launch_bounds__(kBlock, LPQ == 1 ? kWavesGather : kWavesWide) void
+__global__ __launch_bounds__(kBlock, (LPQ == 1 && VEC <= 4) ? kWavesGather : kWavesWide) void
 query_forward_kernel(
         QDev a, T* __restrict__ out) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -462,7 +484,7 @@ __device__ __forceinline__ QueryInputs front_inputs(const QDev& a, const FrontDe
 }
 
 template <typename T, int VEC, int LPQ, bool LDS, bool AUX>
-__global__ __launch_bounds__(kBlock, LPQ == 1 ? kWavesGather : kWavesWide) void
+__global__ __launch_bounds__(kBlock, (LPQ == 1 && VEC <= 4) ? kWavesGather : kWavesWide) void
 grid_forward_kernel(QDev a, FrontDev f, T* __restrict__ out) {
     extern __shared__ __align__(16) unsigned char smem[];
     Tile* tile_s = reinterpret_cast<Tile*>(smem);
@@ -2308,6 +2330,23 @@ int dispatch_forward(const QDev& d, void* out, hipStream_t s) {
             }
         }
     }
+    if constexpr (sizeof(T) == 4) {
+        // narrow rows that are not a multiple of four channels: one lane takes
+        // the whole row (six channels: two lanes, three each), instead of one
+        // lane per channel with a power of two of lanes per query
+        switch (d.E) {
+            case 2:
+                return launch_forward<float, 2, 1>(d, out, s);
+            case 3:
+                return launch_forward<float, 3, 1>(d, out, s);
+            case 5:
+                return launch_forward<float, 5, 1>(d, out, s);
+            case 6:
+                return launch_forward<float, 3, 2>(d, out, s);
+            default:
+                break;
+        }
+    }
     switch (pow2_ceil(d.E)) {
         case 1:
             return launch_forward<T, 1, 1>(d, out, s);
@@ -2336,6 +2375,23 @@ int dispatch_grid_forward(const QDev& d, const FrontDev& f, void* out, hipStream
                 default:
                     return launch_grid_forward<float, 4, 4>(d, f, out, s);
             }
+        }
+    }
+    if constexpr (sizeof(T) == 4) {
+        // narrow rows that are not a multiple of four channels: one lane takes
+        // the whole row (six channels: two lanes, three each), instead of one
+        // lane per channel with a power of two of lanes per query
+        switch (d.E) {
+            case 2:
+                return launch_grid_forward<float, 2, 1>(d, f, out, s);
+            case 3:
+                return launch_grid_forward<float, 3, 1>(d, f, out, s);
+            case 5:
+                return launch_grid_forward<float, 5, 1>(d, f, out, s);
+            case 6:
+                return launch_grid_forward<float, 3, 2>(d, f, out, s);
+            default:
+                break;
         }
     }
     switch (pow2_ceil(d.E)) {
