@@ -120,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "7423550822a44250c202da61659f53a81d3722cff450c3ad48ff1de65fa01fa1",
+    "csrc_sha256": "77d2cdf9c3eb9e196afa1a80d0c5e871a2f8fb2ed516975009fa10c025921e73",
 }
 
 
