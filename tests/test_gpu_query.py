@@ -96,7 +96,7 @@ def _compare_all(ash, oracle, grid, x, interpolation, seed=0):
 
 
 @pytest.mark.parametrize("interpolation", ["linear", "smooth_step"])
-@pytest.mark.parametrize("embedding_dim", [1, 2, 3, 4, 5, 8, 12, 16])
+@pytest.mark.parametrize("embedding_dim", [1, 2, 3, 4, 5, 6, 7, 8, 12, 16])
 def test_all_embedding_dims_fp32(gpu_ash, oracle, interpolation, embedding_dim):
     grid = _make_grid(gpu_ash, 4, embedding_dim, 1, seed=embedding_dim, holes=3)
     x = _queries(4, 1, 6000, seed=100 + embedding_dim, margin=2.0)
