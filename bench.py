@@ -120,33 +120,35 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "77d2cdf9c3eb9e196afa1a80d0c5e871a2f8fb2ed516975009fa10c025921e73",
+    "csrc_sha256": "062abb5f4f7c92c05127c09a1bd3aa03abe4543dfbf1671920a06bcc3cef42c0",
 }
 
 
 def csrc_fingerprint() -> str:
-    """SHA-256 over the kernel sources of libash_hip.so (names and contents)."""
-    import hashlib
+    """SHA-256 over the kernel sources of libash_hip.so (names and contents),
+    as the build computes it and compiles it into the library."""
+    import importlib.util
 
-    csrc = os.path.join(ROOT, "torch-ash_amd", "csrc")
-    h = hashlib.sha256()
-    for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h")):
-            h.update(name.encode())
-            with open(os.path.join(csrc, name), "rb") as f:
-                h.update(f.read())
-    return h.hexdigest()
+    spec = importlib.util.spec_from_file_location(
+        "ash_build", os.path.join(ROOT, "torch-ash_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    return build.source_fingerprint()
 
 
-def attach_counters(kernels, default_sizes: bool):
+def attach_counters(kernels, default_sizes: bool, library: str):
     """Adds the separately collected counter figures to the kernel entries when
-    they describe this run; returns what the JSON line says about them."""
+    they describe this run; returns what the JSON line says about them.
+    `library`: the fingerprint compiled into the library that ran."""
     current = csrc_fingerprint()
-    note = dict(COUNTERS_SOURCE, measured_in_this_run=False, csrc_sha256_of_this_run=current)
-    note["attached"] = bool(default_sizes and current == COUNTERS_SOURCE["csrc_sha256"])
+    note = dict(COUNTERS_SOURCE, measured_in_this_run=False, csrc_sha256_of_this_run=current,
+                csrc_sha256_of_the_library=library)
+    note["attached"] = bool(default_sizes and library == current == COUNTERS_SOURCE["csrc_sha256"])
     if not note["attached"]:
-        note["why_not"] = ("other sizes than the counters were collected at" if not default_sizes
-                           else "the kernel sources changed since the counters were collected")
+        note["why_not"] = (
+            "other sizes than the counters were collected at" if not default_sizes
+            else "the library was not built from the kernel sources beside it" if library != current
+            else "the kernel sources changed since the counters were collected")
         return note
     for name, (traffic, hit_rate, atomics) in MEASURED_COUNTERS.items():
         entry = kernels.get(name)
@@ -1009,7 +1011,8 @@ def main():
     if not args.no_fusion:
         kernels["cfg5_fusion"] = bench_fusion(torch, ash, workloads, args, dev)
     counters_note = attach_counters(
-        kernels, args.keys == 16_000_000 and args.capacity == 24_000_000)
+        kernels, args.keys == 16_000_000 and args.capacity == 24_000_000,
+        ash.common.load_library().ash_source_fingerprint().decode())
     dominant = max((kernels["api_insert_path"], "find", "items"), key=lambda k: kernels[k]["ms"])
     roof = dict(kernels[dominant])
     table_bytes = (args.capacity + 5) // 6 * 128

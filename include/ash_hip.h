@@ -46,6 +46,12 @@ const char* ash_last_error(void);
 /* ABI version, bumped on incompatible changes. */
 int ash_abi_version(void);
 
+/* SHA-256 (hex) over the kernel sources this library was built from, as the
+ * build computes it (names and contents of the .hip and .h files under
+ * csrc/), or "unknown".  For benchmarks and tests to tell a library that does
+ * not belong to the sources beside it.  No counterpart in the reference. */
+const char* ash_source_fingerprint(void);
+
 /* ------------------------------------------------------------------ hash map */
 
 /* Storage needed for a table of `capacity` entries with `key_dim` int32 key

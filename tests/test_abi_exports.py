@@ -38,6 +38,19 @@ def test_abi_version(lib):
     assert lib.ash_abi_version() == 1
 
 
+def test_library_is_built_from_the_sources_beside_it(lib):
+    """The build compiles a fingerprint of the kernel sources into the library:
+    a library left over from other sources (an edit without a rebuild) fails
+    here instead of being measured or tested in their name."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location(
+        "ash_build", os.path.join(ROOT, "torch-ash_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    assert lib.ash_source_fingerprint().decode() == build.source_fingerprint()
+
+
 def _error(lib):
     return lib.ash_last_error().decode()
 

@@ -56,6 +56,7 @@ class _QueryArgs(ctypes.Structure):
 _SIGNATURES = {
     "ash_last_error": (ctypes.c_char_p, []),
     "ash_abi_version": (ctypes.c_int, []),
+    "ash_source_fingerprint": (ctypes.c_char_p, []),
     "ash_map_workspace_bytes": (
         ctypes.c_int,
         [ctypes.c_int, _I64, ctypes.POINTER(_I64), ctypes.POINTER(_I64)],

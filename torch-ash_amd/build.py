@@ -49,6 +49,22 @@ def compile_flags():
     ]
 
 
+def source_fingerprint() -> str:
+    """SHA-256 over the kernel sources (names and contents of csrc/*.hip and
+    csrc/*.h).  It is compiled into the library (ash_source_fingerprint), so
+    that a benchmark or a test can tell a library that was not built from the
+    sources beside it."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
 def is_stale() -> bool:
     if not os.path.exists(OUT):
         return True
@@ -62,11 +78,14 @@ def build(force: bool = False, verbose: bool = True) -> str:
         return OUT
     os.makedirs(OUT_DIR, exist_ok=True)
     hipcc = hipcc_path()
+    stamp = f'-DASH_SOURCE_FINGERPRINT="{source_fingerprint()}"'
     objs = []
     procs = []
     for src in SOURCES:
         obj = os.path.join(OUT_DIR, src.replace(".hip", ".o"))
         cmd = [hipcc, *compile_flags(), "-c", os.path.join(CSRC, src), "-o", obj]
+        if src == "ash_map.hip":
+            cmd.insert(1, stamp)
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd)))

@@ -1904,6 +1904,13 @@ const char* ash_last_error(void) { return g_last_error.c_str(); }
 
 int ash_abi_version(void) { return 1; }
 
+// The build passes the fingerprint of the kernel sources it compiles
+// (torch-ash_amd/build.py: source_fingerprint).
+#ifndef ASH_SOURCE_FINGERPRINT
+#define ASH_SOURCE_FINGERPRINT "unknown"
+#endif
+const char* ash_source_fingerprint(void) { return ASH_SOURCE_FINGERPRINT; }
+
 int ash_map_workspace_bytes(int key_dim, int64_t capacity, int64_t* table_bytes,
                             int64_t* general_bytes) {
     if (key_dim < 1 || key_dim > 4) ASH_FAIL("key_dim must be in 1..4");
