@@ -113,10 +113,34 @@ __device__ __forceinline__ float2 folded(const float2 old, const CellObservation
     return out;
 }
 
+// The same for a row of distance, colour and weight (five channels, 20 bytes,
+// 4-byte aligned: moved as 16 + 4 bytes); without a colour image the three
+// colour channels keep what they hold.
+struct alignas(4) Row5 {
+    float v[5];
+};
+
+__device__ __forceinline__ Row5 folded(const Row5& old, const CellObservation& o, bool colour) {
+    const float w_sum = old.v[4];
+    const float w_new = __fadd_rn(w_sum, o.weight);
+    const float denom = __fadd_rn(w_new, 1e-6f);
+    Row5 out = old;
+    out.v[0] = __fdiv_rn(__fadd_rn(__fmul_rn(old.v[0], w_sum), __fmul_rn(o.sdf, o.weight)), denom);
+    if (colour) {
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+            out.v[1 + q] = __fdiv_rn(
+                    __fadd_rn(__fmul_rn(old.v[1 + q], w_sum), __fmul_rn(o.rgb[q], o.weight)), denom);
+        }
+    }
+    out.v[4] = w_new;
+    return out;
+}
+
 // The update of cell `cell` of the block stored in row `row` of the
 // embeddings, whose block coordinates are bx, by, bz.  E: channels per row
-// when known at compile time (2: one 8-byte access per row), else 0 and a.e is
-// used.  Either way the arithmetic of the update is the same sequence of fp32
+// when known at compile time (2: one 8-byte access per row; 5: 16 + 4 bytes),
+// else 0 and a.e is used.  Either way the arithmetic of the update is the same sequence of fp32
 // operations.
 template <int G, int E>
 __device__ __forceinline__ void integrate_cell_at(const IntegrateArgs& a, int64_t row, int cell,
@@ -127,6 +151,9 @@ __device__ __forceinline__ void integrate_cell_at(const IntegrateArgs& a, int64_
     if constexpr (E == 2) {
         float2* e2 = reinterpret_cast<float2*>(e);
         *e2 = folded(*e2, o);
+    } else if constexpr (E == 5) {
+        Row5* e5 = reinterpret_cast<Row5*>(e);
+        *e5 = folded(*e5, o, a.color != nullptr);
     } else {
         const float w_sum = e[ne - 1];
         const float w_new = __fadd_rn(w_sum, o.weight);
@@ -229,6 +256,19 @@ __global__ __launch_bounds__(kBlock) void integrate_depth_flagged_kernel(
                     rows[cell] = folded(old0, o0);
                     if (two) rows[other] = folded(old1, o1);
                 }
+            } else if constexpr (E == 5) {
+                Row5* rows = reinterpret_cast<Row5*>(a.emb) + static_cast<int64_t>(r) * m;
+                const bool colour = a.color != nullptr;
+                for (int cell = threadIdx.x; cell < m; cell += 2 * kBlock) {
+                    const int other = cell + kBlock;
+                    const bool two = other < m;
+                    const Row5 old0 = rows[cell];
+                    const Row5 old1 = rows[two ? other : cell];
+                    const CellObservation o0 = observe_cell<G>(a, cell, bx, by, bz);
+                    const CellObservation o1 = observe_cell<G>(a, two ? other : cell, bx, by, bz);
+                    rows[cell] = folded(old0, o0, colour);
+                    if (two) rows[other] = folded(old1, o1, colour);
+                }
             } else {
                 for (int cell = threadIdx.x; cell < m; cell += kBlock) {
                     integrate_cell_at<G, E>(a, r, cell, bx, by, bz);
@@ -310,6 +350,10 @@ extern "C" int ash_grid_integrate_depth_touched(
         integrate_depth_counted_kernel<8, 2><<<static_cast<unsigned>(blocks), kBlock, 0,
                                                static_cast<hipStream_t>(stream)>>>(
                 a, map->d.ctr + kCtrTouched);
+    } else if (a.g == 8 && a.e == 5) {
+        integrate_depth_counted_kernel<8, 5><<<static_cast<unsigned>(blocks), kBlock, 0,
+                                               static_cast<hipStream_t>(stream)>>>(
+                a, map->d.ctr + kCtrTouched);
     } else {
         integrate_depth_counted_kernel<0, 0><<<static_cast<unsigned>(blocks), kBlock, 0,
                                                static_cast<hipStream_t>(stream)>>>(
@@ -346,6 +390,9 @@ extern "C" int ash_grid_integrate_depth_flagged(
     if (a.g == 8 && a.e == 2) {
         integrate_depth_flagged_kernel<8, 2><<<static_cast<unsigned>(groups), kBlock, 0,
                                                static_cast<hipStream_t>(stream)>>>(a, touched);
+    } else if (a.g == 8 && a.e == 5) {
+        integrate_depth_flagged_kernel<8, 5><<<static_cast<unsigned>(groups), kBlock, 0,
+                                               static_cast<hipStream_t>(stream)>>>(a, touched);
     } else {
         integrate_depth_flagged_kernel<0, 0><<<static_cast<unsigned>(groups), kBlock, 0,
                                                static_cast<hipStream_t>(stream)>>>(a, touched);
@@ -375,6 +422,9 @@ extern "C" int ash_grid_integrate_depth(
     if (blocks > 0x7FFFFFFFll) ASH_FAIL("too many cells in one call");
     if (a.g == 8 && a.e == 2) {
         integrate_depth_kernel<8, 2><<<static_cast<unsigned>(blocks), kBlock, 0,
+                                       static_cast<hipStream_t>(stream)>>>(a);
+    } else if (a.g == 8 && a.e == 5) {
+        integrate_depth_kernel<8, 5><<<static_cast<unsigned>(blocks), kBlock, 0,
                                        static_cast<hipStream_t>(stream)>>>(a);
     } else {
         integrate_depth_kernel<0, 0><<<static_cast<unsigned>(blocks), kBlock, 0,
