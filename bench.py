@@ -120,7 +120,7 @@ MEASURED_COUNTERS = {
 COUNTERS_SOURCE = {
     "profiles": ["profiles/bench_hbm_traffic_pmc.md",
                  "profiles/bench_l2_hit_rate_and_atomics_pmc.md"],
-    "csrc_sha256": "062abb5f4f7c92c05127c09a1bd3aa03abe4543dfbf1671920a06bcc3cef42c0",
+    "csrc_sha256": "c6faef7718351d8d76b6af8431f0d453eaf253c59e8058507d7d4a72540cd714",
 }
 
 
